@@ -1,0 +1,278 @@
+/*
+ * puppygrad_hip.h — C ABI of libpuppygrad_hip.so, the MI355X (gfx950) GPT-2
+ * inference backend for puppygrad.
+ *
+ * Each entry point names the puppygrad interface it stands in for (paths are
+ * relative to the puppygrad source tree, `src/...:line`).  All functions return
+ * a pg_status; on failure pg_last_error_message() holds a message whose wording
+ * follows the reference's Gpt2Error strings.  Nothing throws or aborts across
+ * this boundary.  All pointers are plain host pointers unless stated.
+ *
+ * Threading: a pg_gpt2_model is immutable after creation and may be shared by
+ * threads that use distinct caches (the reference takes `&self`,
+ * src/models/gpt2/rust.rs:906-941).  A pg_kv_cache owns its activation scratch,
+ * its logits buffer and its HIP stream, and is single-threaded (`&mut cache`).
+ */
+#ifndef PUPPYGRAD_HIP_H
+#define PUPPYGRAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Gpt2Error variants (src/models/gpt2/error.rs:4-10) plus PG_BACKEND for a HIP
+ * runtime failure, which the Rust adapter maps to Gpt2Error::Asset. */
+typedef enum pg_status {
+  PG_OK = 0,
+  PG_ASSET = 1,
+  PG_INVALID_CONFIG = 2,
+  PG_INVALID_INPUT = 3,
+  PG_INVALID_WEIGHTS = 4,
+  PG_BACKEND = 5
+} pg_status;
+
+/* Thread-local message of the last failing call on this thread. */
+const char* pg_last_error_message(void);
+
+/* Gpt2Config (src/models/gpt2/rust.rs:30-39). */
+typedef struct pg_gpt2_config {
+  uint64_t vocab_size;
+  uint64_t n_positions;
+  uint64_t n_embd;
+  uint64_t n_layer;
+  uint64_t n_head;
+  uint64_t n_inner;
+  float layer_norm_epsilon;
+} pg_gpt2_config;
+
+/* A flat f32 host tensor; len counts elements. */
+typedef struct pg_tensor {
+  const float* data;
+  uint64_t len;
+} pg_tensor;
+
+/* Gpt2BlockWeights (src/models/gpt2/rust.rs:111-125).  Matrices are in the HF
+ * Conv1D [in,out] layout, exactly as Gpt2Model::new receives them
+ * (src/models/gpt2/rust.rs:724-760, 799-825). */
+typedef struct pg_gpt2_block_view {
+  pg_tensor ln_1_g, ln_1_b;
+  pg_tensor c_attn_w, c_attn_b;
+  pg_tensor c_proj_w, c_proj_b;
+  pg_tensor ln_2_g, ln_2_b;
+  pg_tensor c_fc_w, c_fc_b;
+  pg_tensor c_proj_mlp_w, c_proj_mlp_b;
+} pg_gpt2_block_view;
+
+/* Gpt2Weights (src/models/gpt2/rust.rs:102-109). */
+typedef struct pg_gpt2_weights_view {
+  pg_tensor wte, wpe, ln_f_g, ln_f_b;
+  const pg_gpt2_block_view* blocks;
+  uint64_t n_blocks;
+} pg_gpt2_weights_view;
+
+/* Stands where Gpt2RustConfig does in Gpt2BackendConfig::Rust(..)
+ * (src/models/gpt2/options.rs:15-18, 54-96): the per-backend knobs. */
+typedef enum pg_weight_storage { PG_STORE_F32 = 0, PG_STORE_BF16 = 1 } pg_weight_storage;
+typedef enum pg_decode_path {
+  PG_DECODE_AUTO = 0,       /* persistent kernel when the device can co-schedule it */
+  PG_DECODE_KERNELS = 1,    /* one launch per fused op */
+  PG_DECODE_PERSISTENT = 2  /* one launch per token */
+} pg_decode_path;
+typedef struct pg_hip_options {
+  int32_t device;          /* HIP device ordinal */
+  uint32_t weight_storage; /* pg_weight_storage: how the dense matrices and wte are kept in HBM */
+  uint32_t decode_path;    /* pg_decode_path */
+  uint32_t reserved;
+} pg_hip_options;
+
+typedef struct pg_gpt2_model pg_gpt2_model;
+typedef struct pg_kv_cache pg_kv_cache;
+typedef struct pg_logits pg_logits;
+
+/* Gpt2Model::new_with_rust_config (src/models/gpt2/rust.rs:803-825): validates
+ * config (rust.rs:60-95) and weight lengths (rust.rs:1279-1343), uploads every
+ * tensor once and stores the dense matrices as [out,in] (rust.rs:1345-1352).
+ * The caller keeps its host buffers.  options may be NULL for defaults. */
+pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_view* weights,
+                         const pg_hip_options* options, pg_gpt2_model** out);
+void pg_gpt2_destroy(pg_gpt2_model* model);
+/* Gpt2Model.config (src/models/gpt2/rust.rs:143). */
+pg_status pg_gpt2_get_config(const pg_gpt2_model* model, pg_gpt2_config* out);
+/* Gpt2BackendConfig::describe (src/models/gpt2/options.rs:37-51). */
+pg_status pg_gpt2_describe(const pg_gpt2_model* model, char* dst, size_t cap);
+
+/* Gpt2Model::new_kv_cache / Gpt2KvCache::new (src/models/gpt2/rust.rs:902-904,
+ * 186-200): K and V are [layer][batch][head][position][head_dim] f32 in HBM,
+ * zero-filled at full n_positions.  batch = 1 is the reference's cache. */
+pg_status pg_kv_cache_create(const pg_gpt2_model* model, uint32_t batch, pg_kv_cache** out);
+void pg_kv_cache_destroy(pg_kv_cache* cache);
+/* KvCache trait (src/models/autoregressive.rs:1-7). */
+pg_status pg_kv_cache_clear(pg_kv_cache* cache);
+uint64_t pg_kv_cache_seq_len(const pg_kv_cache* cache);
+uint64_t pg_kv_cache_max_seq_len(const pg_kv_cache* cache);
+uint32_t pg_kv_cache_batch(const pg_kv_cache* cache);
+/* The reference's `pub seq_len` field (src/models/gpt2/rust.rs:180); n must not
+ * exceed max_seq_len.  Used to rewind a prefilled cache. */
+pg_status pg_kv_cache_set_seq_len(pg_kv_cache* cache, uint64_t n);
+/* Copies one layer's K (which=0) or V (which=1) panel of sequence `b` to host:
+ * [head][position][head_dim], the layout of Gpt2LayerKvCache
+ * (src/models/gpt2/rust.rs:251-266, kv_index at 1851-1855). */
+pg_status pg_kv_cache_read_layer(const pg_kv_cache* cache, uint32_t b, uint32_t layer,
+                                 uint32_t which, float* dst, size_t len);
+
+/* AutoregressiveDecoder::prefill / Gpt2Model::prefill
+ * (src/models/autoregressive.rs:18-22, src/models/gpt2/rust.rs:906-927):
+ * validates ids (rust.rs:1029-1051), clears the cache, runs the prompt and
+ * returns the logits of the last position.  The cache must have batch 1.  The
+ * returned handle is owned by the cache and stays valid until the next call
+ * that takes this cache. */
+pg_status pg_gpt2_prefill(const pg_gpt2_model* model, pg_kv_cache* cache, const uint32_t* ids,
+                          size_t n, pg_logits** out);
+/* AutoregressiveDecoder::forward_one / Gpt2Model::forward_one
+ * (src/models/autoregressive.rs:24-28, src/models/gpt2/rust.rs:929-1006). */
+pg_status pg_gpt2_forward_one(const pg_gpt2_model* model, pg_kv_cache* cache, uint32_t id,
+                              pg_logits** out);
+/* Gpt2Model::forward (src/models/gpt2/rust.rs:831-882): logits for all n
+ * positions, written to host memory `dst` as [n][vocab_size]. */
+pg_status pg_gpt2_forward(const pg_gpt2_model* model, const uint32_t* ids, size_t n, float* dst,
+                          size_t dst_len);
+
+/* Batched forms: `ids` is [batch][n] (prefill) or [batch] (forward_one); every
+ * sequence of the cache advances together and the logits handle has `batch`
+ * rows.  No reference counterpart beyond running the calls above per sequence. */
+pg_status pg_gpt2_prefill_batch(const pg_gpt2_model* model, pg_kv_cache* cache,
+                                const uint32_t* ids, size_t n, pg_logits** out);
+pg_status pg_gpt2_forward_one_batch(const pg_gpt2_model* model, pg_kv_cache* cache,
+                                    const uint32_t* ids, pg_logits** out);
+
+/* The associated type `Logits` of AutoregressiveDecoder
+ * (src/models/autoregressive.rs:11): a device-resident [rows][vocab] f32 buffer. */
+uint32_t pg_logits_rows(const pg_logits* logits);
+uint64_t pg_logits_vocab(const pg_logits* logits);
+/* argmax_logits (src/models/generation.rs:269-279) on the device: strict '>'
+ * from -inf, lowest index wins ties, NaN never wins, no finite/inf winner -> 0.
+ * out receives one id per row. */
+pg_status pg_logits_argmax(pg_logits* logits, uint32_t* out);
+/* Legacy Vec<f32> view (src/models/gpt2/rust.rs:1005): copies [rows][vocab]. */
+pg_status pg_logits_copy_to_host(pg_logits* logits, float* dst, size_t len);
+
+/* TextGenerationConfig sampling fields (src/models/generation.rs:61-71). */
+typedef struct pg_sampling {
+  float temperature;
+  int32_t has_top_p;
+  float top_p;
+  int32_t has_top_k;
+  uint64_t top_k;
+  float repeat_penalty;
+  uint64_t repeat_last_n;
+} pg_sampling;
+/* TextGenerationConfig::validate (src/models/generation.rs:91-117), messages
+ * prefixed "generation " as Gpt2GenerationConfig::validate does
+ * (src/models/gpt2/options.rs:176-180). */
+pg_status pg_sampling_validate(const pg_sampling* sampling);
+/* SmallRng (src/models/generation.rs:244-267): the state after
+ * LogitsSampler::new(seed). */
+typedef struct pg_rng_state {
+  uint64_t state;
+} pg_rng_state;
+void pg_rng_seed(pg_rng_state* rng, uint64_t seed);
+uint64_t pg_rng_next_u64(pg_rng_state* rng);
+double pg_rng_next_unit_f64(pg_rng_state* rng);
+/* LogitsSampler::select_next_token (src/models/generation.rs:221-241) on row
+ * `row` of the logits: repeat penalty over the last repeat_last_n history ids,
+ * argmax when temperature <= 0, otherwise top-k / top-p / inverse-CDF sampling
+ * (generation.rs:281-362). */
+pg_status pg_logits_sample(pg_logits* logits, uint32_t row, const uint32_t* history, size_t n_hist,
+                           const pg_sampling* sampling, pg_rng_state* rng, uint32_t* out);
+
+/* GenerationStats (src/models/generation.rs:129-138) and the f32-path buckets of
+ * Gpt2OperationProfile (src/models/gpt2/rust.rs:336-347), in seconds.  gpu_decode_s
+ * is the decode span measured with HIP events on the cache's stream. */
+typedef struct pg_generation_stats {
+  uint64_t prompt_tokens;
+  uint64_t generated_tokens;
+  double prefill_s;
+  double decode_s;
+  double first_token_s;
+  double gpu_decode_s;
+} pg_generation_stats;
+
+/* The greedy loop of autoregressive::generate (src/models/autoregressive.rs:61-87)
+ * with the token kept on the device between steps: starting from the logits the
+ * cache currently holds (after prefill or forward_one), selects up to max_new
+ * tokens by argmax, running forward_one after each except the last
+ * (src/models/gpt2/rust.rs:518-528), stopping at n_positions
+ * (rust.rs:496-498) and, if eos >= 0, before emitting eos (rust.rs:503-505).
+ * out_ids must hold max_new entries.  stats may be NULL. */
+pg_status pg_gpt2_decode_greedy(const pg_gpt2_model* model, pg_kv_cache* cache, uint32_t max_new,
+                                int64_t eos, uint32_t* out_ids, uint32_t* out_n,
+                                pg_generation_stats* stats);
+/* Batched greedy decode: `batch` sequences step together for exactly `steps`
+ * tokens (no EOS); out_ids is [steps][batch]. */
+pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* model, pg_kv_cache* cache,
+                                      uint32_t steps, uint32_t* out_ids,
+                                      pg_generation_stats* stats);
+
+/* Gpt2Runtime::stream_token_ids_with_stats with the tokenizer bypassed
+ * (src/models/gpt2/rust.rs:548-634): prefill, then select / EOS-check / push /
+ * on_token / forward_one until max_new_tokens, n_positions or EOS.  on_token may
+ * be NULL; a non-zero return from it stops generation and is reported as
+ * PG_INVALID_INPUT.  out_ids must hold n + max_new entries and receives prompt
+ * plus generated ids. */
+typedef int (*pg_on_token)(uint32_t token_id, void* user);
+pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* model, const uint32_t* ids,
+                                              size_t n, uint32_t max_new, int64_t eos,
+                                              const pg_sampling* sampling, uint64_t seed,
+                                              pg_on_token on_token, void* user, uint32_t* out_ids,
+                                              size_t* out_n, pg_generation_stats* stats);
+
+/* Op-level entry points with the semantics of src/models/cpu.rs; operands are
+ * host pointers, the work runs on `device`.  They exist for kernel parity tests
+ * and as the seam for other models that share these kernels. */
+/* transposed_dense_projection_into (cpu.rs:58-75): weight is [out,in]. */
+pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in_features,
+                      uint64_t out_features, const float* weight, const float* bias, float* out);
+/* layer_norm_in_place (cpu.rs:119-143). */
+pg_status pg_op_layer_norm(int32_t device, float* x, uint64_t rows, uint64_t cols,
+                           const float* gamma, const float* beta, float eps);
+/* gelu_in_place (cpu.rs:145-150). */
+pg_status pg_op_gelu(int32_t device, float* values, uint64_t n);
+/* softmax_in_place (cpu.rs:152-165) applied to each of `rows` rows of `cols`. */
+pg_status pg_op_softmax(int32_t device, float* values, uint64_t rows, uint64_t cols);
+/* add_in_place (cpu.rs:167-171). */
+pg_status pg_op_add(int32_t device, float* dst, const float* src, uint64_t n);
+/* cached_self_attention_into (src/models/gpt2/rust.rs:1662-1741): writes this
+ * token's K and V at `pos` into keys/values ([head][max_seq_len][head_dim], host,
+ * updated in place) and returns the attention output for the C-float query. */
+pg_status pg_op_attention_decode(int32_t device, const float* qkv, uint64_t pos, float* keys,
+                                 float* values, uint64_t max_seq_len, uint64_t n_head,
+                                 uint64_t head_dim, float* out);
+/* argmax_logits (src/models/generation.rs:269-279) on a host vector. */
+pg_status pg_op_argmax(int32_t device, const float* values, uint64_t n, uint32_t* out);
+
+/* Seeded synthetic inputs for benchmarks and tests (no reference counterpart;
+ * the draw is the reference's splitmix64, src/models/generation.rs:244-267).
+ * Element i of the stream uses draws 2i and 2i+1 of SmallRng::new(seed):
+ * u1 = ((d0>>11)+1)/2^53, u2 = (d1>>11)/2^53, z = sqrt(-2 ln u1) cos(2 pi u2),
+ * value = (float)(z * std).  `first` is the stream index of dst[0]. */
+void pg_synth_normal_f32(float* dst, uint64_t n, uint64_t seed, uint64_t first, double std);
+/* ids[i] = next_u64() % vocab from SmallRng::new(seed). */
+void pg_synth_token_ids(uint32_t* dst, uint64_t n, uint64_t seed, uint64_t vocab);
+
+/* Device facts for the benchmark harness. */
+typedef struct pg_device_info {
+  char name[128];
+  char arch[64];
+  uint32_t compute_units;
+  uint64_t total_mem_bytes;
+  uint32_t lds_bytes_per_block;
+} pg_device_info;
+pg_status pg_device_query(int32_t device, pg_device_info* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PUPPYGRAD_HIP_H */

@@ -1,0 +1,377 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes wrapper of the CPU oracle (oracle/pg_oracle.cpp).
+
+The oracle restates puppygrad's CPU GPT-2 path (see the header of pg_oracle.cpp
+for the reference file:line of every function and for how each part is pinned).
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import this
+package; nothing under puppygrad_amd/ does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+from typing import Optional, Sequence
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent
+LIB_PATH = ORACLE_DIR / "libpg_oracle.so"
+
+_f32p = C.POINTER(C.c_float)
+_u32p = C.POINTER(C.c_uint32)
+
+
+class OracleError(Exception):
+    def __init__(self, status: int, msg: str):
+        super().__init__(msg)
+        self.status = status
+        self.msg = msg
+
+
+class orc_config(C.Structure):
+    _fields_ = [("vocab_size", C.c_uint64), ("n_positions", C.c_uint64), ("n_embd", C.c_uint64),
+                ("n_layer", C.c_uint64), ("n_head", C.c_uint64), ("n_inner", C.c_uint64),
+                ("layer_norm_epsilon", C.c_float)]
+
+
+class orc_tensor(C.Structure):
+    _fields_ = [("data", _f32p), ("len", C.c_uint64)]
+
+
+BLOCK_FIELDS = ["ln_1_g", "ln_1_b", "c_attn_w", "c_attn_b", "c_proj_w", "c_proj_b", "ln_2_g",
+                "ln_2_b", "c_fc_w", "c_fc_b", "c_proj_mlp_w", "c_proj_mlp_b"]
+
+
+class orc_block_view(C.Structure):
+    _fields_ = [(n, orc_tensor) for n in BLOCK_FIELDS]
+
+
+class orc_weights_view(C.Structure):
+    _fields_ = [("wte", orc_tensor), ("wpe", orc_tensor), ("ln_f_g", orc_tensor),
+                ("ln_f_b", orc_tensor), ("blocks", C.POINTER(orc_block_view)),
+                ("n_blocks", C.c_uint64)]
+
+
+class orc_rust_config(C.Structure):
+    """Gpt2RustConfig (src/models/gpt2/options.rs:54-96)."""
+    _fields_ = [("threads", C.c_uint64), ("dense_parallel_threshold", C.c_uint64),
+                ("qkv_chunk_size", C.c_uint64), ("attention_projection_chunk_size", C.c_uint64),
+                ("mlp_fc_chunk_size", C.c_uint64), ("mlp_projection_chunk_size", C.c_uint64),
+                ("logits_chunk_size", C.c_uint64),
+                ("attention_head_parallel_threshold", C.c_uint64)]
+
+
+def rust_config(threads: int = 1, **kw) -> orc_rust_config:
+    d = dict(threads=threads, dense_parallel_threshold=262_144, qkv_chunk_size=48,
+             attention_projection_chunk_size=64, mlp_fc_chunk_size=128,
+             mlp_projection_chunk_size=64, logits_chunk_size=256,
+             attention_head_parallel_threshold=4_096)
+    d.update(kw)
+    return orc_rust_config(**d)
+
+
+class orc_sampling(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("has_top_p", C.c_int32), ("top_p", C.c_float),
+                ("has_top_k", C.c_int32), ("top_k", C.c_uint64), ("repeat_penalty", C.c_float),
+                ("repeat_last_n", C.c_uint64), ("seed", C.c_uint64)]
+
+
+def sampling(temperature=0.0, top_p=None, top_k=None, seed=299_792_458, repeat_penalty=1.0,
+             repeat_last_n=128) -> orc_sampling:
+    return orc_sampling(temperature, int(top_p is not None), top_p or 0.0,
+                        int(top_k is not None), top_k or 0, repeat_penalty, repeat_last_n, seed)
+
+
+class orc_stats(C.Structure):
+    _fields_ = [("prompt_tokens", C.c_uint64), ("generated_tokens", C.c_uint64),
+                ("prefill_s", C.c_double), ("decode_s", C.c_double),
+                ("first_token_s", C.c_double), ("layer_norm_s", C.c_double),
+                ("qkv_projection_s", C.c_double), ("attention_s", C.c_double),
+                ("attention_projection_s", C.c_double), ("mlp_fc_projection_s", C.c_double),
+                ("mlp_projection_s", C.c_double), ("final_logits_s", C.c_double)]
+
+
+_lib = None
+
+
+def build(force: bool = False) -> Path:
+    if force or not LIB_PATH.exists():
+        subprocess.run(["make", "-C", str(ORACLE_DIR), "-B" if force else "-s"], check=True,
+                       stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(str(LIB_PATH))
+        L.orc_last_error.restype = C.c_char_p
+        L.orc_dot.restype = C.c_float
+        L.orc_dot_scalar.restype = C.c_float
+        L.orc_argmax.restype = C.c_uint64
+        for name in ("orc_rng_new", "orc_rng_next_u64", "orc_cache_seq_len",
+                     "orc_cache_max_seq_len"):
+            getattr(L, name).restype = C.c_uint64
+        L.orc_rng_next_unit_f64.restype = C.c_double
+        L.orc_rng_new.argtypes = [C.c_uint64]
+        _lib = L
+    return _lib
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise OracleError(status, lib().orc_last_error().decode())
+
+
+def _f(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(_f32p)
+
+
+def _u(ids) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(ids, dtype=np.uint32).reshape(-1))
+
+
+# ---- src/models/cpu.rs ---------------------------------------------------------
+
+def dot(a, b) -> float:
+    a, b = _f(a), _f(b)
+    return float(lib().orc_dot(_p(a), _p(b), C.c_uint64(a.size)))
+
+
+def dot_scalar(a, b) -> float:
+    a, b = _f(a), _f(b)
+    return float(lib().orc_dot_scalar(_p(a), _p(b), C.c_uint64(a.size)))
+
+
+def transposed_dense(x, rows, in_f, out_f, w, bias) -> np.ndarray:
+    x, w, bias = _f(x), _f(w), _f(bias)
+    out = np.empty(rows * out_f, np.float32)
+    lib().orc_transposed_dense(_p(x), C.c_uint64(rows), C.c_uint64(in_f), C.c_uint64(out_f),
+                               _p(w), _p(bias), _p(out))
+    return out
+
+
+def dense(x, rows, in_f, out_f, w, bias) -> np.ndarray:
+    x, w, bias = _f(x), _f(w), _f(bias)
+    out = np.empty(rows * out_f, np.float32)
+    lib().orc_dense(_p(x), C.c_uint64(rows), C.c_uint64(in_f), C.c_uint64(out_f), _p(w),
+                    _p(bias), _p(out))
+    return out
+
+
+def layer_norm(x, rows, cols, gamma, beta, eps) -> np.ndarray:
+    out = _f(x).copy()
+    g, b = _f(gamma), _f(beta)
+    lib().orc_layer_norm(_p(out), C.c_uint64(rows), C.c_uint64(cols), _p(g), _p(b),
+                         C.c_float(eps))
+    return out
+
+
+def gelu(v) -> np.ndarray:
+    out = _f(v).copy()
+    lib().orc_gelu(_p(out), C.c_uint64(out.size))
+    return out
+
+
+def softmax(v) -> np.ndarray:
+    out = _f(v).copy()
+    lib().orc_softmax(_p(out), C.c_uint64(out.size))
+    return out
+
+
+def add(dst, src) -> np.ndarray:
+    out, s = _f(dst).copy(), _f(src)
+    lib().orc_add(_p(out), _p(s), C.c_uint64(out.size))
+    return out
+
+
+def transpose_in_out(w, in_f, out_f) -> np.ndarray:
+    w = _f(w)
+    out = np.empty(in_f * out_f, np.float32)
+    lib().orc_transpose_in_out(_p(w), C.c_uint64(in_f), C.c_uint64(out_f), _p(out))
+    return out
+
+
+def argmax_logits(v) -> int:
+    v = _f(v)
+    return int(lib().orc_argmax(_p(v), C.c_uint64(v.size)))
+
+
+def pool_chunk_ids(threads: int, length: int, chunk_size: int) -> np.ndarray:
+    out = np.empty(length, np.float32)
+    lib().orc_pool_chunk_ids(C.c_uint64(threads), C.c_uint64(length), C.c_uint64(chunk_size),
+                             _p(out))
+    return out
+
+
+# ---- src/models/generation.rs -----------------------------------------------------
+
+class SmallRng:
+    def __init__(self, seed: int):
+        self.state = C.c_uint64(lib().orc_rng_new(seed))
+
+    def next_u64(self) -> int:
+        return int(lib().orc_rng_next_u64(C.byref(self.state)))
+
+    def next_unit_f64(self) -> float:
+        return float(lib().orc_rng_next_unit_f64(C.byref(self.state)))
+
+
+class LogitsSampler:
+    def __init__(self, seed: int):
+        self.rng = SmallRng(seed)
+
+    def select_next_token(self, logits, history: Sequence[int], cfg: orc_sampling) -> int:
+        v, h = _f(logits), _u(history)
+        out = C.c_uint64()
+        _check(lib().orc_select_next_token(C.byref(self.rng.state), _p(v), C.c_uint64(v.size),
+                                           h.ctypes.data_as(_u32p), C.c_uint64(h.size),
+                                           C.byref(cfg), C.byref(out)))
+        return int(out.value)
+
+
+def validate_generation(cfg: orc_sampling) -> None:
+    _check(lib().orc_validate_generation(C.byref(cfg)))
+
+
+# ---- src/models/gpt2/rust.rs ---------------------------------------------------------
+
+def _tensor(a, keep) -> orc_tensor:
+    a = _f(a).reshape(-1)
+    keep.append(a)
+    return orc_tensor(_p(a), a.size)
+
+
+class Cache:
+    def __init__(self, model: "Model"):
+        h = C.c_void_p()
+        _check(lib().orc_cache_create(model._h, C.byref(h)))
+        self._h, self._model = h, model
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().orc_cache_destroy(self._h)
+            self._h = None
+
+    @property
+    def seq_len(self) -> int:
+        return int(lib().orc_cache_seq_len(self._h))
+
+    @seq_len.setter
+    def seq_len(self, n: int):
+        lib().orc_cache_set_seq_len(self._h, C.c_uint64(n))
+
+    @property
+    def max_seq_len(self) -> int:
+        return int(lib().orc_cache_max_seq_len(self._h))
+
+    def clear(self):
+        lib().orc_cache_clear(self._h)
+
+    def read_layer(self, layer: int, which: int) -> np.ndarray:
+        cfg = self._model.config
+        out = np.empty((cfg.n_head, cfg.n_positions, cfg.n_embd // cfg.n_head), np.float32)
+        lib().orc_cache_read(self._h, C.c_uint64(layer), C.c_int(which), _p(out))
+        return out
+
+
+class Model:
+    """Gpt2Model::new_with_rust_config (rust.rs:803-825).  `config` and `weights`
+    are any objects with the reference's field names (Gpt2Config / Gpt2Weights)."""
+
+    def __init__(self, config, weights, rc: Optional[orc_rust_config] = None):
+        keep: list = []
+        n_inner = config.n_inner if config.n_inner is not None else 4 * config.n_embd
+        cfg = orc_config(config.vocab_size, config.n_positions, config.n_embd, config.n_layer,
+                         config.n_head, n_inner, config.layer_norm_epsilon)
+        blocks = (orc_block_view * max(len(weights.blocks), 1))()
+        for i, b in enumerate(weights.blocks):
+            for name in BLOCK_FIELDS:
+                setattr(blocks[i], name, _tensor(getattr(b, name), keep))
+        view = orc_weights_view(_tensor(weights.wte, keep), _tensor(weights.wpe, keep),
+                                _tensor(weights.ln_f_g, keep), _tensor(weights.ln_f_b, keep),
+                                C.cast(blocks, C.POINTER(orc_block_view)), len(weights.blocks))
+        h = C.c_void_p()
+        rcv = rc if rc is not None else rust_config(1)
+        _check(lib().orc_gpt2_create(C.byref(cfg), C.byref(view), C.byref(rcv), C.byref(h)))
+        self._h = h
+        self.config = config
+        self.vocab = config.vocab_size
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().orc_gpt2_destroy(self._h)
+            self._h = None
+
+    def new_kv_cache(self) -> Cache:
+        return Cache(self)
+
+    def forward(self, ids) -> np.ndarray:
+        ids = _u(ids)
+        out = np.empty((max(ids.size, 1), self.vocab), np.float32)
+        _check(lib().orc_gpt2_forward(self._h, ids.ctypes.data_as(_u32p), C.c_uint64(ids.size),
+                                      _p(out)))
+        return out[:ids.size]
+
+    def prefill(self, ids, cache: Cache) -> np.ndarray:
+        ids = _u(ids)
+        out = np.empty(self.vocab, np.float32)
+        _check(lib().orc_gpt2_prefill(self._h, cache._h, ids.ctypes.data_as(_u32p),
+                                      C.c_uint64(ids.size), _p(out)))
+        return out
+
+    def forward_one(self, token_id: int, cache: Cache) -> np.ndarray:
+        out = np.empty(self.vocab, np.float32)
+        _check(lib().orc_gpt2_forward_one(self._h, cache._h, C.c_uint32(token_id), _p(out)))
+        return out
+
+    def generate(self, ids, max_new: int):
+        """autoregressive::generate (autoregressive.rs:61-87)."""
+        ids = _u(ids)
+        out = np.empty(ids.size + max_new + 1, np.uint32)
+        n = C.c_uint64()
+        _check(lib().orc_generate(self._h, ids.ctypes.data_as(_u32p), C.c_uint64(ids.size),
+                                  C.c_uint64(max_new), out.ctypes.data_as(_u32p), C.byref(n)))
+        return [int(t) for t in out[:n.value]]
+
+    def generate_greedy(self, ids, max_new: int):
+        """Gpt2Model::generate_greedy (rust.rs:884-900)."""
+        ids = _u(ids)
+        out = np.empty(ids.size + max_new + 1, np.uint32)
+        n = C.c_uint64()
+        _check(lib().orc_generate_greedy_full(self._h, ids.ctypes.data_as(_u32p),
+                                              C.c_uint64(ids.size), C.c_uint64(max_new),
+                                              out.ctypes.data_as(_u32p), C.byref(n)))
+        return [int(t) for t in out[:n.value]]
+
+    def stream_token_ids_with_stats(self, ids, max_new: int, eos: Optional[int],
+                                    cfg: Optional[orc_sampling] = None, want_logits=False):
+        """rust.rs:548-634.  Returns (tokens, stats, per_step_logits|None, top2_gap)."""
+        ids = _u(ids)
+        cfg = cfg if cfg is not None else sampling()
+        out = np.empty(ids.size + max_new + 1, np.uint32)
+        n = C.c_uint64()
+        st = orc_stats()
+        logits = np.zeros((max(max_new, 1), self.vocab), np.float32) if want_logits else None
+        gap = np.zeros(max(max_new, 1), np.float32)
+        _check(lib().orc_stream_token_ids_with_stats(
+            self._h, ids.ctypes.data_as(_u32p), C.c_uint64(ids.size), C.c_uint64(max_new),
+            C.c_int64(-1 if eos is None else eos), C.byref(cfg), out.ctypes.data_as(_u32p),
+            C.byref(n), C.byref(st), _p(logits) if want_logits else None, _p(gap)))
+        g = st.generated_tokens
+        return ([int(t) for t in out[:n.value]], st,
+                logits[:g] if want_logits else None, gap[:g])
+
+    def timed_forward_steps(self, cache: Cache, start_len: int, ids, want_logits=False):
+        ids = _u(ids)
+        sec = C.c_double()
+        out = np.empty(self.vocab, np.float32) if want_logits else None
+        _check(lib().orc_timed_forward_steps(self._h, cache._h, C.c_uint64(start_len),
+                                             ids.ctypes.data_as(_u32p), C.c_uint64(ids.size),
+                                             C.byref(sec), _p(out) if want_logits else None))
+        return sec.value, out

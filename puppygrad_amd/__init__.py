@@ -1,0 +1,14 @@
+"""puppygrad_amd: MI355X (gfx950) GPT-2 inference backend for puppygrad.
+
+The product is libpuppygrad_hip.so (C ABI in include/puppygrad_hip.h); this
+package is its Python host-side mirror, used by the tests and the benchmark.
+"""
+from .gpt2 import (GPT2_EOS_TOKEN_ID, DeviceLogits, GenerationStats, Gpt2BlockWeights, Gpt2Config,
+                   Gpt2Error, Gpt2GenerationConfig, Gpt2HipConfig, Gpt2KvCache, Gpt2Model,
+                   Gpt2Output, Gpt2Weights, LogitsSampler, TextGenerationConfig, argmax_logits,
+                   generate)
+
+__all__ = ["GPT2_EOS_TOKEN_ID", "DeviceLogits", "GenerationStats", "Gpt2BlockWeights",
+           "Gpt2Config", "Gpt2Error", "Gpt2GenerationConfig", "Gpt2HipConfig", "Gpt2KvCache",
+           "Gpt2Model", "Gpt2Output", "Gpt2Weights", "LogitsSampler", "TextGenerationConfig",
+           "argmax_logits", "generate"]

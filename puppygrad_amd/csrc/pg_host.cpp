@@ -1,0 +1,1113 @@
+// Host side of libpuppygrad_hip.so: handle types, the reference's validation
+// and error wording, weight upload, and the forward / generation drivers that
+// sequence the kernels in pg_kernels.hip.  The public contract is
+// include/puppygrad_hip.h; reference citations (`src/...:line`) name the
+// puppygrad code each piece mirrors.
+#include "../../include/puppygrad_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "pg_kernels.h"
+
+namespace {
+
+thread_local std::string g_err;
+
+pg_status fail(pg_status s, const std::string& msg) {
+  g_err = msg;
+  return s;
+}
+
+#define PG_HIP(expr)                                                                  \
+  do {                                                                                \
+    hipError_t e__ = (expr);                                                          \
+    if (e__ != hipSuccess)                                                            \
+      return fail(PG_BACKEND, std::string("HIP error: ") + hipGetErrorString(e__) +   \
+                                  " at " #expr);                                      \
+  } while (0)
+
+using Clock = std::chrono::steady_clock;
+double since(Clock::time_point t0) {
+  return std::chrono::duration<double>(Clock::now() - t0).count();
+}
+
+struct Cfg {
+  size_t V, P, C, L, H, I;
+  float eps;
+  size_t hd() const { return C / H; }
+};
+
+}  // namespace
+
+struct pg_gpt2_model {
+  Cfg cfg;
+  int device = 0;
+  int num_cus = 0;
+  pg_hip_options opts{};
+  float* arena = nullptr;  // one allocation holding every tensor
+  size_t arena_floats = 0;
+  float *wte = nullptr, *wpe = nullptr, *ln_f_g = nullptr, *ln_f_b = nullptr;
+  std::vector<pgk::LayerW> layers;
+};
+
+struct pg_logits {
+  pg_kv_cache* owner;
+  float* data;  // device [rows][vocab]
+  uint32_t rows;
+  uint64_t vocab;
+};
+
+struct pg_kv_cache {
+  Cfg cfg;
+  int device = 0;
+  int num_cus = 0;
+  uint32_t B = 1;
+  size_t seq_len = 0;
+  float* kv = nullptr;  // [L][2][B][H][P][hd]
+  // per-sequence activation scratch, [B][...]
+  float *x = nullptr, *q = nullptr, *hbuf = nullptr, *part_acc = nullptr, *part_m = nullptr,
+        *part_l = nullptr, *logits_buf = nullptr;
+  uint32_t* d_tok = nullptr;      // [B] token the next step embeds
+  uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
+  uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  pg_logits logits{};
+  bool logits_valid = false;
+
+  float* k_panel(size_t l, size_t b) const {
+    return kv + (((l * 2 + 0) * B + b) * cfg.H) * cfg.P * cfg.hd();
+  }
+  float* v_panel(size_t l, size_t b) const {
+    return kv + (((l * 2 + 1) * B + b) * cfg.H) * cfg.P * cfg.hd();
+  }
+};
+
+namespace {
+
+// Gpt2Config::validate (src/models/gpt2/rust.rs:60-95).
+pg_status validate_config(const pg_gpt2_config& c) {
+  if (c.vocab_size == 0) return fail(PG_INVALID_CONFIG, "vocab_size must be > 0");
+  if (c.n_positions == 0) return fail(PG_INVALID_CONFIG, "n_positions must be > 0");
+  if (c.n_embd == 0) return fail(PG_INVALID_CONFIG, "n_embd must be > 0");
+  if (c.n_layer == 0) return fail(PG_INVALID_CONFIG, "n_layer must be > 0");
+  if (c.n_head == 0) return fail(PG_INVALID_CONFIG, "n_head must be > 0");
+  if (c.n_inner == 0) return fail(PG_INVALID_CONFIG, "n_inner must be > 0");
+  if (c.n_embd % c.n_head != 0)
+    return fail(PG_INVALID_CONFIG, "n_embd " + std::to_string(c.n_embd) +
+                                       " must be divisible by n_head " +
+                                       std::to_string(c.n_head));
+  if (!(c.layer_norm_epsilon > 0.0f))
+    return fail(PG_INVALID_CONFIG, "layer_norm_epsilon must be > 0");
+  // Limits of this backend (no reference counterpart): vectors are staged in
+  // 64 KiB of LDS and indices are 32-bit.
+  const uint64_t lds_floats = 16384;
+  if (c.n_embd > lds_floats || c.n_inner > lds_floats || c.n_positions > lds_floats)
+    return fail(PG_INVALID_CONFIG,
+                "hip backend supports n_embd, n_inner and n_positions up to 16384");
+  if (c.vocab_size > (1ull << 31) || c.n_layer > 4096)
+    return fail(PG_INVALID_CONFIG, "hip backend supports vocab_size < 2^31 and n_layer <= 4096");
+  return PG_OK;
+}
+
+// expect_len (src/models/gpt2/rust.rs:1335-1343).
+pg_status expect_len(const std::string& name, const pg_tensor& t, size_t expected) {
+  if (t.len != expected)
+    return fail(PG_INVALID_WEIGHTS, name + " len " + std::to_string(t.len) +
+                                        " does not match expected " + std::to_string(expected));
+  if (expected && !t.data) return fail(PG_INVALID_WEIGHTS, name + " data pointer is null");
+  return PG_OK;
+}
+
+// validate_weights (src/models/gpt2/rust.rs:1279-1333).
+pg_status validate_weights(const Cfg& c, const pg_gpt2_weights_view& w) {
+  pg_status s;
+  if ((s = expect_len("wte", w.wte, c.V * c.C))) return s;
+  if ((s = expect_len("wpe", w.wpe, c.P * c.C))) return s;
+  if ((s = expect_len("ln_f_g", w.ln_f_g, c.C))) return s;
+  if ((s = expect_len("ln_f_b", w.ln_f_b, c.C))) return s;
+  if (w.n_blocks != c.L)
+    return fail(PG_INVALID_WEIGHTS, "blocks len " + std::to_string(w.n_blocks) +
+                                        " does not match n_layer " + std::to_string(c.L));
+  for (size_t i = 0; i < c.L; ++i) {
+    const pg_gpt2_block_view& b = w.blocks[i];
+    std::string p = "blocks[" + std::to_string(i) + "]";
+    if ((s = expect_len(p + ".ln_1_g", b.ln_1_g, c.C))) return s;
+    if ((s = expect_len(p + ".ln_1_b", b.ln_1_b, c.C))) return s;
+    if ((s = expect_len(p + ".c_attn_w", b.c_attn_w, c.C * 3 * c.C))) return s;
+    if ((s = expect_len(p + ".c_attn_b", b.c_attn_b, 3 * c.C))) return s;
+    if ((s = expect_len(p + ".c_proj_w", b.c_proj_w, c.C * c.C))) return s;
+    if ((s = expect_len(p + ".c_proj_b", b.c_proj_b, c.C))) return s;
+    if ((s = expect_len(p + ".ln_2_g", b.ln_2_g, c.C))) return s;
+    if ((s = expect_len(p + ".ln_2_b", b.ln_2_b, c.C))) return s;
+    if ((s = expect_len(p + ".c_fc_w", b.c_fc_w, c.C * c.I))) return s;
+    if ((s = expect_len(p + ".c_fc_b", b.c_fc_b, c.I))) return s;
+    if ((s = expect_len(p + ".c_proj_mlp_w", b.c_proj_mlp_w, c.I * c.C))) return s;
+    if ((s = expect_len(p + ".c_proj_mlp_b", b.c_proj_mlp_b, c.C))) return s;
+  }
+  return PG_OK;
+}
+
+size_t round_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+pg_status select_device(int device) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n == 0)
+    return fail(PG_BACKEND, "no HIP device available: the hip backend needs an AMD GPU");
+  if (device < 0 || device >= n)
+    return fail(PG_INVALID_CONFIG, "hip device " + std::to_string(device) +
+                                       " out of range for " + std::to_string(n) + " devices");
+  PG_HIP(hipSetDevice(device));
+  return PG_OK;
+}
+
+// validate_input (src/models/gpt2/rust.rs:1029-1051).
+pg_status validate_input(const Cfg& c, const uint32_t* ids, size_t n) {
+  if (n == 0 || !ids) return fail(PG_INVALID_INPUT, "input_ids must not be empty");
+  if (n > c.P)
+    return fail(PG_INVALID_INPUT, "sequence length " + std::to_string(n) +
+                                      " exceeds n_positions " + std::to_string(c.P));
+  for (size_t i = 0; i < n; ++i)
+    if (ids[i] >= c.V)
+      return fail(PG_INVALID_INPUT, "token id " + std::to_string(ids[i]) + " at index " +
+                                        std::to_string(i) + " exceeds vocab_size " +
+                                        std::to_string(c.V));
+  return PG_OK;
+}
+
+// Gpt2KvCache::check_compatible (src/models/gpt2/rust.rs:206-234).
+pg_status check_compatible(const pg_gpt2_model* m, const pg_kv_cache* c) {
+  if (c->cfg.L != m->cfg.L)
+    return fail(PG_INVALID_INPUT, "cache layer count " + std::to_string(c->cfg.L) +
+                                      " does not match n_layer " + std::to_string(m->cfg.L));
+  if (c->cfg.P != m->cfg.P)
+    return fail(PG_INVALID_INPUT, "cache max_seq_len " + std::to_string(c->cfg.P) +
+                                      " does not match n_positions " + std::to_string(m->cfg.P));
+  if (c->cfg.H != m->cfg.H)
+    return fail(PG_INVALID_INPUT, "cache n_head " + std::to_string(c->cfg.H) +
+                                      " does not match n_head " + std::to_string(m->cfg.H));
+  if (c->cfg.hd() != m->cfg.hd())
+    return fail(PG_INVALID_INPUT, "cache head_dim " + std::to_string(c->cfg.hd()) +
+                                      " does not match head_dim " + std::to_string(m->cfg.hd()));
+  if (c->device != m->device)
+    return fail(PG_INVALID_INPUT, "cache lives on device " + std::to_string(c->device) +
+                                      " but the model is on device " + std::to_string(m->device));
+  return PG_OK;
+}
+
+// One cached decoder step for sequence b (forward_one_profiled_with_scratch,
+// src/models/gpt2/rust.rs:943-1006, block at 1136-1250) as a chain of fused
+// launches on the cache's stream.  The token comes from tok_ptr (device) when
+// it is non-null.  With want_logits false the final LayerNorm and lm_head are
+// skipped (prefill discards those logits, rust.rs:922-926).
+pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
+                              const uint32_t* tok_ptr, uint32_t tok, size_t pos,
+                              bool want_logits) {
+  const Cfg& g = m->cfg;
+  const int C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
+  hipStream_t s = c->stream;
+  float* x = c->x + b * g.C;
+  float* q = c->q + b * g.C;
+  float* hb = c->hbuf + b * g.I;
+  const size_t part_stride = (size_t)H * pgk::kMaxSplits;
+  float* pa = c->part_acc + b * part_stride * hd;
+  float* pm = c->part_m + b * part_stride;
+  float* pl = c->part_l + b * part_stride;
+  const int nsplit = hd == pgk::kHeadDim ? pgk::choose_nsplit((int)pos + 1, H, m->num_cus) : 1;
+
+  PG_HIP(pgk::launch_embed(x, m->wte, m->wpe, tok_ptr, tok, (int)pos, C, s));
+  for (size_t l = 0; l < g.L; ++l) {
+    const pgk::LayerW& w = m->layers[l];
+    pgk::GemvArgs a{};
+    // LN1 + c_attn + K/V append
+    a.W = w.c_attn_w; a.bias = w.c_attn_b; a.x = x; a.y = q; a.K = C; a.nout = 3 * C;
+    a.ln_g = w.ln_1_g; a.ln_b = w.ln_1_b; a.eps = g.eps;
+    a.kcache = c->k_panel(l, b); a.vcache = c->v_panel(l, b);
+    a.pos = (int)pos; a.P = P; a.C = C; a.head_dim = hd;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_QKV, s));
+    // attention over keys [0, pos]
+    PG_HIP(pgk::launch_attn_decode(q, c->k_panel(l, b), c->v_panel(l, b), (int)pos, P, H, hd,
+                                   nsplit, pa, pm, pl, s));
+    // merge splits + c_proj + residual
+    a = pgk::GemvArgs{};
+    a.W = w.c_proj_w; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
+    a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
+    // LN2 + c_fc + GELU
+    a = pgk::GemvArgs{};
+    a.W = w.c_fc_w; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
+    a.ln_g = w.ln_2_g; a.ln_b = w.ln_2_b; a.eps = g.eps;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_GELU, s));
+    // mlp c_proj + residual
+    a = pgk::GemvArgs{};
+    a.W = w.c_proj_mlp_w; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
+    a.nout = C;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
+  }
+  if (want_logits) {
+    pgk::GemvArgs a{};
+    a.W = m->wte; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
+    a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+  }
+  return PG_OK;
+}
+
+pg_status check_step(const pg_gpt2_model* m, const pg_kv_cache* c) {
+  // rust.rs:957-962
+  if (c->seq_len >= c->cfg.P)
+    return fail(PG_INVALID_INPUT, "cache is full at seq_len " + std::to_string(c->seq_len));
+  (void)m;
+  return PG_OK;
+}
+
+pg_status finish_logits(pg_kv_cache* c, pg_logits** out) {
+  c->logits.owner = c;
+  c->logits.data = c->logits_buf;
+  c->logits.rows = c->B;
+  c->logits.vocab = c->cfg.V;
+  c->logits_valid = true;
+  if (out) *out = &c->logits;
+  return PG_OK;
+}
+
+// ---- host sampler: src/models/generation.rs:281-362 --------------------------
+
+void apply_repeat_penalty(std::vector<float>& logits, const uint32_t* history, size_t n_hist,
+                          float penalty, uint64_t last_n) {
+  if (penalty == 1.0f || last_n == 0) return;
+  std::vector<uint32_t> seen;
+  size_t take = (size_t)std::min<uint64_t>(last_n, n_hist);
+  for (size_t j = 0; j < take; ++j) {
+    uint32_t t = history[n_hist - 1 - j];
+    if (t >= logits.size() || std::find(seen.begin(), seen.end(), t) != seen.end()) continue;
+    seen.push_back(t);
+    if (logits[t] < 0.0f)
+      logits[t] *= penalty;
+    else
+      logits[t] /= penalty;
+  }
+}
+
+size_t argmax_host(const float* v, size_t n) {
+  size_t bi = 0;
+  float best = -INFINITY;
+  for (size_t i = 0; i < n; ++i)
+    if (v[i] > best) {
+      best = v[i];
+      bi = i;
+    }
+  return bi;
+}
+
+inline int32_t total_order_key(float f) {
+  int32_t b;
+  std::memcpy(&b, &f, 4);
+  b ^= (int32_t)(((uint32_t)(b >> 31)) >> 1);
+  return b;
+}
+
+pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg,
+                        pg_rng_state* rng, uint32_t* out) {
+  std::vector<std::pair<uint32_t, float>> cand;
+  for (size_t i = 0; i < logits.size(); ++i)
+    if (std::isfinite(logits[i])) cand.emplace_back((uint32_t)i, logits[i]);
+  if (cand.empty())
+    return fail(PG_INVALID_INPUT,
+                "token sampling failed: cannot sample from empty or non-finite logits");
+  std::stable_sort(cand.begin(), cand.end(), [](const auto& l, const auto& r) {
+    return total_order_key(r.second) < total_order_key(l.second);
+  });
+  if (cfg.has_top_k) cand.resize((size_t)std::min<uint64_t>(cfg.top_k, cand.size()));
+  const double T = (double)cfg.temperature;
+  const double max_logit = (double)cand[0].second / T;
+  std::vector<std::pair<uint32_t, double>> w;
+  w.reserve(cand.size());
+  for (auto& c : cand) w.emplace_back(c.first, std::exp((double)c.second / T - max_logit));
+  if (cfg.has_top_p) {
+    double full = 0.0;
+    for (auto& e : w) full += e.second;
+    if (full > 0.0) {
+      double cum = 0.0;
+      size_t keep = 0;
+      for (auto& e : w) {
+        cum += e.second;
+        keep += 1;
+        if (cum / full >= (double)cfg.top_p) break;
+      }
+      w.resize(std::max<size_t>(keep, 1));
+    }
+  }
+  double total = 0.0;
+  for (auto& e : w) total += e.second;
+  if (total <= 0.0 || !std::isfinite(total)) {
+    *out = w[0].first;
+    return PG_OK;
+  }
+  uint32_t fallback = w.back().first;
+  double target = pg_rng_next_unit_f64(rng) * total;
+  for (auto& e : w) {
+    target -= e.second;
+    if (target <= 0.0) {
+      *out = e.first;
+      return PG_OK;
+    }
+  }
+  *out = fallback;
+  return PG_OK;
+}
+
+struct DevBuf {
+  float* p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+  pg_status alloc(size_t n) {
+    PG_HIP(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(float)));
+    return PG_OK;
+  }
+};
+
+}  // namespace
+
+extern "C" {
+
+const char* pg_last_error_message(void) { return g_err.c_str(); }
+
+pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_view* weights,
+                         const pg_hip_options* options, pg_gpt2_model** out) {
+  if (!config || !weights || !out) return fail(PG_INVALID_INPUT, "null argument");
+  *out = nullptr;
+  pg_status s;
+  if ((s = validate_config(*config))) return s;
+  Cfg g{config->vocab_size, config->n_positions, config->n_embd,          config->n_layer,
+        config->n_head,     config->n_inner,     config->layer_norm_epsilon};
+  if ((s = validate_weights(g, *weights))) return s;
+  pg_hip_options opts{};
+  if (options) opts = *options;
+  if (opts.weight_storage != PG_STORE_F32)
+    return fail(PG_INVALID_CONFIG, "hip backend weight_storage: only f32 is implemented");
+  if (opts.decode_path > PG_DECODE_PERSISTENT)
+    return fail(PG_INVALID_CONFIG, "hip backend decode_path out of range");
+  if ((s = select_device(opts.device))) return s;
+
+  auto m = std::make_unique<pg_gpt2_model>();
+  m->cfg = g;
+  m->device = opts.device;
+  m->opts = opts;
+  hipDeviceProp_t prop;
+  PG_HIP(hipGetDeviceProperties(&prop, opts.device));
+  m->num_cus = prop.multiProcessorCount;
+
+  // One arena; every tensor starts on a 256-byte boundary.
+  const size_t A = 64;
+  size_t total = round_up(g.V * g.C, A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A);
+  const size_t per_layer = 6 * round_up(g.C, A) + round_up(3 * g.C * g.C, A) +
+                           round_up(3 * g.C, A) + round_up(g.C * g.C, A) +
+                           2 * round_up(g.C * g.I, A) + round_up(g.I, A);
+  total += g.L * per_layer;
+  PG_HIP(hipMalloc(&m->arena, total * sizeof(float)));
+  m->arena_floats = total;
+  struct Guard {
+    pg_gpt2_model* m;
+    bool ok = false;
+    ~Guard() {
+      if (!ok && m->arena) (void)hipFree(m->arena);
+    }
+  } guard{m.get()};
+
+  size_t off = 0;
+  auto place = [&](size_t n) {
+    float* p = m->arena + off;
+    off += round_up(n, A);
+    return p;
+  };
+  auto upload = [&](float* dst, const pg_tensor& t) -> pg_status {
+    PG_HIP(hipMemcpy(dst, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
+    return PG_OK;
+  };
+  DevBuf staging;
+  if ((s = staging.alloc(std::max(3 * g.C * g.C, g.C * g.I)))) return s;
+  // transpose_dense_weights (src/models/gpt2/rust.rs:1345-1352): [in,out] -> [out,in].
+  auto upload_t = [&](float* dst, const pg_tensor& t, size_t in_f, size_t out_f) -> pg_status {
+    PG_HIP(hipMemcpy(staging.p, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
+    PG_HIP(pgk::launch_transpose(staging.p, dst, (int)in_f, (int)out_f, nullptr));
+    PG_HIP(hipStreamSynchronize(nullptr));
+    return PG_OK;
+  };
+
+  m->wte = place(g.V * g.C);
+  m->wpe = place(g.P * g.C);
+  m->ln_f_g = place(g.C);
+  m->ln_f_b = place(g.C);
+  if ((s = upload(m->wte, weights->wte))) return s;
+  if ((s = upload(m->wpe, weights->wpe))) return s;
+  if ((s = upload(m->ln_f_g, weights->ln_f_g))) return s;
+  if ((s = upload(m->ln_f_b, weights->ln_f_b))) return s;
+  m->layers.resize(g.L);
+  for (size_t l = 0; l < g.L; ++l) {
+    const pg_gpt2_block_view& b = weights->blocks[l];
+    float* ln_1_g = place(g.C);
+    float* ln_1_b = place(g.C);
+    float* c_attn_w = place(3 * g.C * g.C);
+    float* c_attn_b = place(3 * g.C);
+    float* c_proj_w = place(g.C * g.C);
+    float* c_proj_b = place(g.C);
+    float* ln_2_g = place(g.C);
+    float* ln_2_b = place(g.C);
+    float* c_fc_w = place(g.C * g.I);
+    float* c_fc_b = place(g.I);
+    float* c_proj_mlp_w = place(g.I * g.C);
+    float* c_proj_mlp_b = place(g.C);
+    if ((s = upload(ln_1_g, b.ln_1_g))) return s;
+    if ((s = upload(ln_1_b, b.ln_1_b))) return s;
+    if ((s = upload_t(c_attn_w, b.c_attn_w, g.C, 3 * g.C))) return s;
+    if ((s = upload(c_attn_b, b.c_attn_b))) return s;
+    if ((s = upload_t(c_proj_w, b.c_proj_w, g.C, g.C))) return s;
+    if ((s = upload(c_proj_b, b.c_proj_b))) return s;
+    if ((s = upload(ln_2_g, b.ln_2_g))) return s;
+    if ((s = upload(ln_2_b, b.ln_2_b))) return s;
+    if ((s = upload_t(c_fc_w, b.c_fc_w, g.C, g.I))) return s;
+    if ((s = upload(c_fc_b, b.c_fc_b))) return s;
+    if ((s = upload_t(c_proj_mlp_w, b.c_proj_mlp_w, g.I, g.C))) return s;
+    if ((s = upload(c_proj_mlp_b, b.c_proj_mlp_b))) return s;
+    m->layers[l] = pgk::LayerW{ln_1_g, ln_1_b, c_attn_w, c_attn_b, c_proj_w,     c_proj_b,
+                               ln_2_g, ln_2_b, c_fc_w,   c_fc_b,   c_proj_mlp_w, c_proj_mlp_b};
+  }
+  guard.ok = true;
+  *out = m.release();
+  return PG_OK;
+}
+
+void pg_gpt2_destroy(pg_gpt2_model* m) {
+  if (!m) return;
+  if (hipSetDevice(m->device) == hipSuccess && m->arena) (void)hipFree(m->arena);
+  delete m;
+}
+
+pg_status pg_gpt2_get_config(const pg_gpt2_model* m, pg_gpt2_config* out) {
+  if (!m || !out) return fail(PG_INVALID_INPUT, "null argument");
+  *out = pg_gpt2_config{m->cfg.V, m->cfg.P, m->cfg.C, m->cfg.L, m->cfg.H, m->cfg.I, m->cfg.eps};
+  return PG_OK;
+}
+
+pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
+  if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
+  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=f32)", m->device,
+                m->num_cus);
+  return PG_OK;
+}
+
+pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache** out) {
+  if (!m || !out) return fail(PG_INVALID_INPUT, "null argument");
+  *out = nullptr;
+  if (batch == 0) return fail(PG_INVALID_INPUT, "cache batch must be > 0");
+  pg_status s;
+  if ((s = select_device(m->device))) return s;
+  const Cfg& g = m->cfg;
+  auto c = std::make_unique<pg_kv_cache>();
+  c->cfg = g;
+  c->device = m->device;
+  c->num_cus = m->num_cus;
+  c->B = batch;
+  const size_t B = batch, hd = g.hd();
+  const size_t kv_floats = g.L * 2 * B * g.H * g.P * hd;
+  const size_t parts = B * g.H * pgk::kMaxSplits;
+  struct Guard {
+    pg_kv_cache* c;
+    bool ok = false;
+    ~Guard() {
+      if (!ok) pg_kv_cache_destroy(c);
+    }
+  };
+  pg_kv_cache* raw = c.release();
+  Guard guard{raw};
+  PG_HIP(hipStreamCreateWithFlags(&raw->stream, hipStreamNonBlocking));
+  PG_HIP(hipEventCreate(&raw->ev0));
+  PG_HIP(hipEventCreate(&raw->ev1));
+  PG_HIP(hipMalloc(&raw->kv, kv_floats * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->x, B * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->q, B * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->hbuf, B * g.I * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->part_acc, parts * hd * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->part_m, parts * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->part_l, parts * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->logits_buf, B * g.V * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->d_tok, B * sizeof(uint32_t)));
+  PG_HIP(hipMalloc(&raw->d_out_ids, g.P * B * sizeof(uint32_t)));
+  PG_HIP(hipHostMalloc(&raw->h_ids, g.P * B * sizeof(uint32_t), hipHostMallocDefault));
+  // Gpt2LayerKvCache::new zero-fills (src/models/gpt2/rust.rs:258-266).
+  PG_HIP(pgk::launch_fill_zero(raw->kv, kv_floats, raw->stream));
+  PG_HIP(hipStreamSynchronize(raw->stream));
+  guard.ok = true;
+  *out = raw;
+  return PG_OK;
+}
+
+void pg_kv_cache_destroy(pg_kv_cache* c) {
+  if (!c) return;
+  if (hipSetDevice(c->device) == hipSuccess) {
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    (void)hipFree(c->kv);
+    (void)hipFree(c->x);
+    (void)hipFree(c->q);
+    (void)hipFree(c->hbuf);
+    (void)hipFree(c->part_acc);
+    (void)hipFree(c->part_m);
+    (void)hipFree(c->part_l);
+    (void)hipFree(c->logits_buf);
+    (void)hipFree(c->d_tok);
+    (void)hipFree(c->d_out_ids);
+    if (c->h_ids) (void)hipHostFree(c->h_ids);
+    if (c->ev0) (void)hipEventDestroy(c->ev0);
+    if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+  }
+  delete c;
+}
+
+pg_status pg_kv_cache_clear(pg_kv_cache* c) {
+  if (!c) return fail(PG_INVALID_INPUT, "null argument");
+  c->seq_len = 0;  // Gpt2KvCache::clear resets seq_len only (rust.rs:202-204)
+  c->logits_valid = false;
+  return PG_OK;
+}
+uint64_t pg_kv_cache_seq_len(const pg_kv_cache* c) { return c ? c->seq_len : 0; }
+uint64_t pg_kv_cache_max_seq_len(const pg_kv_cache* c) { return c ? c->cfg.P : 0; }
+uint32_t pg_kv_cache_batch(const pg_kv_cache* c) { return c ? c->B : 0; }
+pg_status pg_kv_cache_set_seq_len(pg_kv_cache* c, uint64_t n) {
+  if (!c) return fail(PG_INVALID_INPUT, "null argument");
+  if (n > c->cfg.P)
+    return fail(PG_INVALID_INPUT, "seq_len " + std::to_string(n) + " exceeds max_seq_len " +
+                                      std::to_string(c->cfg.P));
+  c->seq_len = n;
+  c->logits_valid = false;
+  return PG_OK;
+}
+
+pg_status pg_kv_cache_read_layer(const pg_kv_cache* c, uint32_t b, uint32_t layer, uint32_t which,
+                                 float* dst, size_t len) {
+  if (!c || !dst) return fail(PG_INVALID_INPUT, "null argument");
+  const size_t panel = c->cfg.H * c->cfg.P * c->cfg.hd();
+  if (b >= c->B || layer >= c->cfg.L || which > 1 || len != panel)
+    return fail(PG_INVALID_INPUT, "cache panel index or length out of range");
+  pg_status s;
+  if ((s = select_device(c->device))) return s;
+  PG_HIP(hipStreamSynchronize(c->stream));
+  const float* src = which ? c->v_panel(layer, b) : c->k_panel(layer, b);
+  PG_HIP(hipMemcpy(dst, src, panel * sizeof(float), hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_gpt2_prefill_batch(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* ids,
+                                size_t n, pg_logits** out) {
+  if (!m || !c) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  for (size_t b = 0; b < c->B; ++b)
+    if ((s = validate_input(m->cfg, ids ? ids + b * n : nullptr, n))) return s;
+  if ((s = check_compatible(m, c))) return s;
+  if ((s = select_device(m->device))) return s;
+  c->seq_len = 0;  // cache.clear() (rust.rs:918)
+  c->logits_valid = false;
+  for (size_t b = 0; b < c->B; ++b)
+    for (size_t i = 0; i < n; ++i)
+      if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b * n + i], i, i + 1 == n))) return s;
+  PG_HIP(hipStreamSynchronize(c->stream));
+  c->seq_len = n;
+  return finish_logits(c, out);
+}
+
+pg_status pg_gpt2_prefill(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* ids, size_t n,
+                          pg_logits** out) {
+  if (!m || !c) return fail(PG_INVALID_INPUT, "null argument");
+  if (c->B != 1) return fail(PG_INVALID_INPUT, "prefill needs a cache of batch 1");
+  return pg_gpt2_prefill_batch(m, c, ids, n, out);
+}
+
+pg_status pg_gpt2_forward_one_batch(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* ids,
+                                    pg_logits** out) {
+  if (!m || !c || !ids) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = check_compatible(m, c))) return s;
+  for (size_t b = 0; b < c->B; ++b)
+    if (ids[b] >= m->cfg.V)  // rust.rs:951-956
+      return fail(PG_INVALID_INPUT, "token id " + std::to_string(ids[b]) +
+                                        " exceeds vocab_size " + std::to_string(m->cfg.V));
+  if ((s = check_step(m, c))) return s;
+  if ((s = select_device(m->device))) return s;
+  for (size_t b = 0; b < c->B; ++b)
+    if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b], c->seq_len, true))) return s;
+  PG_HIP(hipStreamSynchronize(c->stream));
+  c->seq_len += 1;  // rust.rs:1004
+  return finish_logits(c, out);
+}
+
+pg_status pg_gpt2_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t id,
+                              pg_logits** out) {
+  if (!m || !c) return fail(PG_INVALID_INPUT, "null argument");
+  if (c->B != 1) return fail(PG_INVALID_INPUT, "forward_one needs a cache of batch 1");
+  return pg_gpt2_forward_one_batch(m, c, &id, out);
+}
+
+pg_status pg_gpt2_forward(const pg_gpt2_model* m, const uint32_t* ids, size_t n, float* dst,
+                          size_t dst_len) {
+  if (!m || !dst) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = validate_input(m->cfg, ids, n))) return s;
+  if (dst_len != n * m->cfg.V)
+    return fail(PG_INVALID_INPUT, "logits buffer length " + std::to_string(dst_len) +
+                                      " does not match seq_len * vocab_size " +
+                                      std::to_string(n * m->cfg.V));
+  pg_kv_cache* c = nullptr;
+  if ((s = pg_kv_cache_create(m, 1, &c))) return s;
+  std::unique_ptr<pg_kv_cache, void (*)(pg_kv_cache*)> holder(c, pg_kv_cache_destroy);
+  for (size_t i = 0; i < n; ++i) {
+    if ((s = enqueue_forward_one(m, c, 0, nullptr, ids[i], i, true))) return s;
+    PG_HIP(hipMemcpyAsync(dst + i * m->cfg.V, c->logits_buf, m->cfg.V * sizeof(float),
+                          hipMemcpyDeviceToHost, c->stream));
+  }
+  PG_HIP(hipStreamSynchronize(c->stream));
+  return PG_OK;
+}
+
+uint32_t pg_logits_rows(const pg_logits* l) { return l ? l->rows : 0; }
+uint64_t pg_logits_vocab(const pg_logits* l) { return l ? l->vocab : 0; }
+
+pg_status pg_logits_argmax(pg_logits* l, uint32_t* out) {
+  if (!l || !out) return fail(PG_INVALID_INPUT, "null argument");
+  pg_kv_cache* c = l->owner;
+  if (!c->logits_valid) return fail(PG_INVALID_INPUT, "logits handle is stale");
+  pg_status s;
+  if ((s = select_device(c->device))) return s;
+  for (uint32_t r = 0; r < l->rows; ++r)
+    PG_HIP(pgk::launch_argmax(l->data + (size_t)r * l->vocab, (int)l->vocab, c->d_tok + r,
+                              c->stream));
+  PG_HIP(hipMemcpyAsync(c->h_ids, c->d_tok, l->rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                        c->stream));
+  PG_HIP(hipStreamSynchronize(c->stream));
+  std::memcpy(out, c->h_ids, l->rows * sizeof(uint32_t));
+  return PG_OK;
+}
+
+pg_status pg_logits_copy_to_host(pg_logits* l, float* dst, size_t len) {
+  if (!l || !dst) return fail(PG_INVALID_INPUT, "null argument");
+  pg_kv_cache* c = l->owner;
+  if (!c->logits_valid) return fail(PG_INVALID_INPUT, "logits handle is stale");
+  if (len != (size_t)l->rows * l->vocab)
+    return fail(PG_INVALID_INPUT, "logits copy length does not match rows * vocab");
+  pg_status s;
+  if ((s = select_device(c->device))) return s;
+  PG_HIP(hipStreamSynchronize(c->stream));
+  PG_HIP(hipMemcpy(dst, l->data, len * sizeof(float), hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_sampling_validate(const pg_sampling* c) {
+  if (!c) return fail(PG_INVALID_INPUT, "null argument");
+  if (!std::isfinite(c->temperature) || c->temperature < 0.0f)
+    return fail(PG_INVALID_CONFIG, "generation temperature must be finite and >= 0");
+  if (c->has_top_p && (!std::isfinite(c->top_p) || c->top_p <= 0.0f || c->top_p > 1.0f))
+    return fail(PG_INVALID_CONFIG, "generation top_p must be finite and in (0, 1]");
+  if (c->has_top_k && c->top_k == 0)
+    return fail(PG_INVALID_CONFIG, "generation top_k must be > 0");
+  if (!std::isfinite(c->repeat_penalty) || c->repeat_penalty <= 0.0f)
+    return fail(PG_INVALID_CONFIG, "generation repeat_penalty must be finite and > 0");
+  return PG_OK;
+}
+
+void pg_rng_seed(pg_rng_state* rng, uint64_t seed) { rng->state = seed ^ 0x9e3779b97f4a7c15ULL; }
+uint64_t pg_rng_next_u64(pg_rng_state* rng) {
+  rng->state += 0x9e3779b97f4a7c15ULL;
+  uint64_t v = rng->state;
+  v = (v ^ (v >> 30)) * 0xbf58476d1ce4e5b9ULL;
+  v = (v ^ (v >> 27)) * 0x94d049bb133111ebULL;
+  return v ^ (v >> 31);
+}
+double pg_rng_next_unit_f64(pg_rng_state* rng) {
+  return (double)(pg_rng_next_u64(rng) >> 11) * (1.0 / (double)(1ULL << 53));
+}
+
+pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, size_t n_hist,
+                           const pg_sampling* sampling, pg_rng_state* rng, uint32_t* out) {
+  if (!l || !sampling || !rng || !out) return fail(PG_INVALID_INPUT, "null argument");
+  if (row >= l->rows) return fail(PG_INVALID_INPUT, "logits row out of range");
+  pg_kv_cache* c = l->owner;
+  if (!c->logits_valid) return fail(PG_INVALID_INPUT, "logits handle is stale");
+  pg_status s;
+  if ((s = select_device(c->device))) return s;
+  const bool penalised = !(sampling->repeat_penalty == 1.0f || sampling->repeat_last_n == 0);
+  if (sampling->temperature <= 0.0f && !penalised) {
+    // Pure greedy: argmax on the device, only the id crosses to the host.
+    PG_HIP(pgk::launch_argmax(l->data + (size_t)row * l->vocab, (int)l->vocab, c->d_tok + row,
+                              c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_ids, c->d_tok + row, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));
+    *out = c->h_ids[0];
+    return PG_OK;
+  }
+  std::vector<float> adjusted(l->vocab);
+  PG_HIP(hipStreamSynchronize(c->stream));
+  PG_HIP(hipMemcpy(adjusted.data(), l->data + (size_t)row * l->vocab, l->vocab * sizeof(float),
+                   hipMemcpyDeviceToHost));
+  apply_repeat_penalty(adjusted, history, n_hist, sampling->repeat_penalty,
+                       sampling->repeat_last_n);
+  if (sampling->temperature <= 0.0f) {
+    *out = (uint32_t)argmax_host(adjusted.data(), adjusted.size());
+    return PG_OK;
+  }
+  return sample_logits(adjusted, *sampling, rng, out);
+}
+
+pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t steps,
+                                      uint32_t* out_ids, pg_generation_stats* stats) {
+  if (!m || !c || !out_ids) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = check_compatible(m, c))) return s;
+  if (!c->logits_valid)
+    return fail(PG_INVALID_INPUT, "decode needs logits from prefill or forward_one");
+  if ((s = select_device(m->device))) return s;
+  const size_t B = c->B, V = m->cfg.V;
+  // Selecting a token needs no cache slot; each forward after it does.
+  size_t room = c->cfg.P - c->seq_len;  // forwards still possible
+  size_t n_steps = std::min<size_t>(steps, room + 1);
+  auto t0 = Clock::now();
+  PG_HIP(hipEventRecord(c->ev0, c->stream));
+  for (size_t i = 0; i < n_steps; ++i) {
+    for (size_t b = 0; b < B; ++b)
+      PG_HIP(pgk::launch_argmax(c->logits_buf + b * V, (int)V, c->d_tok + b, c->stream));
+    PG_HIP(hipMemcpyAsync(c->d_out_ids + i * B, c->d_tok, B * sizeof(uint32_t),
+                          hipMemcpyDeviceToDevice, c->stream));
+    bool needs_next = i + 1 < n_steps;  // rust.rs:518-528: no forward after the last token
+    if (needs_next) {
+      for (size_t b = 0; b < B; ++b)
+        if ((s = enqueue_forward_one(m, c, b, c->d_tok + b, 0, c->seq_len, true))) return s;
+      c->seq_len += 1;
+    }
+  }
+  PG_HIP(hipEventRecord(c->ev1, c->stream));
+  PG_HIP(hipMemcpyAsync(c->h_ids, c->d_out_ids, n_steps * B * sizeof(uint32_t),
+                        hipMemcpyDeviceToHost, c->stream));
+  PG_HIP(hipStreamSynchronize(c->stream));
+  std::memcpy(out_ids, c->h_ids, n_steps * B * sizeof(uint32_t));
+  c->logits_valid = false;  // the logits the last selection used are consumed
+  if (stats) {
+    float ms = 0.0f;
+    PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    stats->generated_tokens = n_steps;
+    stats->decode_s = since(t0);
+    stats->gpu_decode_s = ms * 1e-3;
+  }
+  return PG_OK;
+}
+
+pg_status pg_gpt2_decode_greedy(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t max_new,
+                                int64_t eos, uint32_t* out_ids, uint32_t* out_n,
+                                pg_generation_stats* stats) {
+  if (!m || !c || !out_ids || !out_n) return fail(PG_INVALID_INPUT, "null argument");
+  if (c->B != 1) return fail(PG_INVALID_INPUT, "decode_greedy needs a cache of batch 1");
+  if (eos >= 0 && (uint64_t)eos >= m->cfg.V)
+    return fail(PG_INVALID_CONFIG, "generation eos_token_id " + std::to_string(eos) +
+                                       " is outside vocab_size " + std::to_string(m->cfg.V));
+  *out_n = 0;
+  if (max_new == 0) return PG_OK;
+  const size_t start_len = c->seq_len;
+  size_t room = c->cfg.P - c->seq_len;
+  size_t n_steps = std::min<size_t>(max_new, room + 1);
+  std::vector<uint32_t> ids(n_steps);
+  pg_generation_stats st{};
+  pg_status s = pg_gpt2_decode_greedy_batch(m, c, (uint32_t)n_steps, ids.data(), &st);
+  if (s) return s;
+  size_t n = st.generated_tokens;
+  if (eos >= 0) {
+    // EOS is tested before the push (rust.rs:503-505): drop it and what follows,
+    // and rewind the cache to the forwards the reference would have run.
+    for (size_t i = 0; i < n; ++i)
+      if (ids[i] == (uint32_t)eos) {
+        n = i;
+        c->seq_len = start_len + i;
+        break;
+      }
+  }
+  std::memcpy(out_ids, ids.data(), n * sizeof(uint32_t));
+  *out_n = (uint32_t)n;
+  if (stats) {
+    *stats = st;
+    stats->generated_tokens = n;
+  }
+  return PG_OK;
+}
+
+pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint32_t* ids,
+                                              size_t n, uint32_t max_new, int64_t eos,
+                                              const pg_sampling* sampling, uint64_t seed,
+                                              pg_on_token on_token, void* user, uint32_t* out_ids,
+                                              size_t* out_n, pg_generation_stats* stats) {
+  if (!m || !sampling || !out_ids || !out_n) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = pg_sampling_validate(sampling))) return s;
+  if (eos >= 0 && (uint64_t)eos >= m->cfg.V)  // rust.rs:558-566
+    return fail(PG_INVALID_CONFIG, "generation eos_token_id " + std::to_string(eos) +
+                                       " is outside vocab_size " + std::to_string(m->cfg.V));
+  pg_kv_cache* c = nullptr;
+  if ((s = pg_kv_cache_create(m, 1, &c))) return s;
+  std::unique_ptr<pg_kv_cache, void (*)(pg_kv_cache*)> holder(c, pg_kv_cache_destroy);
+  auto first_start = Clock::now();
+  auto prefill_start = Clock::now();
+  pg_logits* logits = nullptr;
+  if ((s = pg_gpt2_prefill(m, c, ids, n, &logits))) return s;
+  double prefill_s = since(prefill_start);
+  std::vector<uint32_t> output(ids, ids + n);
+  auto decode_start = Clock::now();
+  double first_token_s = -1.0;
+  uint64_t generated = 0;
+  pg_rng_state rng;
+  pg_rng_seed(&rng, seed);
+  for (uint32_t it = 0; it < max_new; ++it) {
+    if (output.size() >= m->cfg.P) break;
+    uint32_t tok = 0;
+    if ((s = pg_logits_sample(logits, 0, output.data(), output.size(), sampling, &rng, &tok)))
+      return s;
+    if (eos >= 0 && (uint32_t)eos == tok) break;
+    output.push_back(tok);
+    if (on_token && on_token(tok, user) != 0)
+      return fail(PG_INVALID_INPUT, "on_token callback stopped generation");
+    generated += 1;
+    if (first_token_s < 0) first_token_s = since(first_start);
+    bool needs_next = generated < max_new && output.size() < m->cfg.P;
+    if (needs_next)
+      if ((s = pg_gpt2_forward_one(m, c, tok, &logits))) return s;
+  }
+  double decode_s = since(decode_start);
+  std::memcpy(out_ids, output.data(), output.size() * sizeof(uint32_t));
+  *out_n = output.size();
+  if (stats) {
+    stats->prompt_tokens = n;
+    stats->generated_tokens = generated;
+    stats->prefill_s = prefill_s;
+    stats->decode_s = decode_s;
+    stats->first_token_s = first_token_s;
+    stats->gpu_decode_s = 0.0;
+  }
+  return PG_OK;
+}
+
+// ---- op-level entry points ---------------------------------------------------
+
+pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in_f,
+                      uint64_t out_f, const float* weight, const float* bias, float* out) {
+  if (!x || !weight || !bias || !out) return fail(PG_INVALID_INPUT, "null argument");
+  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30))
+    return fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  DevBuf dx, dw, db, dy;
+  if ((s = dx.alloc(rows * in_f)) || (s = dw.alloc(in_f * out_f)) || (s = db.alloc(out_f)) ||
+      (s = dy.alloc(rows * out_f)))
+    return s;
+  PG_HIP(hipMemcpy(dx.p, x, rows * in_f * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(dw.p, weight, in_f * out_f * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(db.p, bias, out_f * 4, hipMemcpyHostToDevice));
+  for (uint64_t r = 0; r < rows; ++r) {
+    pgk::GemvArgs a{};
+    a.W = dw.p; a.bias = db.p; a.x = dx.p + r * in_f; a.y = dy.p + r * out_f;
+    a.K = (int)in_f; a.nout = (int)out_f;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_BIAS, nullptr));
+  }
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(out, dy.p, rows * out_f * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_layer_norm(int32_t device, float* x, uint64_t rows, uint64_t cols,
+                           const float* gamma, const float* beta, float eps) {
+  if (!x || !gamma || !beta) return fail(PG_INVALID_INPUT, "null argument");
+  if (cols == 0 || cols > 16384 || rows > (1u << 30))
+    return fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16384]");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0) return PG_OK;
+  DevBuf dx, dg, db;
+  if ((s = dx.alloc(rows * cols)) || (s = dg.alloc(cols)) || (s = db.alloc(cols))) return s;
+  PG_HIP(hipMemcpy(dx.p, x, rows * cols * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(dg.p, gamma, cols * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(db.p, beta, cols * 4, hipMemcpyHostToDevice));
+  PG_HIP(pgk::launch_layer_norm(dx.p, (int)rows, (int)cols, dg.p, db.p, eps, nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(x, dx.p, rows * cols * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_gelu(int32_t device, float* v, uint64_t n) {
+  if (!v) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (n == 0) return PG_OK;
+  DevBuf d;
+  if ((s = d.alloc(n))) return s;
+  PG_HIP(hipMemcpy(d.p, v, n * 4, hipMemcpyHostToDevice));
+  PG_HIP(pgk::launch_gelu(d.p, n, nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(v, d.p, n * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_softmax(int32_t device, float* v, uint64_t rows, uint64_t cols) {
+  if (!v) return fail(PG_INVALID_INPUT, "null argument");
+  if (rows > (1u << 30) || cols > (1u << 30))
+    return fail(PG_INVALID_INPUT, "softmax: rows/cols too large");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0 || cols == 0) return PG_OK;
+  DevBuf d;
+  if ((s = d.alloc(rows * cols))) return s;
+  PG_HIP(hipMemcpy(d.p, v, rows * cols * 4, hipMemcpyHostToDevice));
+  PG_HIP(pgk::launch_softmax(d.p, (int)rows, (int)cols, nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(v, d.p, rows * cols * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_add(int32_t device, float* dst, const float* src, uint64_t n) {
+  if (!dst || !src) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (n == 0) return PG_OK;
+  DevBuf a, b;
+  if ((s = a.alloc(n)) || (s = b.alloc(n))) return s;
+  PG_HIP(hipMemcpy(a.p, dst, n * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(b.p, src, n * 4, hipMemcpyHostToDevice));
+  PG_HIP(pgk::launch_add(a.p, b.p, n, nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(dst, a.p, n * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_attention_decode(int32_t device, const float* qkv, uint64_t pos, float* keys,
+                                 float* values, uint64_t max_seq_len, uint64_t n_head,
+                                 uint64_t head_dim, float* out) {
+  if (!qkv || !keys || !values || !out) return fail(PG_INVALID_INPUT, "null argument");
+  if (n_head == 0 || head_dim == 0 || max_seq_len == 0 || max_seq_len > 16384 ||
+      n_head * head_dim > 16384)
+    return fail(PG_INVALID_INPUT, "attention: dimensions out of range");
+  if (pos >= max_seq_len)
+    return fail(PG_INVALID_INPUT, "cache is full at seq_len " + std::to_string(pos));
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  const size_t C = n_head * head_dim, panel = n_head * max_seq_len * head_dim;
+  hipDeviceProp_t prop;
+  PG_HIP(hipGetDeviceProperties(&prop, device));
+  const int nsplit = head_dim == (uint64_t)pgk::kHeadDim
+                         ? pgk::choose_nsplit((int)pos + 1, (int)n_head, prop.multiProcessorCount)
+                         : 1;
+  DevBuf dq, dk, dv, pa, pm, pl, dout;
+  if ((s = dq.alloc(3 * C)) || (s = dk.alloc(panel)) || (s = dv.alloc(panel)) ||
+      (s = pa.alloc(n_head * nsplit * head_dim)) || (s = pm.alloc(n_head * nsplit)) ||
+      (s = pl.alloc(n_head * nsplit)) || (s = dout.alloc(C)))
+    return s;
+  PG_HIP(hipMemcpy(dq.p, qkv, 3 * C * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(dk.p, keys, panel * 4, hipMemcpyHostToDevice));
+  PG_HIP(hipMemcpy(dv.p, values, panel * 4, hipMemcpyHostToDevice));
+  // K/V append (rust.rs:1677-1683): strided copy of this token's rows.
+  PG_HIP(hipMemcpy2D(dk.p + pos * head_dim, max_seq_len * head_dim * 4, dq.p + C, head_dim * 4,
+                     head_dim * 4, n_head, hipMemcpyDeviceToDevice));
+  PG_HIP(hipMemcpy2D(dv.p + pos * head_dim, max_seq_len * head_dim * 4, dq.p + 2 * C,
+                     head_dim * 4, head_dim * 4, n_head, hipMemcpyDeviceToDevice));
+  PG_HIP(pgk::launch_attn_decode(dq.p, dk.p, dv.p, (int)pos, (int)max_seq_len, (int)n_head,
+                                 (int)head_dim, nsplit, pa.p, pm.p, pl.p, nullptr));
+  PG_HIP(pgk::launch_attn_finish(pa.p, pm.p, pl.p, (int)n_head, (int)head_dim, nsplit, dout.p,
+                                 nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(out, dout.p, C * 4, hipMemcpyDeviceToHost));
+  PG_HIP(hipMemcpy(keys, dk.p, panel * 4, hipMemcpyDeviceToHost));
+  PG_HIP(hipMemcpy(values, dv.p, panel * 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+pg_status pg_op_argmax(int32_t device, const float* v, uint64_t n, uint32_t* out) {
+  if (!v || !out) return fail(PG_INVALID_INPUT, "null argument");
+  if (n > (1u << 30)) return fail(PG_INVALID_INPUT, "argmax: too many values");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (n == 0) {
+    *out = 0;
+    return PG_OK;
+  }
+  DevBuf d, r;
+  if ((s = d.alloc(n)) || (s = r.alloc(1))) return s;
+  PG_HIP(hipMemcpy(d.p, v, n * 4, hipMemcpyHostToDevice));
+  PG_HIP(pgk::launch_argmax(d.p, (int)n, reinterpret_cast<uint32_t*>(r.p), nullptr));
+  PG_HIP(hipStreamSynchronize(nullptr));
+  PG_HIP(hipMemcpy(out, r.p, 4, hipMemcpyDeviceToHost));
+  return PG_OK;
+}
+
+// ---- synthetic inputs ---------------------------------------------------------
+
+static inline uint64_t splitmix_at(uint64_t seed, uint64_t j) {
+  // Output number j (0-based) of SmallRng::new(seed): the state is a counter.
+  uint64_t v = (seed ^ 0x9e3779b97f4a7c15ULL) + (j + 1) * 0x9e3779b97f4a7c15ULL;
+  v = (v ^ (v >> 30)) * 0xbf58476d1ce4e5b9ULL;
+  v = (v ^ (v >> 27)) * 0x94d049bb133111ebULL;
+  return v ^ (v >> 31);
+}
+
+void pg_synth_normal_f32(float* dst, uint64_t n, uint64_t seed, uint64_t first, double std_) {
+  const double inv53 = 1.0 / (double)(1ULL << 53);
+  const double two_pi = 6.283185307179586476925286766559;
+  auto work = [&](uint64_t lo, uint64_t hi) {
+    for (uint64_t i = lo; i < hi; ++i) {
+      uint64_t e = first + i;
+      double u1 = (double)((splitmix_at(seed, 2 * e) >> 11) + 1) * inv53;
+      double u2 = (double)(splitmix_at(seed, 2 * e + 1) >> 11) * inv53;
+      double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(two_pi * u2);
+      dst[i] = (float)(z * std_);
+    }
+  };
+  unsigned hw = std::thread::hardware_concurrency();
+  unsigned nt = std::max(1u, std::min(hw ? hw : 1u, 16u));
+  if (n < (1u << 16)) nt = 1;
+  if (nt == 1) {
+    work(0, n);
+    return;
+  }
+  std::vector<std::thread> th;
+  uint64_t per = (n + nt - 1) / nt;
+  for (unsigned t = 0; t < nt; ++t) {
+    uint64_t lo = std::min<uint64_t>(n, t * per), hi = std::min<uint64_t>(n, lo + per);
+    if (lo < hi) th.emplace_back(work, lo, hi);
+  }
+  for (auto& t : th) t.join();
+}
+
+void pg_synth_token_ids(uint32_t* dst, uint64_t n, uint64_t seed, uint64_t vocab) {
+  for (uint64_t i = 0; i < n; ++i) dst[i] = (uint32_t)(splitmix_at(seed, i) % vocab);
+}
+
+pg_status pg_device_query(int32_t device, pg_device_info* out) {
+  if (!out) return fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  hipDeviceProp_t prop;
+  PG_HIP(hipGetDeviceProperties(&prop, device));
+  std::memset(out, 0, sizeof(*out));
+  std::snprintf(out->name, sizeof(out->name), "%s", prop.name);
+  std::snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+  out->compute_units = (uint32_t)prop.multiProcessorCount;
+  out->total_mem_bytes = prop.totalGlobalMem;
+  out->lds_bytes_per_block = (uint32_t)prop.sharedMemPerBlock;
+  return PG_OK;
+}
+
+}  // extern "C"

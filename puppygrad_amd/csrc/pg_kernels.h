@@ -1,0 +1,81 @@
+// Launchers for the gfx950 kernels of the GPT-2 decode/prefill path.
+// Internal to libpuppygrad_hip.so; the public surface is include/puppygrad_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pgk {
+
+constexpr int kHeadDim = 64;       // every GPT-2 size has head_dim 64; other sizes use the generic path
+constexpr int kMaxSplits = 32;     // upper bound on key splits per head in decode attention
+
+// Device-side view of one transformer block.  Matrices are [out,in] row-major.
+struct LayerW {
+  const float *ln_1_g, *ln_1_b;
+  const float *c_attn_w, *c_attn_b;   // [3C][C], [3C]
+  const float *c_proj_w, *c_proj_b;   // [C][C], [C]
+  const float *ln_2_g, *ln_2_b;
+  const float *c_fc_w, *c_fc_b;       // [I][C], [I]
+  const float *c_proj_mlp_w, *c_proj_mlp_b;  // [C][I], [C]
+};
+
+enum Prologue : int { PRO_NONE = 0, PRO_LN = 1, PRO_ATTN_COMBINE = 2 };
+enum Epilogue : int { EPI_BIAS = 0, EPI_GELU = 1, EPI_RESID = 2, EPI_QKV = 3 };
+
+// y = epilogue(bias + W . prologue(x)) for one input vector.
+struct GemvArgs {
+  const float* W;      // [nout][K]
+  const float* bias;   // [nout] or nullptr (treated as 0)
+  const float* x;      // [K] input (PRO_NONE / PRO_LN)
+  float* y;            // [nout] output (EPI_BIAS / EPI_GELU / EPI_RESID); q for EPI_QKV
+  int K;
+  int nout;
+  // PRO_LN
+  const float* ln_g;
+  const float* ln_b;
+  float eps;
+  // PRO_ATTN_COMBINE: partial attention results per (head, split)
+  const float* part_acc;  // [H][nsplit][hd]
+  const float* part_m;    // [H][nsplit]
+  const float* part_l;    // [H][nsplit]
+  int nsplit;
+  int head_dim;
+  // EPI_RESID
+  const float* resid;  // [nout]
+  // EPI_QKV: rows [C,2C) go to kcache, [2C,3C) to vcache at position pos
+  float* kcache;  // [H][P][hd]
+  float* vcache;
+  int pos;
+  int P;
+  int C;
+};
+
+hipError_t launch_gemv(const GemvArgs& a, int prologue, int epilogue, hipStream_t s);
+
+// x = wte[tok] + wpe[pos]; tok comes from tok_ptr[0] when tok_ptr != nullptr.
+hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
+                        uint32_t tok, int pos, int C, hipStream_t s);
+
+// Split-key decode attention for one query over keys [0, pos].
+hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
+                              int P, int H, int head_dim, int nsplit, float* part_acc,
+                              float* part_m, float* part_l, hipStream_t s);
+int choose_nsplit(int n_keys, int H, int num_cus);
+
+// out[0] = argmax with the reference's tie/NaN rules.
+hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s);
+
+// Stand-alone forms of the cpu.rs ops (rows handled one block each).
+hipError_t launch_layer_norm(float* x, int rows, int cols, const float* g, const float* b,
+                             float eps, hipStream_t s);
+hipError_t launch_gelu(float* v, size_t n, hipStream_t s);
+hipError_t launch_softmax(float* v, int rows, int cols, hipStream_t s);
+hipError_t launch_add(float* dst, const float* src, size_t n, hipStream_t s);
+// dst[o*in + i] = src[i*out + o]
+hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, hipStream_t s);
+// Attention output from a single split's (acc, m, l): out = acc / l per head.
+hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
+                              int H, int head_dim, int nsplit, float* out, hipStream_t s);
+hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
+
+}  // namespace pgk

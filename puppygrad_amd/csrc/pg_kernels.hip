@@ -1,0 +1,529 @@
+// gfx950 kernels for the GPT-2 decode path, one launch per fused op.
+//
+// Semantics follow puppygrad's CPU kernels (src/models/cpu.rs) and its cached
+// forward (src/models/gpt2/rust.rs:1136-1250, 1662-1741); each kernel names the
+// function it covers.  All arithmetic is f32 with f32 accumulation.
+//
+// Shapes the launchers assume are checked on the host before any launch
+// (pg_host.cpp); kernels themselves guard only the ragged tails.
+#include "pg_kernels.h"
+
+#include <math.h>
+
+namespace pgk {
+
+namespace {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;  // 4 wavefronts of 64 lanes
+constexpr int kWaves = kBlock / 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+// Sum over the block; every thread receives the result.  red holds kWaves floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();  // red may still be read from a previous reduction
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) t += red[w];
+  return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) t = fmaxf(t, red[w]);
+  return t;
+}
+
+// gelu_in_place (cpu.rs:145-150).
+__device__ __forceinline__ float gelu_tanh(float x) {
+  return 0.5f * x * (1.0f + tanhf(0.7978846f * (x + 0.044715f * x * x * x)));
+}
+
+// layer_norm_in_place (cpu.rs:119-143) on a vector already staged in LDS:
+// two-pass mean / biased variance, eps inside the sqrt.
+__device__ __forceinline__ void ln_in_lds(float* sx, int K, const float* g, const float* b,
+                                          float eps, float* red) {
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < K; i += kBlock) s += sx[i];
+  float mean = block_sum(s, red) / (float)K;
+  float v = 0.0f;
+  for (int i = threadIdx.x; i < K; i += kBlock) {
+    float d = sx[i] - mean;
+    v += d * d;
+  }
+  float var = block_sum(v, red) / (float)K;
+  float inv = 1.0f / sqrtf(var + eps);
+  for (int i = threadIdx.x; i < K; i += kBlock) sx[i] = (sx[i] - mean) * inv * g[i] + b[i];
+  __syncthreads();
+}
+
+// Merge of per-split attention partials (acc, m, l) into the attention output
+// for element i = h*hd + d:  sum_s e^{m_s-M} acc_s[d] / sum_s e^{m_s-M} l_s.
+__device__ __forceinline__ float attn_combine_elem(const float* part_acc, const float* part_m,
+                                                   const float* part_l, int nsplit, int hd,
+                                                   int i) {
+  int h = i / hd, d = i - h * hd;
+  const float* m = part_m + h * nsplit;
+  const float* l = part_l + h * nsplit;
+  float M = m[0];
+  for (int s = 1; s < nsplit; ++s) M = fmaxf(M, m[s]);
+  float num = 0.0f, den = 0.0f;
+  for (int s = 0; s < nsplit; ++s) {
+    float w = expf(m[s] - M);
+    den += w * l[s];
+    num += w * part_acc[(size_t)(h * nsplit + s) * hd + d];
+  }
+  return num / den;
+}
+
+// transposed_dense_projection_into (cpu.rs:58-75) for one row of x, with the
+// producer of x (LayerNorm or the attention merge) and the consumer of y
+// (GELU, residual add, K/V cache append) folded in.  One wavefront owns RPW
+// weight rows; lanes stride over the row in float4 and reduce at the end.
+template <int PRO, int EPI, int RPW, bool VEC4>
+__global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
+  extern __shared__ float sx[];  // K floats
+  __shared__ float red[kWaves];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = a.K;
+
+  if (PRO == PRO_ATTN_COMBINE) {
+    for (int i = tid; i < K; i += kBlock)
+      sx[i] = attn_combine_elem(a.part_acc, a.part_m, a.part_l, a.nsplit, a.head_dim, i);
+  } else {
+    for (int i = tid; i < K; i += kBlock) sx[i] = a.x[i];
+  }
+  __syncthreads();
+  if (PRO == PRO_LN) ln_in_lds(sx, K, a.ln_g, a.ln_b, a.eps, red);
+
+  const int row0 = (blockIdx.x * kWaves + wave) * RPW;
+  if (row0 >= a.nout) return;
+  float acc[RPW];
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) acc[r] = 0.0f;
+
+  if (VEC4) {
+    const int K4 = K >> 2;
+    const float4* sx4 = reinterpret_cast<const float4*>(sx);
+    const f4* W4 = reinterpret_cast<const f4*>(a.W);
+#pragma unroll 2
+    for (int j = lane; j < K4; j += 64) {
+      float4 xv = sx4[j];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) {
+          f4 w = __builtin_nontemporal_load(&W4[(size_t)row * K4 + j]);
+          acc[r] += w.x * xv.x + w.y * xv.y + w.z * xv.z + w.w * xv.w;
+        }
+      }
+    }
+  } else {
+    for (int j = lane; j < K; j += 64) {
+      float xv = sx[j];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) acc[r] += a.W[(size_t)row * K + j] * xv;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) acc[r] = wave_sum(acc[r]);
+
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      int o = row0 + r;
+      if (o >= a.nout) break;
+      float v = (a.bias ? a.bias[o] : 0.0f) + acc[r];
+      if (EPI == EPI_BIAS) {
+        a.y[o] = v;
+      } else if (EPI == EPI_GELU) {
+        a.y[o] = gelu_tanh(v);
+      } else if (EPI == EPI_RESID) {
+        a.y[o] = a.resid[o] + v;  // add_in_place (cpu.rs:167-171)
+      } else {  // EPI_QKV: K/V append of cached_self_attention_into (rust.rs:1677-1683)
+        if (o < a.C) {
+          a.y[o] = v;
+        } else {
+          int which = o >= 2 * a.C;
+          int c = o - (which ? 2 * a.C : a.C);
+          int h = c / a.head_dim, d = c - h * a.head_dim;
+          float* dst = which ? a.vcache : a.kcache;
+          dst[((size_t)h * a.P + a.pos) * a.head_dim + d] = v;
+        }
+      }
+    }
+  }
+}
+
+// Embedding of one token (rust.rs:966-974).
+__global__ void k_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
+                        uint32_t tok, int pos, int C) {
+  uint32_t t = tok_ptr ? tok_ptr[0] : tok;
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < C) x[i] = wte[(size_t)t * C + i] + wpe[(size_t)pos * C + i];
+}
+
+// cached_self_attention_into (rust.rs:1721-1740) for head_dim 64, keys split
+// over blockIdx.x.  A block scores its keys with 16 lanes per key (float4 each),
+// takes the max-subtracted exponentials (softmax_in_place, cpu.rs:152-165) and
+// accumulates p.V; the per-split (acc, m, l) are merged by the consumer.
+__global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restrict__ q,
+                                                          const float* __restrict__ kcache,
+                                                          const float* __restrict__ vcache,
+                                                          int pos, int P, int nsplit,
+                                                          float* part_acc, float* part_m,
+                                                          float* part_l) {
+  extern __shared__ float sc[];  // scores of this split
+  __shared__ float red[kWaves];
+  __shared__ float accs[kWaves][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.x, h = blockIdx.y;
+  const int n = pos + 1;
+  const int per = (n + nsplit - 1) / nsplit;
+  const int k0 = split * per;
+  const int k1 = min(n, k0 + per);
+  const size_t pidx = (size_t)h * nsplit + split;
+  if (k0 >= k1) {  // empty split: contributes nothing to the merge
+    if (tid < 64) part_acc[pidx * 64 + tid] = 0.0f;
+    if (tid == 0) {
+      part_m[pidx] = -INFINITY;
+      part_l[pidx] = 0.0f;
+    }
+    return;
+  }
+  const int sub = lane >> 4, d4 = lane & 15;
+  const float4 qv = reinterpret_cast<const float4*>(q + h * 64)[d4];
+  const float4* K4 = reinterpret_cast<const float4*>(kcache + (size_t)h * P * 64);
+  const float4* V4 = reinterpret_cast<const float4*>(vcache + (size_t)h * P * 64);
+  const float scale = 1.0f / sqrtf(64.0f);
+
+  float mx = -INFINITY;
+  for (int k = k0 + wave * 4 + sub; k < k1; k += kWaves * 4) {
+    float4 kv = K4[(size_t)k * 16 + d4];
+    float s = qv.x * kv.x + qv.y * kv.y + qv.z * kv.z + qv.w * kv.w;
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    s += __shfl_xor(s, 4, 64);
+    s += __shfl_xor(s, 8, 64);
+    s *= scale;
+    if (d4 == 0) sc[k - k0] = s;
+    mx = fmaxf(mx, s);
+  }
+  mx = block_max(mx, red);  // includes the barrier that publishes sc[]
+
+  float lsum = 0.0f;
+  for (int i = tid; i < k1 - k0; i += kBlock) {
+    float p = expf(sc[i] - mx);
+    sc[i] = p;
+    lsum += p;
+  }
+  lsum = block_sum(lsum, red);
+
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = k0 + wave * 4 + sub; k < k1; k += kWaves * 4) {
+    float p = sc[k - k0];
+    float4 vv = V4[(size_t)k * 16 + d4];
+    acc.x += p * vv.x;
+    acc.y += p * vv.y;
+    acc.z += p * vv.z;
+    acc.w += p * vv.w;
+  }
+#pragma unroll
+  for (int off = 16; off <= 32; off <<= 1) {
+    acc.x += __shfl_xor(acc.x, off, 64);
+    acc.y += __shfl_xor(acc.y, off, 64);
+    acc.z += __shfl_xor(acc.z, off, 64);
+    acc.w += __shfl_xor(acc.w, off, 64);
+  }
+  if (sub == 0) reinterpret_cast<float4*>(accs[wave])[d4] = acc;
+  __syncthreads();
+  if (tid < 64) {
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) t += accs[w][tid];
+    part_acc[pidx * 64 + tid] = t;
+  }
+  if (tid == 0) {
+    part_m[pidx] = mx;
+    part_l[pidx] = lsum;
+  }
+}
+
+// Same computation for any head_dim: one block per head, one split.
+__global__ __launch_bounds__(kBlock) void k_attn_decode_any(const float* q, const float* kcache,
+                                                            const float* vcache, int pos, int P,
+                                                            int hd, float* part_acc, float* part_m,
+                                                            float* part_l) {
+  extern __shared__ float sc[];
+  __shared__ float red[kWaves];
+  const int tid = threadIdx.x, h = blockIdx.y;
+  const int n = pos + 1;
+  const float scale = 1.0f / sqrtf((float)hd);
+  const float* Kh = kcache + (size_t)h * P * hd;
+  const float* Vh = vcache + (size_t)h * P * hd;
+  float mx = -INFINITY;
+  for (int k = tid; k < n; k += kBlock) {
+    float s = 0.0f;
+    for (int d = 0; d < hd; ++d) s += q[h * hd + d] * Kh[(size_t)k * hd + d];
+    s *= scale;
+    sc[k] = s;
+    mx = fmaxf(mx, s);
+  }
+  mx = block_max(mx, red);
+  float lsum = 0.0f;
+  for (int k = tid; k < n; k += kBlock) {
+    float p = expf(sc[k] - mx);
+    sc[k] = p;
+    lsum += p;
+  }
+  lsum = block_sum(lsum, red);
+  for (int d = tid; d < hd; d += kBlock) {
+    float t = 0.0f;
+    for (int k = 0; k < n; ++k) t += sc[k] * Vh[(size_t)k * hd + d];
+    part_acc[(size_t)h * hd + d] = t;
+  }
+  if (tid == 0) {
+    part_m[h] = mx;
+    part_l[h] = lsum;
+  }
+}
+
+__global__ void k_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
+                              int C, int hd, int nsplit, float* out) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < C) out[i] = attn_combine_elem(part_acc, part_m, part_l, nsplit, hd, i);
+}
+
+// argmax_logits (generation.rs:269-279): strict '>' from -inf, first maximum
+// wins, NaN never wins; with no winner the answer is 0.
+struct Best {
+  float v;
+  uint32_t i;
+};
+__device__ __forceinline__ Best better(Best a, Best b) {
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+__global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t* out) {
+  __shared__ float sv[16];
+  __shared__ uint32_t si[16];
+  Best b{-INFINITY, 0xffffffffu};
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    float x = v[i];
+    if (x > b.v) {
+      b.v = x;
+      b.i = (uint32_t)i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(b.v, off, 64), (uint32_t)__shfl_xor((int)b.i, off, 64)};
+    b = better(b, o);
+  }
+  int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    sv[wave] = b.v;
+    si[wave] = b.i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best r{sv[0], si[0]};
+    for (int w = 1; w < 16; ++w) r = better(r, Best{sv[w], si[w]});
+    out[0] = (r.i == 0xffffffffu) ? 0u : r.i;
+  }
+}
+
+// ---- stand-alone cpu.rs ops -------------------------------------------------
+
+__global__ __launch_bounds__(kBlock) void k_layer_norm(float* x, int cols, const float* g,
+                                                       const float* b, float eps) {
+  extern __shared__ float sx[];
+  __shared__ float red[kWaves];
+  float* row = x + (size_t)blockIdx.x * cols;
+  for (int i = threadIdx.x; i < cols; i += kBlock) sx[i] = row[i];
+  __syncthreads();
+  ln_in_lds(sx, cols, g, b, eps, red);
+  for (int i = threadIdx.x; i < cols; i += kBlock) row[i] = sx[i];
+}
+
+__global__ void k_gelu(float* v, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[i] = gelu_tanh(v[i]);
+}
+
+__global__ __launch_bounds__(kBlock) void k_softmax(float* v, int cols) {
+  __shared__ float red[kWaves];
+  float* row = v + (size_t)blockIdx.x * cols;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < cols; i += kBlock) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, red);
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += kBlock) {
+    float e = expf(row[i] - mx);
+    row[i] = e;
+    s += e;
+  }
+  s = block_sum(s, red);
+  for (int i = threadIdx.x; i < cols; i += kBlock) row[i] /= s;
+}
+
+__global__ void k_add(float* dst, const float* src, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] += src[i];
+}
+
+__global__ void k_fill_zero(float* p, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = 0.0f;
+}
+
+// transpose_in_out (cpu.rs:281-289): 32x32 tiles through LDS.
+__global__ void k_transpose(const float* src, float* dst, int in_f, int out_f) {
+  __shared__ float tile[32][33];
+  int o0 = blockIdx.x * 32, i0 = blockIdx.y * 32;
+  int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 256 threads: 8 rows per pass
+  for (int r = ty; r < 32; r += 8) {
+    int i = i0 + r, o = o0 + tx;
+    if (i < in_f && o < out_f) tile[r][tx] = src[(size_t)i * out_f + o];
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    int o = o0 + r, i = i0 + tx;
+    if (i < in_f && o < out_f) dst[(size_t)o * in_f + i] = tile[tx][r];
+  }
+}
+
+template <int PRO, int EPI>
+hipError_t launch_gemv_pe(const GemvArgs& a, hipStream_t s) {
+  const bool vec4 = (a.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.W) & 15) == 0);
+  const size_t lds = (size_t)a.K * sizeof(float);
+  // Two rows per wavefront once there are enough rows to fill the chip with
+  // 8-row blocks; otherwise one row per wavefront.
+  const bool two = a.nout >= 4096;
+  const int rpw = two ? 2 : 1;
+  const int blocks = (a.nout + kWaves * rpw - 1) / (kWaves * rpw);
+  if (vec4) {
+    if (two)
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, true>), dim3(blocks), dim3(kBlock), lds, s, a);
+    else
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, true>), dim3(blocks), dim3(kBlock), lds, s, a);
+  } else {
+    hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, false>), dim3((a.nout + kWaves - 1) / kWaves),
+                       dim3(kBlock), lds, s, a);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gemv(const GemvArgs& a, int prologue, int epilogue, hipStream_t s) {
+#define PG_CASE(P, E) \
+  if (prologue == P && epilogue == E) return launch_gemv_pe<P, E>(a, s);
+  PG_CASE(PRO_NONE, EPI_BIAS)
+  PG_CASE(PRO_NONE, EPI_RESID)
+  PG_CASE(PRO_NONE, EPI_GELU)
+  PG_CASE(PRO_LN, EPI_BIAS)
+  PG_CASE(PRO_LN, EPI_GELU)
+  PG_CASE(PRO_LN, EPI_QKV)
+  PG_CASE(PRO_ATTN_COMBINE, EPI_RESID)
+#undef PG_CASE
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
+                        uint32_t tok, int pos, int C, hipStream_t s) {
+  hipLaunchKernelGGL(k_embed, dim3((C + 255) / 256), dim3(256), 0, s, x, wte, wpe, tok_ptr, tok,
+                     pos, C);
+  return hipGetLastError();
+}
+
+int choose_nsplit(int n_keys, int H, int num_cus) {
+  // Enough (head, split) blocks to cover the CUs about twice, at least 16 keys each.
+  int want = (2 * num_cus + H - 1) / H;
+  int by_len = (n_keys + 15) / 16;
+  int ns = want < by_len ? want : by_len;
+  if (ns < 1) ns = 1;
+  if (ns > kMaxSplits) ns = kMaxSplits;
+  return ns;
+}
+
+hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
+                              int P, int H, int head_dim, int nsplit, float* part_acc,
+                              float* part_m, float* part_l, hipStream_t s) {
+  if (head_dim == kHeadDim) {
+    int per = (pos + 1 + nsplit - 1) / nsplit;
+    hipLaunchKernelGGL(k_attn_decode64, dim3(nsplit, H), dim3(kBlock), per * sizeof(float), s, q,
+                       kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l);
+  } else {
+    hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H), dim3(kBlock), (pos + 1) * sizeof(float), s,
+                       q, kcache, vcache, pos, P, head_dim, part_acc, part_m, part_l);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
+                              int H, int head_dim, int nsplit, float* out, hipStream_t s) {
+  int C = H * head_dim;
+  hipLaunchKernelGGL(k_attn_finish, dim3((C + 255) / 256), dim3(256), 0, s, part_acc, part_m,
+                     part_l, C, head_dim, nsplit, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s) {
+  hipLaunchKernelGGL(k_argmax, dim3(1), dim3(1024), 0, s, v, n, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_layer_norm(float* x, int rows, int cols, const float* g, const float* b,
+                             float eps, hipStream_t s) {
+  hipLaunchKernelGGL(k_layer_norm, dim3(rows), dim3(kBlock), cols * sizeof(float), s, x, cols, g,
+                     b, eps);
+  return hipGetLastError();
+}
+hipError_t launch_gelu(float* v, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_gelu, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, v, n);
+  return hipGetLastError();
+}
+hipError_t launch_softmax(float* v, int rows, int cols, hipStream_t s) {
+  hipLaunchKernelGGL(k_softmax, dim3(rows), dim3(kBlock), 0, s, v, cols);
+  return hipGetLastError();
+}
+hipError_t launch_add(float* dst, const float* src, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_add, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dst, src, n);
+  return hipGetLastError();
+}
+hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, hipStream_t s) {
+  hipLaunchKernelGGL(k_transpose, dim3((out_f + 31) / 32, (in_f + 31) / 32), dim3(256), 0, s, src,
+                     dst, in_f, out_f);
+  return hipGetLastError();
+}
+hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s) {
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks == 0) blocks = 1;
+  hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)blocks), dim3(256), 0, s, p, n);
+  return hipGetLastError();
+}
+
+}  // namespace pgk

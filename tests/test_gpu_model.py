@@ -1,0 +1,213 @@
+"""The HIP backend behind the reference's model API: the reference's own GPT-2
+unit tests (src/models/gpt2/rust.rs:1865-2020) re-run on it, plus logit parity
+with the oracle and the Hugging Face golden vectors."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import ABS_TOL, REL_TOL, assert_logits_close, load_golden, small_cases
+from puppygrad_amd import (Gpt2Error, Gpt2GenerationConfig, Gpt2Model, LogitsSampler,
+                           TextGenerationConfig, generate, synth)
+
+pytestmark = pytest.mark.gpu
+
+
+def tiny():
+    cfg = synth.tiny_config()
+    return cfg, Gpt2Model.new(cfg, synth.tiny_weights(cfg))
+
+
+def test_validates_weight_shapes():
+    cfg = synth.tiny_config()
+    w = synth.tiny_weights(cfg)
+    w.wte = w.wte[:-1]
+    with pytest.raises(Gpt2Error) as e:
+        Gpt2Model.new(cfg, w)
+    assert "wte len" in str(e.value) and e.value.kind == "InvalidWeights"
+
+
+def test_forward_returns_logits_for_each_position():
+    cfg, model = tiny()
+    out = model.forward([1, 2, 3])
+    assert out.seq_len == 3 and out.vocab_size == cfg.vocab_size
+    assert out.logits.shape == (3, cfg.vocab_size) and np.isfinite(out.logits).all()
+
+
+def test_greedy_generation_appends_tokens_until_context_limit():
+    cfg, model = tiny()
+    tokens = model.generate_greedy([0, 1], 10)
+    assert len(tokens) == cfg.n_positions and tokens[:2] == [0, 1]
+    assert all(t < cfg.vocab_size for t in tokens)
+
+
+def test_cached_prefill_matches_full_forward_last_logits():
+    cfg, model = tiny()
+    full = model.forward([1, 2, 3])
+    cache = model.new_kv_cache()
+    cached = model.prefill([1, 2, 3], cache).to_host()
+    assert cache.seq_len == 3
+    np.testing.assert_allclose(cached, full.last_logits(), atol=1e-5, rtol=0)
+
+
+def test_cached_greedy_generation_matches_full_generation():
+    _, model = tiny()
+    assert model.generate_greedy_cached([0, 1], 3) == model.generate_greedy([0, 1], 3)
+
+
+def test_streams_generated_tokens_in_order():
+    _, model = tiny()
+    streamed = []
+    tokens = model.stream_greedy_tokens([0, 1], 3, streamed.append)
+    assert tokens[:2] == [0, 1] and streamed == tokens[2:]
+
+
+def test_implements_generic_autoregressive_decoder():
+    _, model = tiny()
+    assert generate(model, [0, 1], 3, lambda _t: None) == model.generate_greedy_cached([0, 1], 3)
+
+
+def test_gpt2_cache_exposes_generic_kv_cache_contract():
+    cfg, model = tiny()
+    cache = model.new_kv_cache()
+    cache.seq_len = 2
+    assert cache.seq_len == 2 and cache.max_seq_len == cfg.n_positions
+    cache.clear()
+    assert cache.seq_len == 0
+
+
+def test_tokens_match_oracle_on_tiny():
+    cfg, model = tiny()
+    ref = oracle.Model(cfg, synth.tiny_weights(cfg))
+    assert model.generate_greedy_cached([0, 1], 3) == ref.generate([0, 1], 3)
+    toks, stats = model.stream_token_ids_with_stats([0, 1], Gpt2GenerationConfig(10))
+    want, st, _, _ = ref.stream_token_ids_with_stats([0, 1], 10, 50256 if cfg.vocab_size > 50256 else None)
+    assert toks == want and stats.generated_tokens == st.generated_tokens == 3
+
+
+def test_error_surface():
+    cfg, model = tiny()
+    cache = model.new_kv_cache()
+    with pytest.raises(Gpt2Error, match="input_ids must not be empty"):
+        model.prefill([], cache)
+    with pytest.raises(Gpt2Error, match="exceeds n_positions"):
+        model.prefill([0] * 6, cache)
+    with pytest.raises(Gpt2Error, match="at index 1 exceeds vocab_size"):
+        model.prefill([0, 8], cache)
+    with pytest.raises(Gpt2Error, match="exceeds vocab_size"):
+        model.forward_one(8, cache)
+    model.prefill([0, 1, 2, 3, 4], cache)
+    with pytest.raises(Gpt2Error, match="cache is full at seq_len 5"):
+        model.forward_one(1, cache)
+    other = Gpt2Model.new(synth.Gpt2Config(vocab_size=8, n_positions=6, n_embd=4, n_layer=1, n_head=2),
+                          synth.random_weights(synth.Gpt2Config(vocab_size=8, n_positions=6, n_embd=4,
+                                                                n_layer=1, n_head=2), 1))
+    with pytest.raises(Gpt2Error, match="cache max_seq_len 5 does not match n_positions 6"):
+        other.forward_one(1, cache)
+    bad = synth.tiny_config()
+    bad.n_head = 3
+    with pytest.raises(Gpt2Error, match="must be divisible by n_head"):
+        Gpt2Model.new(bad, synth.tiny_weights(synth.tiny_config()))
+    with pytest.raises(Gpt2Error, match="outside vocab_size"):
+        model.stream_token_ids_with_stats([0, 1], TextGenerationConfig(2, eos_token_id=8))
+    with pytest.raises(Gpt2Error, match="top_p"):
+        model.stream_token_ids_with_stats([0, 1], TextGenerationConfig(2, top_p=2.0))
+
+
+@pytest.mark.parametrize("case", small_cases(), ids=lambda c: c[0])
+def test_logits_match_oracle_small(case):
+    _, cfg, w, ids = case
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
+    assert_logits_close(model.forward(ids).logits, ref.forward(ids))
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    for tok in [1, 0, 5]:
+        if cache.seq_len >= cfg.n_positions:
+            break
+        assert_logits_close(model.forward_one(tok, cache).to_host(), ref.forward_one(tok, rcache))
+    for layer in range(cfg.n_layer):  # K/V cache layout is the reference's kv_index
+        for which in (0, 1):
+            np.testing.assert_allclose(cache.read_layer(layer, which)[:, :cache.seq_len],
+                                       rcache.read_layer(layer, which)[:, :rcache.seq_len],
+                                       atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["hf_c128_l2", "hf_c192_l3_h3", "hf_gpt2_small"])
+def test_logits_match_hf_golden(name):
+    cfg, w, z = load_golden(name)
+    model = Gpt2Model.new(cfg, w)
+    ids = z["ids"]
+    if cfg.vocab_size > 1000:
+        cache = model.new_kv_cache()
+        logits = model.prefill(ids, cache)
+        assert model.select_next_token(logits) == int(z["argmax"])
+        got = logits.to_host()[z["cols"]][None]
+    else:
+        got = model.forward(ids).logits[np.ix_(z["rows"], z["cols"])]
+    assert_logits_close(got, z["logits"])
+
+
+def test_sampler_on_device_logits_matches_oracle():
+    _, cfg, w, ids = small_cases()[1]
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    rlogits = ref.prefill(ids, rcache)
+    for kw in [dict(), dict(repeat_penalty=1.7), dict(temperature=0.9), dict(temperature=0.7, top_k=5),
+               dict(temperature=1.1, top_p=0.8), dict(temperature=0.8, top_k=20, top_p=0.5, repeat_penalty=1.3)]:
+        for seed in (1, 299792458):
+            g = TextGenerationConfig(1, seed=seed, **kw)
+            got = LogitsSampler(seed).select_next_token(logits, ids, g)
+            want = oracle.LogitsSampler(seed).select_next_token(
+                rlogits, ids, oracle.sampling(seed=seed, **kw))
+            assert got == want, (kw, seed)
+
+
+def test_sampled_stream_matches_oracle():
+    _, cfg, w, ids = small_cases()[1]
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
+    g = TextGenerationConfig(12, temperature=0.9, top_k=30, top_p=0.95, repeat_penalty=1.2, seed=7)
+    toks, stats = model.stream_token_ids_with_stats(ids, g)
+    want, st, _, _ = ref.stream_token_ids_with_stats(
+        ids, 12, None, oracle.sampling(temperature=0.9, top_k=30, top_p=0.95, repeat_penalty=1.2, seed=7))
+    assert toks == want and stats.generated_tokens == st.generated_tokens
+
+
+def greedy_with_teacher_forcing(model, ref, ids, max_new, check_every=1):
+    """Runs the oracle's greedy stream and replays its tokens through the HIP
+    model, comparing logits at each step; returns (#steps, #argmax mismatches
+    that the oracle's top-2 gap explains, #unexplained)."""
+    want, st, rlogits, gaps = ref.stream_token_ids_with_stats(ids, max_new, None, want_logits=True)
+    cache = model.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    explained = unexplained = 0
+    for step in range(st.generated_tokens):
+        if step % check_every == 0:
+            assert_logits_close(logits.to_host(), rlogits[step], what=f"step {step}")
+        tok = model.select_next_token(logits)
+        ref_tok = want[len(ids) + step]
+        if tok != ref_tok:
+            if gaps[step] <= 2 * (ABS_TOL + REL_TOL * abs(float(rlogits[step].max()))):
+                explained += 1
+            else:
+                unexplained += 1
+        if step + 1 < st.generated_tokens:
+            logits = model.forward_one(ref_tok, cache)  # teacher-force the reference's token
+    return st.generated_tokens, explained, unexplained, want
+
+
+def test_config1_gpt2_small_greedy_decode_parity():
+    """BASELINE config 1: 124M, 32 prompt ids, 128 greedy tokens with KV cache."""
+    cfg = synth.Gpt2Config(**synth.GPT2_SMALL)
+    w = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 1)
+    ids = list(synth.token_ids(32, synth.TOKEN_SEED_BASE + 1, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(8))
+    steps, explained, unexplained, want = greedy_with_teacher_forcing(model, ref, ids, 128)
+    assert steps == 128 and unexplained == 0
+    # the fused on-device loop yields the same ids wherever no near-tie intervened
+    cache = model.new_kv_cache()
+    model.prefill(ids, cache)
+    got, stats = model.decode_greedy(cache, 128)
+    assert stats.generated_tokens == 128 and len(got) == 128
+    if explained == 0:
+        assert got == want[32:]
+    assert cache.seq_len == 32 + 127  # the forward after the last token is skipped

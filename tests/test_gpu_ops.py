@@ -1,0 +1,126 @@
+"""HIP kernels against the oracle, op by op, through the C ABI (pg_op_*)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from puppygrad_amd import _lib
+from puppygrad_amd.synth import patterned
+
+pytestmark = pytest.mark.gpu
+
+
+def L():
+    return _lib.load()
+
+
+def ok(status):
+    assert status == 0, L().pg_last_error_message().decode()
+
+
+def hip_dense(x, rows, k, n, w, b):
+    out = np.empty(rows * n, np.float32)
+    ok(L().pg_op_dense(0, _lib.f32p(x), rows, k, n, _lib.f32p(w), _lib.f32p(b), _lib.f32p(out)))
+    return out
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 768, 2304), (1, 768, 768), (1, 3072, 768), (1, 1600, 4800),
+                                      (1, 6400, 1600), (2, 1024, 4096), (1, 4, 12), (3, 37, 5),
+                                      (1, 100, 1), (1, 1600, 50257), (1, 8, 4)])
+def test_dense_matches_oracle(rows, k, n):
+    rng = np.random.default_rng(k * 31 + n)
+    x = rng.standard_normal(rows * k).astype(np.float32)
+    w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    got = hip_dense(x, rows, k, n, w, b)
+    want = oracle.transposed_dense(x, rows, k, n, w, b)
+    np.testing.assert_allclose(got, want, atol=2e-5, rtol=1e-5)
+
+
+def test_dense_reference_unit_vector():
+    # src/models/cpu.rs:312-327
+    x, weight = patterned(6, 0.2), patterned(12, 0.1)
+    bias = np.array([0.5, -0.25, 0.125, 0.0], np.float32)
+    t = oracle.transpose_in_out(weight, 3, 4)
+    np.testing.assert_allclose(hip_dense(x, 2, 3, 4, t, bias), oracle.dense(x, 2, 3, 4, weight, bias),
+                               atol=1e-6, rtol=0)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 4), (1, 768), (3, 1600), (5, 37), (2, 6400)])
+def test_layer_norm_matches_oracle(rows, cols):
+    rng = np.random.default_rng(cols)
+    x = (rng.standard_normal(rows * cols) * 3 + 1.5).astype(np.float32)
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    got = x.copy()
+    ok(L().pg_op_layer_norm(0, _lib.f32p(got), rows, cols, _lib.f32p(g), _lib.f32p(b), 1e-5))
+    np.testing.assert_allclose(got, oracle.layer_norm(x, rows, cols, g, b, 1e-5), atol=5e-6, rtol=1e-5)
+
+
+def test_gelu_softmax_add_match_oracle():
+    x = np.linspace(-8, 8, 4001).astype(np.float32)
+    got = x.copy()
+    ok(L().pg_op_gelu(0, _lib.f32p(got), got.size))
+    np.testing.assert_allclose(got, oracle.gelu(x), atol=1e-6, rtol=1e-5)
+    rng = np.random.default_rng(5)
+    for n in [1, 2, 33, 1024, 5000]:
+        v = (rng.standard_normal(n) * 4).astype(np.float32)
+        got = v.copy()
+        ok(L().pg_op_softmax(0, _lib.f32p(got), 1, n))
+        np.testing.assert_allclose(got, oracle.softmax(v), atol=1e-7, rtol=1e-5)
+    a, b = patterned(1000, 0.5), patterned(1000, -0.25)
+    got = a.copy()
+    ok(L().pg_op_add(0, _lib.f32p(got), _lib.f32p(b), got.size))
+    np.testing.assert_array_equal(got, oracle.add(a, b))
+
+
+def oracle_attention(qkv, pos, keys, values, P, H, hd):
+    """cached_self_attention_into restated with the oracle's softmax (rust.rs:1662-1741)."""
+    C_ = H * hd
+    k, v = keys.reshape(H, P, hd).copy(), values.reshape(H, P, hd).copy()
+    k[:, pos] = qkv[C_:2 * C_].reshape(H, hd)
+    v[:, pos] = qkv[2 * C_:].reshape(H, hd)
+    out = np.zeros(C_, np.float32)
+    scale = np.float32(1.0) / np.sqrt(np.float32(hd))
+    for h in range(H):
+        s = np.array([oracle.dot_scalar(qkv[h * hd:(h + 1) * hd], k[h, j]) for j in range(pos + 1)],
+                     np.float32) * scale
+        p = oracle.softmax(s)
+        out[h * hd:(h + 1) * hd] = (p[:, None].astype(np.float64) * v[h, :pos + 1]).sum(0)
+    return out, k, v
+
+
+@pytest.mark.parametrize("H,hd,P,pos", [(2, 2, 5, 0), (2, 2, 5, 4), (12, 64, 1024, 0), (12, 64, 1024, 31),
+                                        (25, 64, 1024, 1023), (16, 64, 1024, 383), (3, 12, 64, 40),
+                                        (1, 64, 128, 17)])
+def test_attention_decode_matches_oracle(H, hd, P, pos):
+    rng = np.random.default_rng(H * 1000 + pos)
+    C_ = H * hd
+    qkv = rng.standard_normal(3 * C_).astype(np.float32)
+    keys = rng.standard_normal(H * P * hd).astype(np.float32)
+    values = rng.standard_normal(H * P * hd).astype(np.float32)
+    want, wk, wv = oracle_attention(qkv, pos, keys, values, P, H, hd)
+    out = np.empty(C_, np.float32)
+    k, v = keys.copy(), values.copy()
+    ok(L().pg_op_attention_decode(0, _lib.f32p(qkv), pos, _lib.f32p(k), _lib.f32p(v), P, H, hd,
+                                  _lib.f32p(out)))
+    np.testing.assert_allclose(out, want, atol=2e-5, rtol=1e-4)
+    np.testing.assert_array_equal(k.reshape(H, P, hd), wk)   # K/V append at kv_index
+    np.testing.assert_array_equal(v.reshape(H, P, hd), wv)
+
+
+def test_argmax_rules_match_oracle():
+    inf, nan = float("inf"), float("nan")
+    cases = [[1.0, 3.0, 3.0, 2.0], [-inf, -inf], [nan, nan, nan], [1.0, nan, 0.5],
+             [nan, 1.0, inf, inf], [-5.0]]
+    rng = np.random.default_rng(9)
+    big = rng.standard_normal(50257).astype(np.float32)
+    big[[777, 40000]] = big.max() + 1.0  # a tie far apart: lowest index wins
+    cases.append(big)
+    cases.append(np.full(50257, -inf, np.float32))
+    for c in cases:
+        v = np.asarray(c, np.float32)
+        out = C.c_uint32()
+        ok(L().pg_op_argmax(0, _lib.f32p(v), v.size, C.byref(out)))
+        assert out.value == oracle.argmax_logits(v)
