@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Headline benchmark: GPT-2 XL 1.5B fp32, batch-1 greedy decode with a KV cache
+prefilled to 896 tokens (BASELINE.json configs[3]), on one MI355X.
+
+A step is one cached decoder forward (one token).  The timed region holds
+weights, KV cache and the first logits resident in HBM; token selection
+(argmax) runs on the device and only the ids return to the host afterwards.
+Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this path runs on one GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def weight_bytes(cfg) -> int:
+    """Bytes of parameters one decode step reads: every block tensor, ln_f, wte
+    (as lm_head) and the two embedding rows."""
+    C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    per_layer = 3 * C_ * C_ + 3 * C_ + C_ * C_ + C_ + 2 * C_ * I + I + C_ + 4 * C_
+    return 4 * (L * per_layer + 2 * C_ + V * C_ + 2 * C_)
+
+
+def kv_bytes(cfg, pos: int) -> int:
+    """K and V rows of positions [0, pos] over all layers."""
+    return 4 * 2 * cfg.n_layer * cfg.n_embd * (pos + 1)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=127)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--model", default="xl", choices=["xl", "medium", "small"])
+    ap.add_argument("--prefill", type=int, default=None, help="tokens in the cache before decode")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this path runs on ONE GPU (batch-1 decode does not shard usefully; see "
+            "DESIGN.md); --gpus must be 1")
+        return 2
+
+    from puppygrad_amd import Gpt2Config, Gpt2HipConfig, Gpt2Model, _lib, synth
+
+    model_kw = {"xl": synth.GPT2_XL, "medium": synth.GPT2_MEDIUM, "small": synth.GPT2_SMALL}[args.model]
+    cfg_no = {"xl": 4, "medium": 3, "small": 1}[args.model]
+    cfg = Gpt2Config(**model_kw)
+    n_prefill = args.prefill if args.prefill is not None else {"xl": 896, "medium": 128, "small": 32}[args.model]
+    room = cfg.n_positions - n_prefill  # tokens one pass can generate
+
+    t0 = time.time()
+    weights = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + cfg_no)
+    ids = synth.token_ids(n_prefill, synth.TOKEN_SEED_BASE + cfg_no, cfg.vocab_size)
+    log(f"[bench] synthetic weights: {time.time() - t0:.1f}s")
+    t0 = time.time()
+    path = {"auto": _lib.PG_DECODE_AUTO, "kernels": _lib.PG_DECODE_KERNELS,
+            "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
+    model = Gpt2Model.new(cfg, weights, Gpt2HipConfig(device=0, decode_path=path))
+    log(f"[bench] upload: {time.time() - t0:.1f}s; backend: {model.describe()}")
+
+    cache = model.new_kv_cache()
+    t0 = time.time()
+    model.prefill(ids, cache)
+    prefill_s = time.time() - t0
+    log(f"[bench] prefill {n_prefill} tokens: {prefill_s:.2f}s")
+
+    def rewind():
+        """Back to the prefilled state with valid logits (one untimed forward)."""
+        cache.seq_len = n_prefill - 1
+        model.forward_one(int(ids[-1]), cache)
+
+    # warmup
+    done = 0
+    while done < args.warmup:
+        n = min(args.warmup - done, room - 1)
+        model.decode_greedy(cache, n + 1)
+        done += n
+        rewind()
+
+    # timed: K forwards in passes of at most room-1 forwards (room tokens)
+    steps_left = args.steps
+    wall = gpu = 0.0
+    tokens = 0
+    kv_total = 0
+    while steps_left > 0:
+        n = min(steps_left, room - 1)
+        start = cache.seq_len
+        toks, st = model.decode_greedy(cache, n + 1)  # n+1 tokens selected, n forwards
+        assert len(toks) == n + 1 and cache.seq_len == start + n
+        wall += st.decode_time
+        gpu += st.gpu_decode_time
+        tokens += n + 1
+        kv_total += sum(kv_bytes(cfg, p) for p in range(start, start + n))
+        steps_left -= n
+        if steps_left > 0:
+            rewind()
+    K = args.steps
+    ms_per_step = wall / K * 1e3
+    gpu_ms_per_step = gpu / K * 1e3
+    tok_s = K / wall  # forwards per second; the reference's tokens/sec adds the free last token
+    algo_bytes = weight_bytes(cfg) + kv_total / K
+    achieved = algo_bytes / (gpu / K) / 1e9
+
+    info = _lib.pg_device_info()
+    _lib.load().pg_device_query(0, C.byref(info))
+
+    result = {
+        "metric": "decode tokens/sec, GPT-2 XL 1.5B fp32 bs=1" if args.model == "xl"
+                  else f"decode tokens/sec, GPT-2 {args.model} fp32 bs=1",
+        "value": round(tok_s, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"GPT-2 {args.model} fp32 B=1 greedy decode, KV cache prefilled to "
+                               f"{n_prefill} tokens, positions {n_prefill}..{n_prefill + min(K, room - 1) - 1}",
+                   "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
+                   "device": info.name.decode(), "compute_units": info.compute_units,
+                   "backend": model.describe()},
+        "reference_metric_tokens_per_s": round(tokens / wall, 2),
+        "gpu_ms_per_step": round(gpu_ms_per_step, 4),
+        "prefill_s": round(prefill_s, 3),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "one decode step (all launches of one token)",
+                     "algorithmic_bytes_per_step": int(algo_bytes)},
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, weights, ids, n_prefill)
+
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def cpu_baseline(cfg, weights, ids, n_prefill):
+    """The oracle (a C++ restatement of the reference's CPU path, AVX dot and
+    round-robin chunked thread pool) timed on this host: a bounded sample of
+    forward_one steps at the benchmark's context length."""
+    import oracle
+    cores = len(os.sched_getaffinity(0))
+    threads = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+    t0 = time.time()
+    ref = oracle.Model(cfg, weights, oracle.rust_config(threads))
+    log(f"[bench] cpu oracle build: {time.time() - t0:.1f}s, threads={threads}")
+    rcache = ref.new_kv_cache()
+    step_ids = [int(ids[i % len(ids)]) for i in range(64)]
+    # 1 warmup step, then as many steps as fit in about 15 s (at least 3)
+    sec, _ = ref.timed_forward_steps(rcache, n_prefill, step_ids[:1])
+    n = int(max(3, min(48, 15.0 / max(sec, 1e-3))))
+    runs = []
+    for _ in range(3):
+        s, _ = ref.timed_forward_steps(rcache, n_prefill, step_ids[:max(1, n // 3)])
+        runs.append(max(1, n // 3) / s)
+    runs.sort()
+    return {"value": round(runs[1], 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"median of 3 runs of {max(1, n // 3)} forward_one steps starting at cache length "
+                      f"{n_prefill} (KV values zero-filled; timing does not depend on them), "
+                      f"default Gpt2RustConfig thresholds"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())
