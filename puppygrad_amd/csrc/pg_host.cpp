@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -58,6 +59,10 @@ struct pg_gpt2_model {
   size_t arena_floats = 0;
   float *wte = nullptr, *wpe = nullptr, *ln_f_g = nullptr, *ln_f_b = nullptr;
   std::vector<pgk::LayerW> layers;
+  pgk::LayerW* d_layers = nullptr;  // the same table in device memory
+  bool persistent = false;          // batch-1 decode runs as one persistent launch
+  int persistent_grid = 0;          // workgroups of that launch (one per CU)
+  int attn_splits = 1;              // key splits per head in the persistent kernel
 };
 
 struct pg_logits {
@@ -84,6 +89,14 @@ struct pg_kv_cache {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   pg_logits logits{};
   bool logits_valid = false;
+  // persistent decode: tagged activation words {epoch, f32} and the launch status
+  unsigned long long *qkv_t = nullptr, *part_t = nullptr, *attn_t = nullptr, *xa_t = nullptr,
+                     *h_t = nullptr, *xm_t = nullptr, *best_t = nullptr;
+  size_t tagged_words = 0;  // total words in the allocation that starts at qkv_t
+  unsigned* status = nullptr;
+  unsigned* h_status = nullptr;  // pinned
+  uint32_t* d_force = nullptr;   // [P] prompt ids for a one-launch prefill
+  unsigned epoch = 1;            // next unused epoch
 
   float* k_panel(size_t l, size_t b) const {
     return kv + (((l * 2 + 0) * B + b) * cfg.H) * cfg.P * cfg.hd();
@@ -261,6 +274,72 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   }
+  return PG_OK;
+}
+
+// Persistent launches are serialised process-wide: two of them resident at once
+// could each hold part of the CUs while waiting for workgroups that cannot start.
+std::mutex g_persistent_mu;
+
+bool use_persistent(const pg_gpt2_model* m, const pg_kv_cache* c) {
+  return m->persistent && c->B == 1 && c->qkv_t != nullptr;
+}
+
+// Runs n_fwd cached decoder steps of sequence 0 in ONE launch of the persistent
+// kernel and waits for it.  Token t is force_ids[t] when force_ids is set (prefill),
+// otherwise the first token comes from d_tok / tok and later ones from the argmax
+// of the previous step.  On return *done is the number of forwards executed and
+// *stopped says whether an EOS token ended the run early.
+pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
+                         bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
+                         size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
+                         size_t* done, bool* stopped, bool timed) {
+  const Cfg& g = m->cfg;
+  const unsigned span = (unsigned)(n_fwd * (g.L + 1) * 8 + 8);
+  if (c->epoch > 0xE0000000u - span) {
+    // epochs would wrap: clear every tag and start over
+    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->qkv_t), c->tagged_words * 2,
+                                 c->stream));
+    c->epoch = 1;
+  }
+  pgk::DecodeParams p{};
+  p.layers = m->d_layers;
+  p.wte = m->wte; p.wpe = m->wpe; p.ln_f_g = m->ln_f_g; p.ln_f_b = m->ln_f_b;
+  p.C = (int)g.C; p.I = (int)g.I; p.H = (int)g.H; p.L = (int)g.L; p.V = (int)g.V; p.P = (int)g.P;
+  p.eps = g.eps;
+  p.kv = c->kv;
+  p.kv_layer_stride = 2 * g.H * g.P * g.hd();
+  p.kv_v_offset = g.H * g.P * g.hd();
+  p.qkv_t = c->qkv_t; p.part_t = c->part_t; p.attn_t = c->attn_t; p.xa_t = c->xa_t;
+  p.h_t = c->h_t; p.xm_t = c->xm_t; p.best_t = c->best_t;
+  p.logits = c->logits_buf;
+  p.d_tok = c->d_tok;
+  p.tok_val = tok;
+  p.tok_from_ptr = tok_from_ptr ? 1 : 0;
+  p.out_ids = out_ids_dev;
+  p.force_ids = force_ids;
+  p.lm_last_only = lm_last_only ? 1 : 0;
+  p.pos0 = (int)pos0;
+  p.n_fwd = (int)n_fwd;
+  p.select_last = select_last ? 1 : 0;
+  p.eos = (int)eos;
+  p.epoch0 = c->epoch;
+  p.ns = m->attn_splits;
+  p.status = c->status;
+  c->epoch += span;
+  std::lock_guard<std::mutex> lk(g_persistent_mu);
+  PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
+  if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
+  PG_HIP(pgk::launch_decode_persistent(p, m->persistent_grid, c->stream));
+  if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
+  PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
+                        c->stream));
+  PG_HIP(hipStreamSynchronize(c->stream));
+  if (c->h_status[0] != 0)
+    return fail(PG_BACKEND, "persistent decode kernel gave up waiting for a dependency "
+                            "(another kernel may be occupying the device)");
+  if (done) *done = c->h_status[1];
+  if (stopped) *stopped = c->h_status[2] != 0;
   return PG_OK;
 }
 
@@ -485,14 +564,55 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     m->layers[l] = pgk::LayerW{ln_1_g, ln_1_b, c_attn_w, c_attn_b, c_proj_w,     c_proj_b,
                                ln_2_g, ln_2_b, c_fc_w,   c_fc_b,   c_proj_mlp_w, c_proj_mlp_b};
   }
+  PG_HIP(hipMalloc(&m->d_layers, g.L * sizeof(pgk::LayerW)));
+  struct Guard2 {
+    pg_gpt2_model* m;
+    bool ok = false;
+    ~Guard2() {
+      if (!ok && m->d_layers) (void)hipFree(m->d_layers);
+    }
+  } guard2{m.get()};
+  PG_HIP(hipMemcpy(m->d_layers, m->layers.data(), g.L * sizeof(pgk::LayerW),
+                   hipMemcpyHostToDevice));
+
+  // The persistent decode kernel covers head_dim 64, n_inner = 4 n_embd and the
+  // row widths it is instantiated for; everything else takes the per-op launches.
+  {
+    const int grid = m->num_cus;
+    int blocks_per_cu = 0;
+    bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_tile_depth((int)g.C) != 0 &&
+                    g.P <= 4096 && grid > 0 && (g.C + grid - 1) / grid <= 64 &&
+                    2 * (size_t)grid <= g.I;
+    if (shape_ok) {
+      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, (int)g.I, &blocks_per_cu));
+      shape_ok = blocks_per_cu >= 1;
+    }
+    if (shape_ok) {
+      int ns = std::min<int>(16, grid / (int)g.H);
+      ns = std::max<int>(ns, (int)((g.P + 127) / 128));
+      ns = std::max(ns, 1);
+      shape_ok = ns <= pgk::kMaxSplits && (size_t)ns * 66 <= g.I;
+      m->attn_splits = ns;
+    }
+    if (opts.decode_path == PG_DECODE_PERSISTENT && !shape_ok)
+      return fail(PG_INVALID_CONFIG,
+                  "hip backend decode_path=persistent needs head_dim 64, n_inner = 4*n_embd and "
+                  "n_embd in (512,1024] or (1536,1792]");
+    m->persistent = shape_ok && opts.decode_path != PG_DECODE_KERNELS;
+    m->persistent_grid = grid;
+  }
   guard.ok = true;
+  guard2.ok = true;
   *out = m.release();
   return PG_OK;
 }
 
 void pg_gpt2_destroy(pg_gpt2_model* m) {
   if (!m) return;
-  if (hipSetDevice(m->device) == hipSuccess && m->arena) (void)hipFree(m->arena);
+  if (hipSetDevice(m->device) == hipSuccess) {
+    if (m->arena) (void)hipFree(m->arena);
+    if (m->d_layers) (void)hipFree(m->d_layers);
+  }
   delete m;
 }
 
@@ -504,8 +624,8 @@ pg_status pg_gpt2_get_config(const pg_gpt2_model* m, pg_gpt2_config* out) {
 
 pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
   if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
-  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=f32)", m->device,
-                m->num_cus);
+  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=f32, decode=%s)", m->device,
+                m->num_cus, m->persistent ? "persistent" : "kernels");
   return PG_OK;
 }
 
@@ -547,6 +667,22 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->d_tok, B * sizeof(uint32_t)));
   PG_HIP(hipMalloc(&raw->d_out_ids, g.P * B * sizeof(uint32_t)));
   PG_HIP(hipHostMalloc(&raw->h_ids, g.P * B * sizeof(uint32_t), hipHostMallocDefault));
+  if (m->persistent && batch == 1) {
+    const size_t n_part = g.H * pgk::kMaxSplits * 66;
+    const size_t words = 3 * g.C + n_part + g.C + g.C + g.I + g.C + 2 * (size_t)m->persistent_grid;
+    PG_HIP(hipMalloc(&raw->qkv_t, words * sizeof(unsigned long long)));
+    raw->tagged_words = words;
+    raw->part_t = raw->qkv_t + 3 * g.C;
+    raw->attn_t = raw->part_t + n_part;
+    raw->xa_t = raw->attn_t + g.C;
+    raw->h_t = raw->xa_t + g.C;
+    raw->xm_t = raw->h_t + g.I;
+    raw->best_t = raw->xm_t + g.C;
+    PG_HIP(hipMalloc(&raw->status, 4 * sizeof(unsigned)));
+    PG_HIP(hipHostMalloc(&raw->h_status, 4 * sizeof(unsigned), hipHostMallocDefault));
+    PG_HIP(hipMalloc(&raw->d_force, g.P * sizeof(uint32_t)));
+    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(raw->qkv_t), words * 2, raw->stream));
+  }
   // Gpt2LayerKvCache::new zero-fills (src/models/gpt2/rust.rs:258-266).
   PG_HIP(pgk::launch_fill_zero(raw->kv, kv_floats, raw->stream));
   PG_HIP(hipStreamSynchronize(raw->stream));
@@ -570,6 +706,10 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->d_tok);
     (void)hipFree(c->d_out_ids);
     if (c->h_ids) (void)hipHostFree(c->h_ids);
+    (void)hipFree(c->qkv_t);
+    (void)hipFree(c->status);
+    (void)hipFree(c->d_force);
+    if (c->h_status) (void)hipHostFree(c->h_status);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -620,6 +760,16 @@ pg_status pg_gpt2_prefill_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   if ((s = select_device(m->device))) return s;
   c->seq_len = 0;  // cache.clear() (rust.rs:918)
   c->logits_valid = false;
+  if (use_persistent(m, c)) {
+    PG_HIP(hipMemcpyAsync(c->d_force, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));  // ids is the caller's pageable memory
+    if ((s = run_persistent(m, c, c->d_force, true, false, 0, 0, n, false, -1, nullptr, nullptr,
+                            nullptr, false)))
+      return s;
+    c->seq_len = n;
+    return finish_logits(c, out);
+  }
   for (size_t b = 0; b < c->B; ++b)
     for (size_t i = 0; i < n; ++i)
       if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b * n + i], i, i + 1 == n))) return s;
@@ -646,6 +796,13 @@ pg_status pg_gpt2_forward_one_batch(const pg_gpt2_model* m, pg_kv_cache* c, cons
                                         " exceeds vocab_size " + std::to_string(m->cfg.V));
   if ((s = check_step(m, c))) return s;
   if ((s = select_device(m->device))) return s;
+  if (use_persistent(m, c)) {
+    if ((s = run_persistent(m, c, nullptr, false, false, ids[0], c->seq_len, 1, false, -1,
+                            nullptr, nullptr, nullptr, false)))
+      return s;
+    c->seq_len += 1;
+    return finish_logits(c, out);
+  }
   for (size_t b = 0; b < c->B; ++b)
     if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b], c->seq_len, true))) return s;
   PG_HIP(hipStreamSynchronize(c->stream));
@@ -673,7 +830,13 @@ pg_status pg_gpt2_forward(const pg_gpt2_model* m, const uint32_t* ids, size_t n,
   if ((s = pg_kv_cache_create(m, 1, &c))) return s;
   std::unique_ptr<pg_kv_cache, void (*)(pg_kv_cache*)> holder(c, pg_kv_cache_destroy);
   for (size_t i = 0; i < n; ++i) {
-    if ((s = enqueue_forward_one(m, c, 0, nullptr, ids[i], i, true))) return s;
+    if (use_persistent(m, c)) {
+      if ((s = run_persistent(m, c, nullptr, false, false, ids[i], i, 1, false, -1, nullptr,
+                              nullptr, nullptr, false)))
+        return s;
+    } else if ((s = enqueue_forward_one(m, c, 0, nullptr, ids[i], i, true))) {
+      return s;
+    }
     PG_HIP(hipMemcpyAsync(dst + i * m->cfg.V, c->logits_buf, m->cfg.V * sizeof(float),
                           hipMemcpyDeviceToHost, c->stream));
   }
@@ -770,46 +933,83 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
   return sample_logits(adjusted, *sampling, rng, out);
 }
 
-pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t steps,
-                                      uint32_t* out_ids, pg_generation_stats* stats) {
-  if (!m || !c || !out_ids) return fail(PG_INVALID_INPUT, "null argument");
+// Shared body of the two greedy-decode entry points.  Selects up to `steps`
+// tokens; token i+1 comes from a forward of token i, and no forward follows the
+// last selected token (src/models/gpt2/rust.rs:518-528).  Generation stops when
+// prompt + generated reaches n_positions (rust.rs:496-498), so at most
+// P - seq_len tokens are selected.  With eos >= 0 the run may end early at the
+// first EOS; ids then still holds the EOS as its last entry and the caller drops it.
+static pg_status decode_core(const pg_gpt2_model* m, pg_kv_cache* c, size_t steps, int64_t eos,
+                             uint32_t* ids, size_t* n_ids, pg_generation_stats* stats) {
   pg_status s;
   if ((s = check_compatible(m, c))) return s;
   if (!c->logits_valid)
     return fail(PG_INVALID_INPUT, "decode needs logits from prefill or forward_one");
   if ((s = select_device(m->device))) return s;
   const size_t B = c->B, V = m->cfg.V;
-  // Selecting a token needs no cache slot; each forward after it does.
-  size_t room = c->cfg.P - c->seq_len;  // forwards still possible
-  size_t n_steps = std::min<size_t>(steps, room + 1);
-  auto t0 = Clock::now();
-  PG_HIP(hipEventRecord(c->ev0, c->stream));
-  for (size_t i = 0; i < n_steps; ++i) {
-    for (size_t b = 0; b < B; ++b)
-      PG_HIP(pgk::launch_argmax(c->logits_buf + b * V, (int)V, c->d_tok + b, c->stream));
-    PG_HIP(hipMemcpyAsync(c->d_out_ids + i * B, c->d_tok, B * sizeof(uint32_t),
-                          hipMemcpyDeviceToDevice, c->stream));
-    bool needs_next = i + 1 < n_steps;  // rust.rs:518-528: no forward after the last token
-    if (needs_next) {
-      for (size_t b = 0; b < B; ++b)
-        if ((s = enqueue_forward_one(m, c, b, c->d_tok + b, 0, c->seq_len, true))) return s;
-      c->seq_len += 1;
-    }
+  const size_t n_steps = std::min<size_t>(steps, c->cfg.P - c->seq_len);
+  *n_ids = 0;
+  if (n_steps == 0) {
+    if (stats) *stats = pg_generation_stats{};
+    return PG_OK;
   }
-  PG_HIP(hipEventRecord(c->ev1, c->stream));
-  PG_HIP(hipMemcpyAsync(c->h_ids, c->d_out_ids, n_steps * B * sizeof(uint32_t),
-                        hipMemcpyDeviceToHost, c->stream));
-  PG_HIP(hipStreamSynchronize(c->stream));
-  std::memcpy(out_ids, c->h_ids, n_steps * B * sizeof(uint32_t));
+  auto t0 = Clock::now();
+  size_t n_out = n_steps;
+  float ms = 0.0f;
+  if (use_persistent(m, c)) {
+    PG_HIP(pgk::launch_argmax(c->logits_buf, (int)V, c->d_tok, c->stream));
+    size_t done = 0;
+    bool stopped = false;
+    if (n_steps > 1) {
+      if ((s = run_persistent(m, c, nullptr, false, true, 0, c->seq_len, n_steps - 1, true, eos,
+                              c->d_out_ids, &done, &stopped, true)))
+        return s;
+      PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
+      n_out = stopped ? done + 1 : n_steps;
+      c->seq_len += done;
+    } else {
+      PG_HIP(hipMemcpyAsync(c->d_out_ids, c->d_tok, sizeof(uint32_t), hipMemcpyDeviceToDevice,
+                            c->stream));
+    }
+    PG_HIP(hipMemcpyAsync(c->h_ids, c->d_out_ids, n_out * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));
+  } else {
+    PG_HIP(hipEventRecord(c->ev0, c->stream));
+    for (size_t i = 0; i < n_steps; ++i) {
+      for (size_t b = 0; b < B; ++b)
+        PG_HIP(pgk::launch_argmax(c->logits_buf + b * V, (int)V, c->d_tok + b, c->stream));
+      PG_HIP(hipMemcpyAsync(c->d_out_ids + i * B, c->d_tok, B * sizeof(uint32_t),
+                            hipMemcpyDeviceToDevice, c->stream));
+      if (i + 1 < n_steps) {
+        for (size_t b = 0; b < B; ++b)
+          if ((s = enqueue_forward_one(m, c, b, c->d_tok + b, 0, c->seq_len, true))) return s;
+        c->seq_len += 1;
+      }
+    }
+    PG_HIP(hipEventRecord(c->ev1, c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_ids, c->d_out_ids, n_steps * B * sizeof(uint32_t),
+                          hipMemcpyDeviceToHost, c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));
+    PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
+  }
+  std::memcpy(ids, c->h_ids, n_out * B * sizeof(uint32_t));
+  *n_ids = n_out;
   c->logits_valid = false;  // the logits the last selection used are consumed
   if (stats) {
-    float ms = 0.0f;
-    PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
-    stats->generated_tokens = n_steps;
+    *stats = pg_generation_stats{};
+    stats->generated_tokens = n_out;
     stats->decode_s = since(t0);
     stats->gpu_decode_s = ms * 1e-3;
   }
   return PG_OK;
+}
+
+pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t steps,
+                                      uint32_t* out_ids, pg_generation_stats* stats) {
+  if (!m || !c || !out_ids) return fail(PG_INVALID_INPUT, "null argument");
+  size_t n = 0;
+  return decode_core(m, c, steps, -1, out_ids, &n, stats);
 }
 
 pg_status pg_gpt2_decode_greedy(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t max_new,
@@ -823,13 +1023,11 @@ pg_status pg_gpt2_decode_greedy(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t
   *out_n = 0;
   if (max_new == 0) return PG_OK;
   const size_t start_len = c->seq_len;
-  size_t room = c->cfg.P - c->seq_len;
-  size_t n_steps = std::min<size_t>(max_new, room + 1);
-  std::vector<uint32_t> ids(n_steps);
+  std::vector<uint32_t> ids(std::max<size_t>(max_new, 1));
   pg_generation_stats st{};
-  pg_status s = pg_gpt2_decode_greedy_batch(m, c, (uint32_t)n_steps, ids.data(), &st);
+  size_t n = 0;
+  pg_status s = decode_core(m, c, max_new, eos, ids.data(), &n, &st);
   if (s) return s;
-  size_t n = st.generated_tokens;
   if (eos >= 0) {
     // EOS is tested before the push (rust.rs:503-505): drop it and what follows,
     // and rewind the cache to the forwards the reference would have run.

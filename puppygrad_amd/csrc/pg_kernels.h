@@ -78,4 +78,34 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
                               int H, int head_dim, int nsplit, float* out, hipStream_t s);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
 
+// ---- persistent batch-1 decode (pg_decode.hip) --------------------------------
+struct DecodeParams {
+  const LayerW* layers;
+  const float *wte, *wpe, *ln_f_g, *ln_f_b;
+  int C, I, H, L, V, P;
+  float eps;
+  float* kv;               // [L][2][H][P][64] of this sequence
+  size_t kv_layer_stride;  // floats from layer l to l+1
+  size_t kv_v_offset;      // floats from the K panel to the V panel of a layer
+  unsigned long long *qkv_t, *part_t, *attn_t, *xa_t, *h_t, *xm_t, *best_t;
+  float* logits;
+  uint32_t* d_tok;
+  uint32_t tok_val;
+  int tok_from_ptr;
+  uint32_t* out_ids;
+  const uint32_t* force_ids;  // if set, token t is force_ids[t] (prefill); no argmax chain
+  int lm_last_only;           // with force_ids: LN_f + lm_head only after the last token
+  int pos0, n_fwd, select_last, eos;
+  unsigned epoch0;
+  int ns;
+  unsigned* status;  // [0] abort, [1] forwards done, [2] stopped at eos
+};
+
+
+// Tile depth the persistent kernel is built for at this n_embd (0: unsupported).
+int persistent_tile_depth(int C);
+size_t persistent_lds_bytes(int C, int I);
+hipError_t persistent_max_blocks_per_cu(int C, int I, int* out);
+hipError_t launch_decode_persistent(const DecodeParams& p, int grid, hipStream_t s);
+
 }  // namespace pgk
