@@ -2,14 +2,19 @@
 // decoder steps (forward_one_profiled_with_scratch, src/models/gpt2/rust.rs:943-1006,
 // block at 1136-1250, attention at 1662-1741) for one or many greedy tokens.
 //
-// Design.  One workgroup per CU streams its share of every weight matrix exactly
-// once per token with nontemporal 16-byte loads.  Workgroups never meet at a grid
-// barrier.  Every activation that crosses workgroups is stored as a 64-bit word
-// {epoch, f32 bits} with one agent-scope atomic store; a consumer polls the words
-// it needs until they carry the epoch of the producing (token, layer, phase).
-// Because weight addresses do not depend on data, each phase issues the loads of
-// its first weight tiles BEFORE it starts polling, so HBM keeps streaming while
-// the dependency chain catches up.
+// Design.  256 workgroups (one per CU) each own a contiguous band of rows of every
+// weight matrix and stream it exactly once per token with nontemporal 16-byte
+// loads.  Workgroups never meet at a grid barrier.  Every activation that crosses
+// workgroups is stored as a 64-bit word {epoch, f32 bits} with one agent-scope
+// atomic store; a consumer polls the words it needs until they carry the epoch of
+// the producing (token, layer, phase).  Weight addresses do not depend on data, so
+// the whole band of the NEXT matrix is requested into registers before the current
+// phase starts waiting: HBM keeps streaming while the dependency chain catches up.
+//
+// A band is treated as a flat array of float4: thread t holds elements
+// t, t+512, t+1024, ...  A wavefront's 64 consecutive float4 lie in at most two
+// rows, so one (or two) DPP wave reductions per 1 KiB give per-chunk partial sums,
+// which are added per row in a fixed order (results do not depend on timing).
 //
 // Per layer:  A  LN1 + c_attn rows            -> qkv_t   (tagged)
 //             B  split-key attention per head -> part_t  (tagged partial acc, m, l)
@@ -32,8 +37,11 @@ namespace {
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+
 constexpr int kThreads = 512;
 constexpr int kWavesP = kThreads / 64;
+constexpr int kGrid = 256;  // workgroups; row bands are computed for exactly this many
 constexpr unsigned kSpinLimit = 1u << 21;
 constexpr int kAttnSteps = 4;  // up to 4*32 = 128 keys per (head, split) item
 
@@ -49,10 +57,27 @@ __device__ __forceinline__ u64 pack_u(unsigned epoch, unsigned v) { return ((u64
 __device__ __forceinline__ unsigned tag_of(u64 w) { return (unsigned)(w >> 32); }
 __device__ __forceinline__ float val_of(u64 w) { return __uint_as_float((unsigned)w); }
 
-__device__ __forceinline__ float wsum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+// Cross-lane adds through DPP (no LDS traffic).  All 64 lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// Sum over each row of 16 lanes; every lane of the row receives it.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_get<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_get<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_get<0x141>(v);  // row_half_mirror
+  v += dpp_get<0x140>(v);  // row_mirror
   return v;
+}
+// Sum over the wavefront; the result is wave-uniform.
+__device__ __forceinline__ float wsum(float v) {
+  v = row16_sum(v);
+  float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (r0 + r1) + (r2 + r3);
 }
 __device__ __forceinline__ float wmax(float v) {
 #pragma unroll
@@ -61,39 +86,49 @@ __device__ __forceinline__ float wmax(float v) {
 }
 
 struct Smem {
-  float red[kWavesP];
+  float red[2][kWavesP];  // alternating buffers: consecutive reductions need one barrier each
   float accs[kWavesP][64];
   float qs[64], kn[64], vn[64];
-  float psum[64 * 4];  // phase F partial sums: [row_local][segment]
   float bestv[kWavesP];
   unsigned besti[kWavesP];
   int ok;
   unsigned tok;
 };
 
+// Block reductions with ONE barrier each.  Two calls in a row must use different
+// buffers (B = 0, 1); a buffer may be reused once another barrier has passed.
+template <int B>
 __device__ __forceinline__ float bsum(float v, Smem& sm) {
   v = wsum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sm.red[threadIdx.x >> 6] = v;
+  if ((threadIdx.x & 63) == 0) sm.red[B][threadIdx.x >> 6] = v;
   __syncthreads();
   float t = 0.0f;
 #pragma unroll
-  for (int w = 0; w < kWavesP; ++w) t += sm.red[w];
+  for (int w = 0; w < kWavesP; ++w) t += sm.red[B][w];
   return t;
 }
+template <int B>
 __device__ __forceinline__ float bmax(float v, Smem& sm) {
   v = wmax(v);
+  if ((threadIdx.x & 63) == 0) sm.red[B][threadIdx.x >> 6] = v;
   __syncthreads();
-  if ((threadIdx.x & 63) == 0) sm.red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = sm.red[0];
+  float t = sm.red[B][0];
 #pragma unroll
-  for (int w = 1; w < kWavesP; ++w) t = fmaxf(t, sm.red[w]);
+  for (int w = 1; w < kWavesP; ++w) t = fmaxf(t, sm.red[B][w]);
   return t;
 }
 
 __device__ __forceinline__ float gelu_tanh(float x) {
   return 0.5f * x * (1.0f + tanhf(0.7978846f * (x + 0.044715f * x * x * x)));
+}
+
+// threadIdx.x behind an empty asm: index arithmetic built on it is recomputed where
+// it is used instead of being hoisted out of the token/layer loops (dozens of
+// loop-invariant 64-bit addresses would otherwise be kept alive and spilled).
+__device__ __forceinline__ int local_tid() {
+  int t = (int)threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
 }
 
 // Waits until src[i] carries `epoch` for every i in [0, n) that this thread owns
@@ -104,10 +139,13 @@ template <int NE>
 __device__ __forceinline__ bool poll_vec(const u64* src, int n, unsigned epoch, float* dst,
                                          unsigned* abort_word) {
   u64 v[NE];
+  const int tid = local_tid();
 #pragma unroll
   for (int e = 0; e < NE; ++e) {
-    int i = threadIdx.x + kThreads * e;
-    v[e] = (i < n) ? PG_LD64(src + i) : pack(epoch, 0.0f);
+    // out-of-range slots re-read the last word: every load is unconditional, so the
+    // compiler can count outstanding loads exactly and never waits for younger ones
+    int i = min(tid + kThreads * e, n - 1);
+    v[e] = PG_LD64(src + i);
   }
   unsigned spins = 0;
   bool good = true;
@@ -116,7 +154,7 @@ __device__ __forceinline__ bool poll_vec(const u64* src, int n, unsigned epoch, 
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
       if (tag_of(v[e]) != epoch) {
-        v[e] = PG_LD64(src + threadIdx.x + kThreads * e);
+        v[e] = PG_LD64(src + min(tid + kThreads * e, n - 1));
         bad = bad || (tag_of(v[e]) != epoch);
       }
     }
@@ -130,11 +168,11 @@ __device__ __forceinline__ bool poll_vec(const u64* src, int n, unsigned epoch, 
       good = false;
       break;
     }
-    __builtin_amdgcn_s_sleep(2);
+    __builtin_amdgcn_s_sleep(1);
   }
 #pragma unroll
   for (int e = 0; e < NE; ++e) {
-    int i = threadIdx.x + kThreads * e;
+    int i = tid + kThreads * e;
     if (i < n) dst[i] = val_of(v[e]);
   }
   return good;
@@ -142,61 +180,150 @@ __device__ __forceinline__ bool poll_vec(const u64* src, int n, unsigned epoch, 
 
 // Makes a per-thread success flag uniform over the workgroup (also a barrier
 // that publishes LDS written by poll_vec).
+// sm.ok starts at 1 and is only ever cleared, so one barrier suffices.
 __device__ __forceinline__ bool all_ok(bool mine, Smem& sm) {
-  __syncthreads();
-  if (threadIdx.x == 0) sm.ok = 1;
-  __syncthreads();
   if (!mine) sm.ok = 0;
   __syncthreads();
   return sm.ok != 0;
 }
 
-// layer_norm_in_place (src/models/cpu.rs:119-143): raw -> xs, both in LDS.
-__device__ __forceinline__ void ln_lds(const float* raw, float* xs, int C, const float* g,
-                                       const float* b, float eps, Smem& sm) {
+// LayerNorm scale/shift of this thread's elements (i = tid + 512*e), fetched ahead
+// of time: a load issued after a weight band would only return behind the band.
+template <int NE>
+struct LnParams {
+  float g[NE], b[NE];
+};
+template <int NE>
+__device__ __forceinline__ void ln_fetch(LnParams<NE>& q, const float* g, const float* b, int C) {
+  const int tid = local_tid();
+#pragma unroll
+  for (int e = 0; e < NE; ++e) {
+    int i = min(tid + kThreads * e, C - 1);  // unconditional loads (see poll_vec)
+    q.g[e] = g[i];
+    q.b[e] = b[i];
+  }
+}
+// layer_norm_in_place (src/models/cpu.rs:119-143): raw -> xs, both in LDS; two-pass
+// mean / biased variance, eps inside the sqrt.  Every wavefront reduces the whole
+// vector on its own (C/64 LDS reads per lane, DPP sums): no block barrier is
+// needed for the statistics, only one at the end to publish xs.
+template <int NE, int C>
+__device__ __forceinline__ void ln_lds(const float* raw, float* xs, const LnParams<NE>& q,
+                                       float eps) {
+  constexpr int NW = cdiv(C, 64);
+  const int tid = local_tid();
+  const int lane = tid & 63;
+  float x[NW];
   float s = 0.0f;
-  for (int i = threadIdx.x; i < C; i += kThreads) s += raw[i];
-  float mean = bsum(s, sm) / (float)C;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    const int i = lane + 64 * j;
+    x[j] = raw[min(i, C - 1)];
+    if (i >= C) x[j] = 0.0f;
+    s += x[j];
+  }
+  const float mean = wsum(s) / (float)C;
   float v = 0.0f;
-  for (int i = threadIdx.x; i < C; i += kThreads) {
-    float d = raw[i] - mean;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    const float d = (lane + 64 * j < C) ? x[j] - mean : 0.0f;
     v += d * d;
   }
-  float var = bsum(v, sm) / (float)C;
-  float inv = 1.0f / sqrtf(var + eps);
-  for (int i = threadIdx.x; i < C; i += kThreads) xs[i] = (raw[i] - mean) * inv * g[i] + b[i];
+  const float var = wsum(v) / (float)C;
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int e = 0; e < NE; ++e) {
+    const int i = tid + kThreads * e;
+    if (i < C) xs[i] = (raw[i] - mean) * inv * q.g[e] + q.b[e];
+  }
   __syncthreads();
 }
-
-template <int J>
-struct Tile {
-  f4 w[J];
-};
 
 // Weight pointers come out of a table in memory; telling the compiler they are
 // global (not generic) addresses gets global_load instead of flat_load.
 typedef const f4 __attribute__((address_space(1)))* gf4p;
 __device__ __forceinline__ gf4p as_global(const f4* p) { return (gf4p)p; }
 
-// One tile = K4s consecutive float4 of a weight row, 64 lanes wide, J deep.
-// The tile is defined on every path (zeros when `valid` is false), so that no
-// stale tile stays live across the phases in between.
+// ---- flat band streaming -------------------------------------------------------
+
+// Requests this thread's share of a band of n4 >= 1 float4 starting at base:
+// elements tid + 512*u.  Loads are unconditional (indices past the end re-read the
+// last element and are never summed): a load under a branch would make the
+// compiler lose count of outstanding loads and wait for ALL of them at the next
+// use of any older one, which serialises the phase behind the band just requested.
+template <int U, int LO = 0, int HI = U>
+__device__ __forceinline__ void band_load(f4 (&w)[U], const f4* base, int n4) {
+  gf4p g = as_global(base);
+  const int tid = local_tid();
+#pragma unroll
+  for (int u = LO; u < HI; ++u) {
+    int f = min(tid + kThreads * u, n4 - 1);
+    w[u] = __builtin_nontemporal_load(g + f);
+  }
+}
+
+// Stage 1 of a band product: every thread multiplies its float4 of the band with
+// the matching float4 of the vector xs (LDS; rows are K4 float4 long) and leaves
+// the scalar product of flat element f in prod[f] (LDS).  About ten instructions
+// per float4: the per-CU instruction issue rate, not HBM, bounds this part.
+template <int U, int K4>
+__device__ __forceinline__ void band_mul(const f4 (&w)[U], const float* xs, float* prod) {
+  const f4* x4 = reinterpret_cast<const f4*>(xs);
+  const int tid = local_tid();
+  constexpr int B = 5;  // LDS reads kept in flight together
+#pragma unroll
+  for (int u0 = 0; u0 < U; u0 += B) {
+    f4 x[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b)
+      if (u0 + b < U) x[b] = x4[(tid + kThreads * (u0 + b)) % K4];
+#pragma unroll
+    for (int b = 0; b < B; ++b)
+      if (u0 + b < U) {
+        const int u = u0 + b;
+        prod[tid + kThreads * u] =
+            (w[u].x * x[b].x + w[u].y * x[b].y) + (w[u].z * x[b].z + w[u].w * x[b].w);
+      }
+  }
+}
+
+// Stage 2: LPR lanes add up the K4 products of one row in a fixed order (lane s
+// takes s, s+LPR, ...; then a DPP tree), so the result does not depend on timing.
+// Returns the row sum on every lane of the group; `row` must be < rows for the
+// value to be meaningful.  All lanes execute it (the DPP tree needs them active).
+template <int K4, int LPR>
+__device__ __forceinline__ float band_row(const float* prod, int row, int rows) {
+  static_assert(LPR == 16 || LPR == 64, "a row is summed by a DPP row or a whole wavefront");
+  constexpr int N = cdiv(K4, LPR);
+  const int sub = local_tid() & (LPR - 1);
+  const float* src = prod + (size_t)min(row, rows - 1) * K4;
+  float v[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const int k = sub + LPR * j;
+    v[j] = src[min(k, K4 - 1)];
+    if (k >= K4) v[j] = 0.0f;
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < N; ++j) s += v[j];
+  return LPR == 16 ? row16_sum(s) : wsum(s);
+}
+
+// ---- row tiles for the long lm_head band -----------------------------------------
+
 template <int J>
-__device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane,
-                                          bool valid = true) {
-  if (valid) {
-    gf4p g = as_global(p);
+struct Tile {
+  f4 w[J];
+};
+// One tile = one weight row, 64 lanes wide, J deep; defined on every path.
+template <int J>
+__device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
+  gf4p g = as_global(p);
 #pragma unroll
-    for (int j = 0; j < J; ++j) {
-      int c = lane + 64 * j;
-      if (j < J - 1 || c < K4s)
-        t.w[j] = __builtin_nontemporal_load(g + c);
-      else
-        t.w[j] = f4{0.f, 0.f, 0.f, 0.f};
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < J; ++j) t.w[j] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < J; ++j) {
+    int c = min(lane + 64 * j, K4s - 1);  // unconditional; load_x zeroes the matching x
+    t.w[j] = __builtin_nontemporal_load(g + c);
   }
 }
 template <int J>
@@ -232,50 +359,264 @@ __device__ __forceinline__ Best better(Best a, Best b) {
   return a;
 }
 
-}  // namespace
-
-namespace {
-
 __device__ __forceinline__ unsigned epoch_of(const DecodeParams& p, int t, int layer, int phase) {
   return p.epoch0 + (unsigned)((t * (p.L + 1) + layer) * 8 + phase);
 }
 
-template <int J>
+// Phases B and B2 of one layer: split-key attention of cached_self_attention_into
+// (src/models/gpt2/rust.rs:1662-1741) for the (head, split) items of this
+// workgroup, then the per-head merge by the workgroup that took split 0.  Out of
+// line so that its registers are allocated apart from the weight bands.
+__device__ __attribute__((noinline)) bool attention_phase(const DecodeParams& p, Smem& sm,
+                                                          float* xs, int t, int l, int pos,
+                                                          float* kc, float* vc) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wg = blockIdx.x;
+  const int G = kGrid, H = p.H, P = p.P, C = p.C;
+  unsigned* abort_word = p.status;
+  {
+    const int ns = p.ns, items = H * ns, n = pos + 1;
+    const int per = (n + ns - 1) / ns;
+    const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
+    const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
+    for (int item = wg; item < items; item += G) {
+      const int h = item / ns, s = item - h * ns;
+      const int k0 = s * per, k1 = min(n, k0 + per);
+      u64* dst = p.part_t + (size_t)item * 66;
+      if (k0 >= k1) {  // empty split: neutral element of the merge
+        if (tid < 64) PG_ST64(dst + tid, pack(epp, 0.0f));
+        if (tid == 64) PG_ST64(dst + 64, pack(epp, -INFINITY));
+        if (tid == 65) PG_ST64(dst + 65, pack(epp, 0.0f));
+        continue;
+      }
+      const bool owns_new = (pos >= k0 && pos < k1);
+      gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
+      gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
+      f4 kr[kAttnSteps], vr[kAttnSteps];
+#pragma unroll
+      for (int i = 0; i < kAttnSteps; ++i) {
+        // unconditional: keys past the split re-read a cached row (position 0 when
+        // nothing is cached yet; the cache is zero-filled at creation) and get weight 0
+        int key = min(k0 + slot + 32 * i, max(pos - 1, 0));
+        kr[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
+        vr[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
+      }
+      // q of this head, and this token's own K/V rows if the split holds pos
+      bool ok = true;
+      {
+        const int part = tid >> 6;  // 0: q, 1: k_new, 2: v_new
+        if (part == 0 || (owns_new && part < 3)) {
+          const u64* src = p.qkv_t + (size_t)part * C + h * 64 + lane;
+          u64 v = PG_LD64(src);
+          unsigned spins = 0;
+          while (tag_of(v) != epq) {
+            if (++spins > kSpinLimit) {
+              ok = false;
+              PG_ST32(abort_word, 1u);
+              break;
+            }
+            if ((spins & 63) == 0 && PG_LD32(abort_word) != 0) {
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            v = PG_LD64(src);
+          }
+          float f = val_of(v);
+          if (part == 0) sm.qs[lane] = f;
+          if (part == 1) {
+            sm.kn[lane] = f;
+            // K append (rust.rs:1677-1683); written through to memory so that a
+            // later token's reader on another XCD cannot miss it in a remote L2
+            PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, f);
+          }
+          if (part == 2) {
+            sm.vn[lane] = f;
+            PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, f);  // V append
+          }
+        }
+      }
+      if (!all_ok(ok, sm)) return false;
+      const f4 qv = reinterpret_cast<const f4*>(sm.qs)[d4];
+      float sc[kAttnSteps];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < kAttnSteps; ++i) {
+        int key = k0 + slot + 32 * i;
+        if (key == pos && key < k1) {
+          kr[i] = reinterpret_cast<const f4*>(sm.kn)[d4];
+          vr[i] = reinterpret_cast<const f4*>(sm.vn)[d4];
+        }
+        float sv = (qv.x * kr[i].x + qv.y * kr[i].y) + (qv.z * kr[i].z + qv.w * kr[i].w);
+        sv = row16_sum(sv);
+        sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
+        sc[i] = (key < k1) ? sv : -INFINITY;
+        mx = fmaxf(mx, sc[i]);
+      }
+      mx = bmax<0>(mx, sm);
+      float lsum = 0.0f;
+      f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < kAttnSteps; ++i) {
+        float pr = expf(sc[i] - mx);  // exp(-inf) = 0 for absent keys
+        if (d4 == 0) lsum += pr;
+        acc += pr * vr[i];
+      }
+      lsum = bsum<1>(lsum, sm);
+#pragma unroll
+      for (int off = 16; off <= 32; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, 64);
+        acc.y += __shfl_xor(acc.y, off, 64);
+        acc.z += __shfl_xor(acc.z, off, 64);
+        acc.w += __shfl_xor(acc.w, off, 64);
+      }
+      if (sub == 0) reinterpret_cast<f4*>(sm.accs[wave])[d4] = acc;
+      __syncthreads();
+      if (tid < 64) {
+        float tsum = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kWavesP; ++wv) tsum += sm.accs[wv][tid];
+        PG_ST64(dst + tid, pack(epp, tsum));
+      }
+      if (tid == 64) PG_ST64(dst + 64, pack(epp, mx));
+      if (tid == 65) PG_ST64(dst + 65, pack(epp, lsum));
+      __syncthreads();
+    }
+    // ---- B2: the workgroup that took split 0 of a head merges that head ----
+    const unsigned epa = epoch_of(p, t, l, 2);
+    for (int item = wg; item < items; item += G) {
+      const int h = item / ns, s = item - h * ns;
+      if (s != 0) continue;
+      float* stage = xs;  // ns*66 floats
+      bool ok = poll_vec<cdiv(kMaxSplits * 66, kThreads)>(p.part_t + (size_t)h * ns * 66,
+                                                          ns * 66, epp, stage, abort_word);
+      if (!all_ok(ok, sm)) return false;
+      if (tid < 64) {
+        float M = stage[64];
+        for (int q = 1; q < ns; ++q) M = fmaxf(M, stage[q * 66 + 64]);
+        float num = 0.0f, den = 0.0f;
+        for (int q = 0; q < ns; ++q) {
+          float wq = expf(stage[q * 66 + 64] - M);
+          den += wq * stage[q * 66 + 65];
+          num += wq * stage[q * 66 + tid];
+        }
+        PG_ST64(p.attn_t + h * 64 + tid, pack(epa, num / den));
+      }
+      __syncthreads();
+    }
+  }
+  return true;
+}
+
+// LN_f + lm_head for this workgroup's band of vocabulary rows, one weight row per
+// wavefront at a time with two rows in flight (the band is ~200 rows deep), plus
+// the band's argmax.  Kept out of line so that its registers are allocated apart
+// from the layer loop's.  Returns false if the wait for its input gave up.
+template <int C_>
+__device__ __attribute__((noinline)) bool lm_head_phase(const DecodeParams& p, Smem& sm, float* xs,
+                                                        float* xraw, int t, int v0, int v1) {
+  constexpr int C = C_, K4 = C_ / 4, J = cdiv(K4, 64), NEC = cdiv(C, kThreads);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wg = blockIdx.x;
+  // parameter fields are read once, before any weight row is requested
+  const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
+  float* const logits = p.logits;
+  u64* const best_t = p.best_t;
+  const float eps = p.eps;
+  const unsigned ep_best = epoch_of(p, t, p.L, 6);
+  LnParams<NEC> lp;
+  ln_fetch<NEC>(lp, p.ln_f_g, p.ln_f_b, C);
+  bool ok = poll_vec<NEC>(p.xm_t, C, epoch_of(p, t, p.L - 1, 5), xraw, p.status);
+  if (!all_ok(ok, sm)) return false;
+  Tile<J> ta, tb;
+  int r = v0 + wave;
+  // rows past the band are clamped to its last row and their products discarded
+  load_tile<J>(ta, wte4 + (size_t)min(r, v1 - 1) * K4, K4, lane);
+  load_tile<J>(tb, wte4 + (size_t)min(r + kWavesP, v1 - 1) * K4, K4, lane);
+  ln_lds<NEC, C>(xraw, xs, lp, eps);
+  f4 xr[J];
+  load_x<J>(xr, xs, K4, lane);
+  Best best{-INFINITY, 0xffffffffu};
+  for (; r < v1; r += 2 * kWavesP) {
+    float va = dot_tile<J>(ta, xr);
+    load_tile<J>(ta, wte4 + (size_t)min(r + 2 * kWavesP, v1 - 1) * K4, K4, lane);
+    if (lane == 0) logits[r] = va;
+    if (va > best.v) best = Best{va, (unsigned)r};
+    int r2 = r + kWavesP;
+    if (r2 < v1) {
+      float vb = dot_tile<J>(tb, xr);
+      load_tile<J>(tb, wte4 + (size_t)min(r2 + 2 * kWavesP, v1 - 1) * K4, K4, lane);
+      if (lane == 0) logits[r2] = vb;
+      if (vb > best.v) best = Best{vb, (unsigned)r2};
+    }
+  }
+  if (lane == 0) {
+    sm.bestv[wave] = best.v;
+    sm.besti[wave] = best.i;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    Best b{sm.bestv[0], sm.besti[0]};
+    for (int wv = 1; wv < kWavesP; ++wv) b = better(b, Best{sm.bestv[wv], sm.besti[wv]});
+    PG_ST64(best_t + 2 * wg, pack(ep_best, b.v));
+    PG_ST64(best_t + 2 * wg + 1, pack_u(ep_best, b.i));
+  }
+  __syncthreads();
+  return true;
+}
+
+#define PG_STAMP(layer, phase)                                                          \
+  do {                                                                                  \
+    if (p.prof && tid == 0 && t + 1 == p.n_fwd)                                         \
+      p.prof[((size_t)wg * (p.L + 1) + (layer)) * 8 + (phase)] = wall_clock64();        \
+  } while (0)
+
+// C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
+template <int C_>
 __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
+  constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
+  constexpr int G = kGrid;
+  constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
+  constexpr int UA = cdiv(RA * K4, kThreads), UD = cdiv(RD * K4, kThreads),
+                UE = cdiv(RE * K4, kThreads), UF = cdiv(RD * C, kThreads);
+  constexpr int J = cdiv(K4, 64);
+  constexpr int NEC = cdiv(C, kThreads), NEI = cdiv(I, kThreads);
+  static_assert(RA <= 32 && RE <= 32 && RD <= 8, "row sums are taken in one pass");
+  static_assert(K4 >= 64, "rows shorter than a wavefront are not handled");
+
   extern __shared__ float dyn[];
   __shared__ Smem sm;
-  float* xs = dyn;          // [I] normalised / staged input of the current GEMV
-  float* xraw = dyn + p.I;  // [C] residual stream entering the current half-block
+  float* xs = dyn;        // [I] normalised / staged input of the current matrix
+  float* xraw = dyn + I;  // [C] residual stream entering the current half-block
+  float* prod = dyn + I + C;  // [512 * max U] per-float4 products of the current band
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wg = blockIdx.x, G = gridDim.x;
-  const int C = p.C, I = p.I, H = p.H, V = p.V, P = p.P;
-  const int K4 = C >> 2;  // float4 per row for K = C, and per segment for K = I = 4C
+  const int wg = blockIdx.x;
+  const int H = p.H, V = p.V, P = p.P;
   unsigned* abort_word = p.status;
   const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
 
-  // row ranges of this workgroup per matrix
-  auto range = [&](int nout, int& r0, int& r1) {
-    r0 = (int)(((long long)wg * nout) / G);
-    r1 = (int)(((long long)(wg + 1) * nout) / G);
-  };
-  int a0, a1, d0, d1, e0, e1, v0, v1;
-  range(3 * C, a0, a1);
-  range(C, d0, d1);
-  range(I, e0, e1);
-  range(V, v0, v1);
+  // row bands of this workgroup
+  const int a0 = (int)(((long long)wg * (3 * C)) / G), a1 = (int)(((long long)(wg + 1) * (3 * C)) / G);
+  const int d0 = (int)(((long long)wg * C) / G), d1 = (int)(((long long)(wg + 1) * C) / G);
+  const int e0 = (int)(((long long)wg * I) / G), e1 = (int)(((long long)(wg + 1) * I) / G);
+  const int v0 = (int)(((long long)wg * V) / G), v1 = (int)(((long long)(wg + 1) * V) / G);
+  const int nA4 = (a1 - a0) * K4, nD4 = (d1 - d0) * K4, nE4 = (e1 - e0) * K4, nF4 = (d1 - d0) * C;
+
+  if (tid == 0) sm.ok = 1;
+  __syncthreads();
+
+  // The out-of-line phases get their own copy of the parameters.  Taking the address
+  // of `p` itself would move it to scratch memory, and every later read of a field
+  // would be a memory load that has to wait for the weight bands in flight.
+  const DecodeParams pc = p;
 
   int t = 0;
   int stopped = 0;
   unsigned tok = 0;
-  Tile<J> pa;  // first tile of the next row-phase (c_attn of a layer, or lm_head)
+  f4 WA[UA];  // c_attn band of the layer about to run
   for (; t < p.n_fwd; ++t) {
     const int pos = p.pos0 + t;
-    {
-      const f4* W4 = reinterpret_cast<const f4*>(p.layers[0].c_attn_w);
-      int r = a0 + wave;
-      load_tile<J>(pa, W4 + (size_t)r * K4, K4, lane, r < a1);
-    }
+    PG_STAMP(p.L, 7);
+    band_load<UA>(WA, reinterpret_cast<const f4*>(p.layers[0].c_attn_w) + (size_t)a0 * K4, nA4);
     // ---- token to embed: given, or the argmax of the previous step's logits ----
     if (p.force_ids) {
       tok = p.force_ids[t];
@@ -284,7 +625,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
     } else {
       // merge the per-workgroup (value, index) pairs in workgroup order
       float* bv = xs;  // 2*G floats of staging
-      bool ok = poll_vec<2>(p.best_t, 2 * G, epoch_of(p, t - 1, p.L, 6), bv, abort_word);
+      bool ok = poll_vec<1>(p.best_t, 2 * G, epoch_of(p, t - 1, p.L, 6), bv, abort_word);
       if (!all_ok(ok, sm)) return;
       if (tid == 0) {
         Best b{-INFINITY, 0xffffffffu};
@@ -308,335 +649,123 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 
       // ================= A: LN1 + c_attn =================
       {
-        const f4* W4 = reinterpret_cast<const f4*>(w.c_attn_w);
-        Tile<J> ta = pa, tb;  // ta was requested during the previous phase F / token start
-        int r = a0 + wave;
-        load_tile<J>(tb, W4 + (size_t)(r + kWavesP) * K4, K4, lane, r + kWavesP < a1);
+        LnParams<NEC> lp;
+        ln_fetch<NEC>(lp, w.ln_1_g, w.ln_1_b, C);
+        const float bias = w.c_attn_b[a0 + min(tid >> 4, a1 - a0 - 1)];
         if (l == 0) {
           // embedding (rust.rs:966-974)
           for (int i = tid; i < C; i += kThreads)
             xraw[i] = p.wte[(size_t)tok * C + i] + p.wpe[(size_t)pos * C + i];
           __syncthreads();
         } else {
-          bool ok = poll_vec<(4 * 64 * J + kThreads - 1) / kThreads>(
-              p.xm_t, C, epoch_of(p, t, l - 1, 5), xraw, abort_word);
+          bool ok = poll_vec<NEC>(p.xm_t, C, epoch_of(p, t, l - 1, 5), xraw, abort_word);
           if (!all_ok(ok, sm)) return;
         }
-        ln_lds(xraw, xs, C, w.ln_1_g, w.ln_1_b, p.eps, sm);
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
-        const unsigned ep = epoch_of(p, t, l, 0);
-        for (; r < a1; r += 2 * kWavesP) {
-          float va = dot_tile<J>(ta, xr);
-          load_tile<J>(ta, W4 + (size_t)(r + 2 * kWavesP) * K4, K4, lane, r + 2 * kWavesP < a1);
-          if (lane == 0) PG_ST64(p.qkv_t + r, pack(ep, w.c_attn_b[r] + va));
-          int r2 = r + kWavesP;
-          if (r2 < a1) {
-            float vb = dot_tile<J>(tb, xr);
-            load_tile<J>(tb, W4 + (size_t)(r2 + 2 * kWavesP) * K4, K4, lane, r2 + 2 * kWavesP < a1);
-            if (lane == 0) PG_ST64(p.qkv_t + r2, pack(ep, w.c_attn_b[r2] + vb));
-          }
+        ln_lds<NEC, C>(xraw, xs, lp, p.eps);
+        band_mul<UA, K4>(WA, xs, prod);
+        __syncthreads();
+        {
+          const int row = tid >> 4;  // 16 lanes per row, 32 rows per pass (RA <= 32)
+          const float sum = band_row<K4, 16>(prod, row, a1 - a0);
+          if ((tid & 15) == 0 && row < a1 - a0)
+            PG_ST64(p.qkv_t + a0 + row, pack(epoch_of(p, t, l, 0), bias + sum));
         }
+        __syncthreads();
       }
+      PG_STAMP(l, 0);
 
       // ================= B: attention over keys [0, pos] =================
-      // c_proj's first tiles are requested now so they stream during attention.
-      const f4* Wd4 = reinterpret_cast<const f4*>(w.c_proj_w);
-      Tile<J> da, db;
-      {
-        int r = d0 + wave;
-        load_tile<J>(da, Wd4 + (size_t)r * K4, K4, lane, r < d1);
-      }
-      {
-        const int ns = p.ns, items = H * ns, n = pos + 1;
-        const int per = (n + ns - 1) / ns;
-        const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
-        const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
-        for (int item = wg; item < items; item += G) {
-          const int h = item / ns, s = item - h * ns;
-          const int k0 = s * per, k1 = min(n, k0 + per);
-          u64* dst = p.part_t + (size_t)item * 66;
-          if (k0 >= k1) {  // empty split: neutral element of the merge
-            if (tid < 64) PG_ST64(dst + tid, pack(epp, 0.0f));
-            if (tid == 64) PG_ST64(dst + 64, pack(epp, -INFINITY));
-            if (tid == 65) PG_ST64(dst + 65, pack(epp, 0.0f));
-            continue;
-          }
-          const bool owns_new = (pos >= k0 && pos < k1);
-          const f4* Kh = reinterpret_cast<const f4*>(kc + (size_t)h * P * 64);
-          const f4* Vh = reinterpret_cast<const f4*>(vc + (size_t)h * P * 64);
-          f4 kr[kAttnSteps], vr[kAttnSteps];
-#pragma unroll
-          for (int i = 0; i < kAttnSteps; ++i) {
-            int key = k0 + slot + 32 * i;
-            if (key < k1 && key < pos) {
-              kr[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
-              vr[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
-            } else {
-              kr[i] = f4{0.f, 0.f, 0.f, 0.f};
-              vr[i] = f4{0.f, 0.f, 0.f, 0.f};
-            }
-          }
-          // q of this head, and this token's own K/V rows if the split holds pos
-          bool ok = true;
-          {
-            const int part = tid >> 6;  // 0: q, 1: k_new, 2: v_new
-            if (part == 0 || (owns_new && part < 3)) {
-              const u64* src = p.qkv_t + (size_t)part * C + h * 64 + lane;
-              u64 v = PG_LD64(src);
-              unsigned spins = 0;
-              while (tag_of(v) != epq) {
-                if (++spins > kSpinLimit) {
-                  ok = false;
-                  PG_ST32(abort_word, 1u);
-                  break;
-                }
-                if ((spins & 63) == 0 && PG_LD32(abort_word) != 0) {
-                  ok = false;
-                  break;
-                }
-                __builtin_amdgcn_s_sleep(2);
-                v = PG_LD64(src);
-              }
-              float f = val_of(v);
-              if (part == 0) sm.qs[lane] = f;
-              if (part == 1) {
-                sm.kn[lane] = f;
-                // K append (rust.rs:1677-1683); written through to memory so that a
-                // later token's reader on another XCD cannot miss it in a remote L2
-                PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, f);
-              }
-              if (part == 2) {
-                sm.vn[lane] = f;
-                PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, f);  // V append
-              }
-            }
-          }
-          if (!all_ok(ok, sm)) return;
-          const f4 qv = reinterpret_cast<const f4*>(sm.qs)[d4];
-          float sc[kAttnSteps];
-          float mx = -INFINITY;
-#pragma unroll
-          for (int i = 0; i < kAttnSteps; ++i) {
-            int key = k0 + slot + 32 * i;
-            if (key == pos && key < k1) {
-              kr[i] = reinterpret_cast<const f4*>(sm.kn)[d4];
-              vr[i] = reinterpret_cast<const f4*>(sm.vn)[d4];
-            }
-            float sv = qv.x * kr[i].x + qv.y * kr[i].y + qv.z * kr[i].z + qv.w * kr[i].w;
-            sv += __shfl_xor(sv, 1, 64);
-            sv += __shfl_xor(sv, 2, 64);
-            sv += __shfl_xor(sv, 4, 64);
-            sv += __shfl_xor(sv, 8, 64);
-            sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
-            sc[i] = (key < k1) ? sv : -INFINITY;
-            mx = fmaxf(mx, sc[i]);
-          }
-          mx = bmax(mx, sm);
-          float lsum = 0.0f;
-          f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int i = 0; i < kAttnSteps; ++i) {
-            float pr = expf(sc[i] - mx);  // exp(-inf) = 0 for absent keys
-            if (d4 == 0) lsum += pr;
-            acc += pr * vr[i];
-          }
-          lsum = bsum(lsum, sm);
-#pragma unroll
-          for (int off = 16; off <= 32; off <<= 1) {
-            acc.x += __shfl_xor(acc.x, off, 64);
-            acc.y += __shfl_xor(acc.y, off, 64);
-            acc.z += __shfl_xor(acc.z, off, 64);
-            acc.w += __shfl_xor(acc.w, off, 64);
-          }
-          if (sub == 0) reinterpret_cast<f4*>(sm.accs[wave])[d4] = acc;
-          __syncthreads();
-          if (tid < 64) {
-            float tsum = 0.0f;
-#pragma unroll
-            for (int wv = 0; wv < kWavesP; ++wv) tsum += sm.accs[wv][tid];
-            PG_ST64(dst + tid, pack(epp, tsum));
-          }
-          if (tid == 64) PG_ST64(dst + 64, pack(epp, mx));
-          if (tid == 65) PG_ST64(dst + 65, pack(epp, lsum));
-          __syncthreads();
-        }
-        // ---- B2: the workgroup that took split 0 of a head merges that head ----
-        const unsigned epa = epoch_of(p, t, l, 2);
-        for (int item = wg; item < items; item += G) {
-          const int h = item / ns, s = item - h * ns;
-          if (s != 0) continue;
-          float* stage = xs;  // ns*66 floats
-          bool ok = poll_vec<(kMaxSplits * 66 + kThreads - 1) / kThreads>(
-              p.part_t + (size_t)h * ns * 66, ns * 66, epp, stage, abort_word);
-          if (!all_ok(ok, sm)) return;
-          if (tid < 64) {
-            float M = stage[64];
-            for (int q = 1; q < ns; ++q) M = fmaxf(M, stage[q * 66 + 64]);
-            float num = 0.0f, den = 0.0f;
-            for (int q = 0; q < ns; ++q) {
-              float wq = expf(stage[q * 66 + 64] - M);
-              den += wq * stage[q * 66 + 65];
-              num += wq * stage[q * 66 + tid];
-            }
-            PG_ST64(p.attn_t + h * 64 + tid, pack(epa, num / den));
-          }
-          __syncthreads();
-        }
-      }
+      f4 WE[UE];  // c_fc band, requested as soon as D's input has arrived
+      if (!attention_phase(pc, sm, xs, t, l, pos, kc, vc)) return;
+      PG_STAMP(l, 2);
 
       // ================= D: c_proj + residual =================
-      const f4* We4 = reinterpret_cast<const f4*>(w.c_fc_w);
-      Tile<J> ea, eb;
       {
-        // c_fc's first tiles are requested before D waits for the attention output
-        int re = e0 + wave;
-        load_tile<J>(ea, We4 + (size_t)re * K4, K4, lane, re < e1);
-        load_tile<J>(db, Wd4 + (size_t)(d0 + wave + kWavesP) * K4, K4, lane, d0 + wave + kWavesP < d1);
+        const float bias = w.c_proj_b[d0 + min(tid >> 4, d1 - d0 - 1)];
+        f4 WD[UD];  // c_proj band: small, requested right before D waits for its input
+        band_load<UD>(WD, reinterpret_cast<const f4*>(w.c_proj_w) + (size_t)d0 * K4, nD4);
         __syncthreads();  // every wave is done with xs of the previous phase
-        bool ok = poll_vec<(4 * 64 * J + kThreads - 1) / kThreads>(
-            p.attn_t, C, epoch_of(p, t, l, 2), xs, abort_word);
+        bool ok = poll_vec<NEC>(p.attn_t, C, epoch_of(p, t, l, 2), xs, abort_word);
         if (!all_ok(ok, sm)) return;
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
-        const unsigned ep = epoch_of(p, t, l, 3);
-        int r = d0 + wave;
-        for (; r < d1; r += 2 * kWavesP) {
-          float va = dot_tile<J>(da, xr);
-          load_tile<J>(da, Wd4 + (size_t)(r + 2 * kWavesP) * K4, K4, lane, r + 2 * kWavesP < d1);
-          if (lane == 0) PG_ST64(p.xa_t + r, pack(ep, xraw[r] + (w.c_proj_b[r] + va)));
-          int r2 = r + kWavesP;
-          if (r2 < d1) {
-            float vb = dot_tile<J>(db, xr);
-            load_tile<J>(db, Wd4 + (size_t)(r2 + 2 * kWavesP) * K4, K4, lane, r2 + 2 * kWavesP < d1);
-            if (lane == 0) PG_ST64(p.xa_t + r2, pack(ep, xraw[r2] + (w.c_proj_b[r2] + vb)));
-          }
+        band_load<UE>(WE, reinterpret_cast<const f4*>(w.c_fc_w) + (size_t)e0 * K4, nE4);
+        band_mul<UD, K4>(WD, xs, prod);
+        __syncthreads();
+        {
+          const int row = tid >> 4;
+          const float sum = band_row<K4, 16>(prod, row, d1 - d0);
+          if ((tid & 15) == 0 && row < d1 - d0)
+            PG_ST64(p.xa_t + d0 + row,
+                    pack(epoch_of(p, t, l, 3), xraw[d0 + row] + (bias + sum)));
         }
+        __syncthreads();
       }
+      PG_STAMP(l, 3);
 
       // ================= E: LN2 + c_fc + GELU =================
-      // F tiles: (row, segment) pairs, 4 segments of C/4 float4 per row of K = 4C.
-      const f4* Wf4 = reinterpret_cast<const f4*>(w.c_proj_mlp_w);
-      const int nF = (d1 - d0) * 4;
-      Tile<J> fa, fb;
+      // mlp c_proj band (rows of K = 4C): the first half is requested before E waits,
+      // the second half once E's own band has been consumed and its registers are free
+      f4 WF[UF];
+      const f4* Wf4 = reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)d0 * C;
       {
-        {
-          int id = wave;
-          load_tile<J>(fa, Wf4 + (size_t)(d0 + (id >> 2)) * C + (size_t)(id & 3) * K4, K4, lane, id < nF);
-          load_tile<J>(eb, We4 + (size_t)(e0 + wave + kWavesP) * K4, K4, lane, e0 + wave + kWavesP < e1);
-        }
-        __syncthreads();  // every wave is done with xraw and xs of phase D
-        bool ok = poll_vec<(4 * 64 * J + kThreads - 1) / kThreads>(
-            p.xa_t, C, epoch_of(p, t, l, 3), xraw, abort_word);
+        LnParams<NEC> lp;
+        ln_fetch<NEC>(lp, w.ln_2_g, w.ln_2_b, C);
+        const float bias = w.c_fc_b[e0 + min(tid >> 4, e1 - e0 - 1)];
+        bool ok = poll_vec<NEC>(p.xa_t, C, epoch_of(p, t, l, 3), xraw, abort_word);
         if (!all_ok(ok, sm)) return;
-        ln_lds(xraw, xs, C, w.ln_2_g, w.ln_2_b, p.eps, sm);
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
-        const unsigned ep = epoch_of(p, t, l, 4);
-        int r = e0 + wave;
-        for (; r < e1; r += 2 * kWavesP) {
-          float va = dot_tile<J>(ea, xr);
-          load_tile<J>(ea, We4 + (size_t)(r + 2 * kWavesP) * K4, K4, lane, r + 2 * kWavesP < e1);
-          if (lane == 0) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(w.c_fc_b[r] + va)));
-          int r2 = r + kWavesP;
-          if (r2 < e1) {
-            float vb = dot_tile<J>(eb, xr);
-            load_tile<J>(eb, We4 + (size_t)(r2 + 2 * kWavesP) * K4, K4, lane, r2 + 2 * kWavesP < e1);
-            if (lane == 0) PG_ST64(p.h_t + r2, pack(ep, gelu_tanh(w.c_fc_b[r2] + vb)));
-          }
+        PG_STAMP(l, 6);
+        band_load<UF, 0, UF / 2>(WF, Wf4, nF4);
+        ln_lds<NEC, C>(xraw, xs, lp, p.eps);
+        band_mul<UE, K4>(WE, xs, prod);
+        PG_STAMP(l, 7);
+        band_load<UF, UF / 2, UF>(WF, Wf4, nF4);
+        __syncthreads();
+        {
+          const int row = tid >> 4;
+          const float sum = band_row<K4, 16>(prod, row, e1 - e0);
+          if ((tid & 15) == 0 && row < e1 - e0)
+            PG_ST64(p.h_t + e0 + row, pack(epoch_of(p, t, l, 4), gelu_tanh(bias + sum)));
         }
+        __syncthreads();
       }
+      PG_STAMP(l, 4);
 
       // ================= F: mlp c_proj + residual =================
+      // The next layer's c_attn band is requested once F's input has arrived.
       {
-        if (l + 1 < p.L) {
-          const f4* Wn4 = reinterpret_cast<const f4*>(p.layers[l + 1].c_attn_w);
-          int r = a0 + wave;
-          load_tile<J>(pa, Wn4 + (size_t)r * K4, K4, lane, r < a1);
-        } else {
-          int r = v0 + wave;
-          load_tile<J>(pa, wte4 + (size_t)r * K4, K4, lane, r < v1);
-        }
-        load_tile<J>(fb, Wf4 + (size_t)(d0 + ((wave + kWavesP) >> 2)) * C +
-                               (size_t)((wave + kWavesP) & 3) * K4, K4, lane, wave + kWavesP < nF);
-        __syncthreads();  // xs is about to be overwritten
-        bool ok = poll_vec<(16 * 64 * J + kThreads - 1) / kThreads>(
-            p.h_t, I, epoch_of(p, t, l, 4), xs, abort_word);
+        const float bias = w.c_proj_mlp_b[d0 + min(tid >> 6, d1 - d0 - 1)];
+        bool ok = poll_vec<NEI>(p.h_t, I, epoch_of(p, t, l, 4), xs, abort_word);
         if (!all_ok(ok, sm)) return;
-        int id = wave;
-        for (; id < nF; id += 2 * kWavesP) {
-          f4 xr[J];
-          load_x<J>(xr, xs + (size_t)(id & 3) * C, K4, lane);
-          float va = dot_tile<J>(fa, xr);
-          int nx = id + 2 * kWavesP;
-          load_tile<J>(fa, Wf4 + (size_t)(d0 + (nx >> 2)) * C + (size_t)(nx & 3) * K4, K4, lane, nx < nF);
-          if (lane == 0) sm.psum[id] = va;
-          int id2 = id + kWavesP;
-          if (id2 < nF) {
-            load_x<J>(xr, xs + (size_t)(id2 & 3) * C, K4, lane);
-            float vb = dot_tile<J>(fb, xr);
-            int nx2 = id2 + 2 * kWavesP;
-            load_tile<J>(fb, Wf4 + (size_t)(d0 + (nx2 >> 2)) * C + (size_t)(nx2 & 3) * K4, K4,
-                           lane, nx2 < nF);
-            if (lane == 0) sm.psum[id2] = vb;
-          }
-        }
+        // The next layer's c_attn band: half now, half once F's own band is consumed
+        // (after the last layer this re-reads its own band: an unconditional request
+        // keeps the load count exact; the data is never used).
+        const f4* Wn4 = reinterpret_cast<const f4*>(p.layers[min(l + 1, p.L - 1)].c_attn_w) +
+                        (size_t)a0 * K4;
+        band_load<UA, 0, UA / 2>(WA, Wn4, nA4);
+        band_mul<UF, C>(WF, xs, prod);
+        band_load<UA, UA / 2, UA>(WA, Wn4, nA4);
         __syncthreads();
-        const unsigned ep = epoch_of(p, t, l, 5);
-        if (tid < d1 - d0) {
-          int r = d0 + tid;
-          float s4 = (sm.psum[4 * tid] + sm.psum[4 * tid + 1]) +
-                     (sm.psum[4 * tid + 2] + sm.psum[4 * tid + 3]);
-          PG_ST64(p.xm_t + r, pack(ep, xraw[r] + (w.c_proj_mlp_b[r] + s4)));
+        {
+          const int row = tid >> 6;  // rows of K = 4C: one wavefront per row (RD <= 8)
+          const float sum = band_row<C, 64>(prod, row, d1 - d0);
+          if ((tid & 63) == 0 && row < d1 - d0)
+            PG_ST64(p.xm_t + d0 + row,
+                    pack(epoch_of(p, t, l, 5), xraw[d0 + row] + (bias + sum)));
         }
         __syncthreads();
       }
+      PG_STAMP(l, 5);
     }  // layers
 
     // ================= LN_f + lm_head (rust.rs:982-1002) =================
     if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
-      Tile<J> ta = pa, tb;  // ta was requested during the last layer's phase F
-      int r = v0 + wave;
-      load_tile<J>(tb, wte4 + (size_t)(r + kWavesP) * K4, K4, lane, r + kWavesP < v1);
-      bool ok = poll_vec<(4 * 64 * J + kThreads - 1) / kThreads>(
-          p.xm_t, C, epoch_of(p, t, p.L - 1, 5), xraw, abort_word);
-      if (!all_ok(ok, sm)) return;
-      ln_lds(xraw, xs, C, p.ln_f_g, p.ln_f_b, p.eps, sm);
-      f4 xr[J];
-      load_x<J>(xr, xs, K4, lane);
-      Best best{-INFINITY, 0xffffffffu};
-      for (; r < v1; r += 2 * kWavesP) {
-        float va = dot_tile<J>(ta, xr);
-        load_tile<J>(ta, wte4 + (size_t)(r + 2 * kWavesP) * K4, K4, lane, r + 2 * kWavesP < v1);
-        if (lane == 0) p.logits[r] = va;
-        if (va > best.v) best = Best{va, (unsigned)r};
-        int r2 = r + kWavesP;
-        if (r2 < v1) {
-          float vb = dot_tile<J>(tb, xr);
-          load_tile<J>(tb, wte4 + (size_t)(r2 + 2 * kWavesP) * K4, K4, lane, r2 + 2 * kWavesP < v1);
-          if (lane == 0) p.logits[r2] = vb;
-          if (vb > best.v) best = Best{vb, (unsigned)r2};
-        }
-      }
-      if (lane == 0) {
-        sm.bestv[wave] = best.v;
-        sm.besti[wave] = best.i;
-      }
-      __syncthreads();
-      if (tid == 0) {
-        Best b{sm.bestv[0], sm.besti[0]};
-        for (int wv = 1; wv < kWavesP; ++wv) b = better(b, Best{sm.bestv[wv], sm.besti[wv]});
-        const unsigned ep = epoch_of(p, t, p.L, 6);
-        PG_ST64(p.best_t + 2 * wg, pack(ep, b.v));
-        PG_ST64(p.best_t + 2 * wg + 1, pack_u(ep, b.i));
-      }
-      __syncthreads();
+      if (!lm_head_phase<C_>(pc, sm, xs, xraw, t, v0, v1)) return;
+      PG_STAMP(p.L, 6);
     }
   }  // tokens
 
   if (!stopped && p.select_last && p.n_fwd > 0) {
     float* bv = xs;
-    bool ok = poll_vec<2>(p.best_t, 2 * G, epoch_of(p, p.n_fwd - 1, p.L, 6), bv, abort_word);
+    bool ok = poll_vec<1>(p.best_t, 2 * G, epoch_of(p, p.n_fwd - 1, p.L, 6), bv, abort_word);
     if (!all_ok(ok, sm)) return;
     if (wg == 0 && tid == 0) {
       Best b{-INFINITY, 0xffffffffu};
@@ -654,33 +783,56 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 
 }  // namespace
 
-int persistent_tile_depth(int C) {
-  int j = (C / 4 + 63) / 64;
-  return (j == 3 || j == 4 || j == 7) ? j : 0;
+// n_embd values the persistent kernel is instantiated for (GPT-2 small, medium, XL).
+bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }
+int persistent_grid() { return kGrid; }
+
+size_t persistent_lds_bytes(int C) {
+  // xs [4C] + xraw [C] + prod [512 * max float4 per thread over the four bands]
+  const int K4 = C / 4, G = kGrid;
+  const int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(4 * C, G);
+  int U = cdiv(RA * K4, kThreads);
+  U = U > cdiv(RD * K4, kThreads) ? U : cdiv(RD * K4, kThreads);
+  U = U > cdiv(RE * K4, kThreads) ? U : cdiv(RE * K4, kThreads);
+  U = U > cdiv(RD * C, kThreads) ? U : cdiv(RD * C, kThreads);
+  return (size_t)(5 * C + kThreads * U) * sizeof(float);
 }
 
-size_t persistent_lds_bytes(int C, int I) { return (size_t)(I + C) * sizeof(float); }
-
-hipError_t launch_decode_persistent(const DecodeParams& p, int grid, hipStream_t s) {
-  const size_t lds = persistent_lds_bytes(p.C, p.I);
-  const int j = persistent_tile_depth(p.C);
-  if (j == 3)
-    hipLaunchKernelGGL(k_decode_persistent<3>, dim3(grid), dim3(kThreads), lds, s, p);
-  else if (j == 4)
-    hipLaunchKernelGGL(k_decode_persistent<4>, dim3(grid), dim3(kThreads), lds, s, p);
-  else if (j == 7)
-    hipLaunchKernelGGL(k_decode_persistent<7>, dim3(grid), dim3(kThreads), lds, s, p);
-  else
-    return hipErrorInvalidValue;
+namespace {
+template <int C_>
+hipError_t launch_one(const DecodeParams& p, hipStream_t s) {
+  const size_t lds = persistent_lds_bytes(C_);
+  // more than the 64 KiB default of dynamic LDS: opt in once per device
+  static thread_local int armed_device = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (armed_device != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_persistent<C_>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    armed_device = dev;
+  }
+  hipLaunchKernelGGL(k_decode_persistent<C_>, dim3(kGrid), dim3(kThreads), lds, s, p);
   return hipGetLastError();
 }
+}  // namespace
 
-hipError_t persistent_max_blocks_per_cu(int C, int I, int* out) {
-  const size_t lds = persistent_lds_bytes(C, I);
-  const int j = persistent_tile_depth(C);
-  if (j == 3) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<3>, kThreads, lds);
-  if (j == 4) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<4>, kThreads, lds);
-  if (j == 7) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<7>, kThreads, lds);
+hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
+  if (p.C == 768) return launch_one<768>(p, s);
+  if (p.C == 1024) return launch_one<1024>(p, s);
+  if (p.C == 1600) return launch_one<1600>(p, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t persistent_max_blocks_per_cu(int C, int* out) {
+  const size_t lds = persistent_lds_bytes(C);
+  if (C == 768)
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<768>, kThreads, lds);
+  if (C == 1024)
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1024>, kThreads, lds);
+  if (C == 1600)
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1600>, kThreads, lds);
   *out = 0;
   return hipSuccess;
 }

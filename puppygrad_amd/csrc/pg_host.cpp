@@ -11,6 +11,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -173,6 +174,17 @@ pg_status validate_weights(const Cfg& c, const pg_gpt2_weights_view& w) {
 
 size_t round_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
 
+struct DevBuf {
+  float* p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+  pg_status alloc(size_t n) {
+    PG_HIP(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(float)));
+    return PG_OK;
+  }
+};
+
 pg_status select_device(int device) {
   int n = 0;
   hipError_t e = hipGetDeviceCount(&n);
@@ -326,15 +338,34 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   p.epoch0 = c->epoch;
   p.ns = m->attn_splits;
   p.status = c->status;
+  // Development aid: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
+  // of the last token of each persistent launch (raw u64, [grid][L+1][8]).
+  const char* prof_path = std::getenv("PG_DECODE_PROF");
+  DevBuf prof;
+  const size_t prof_words = (size_t)m->persistent_grid * (g.L + 1) * 8;
+  if (prof_path) {
+    pg_status ps = prof.alloc(prof_words * 2);
+    if (ps) return ps;
+    PG_HIP(pgk::launch_fill_zero(prof.p, prof_words * 2, c->stream));
+    p.prof = reinterpret_cast<unsigned long long*>(prof.p);
+  }
   c->epoch += span;
   std::lock_guard<std::mutex> lk(g_persistent_mu);
   PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
   if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
-  PG_HIP(pgk::launch_decode_persistent(p, m->persistent_grid, c->stream));
+  PG_HIP(pgk::launch_decode_persistent(p, c->stream));
   if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
   PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
                         c->stream));
   PG_HIP(hipStreamSynchronize(c->stream));
+  if (prof_path) {
+    std::vector<unsigned long long> host(prof_words);
+    PG_HIP(hipMemcpy(host.data(), prof.p, prof_words * 8, hipMemcpyDeviceToHost));
+    if (FILE* f = std::fopen(prof_path, "wb")) {
+      std::fwrite(host.data(), 8, prof_words, f);
+      std::fclose(f);
+    }
+  }
   if (c->h_status[0] != 0)
     return fail(PG_BACKEND, "persistent decode kernel gave up waiting for a dependency "
                             "(another kernel may be occupying the device)");
@@ -447,16 +478,6 @@ pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg
   return PG_OK;
 }
 
-struct DevBuf {
-  float* p = nullptr;
-  ~DevBuf() {
-    if (p) (void)hipFree(p);
-  }
-  pg_status alloc(size_t n) {
-    PG_HIP(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(float)));
-    return PG_OK;
-  }
-};
 
 }  // namespace
 
@@ -576,16 +597,16 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
                    hipMemcpyHostToDevice));
 
   // The persistent decode kernel covers head_dim 64, n_inner = 4 n_embd and the
-  // row widths it is instantiated for; everything else takes the per-op launches.
+  // GPT-2 widths it is instantiated for, on a device that can hold its whole grid
+  // at once; everything else takes the per-op launches.
   {
-    const int grid = m->num_cus;
+    const int grid = pgk::persistent_grid();
     int blocks_per_cu = 0;
-    bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_tile_depth((int)g.C) != 0 &&
-                    g.P <= 4096 && grid > 0 && (g.C + grid - 1) / grid <= 64 &&
-                    2 * (size_t)grid <= g.I;
+    bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
+                    g.P <= 4096 && g.V >= (size_t)grid;
     if (shape_ok) {
-      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, (int)g.I, &blocks_per_cu));
-      shape_ok = blocks_per_cu >= 1;
+      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu));
+      shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
     }
     if (shape_ok) {
       int ns = std::min<int>(16, grid / (int)g.H);
@@ -596,8 +617,8 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     }
     if (opts.decode_path == PG_DECODE_PERSISTENT && !shape_ok)
       return fail(PG_INVALID_CONFIG,
-                  "hip backend decode_path=persistent needs head_dim 64, n_inner = 4*n_embd and "
-                  "n_embd in (512,1024] or (1536,1792]");
+                  "hip backend decode_path=persistent needs head_dim 64, n_inner = 4*n_embd, "
+                  "n_embd in {768, 1024, 1600} and a device that holds 256 workgroups at once");
     m->persistent = shape_ok && opts.decode_path != PG_DECODE_KERNELS;
     m->persistent_grid = grid;
   }

@@ -99,13 +99,18 @@ struct DecodeParams {
   unsigned epoch0;
   int ns;
   unsigned* status;  // [0] abort, [1] forwards done, [2] stopped at eos
+  // Optional [grid][L+1][8] timestamps (100 MHz wall clock) of the last token's phase
+  // completions per workgroup; slot [L][7] holds the token's start.
+  unsigned long long* prof;
 };
 
 
-// Tile depth the persistent kernel is built for at this n_embd (0: unsupported).
-int persistent_tile_depth(int C);
-size_t persistent_lds_bytes(int C, int I);
-hipError_t persistent_max_blocks_per_cu(int C, int I, int* out);
-hipError_t launch_decode_persistent(const DecodeParams& p, int grid, hipStream_t s);
+// n_embd values the persistent kernel is instantiated for, its fixed grid, its
+// dynamic LDS need, and how many of its workgroups fit on one CU.
+bool persistent_supports(int C);
+int persistent_grid();
+size_t persistent_lds_bytes(int C);
+hipError_t persistent_max_blocks_per_cu(int C, int* out);
+hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
 
 }  // namespace pgk
