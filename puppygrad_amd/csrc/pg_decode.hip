@@ -89,6 +89,7 @@ struct Smem {
   float red[2][kWavesP];  // alternating buffers: consecutive reductions need one barrier each
   float accs[kWavesP][64];
   float qs[64], kn[64], vn[64];
+  float psum[64];  // phase F: partial sums of the (row, quarter) tiles
   float bestv[kWavesP];
   unsigned besti[kWavesP];
   int ok;
@@ -570,53 +571,68 @@ __device__ __attribute__((noinline)) bool lm_head_phase(const DecodeParams& p, S
   } while (0)
 
 // C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
+//
+// Each wavefront owns whole weight rows (row-phases A, D, E) or quarter rows of
+// K = 4C (phase F): row r0 + wave + 8*i for i < T.  A row is J float4 per lane; the
+// input vector's matching J float4 sit in registers for the whole phase, so a row
+// costs J loads, 4J multiply-adds and one DPP tree.  All T rows of the NEXT matrix
+// are requested as soon as the current phase's input has arrived.
 template <int C_>
 __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
   constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
   constexpr int G = kGrid;
   constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
-  constexpr int UA = cdiv(RA * K4, kThreads), UD = cdiv(RD * K4, kThreads),
-                UE = cdiv(RE * K4, kThreads), UF = cdiv(RD * C, kThreads);
+  constexpr int TA = cdiv(RA, kWavesP), TD = cdiv(RD, kWavesP), TE = cdiv(RE, kWavesP),
+                TF = cdiv(4 * RD, kWavesP);  // rows (quarter rows for F) per wavefront
   constexpr int J = cdiv(K4, 64);
   constexpr int NEC = cdiv(C, kThreads), NEI = cdiv(I, kThreads);
-  static_assert(RA <= 32 && RE <= 32 && RD <= 8, "row sums are taken in one pass");
-  static_assert(K4 >= 64, "rows shorter than a wavefront are not handled");
+  static_assert(4 * RD <= 64, "phase F partial sums");
 
   extern __shared__ float dyn[];
   __shared__ Smem sm;
   float* xs = dyn;        // [I] normalised / staged input of the current matrix
   float* xraw = dyn + I;  // [C] residual stream entering the current half-block
-  float* prod = dyn + I + C;  // [512 * max U] per-float4 products of the current band
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wg = blockIdx.x;
-  const int H = p.H, V = p.V, P = p.P;
+  const int V = p.V;
   unsigned* abort_word = p.status;
-  const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
 
   // row bands of this workgroup
   const int a0 = (int)(((long long)wg * (3 * C)) / G), a1 = (int)(((long long)(wg + 1) * (3 * C)) / G);
   const int d0 = (int)(((long long)wg * C) / G), d1 = (int)(((long long)(wg + 1) * C) / G);
   const int e0 = (int)(((long long)wg * I) / G), e1 = (int)(((long long)(wg + 1) * I) / G);
   const int v0 = (int)(((long long)wg * V) / G), v1 = (int)(((long long)(wg + 1) * V) / G);
-  const int nA4 = (a1 - a0) * K4, nD4 = (d1 - d0) * K4, nE4 = (e1 - e0) * K4, nF4 = (d1 - d0) * C;
+  const int nF = (d1 - d0) * 4;  // (row, quarter) tiles of phase F
 
   if (tid == 0) sm.ok = 1;
   __syncthreads();
 
   // The out-of-line phases get their own copy of the parameters.  Taking the address
   // of `p` itself would move it to scratch memory, and every later read of a field
-  // would be a memory load that has to wait for the weight bands in flight.
+  // would be a memory load that has to wait for the weight rows in flight.
   const DecodeParams pc = p;
+
+  // Row i of this wavefront in a band [r0, r1), clamped into the band (rows past the
+  // end re-read the last row; their results are dropped).
+  // (the wave index goes through local_tid() so that row addresses are recomputed at
+  // each use instead of being kept alive across the layer loop)
+  auto row_of = [&](int r0, int r1, int i) {
+    return min(r0 + (local_tid() >> 6) + kWavesP * i, r1 - 1);
+  };
 
   int t = 0;
   int stopped = 0;
   unsigned tok = 0;
-  f4 WA[UA];  // c_attn band of the layer about to run
+  Tile<J> WA[TA];  // c_attn rows of the layer about to run
   for (; t < p.n_fwd; ++t) {
     const int pos = p.pos0 + t;
     PG_STAMP(p.L, 7);
-    band_load<UA>(WA, reinterpret_cast<const f4*>(p.layers[0].c_attn_w) + (size_t)a0 * K4, nA4);
+    {
+      const f4* W4 = reinterpret_cast<const f4*>(p.layers[0].c_attn_w);
+#pragma unroll
+      for (int i = 0; i < TA; ++i) load_tile<J>(WA[i], W4 + (size_t)row_of(a0, a1, i) * K4, K4, lane);
+    }
     // ---- token to embed: given, or the argmax of the previous step's logits ----
     if (p.force_ids) {
       tok = p.force_ids[t];
@@ -651,7 +667,10 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
       {
         LnParams<NEC> lp;
         ln_fetch<NEC>(lp, w.ln_1_g, w.ln_1_b, C);
-        const float bias = w.c_attn_b[a0 + min(tid >> 4, a1 - a0 - 1)];
+        float bias[TA];
+#pragma unroll
+        for (int i = 0; i < TA; ++i) bias[i] = w.c_attn_b[row_of(a0, a1, i)];
+        __syncthreads();  // every wave is done with xs / xraw of the previous phase
         if (l == 0) {
           // embedding (rust.rs:966-974)
           for (int i = tid; i < C; i += kThreads)
@@ -662,102 +681,129 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
           if (!all_ok(ok, sm)) return;
         }
         ln_lds<NEC, C>(xraw, xs, lp, p.eps);
-        band_mul<UA, K4>(WA, xs, prod);
-        __syncthreads();
-        {
-          const int row = tid >> 4;  // 16 lanes per row, 32 rows per pass (RA <= 32)
-          const float sum = band_row<K4, 16>(prod, row, a1 - a0);
-          if ((tid & 15) == 0 && row < a1 - a0)
-            PG_ST64(p.qkv_t + a0 + row, pack(epoch_of(p, t, l, 0), bias + sum));
+        f4 xr[J];
+        load_x<J>(xr, xs, K4, lane);
+        const unsigned ep = epoch_of(p, t, l, 0);
+#pragma unroll
+        for (int i = 0; i < TA; ++i) {
+          const int r = a0 + wave + kWavesP * i;
+          const float v = dot_tile<J>(WA[i], xr);
+          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, bias[i] + v));
         }
-        __syncthreads();
       }
       PG_STAMP(l, 0);
 
-      // ================= B: attention over keys [0, pos] =================
-      f4 WE[UE];  // c_fc band, requested as soon as D's input has arrived
+      // ================= B, B2: attention over keys [0, pos] =================
       if (!attention_phase(pc, sm, xs, t, l, pos, kc, vc)) return;
       PG_STAMP(l, 2);
 
       // ================= D: c_proj + residual =================
+      Tile<J> WE[TE];  // c_fc rows, requested as soon as D's input has arrived
       {
-        const float bias = w.c_proj_b[d0 + min(tid >> 4, d1 - d0 - 1)];
-        f4 WD[UD];  // c_proj band: small, requested right before D waits for its input
-        band_load<UD>(WD, reinterpret_cast<const f4*>(w.c_proj_w) + (size_t)d0 * K4, nD4);
+        float bias[TD];
+#pragma unroll
+        for (int i = 0; i < TD; ++i) bias[i] = w.c_proj_b[row_of(d0, d1, i)];
+        Tile<J> WD[TD];  // c_proj rows: few, requested right before D waits for its input
+        {
+          const f4* W4 = reinterpret_cast<const f4*>(w.c_proj_w);
+#pragma unroll
+          for (int i = 0; i < TD; ++i)
+            load_tile<J>(WD[i], W4 + (size_t)row_of(d0, d1, i) * K4, K4, lane);
+        }
         __syncthreads();  // every wave is done with xs of the previous phase
         bool ok = poll_vec<NEC>(p.attn_t, C, epoch_of(p, t, l, 2), xs, abort_word);
         if (!all_ok(ok, sm)) return;
-        band_load<UE>(WE, reinterpret_cast<const f4*>(w.c_fc_w) + (size_t)e0 * K4, nE4);
-        band_mul<UD, K4>(WD, xs, prod);
-        __syncthreads();
         {
-          const int row = tid >> 4;
-          const float sum = band_row<K4, 16>(prod, row, d1 - d0);
-          if ((tid & 15) == 0 && row < d1 - d0)
-            PG_ST64(p.xa_t + d0 + row,
-                    pack(epoch_of(p, t, l, 3), xraw[d0 + row] + (bias + sum)));
+          const f4* W4 = reinterpret_cast<const f4*>(w.c_fc_w);
+#pragma unroll
+          for (int i = 0; i < TE; ++i)
+            load_tile<J>(WE[i], W4 + (size_t)row_of(e0, e1, i) * K4, K4, lane);
         }
-        __syncthreads();
+        f4 xr[J];
+        load_x<J>(xr, xs, K4, lane);
+        const unsigned ep = epoch_of(p, t, l, 3);
+#pragma unroll
+        for (int i = 0; i < TD; ++i) {
+          const int r = d0 + wave + kWavesP * i;
+          const float v = dot_tile<J>(WD[i], xr);
+          if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(ep, xraw[r] + (bias[i] + v)));
+        }
       }
       PG_STAMP(l, 3);
 
       // ================= E: LN2 + c_fc + GELU =================
-      // mlp c_proj band (rows of K = 4C): the first half is requested before E waits,
-      // the second half once E's own band has been consumed and its registers are free
-      f4 WF[UF];
-      const f4* Wf4 = reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)d0 * C;
+      // mlp c_proj quarter rows: a quarter of them is requested once E's input has
+      // arrived, the rest once E's own rows are consumed and their registers are free
+      Tile<J> WF[TF];
+      const f4* Wf4 = reinterpret_cast<const f4*>(w.c_proj_mlp_w);
+      auto f_tile = [&](int i) {  // quarter row (row d0 + id/4, quarter id%4), clamped
+        const int id = min((local_tid() >> 6) + kWavesP * i, nF - 1);
+        return Wf4 + (size_t)(d0 + (id >> 2)) * C + (size_t)(id & 3) * K4;
+      };
       {
         LnParams<NEC> lp;
         ln_fetch<NEC>(lp, w.ln_2_g, w.ln_2_b, C);
-        const float bias = w.c_fc_b[e0 + min(tid >> 4, e1 - e0 - 1)];
+        float bias[TE];
+#pragma unroll
+        for (int i = 0; i < TE; ++i) bias[i] = w.c_fc_b[row_of(e0, e1, i)];
+        __syncthreads();  // every wave is done with xraw (residual of phase D)
         bool ok = poll_vec<NEC>(p.xa_t, C, epoch_of(p, t, l, 3), xraw, abort_word);
         if (!all_ok(ok, sm)) return;
         PG_STAMP(l, 6);
-        band_load<UF, 0, UF / 2>(WF, Wf4, nF4);
+#pragma unroll
+        for (int i = 0; i < TF / 4; ++i) load_tile<J>(WF[i], f_tile(i), K4, lane);
         ln_lds<NEC, C>(xraw, xs, lp, p.eps);
-        band_mul<UE, K4>(WE, xs, prod);
-        PG_STAMP(l, 7);
-        band_load<UF, UF / 2, UF>(WF, Wf4, nF4);
-        __syncthreads();
-        {
-          const int row = tid >> 4;
-          const float sum = band_row<K4, 16>(prod, row, e1 - e0);
-          if ((tid & 15) == 0 && row < e1 - e0)
-            PG_ST64(p.h_t + e0 + row, pack(epoch_of(p, t, l, 4), gelu_tanh(bias + sum)));
+        f4 xr[J];
+        load_x<J>(xr, xs, K4, lane);
+        const unsigned ep = epoch_of(p, t, l, 4);
+#pragma unroll
+        for (int i = 0; i < TE; ++i) {
+          const int r = e0 + wave + kWavesP * i;
+          const float v = dot_tile<J>(WE[i], xr);
+          if (lane == 0 && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(bias[i] + v)));
         }
-        __syncthreads();
+        PG_STAMP(l, 7);
+#pragma unroll
+        for (int i = TF / 4; i < TF; ++i) load_tile<J>(WF[i], f_tile(i), K4, lane);
       }
       PG_STAMP(l, 4);
 
       // ================= F: mlp c_proj + residual =================
-      // The next layer's c_attn band is requested once F's input has arrived.
       {
-        const float bias = w.c_proj_mlp_b[d0 + min(tid >> 6, d1 - d0 - 1)];
+        const float bias = w.c_proj_mlp_b[d0 + min(tid, d1 - d0 - 1)];
+        __syncthreads();  // every wave is done with xs (input of phase E)
         bool ok = poll_vec<NEI>(p.h_t, I, epoch_of(p, t, l, 4), xs, abort_word);
         if (!all_ok(ok, sm)) return;
-        // The next layer's c_attn band: half now, half once F's own band is consumed
-        // (after the last layer this re-reads its own band: an unconditional request
-        // keeps the load count exact; the data is never used).
-        const f4* Wn4 = reinterpret_cast<const f4*>(p.layers[min(l + 1, p.L - 1)].c_attn_w) +
-                        (size_t)a0 * K4;
-        band_load<UA, 0, UA / 2>(WA, Wn4, nA4);
-        band_mul<UF, C>(WF, xs, prod);
-        band_load<UA, UA / 2, UA>(WA, Wn4, nA4);
-        __syncthreads();
-        {
-          const int row = tid >> 6;  // rows of K = 4C: one wavefront per row (RD <= 8)
-          const float sum = band_row<C, 64>(prod, row, d1 - d0);
-          if ((tid & 63) == 0 && row < d1 - d0)
-            PG_ST64(p.xm_t + d0 + row,
-                    pack(epoch_of(p, t, l, 5), xraw[d0 + row] + (bias + sum)));
+        // The next layer's c_attn rows (after the last layer this re-reads its own
+        // rows: an unconditional request keeps the load count exact; unused).  One row
+        // per wavefront now, the rest once F's own tiles are consumed.
+        const f4* Wn4 = reinterpret_cast<const f4*>(p.layers[min(l + 1, p.L - 1)].c_attn_w);
+        load_tile<J>(WA[0], Wn4 + (size_t)row_of(a0, a1, 0) * K4, K4, lane);
+#pragma unroll
+        for (int i = 0; i < TF; ++i) {
+          const int id = wave + kWavesP * i;
+          f4 xr[J];
+          load_x<J>(xr, xs + (size_t)(min(id, nF - 1) & 3) * C, K4, lane);
+          const float v = dot_tile<J>(WF[i], xr);
+          if (lane == 0 && id < nF) sm.psum[id] = v;
         }
+#pragma unroll
+        for (int i = 1; i < TA; ++i)
+          load_tile<J>(WA[i], Wn4 + (size_t)row_of(a0, a1, i) * K4, K4, lane);
         __syncthreads();
+        if (tid < d1 - d0) {
+          const int r = d0 + tid;
+          const float s4 = (sm.psum[4 * tid] + sm.psum[4 * tid + 1]) +
+                           (sm.psum[4 * tid + 2] + sm.psum[4 * tid + 3]);
+          PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), xraw[r] + (bias + s4)));
+        }
       }
       PG_STAMP(l, 5);
     }  // layers
 
     // ================= LN_f + lm_head (rust.rs:982-1002) =================
     if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      __syncthreads();
       if (!lm_head_phase<C_>(pc, sm, xs, xraw, t, v0, v1)) return;
       PG_STAMP(p.L, 6);
     }
@@ -765,6 +811,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 
   if (!stopped && p.select_last && p.n_fwd > 0) {
     float* bv = xs;
+    __syncthreads();
     bool ok = poll_vec<1>(p.best_t, 2 * G, epoch_of(p, p.n_fwd - 1, p.L, 6), bv, abort_word);
     if (!all_ok(ok, sm)) return;
     if (wg == 0 && tid == 0) {
@@ -787,16 +834,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }
 int persistent_grid() { return kGrid; }
 
-size_t persistent_lds_bytes(int C) {
-  // xs [4C] + xraw [C] + prod [512 * max float4 per thread over the four bands]
-  const int K4 = C / 4, G = kGrid;
-  const int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(4 * C, G);
-  int U = cdiv(RA * K4, kThreads);
-  U = U > cdiv(RD * K4, kThreads) ? U : cdiv(RD * K4, kThreads);
-  U = U > cdiv(RE * K4, kThreads) ? U : cdiv(RE * K4, kThreads);
-  U = U > cdiv(RD * C, kThreads) ? U : cdiv(RD * C, kThreads);
-  return (size_t)(5 * C + kThreads * U) * sizeof(float);
-}
+size_t persistent_lds_bytes(int C) { return (size_t)(5 * C) * sizeof(float); }  // xs [4C] + xraw [C]
 
 namespace {
 template <int C_>
