@@ -85,7 +85,7 @@ typedef struct pg_hip_options {
   int32_t device;          /* HIP device ordinal */
   uint32_t weight_storage; /* pg_weight_storage: how the dense matrices and wte are kept in HBM */
   uint32_t decode_path;    /* pg_decode_path */
-  uint32_t reserved;
+  uint32_t prefill_path;   /* 0: GEMM prefill for prompts of 16+ tokens; 1: always token by token */
 } pg_hip_options;
 
 typedef struct pg_gpt2_model pg_gpt2_model;

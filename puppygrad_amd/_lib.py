@@ -42,7 +42,7 @@ class pg_gpt2_weights_view(C.Structure):
 
 class pg_hip_options(C.Structure):
     _fields_ = [("device", C.c_int32), ("weight_storage", C.c_uint32),
-                ("decode_path", C.c_uint32), ("reserved", C.c_uint32)]
+                ("decode_path", C.c_uint32), ("prefill_path", C.c_uint32)]
 
 
 class pg_sampling(C.Structure):

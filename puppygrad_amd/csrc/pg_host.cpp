@@ -374,6 +374,69 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   return PG_OK;
 }
 
+// Sequences at least this long take the GEMM path in prefill / forward.
+constexpr size_t kGemmMinRows = 16;
+
+bool gemm_path_ok(const pg_gpt2_model* m, size_t n) {
+  const Cfg& g = m->cfg;
+  return n >= kGemmMinRows && g.C % 16 == 0 && g.I % 16 == 0 &&
+         (g.hd() == 64 || n * g.H * n * sizeof(float) <= (256u << 20));
+}
+
+// Full-sequence forward of sequence b over ids[0..n) (Gpt2Model::forward,
+// src/models/gpt2/rust.rs:831-882, block_forward at 1053-1134) with MFMA GEMMs and
+// tiled causal attention; K and V of every position land in the cache.  The last
+// position's logits go to the cache's logits row b; with all_logits set, the logits
+// of every position are also copied to dst ([n][V], host).
+pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, const uint32_t* ids,
+                            size_t n, float* all_logits_dst) {
+  const Cfg& g = m->cfg;
+  const int T = (int)n, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
+  hipStream_t s = c->stream;
+  pg_status st;
+  DevBuf X, XN, QKV, ATT, HB, IDS, SCR, LOG;
+  if ((st = X.alloc(n * g.C)) || (st = XN.alloc(n * g.C)) || (st = QKV.alloc(n * 3 * g.C)) ||
+      (st = ATT.alloc(n * g.C)) || (st = HB.alloc(n * g.I)) || (st = IDS.alloc(n)))
+    return st;
+  if (hd != 64 && (st = SCR.alloc(n * g.H * n))) return st;
+  if (all_logits_dst && (st = LOG.alloc(n * g.V))) return st;
+  uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
+  PG_HIP(hipMemcpyAsync(d_ids, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
+  PG_HIP(hipStreamSynchronize(s));  // ids is the caller's pageable memory
+  PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s));
+  auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
+                  int ldc, int N, int K, int epi) -> hipError_t {
+    pgk::GemmArgs a{};
+    a.A = A; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
+    a.M = T; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    return pgk::launch_gemm(a, epi, m->num_cus, s);
+  };
+  for (size_t l = 0; l < g.L; ++l) {
+    const pgk::LayerW& w = m->layers[l];
+    PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, w.ln_1_g, w.ln_1_b, g.eps, s));
+    PG_HIP(gemm(XN.p, C, w.c_attn_w, w.c_attn_b, QKV.p, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
+    PG_HIP(pgk::launch_attn_prefill(QKV.p, T, C, H, hd, P, c->k_panel(l, b), c->v_panel(l, b),
+                                    ATT.p, SCR.p, s));
+    PG_HIP(gemm(ATT.p, C, w.c_proj_w, w.c_proj_b, X.p, C, C, C, pgk::GEMM_RESID));
+    PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, w.ln_2_g, w.ln_2_b, g.eps, s));
+    PG_HIP(gemm(XN.p, C, w.c_fc_w, w.c_fc_b, HB.p, I, I, C, pgk::GEMM_GELU));
+    PG_HIP(gemm(HB.p, I, w.c_proj_mlp_w, w.c_proj_mlp_b, X.p, C, C, I, pgk::GEMM_RESID));
+  }
+  if (all_logits_dst) {
+    PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->ln_f_g, m->ln_f_b, g.eps, s));
+    PG_HIP(gemm(XN.p, C, m->wte, nullptr, LOG.p, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
+    PG_HIP(hipMemcpyAsync(all_logits_dst, LOG.p, n * g.V * sizeof(float), hipMemcpyDeviceToHost,
+                          s));
+  }
+  // last position -> the cache's logits row (LN_f + lm_head, rust.rs:982-1002)
+  pgk::GemvArgs a{};
+  a.W = m->wte; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
+  a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
+  PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+  PG_HIP(hipStreamSynchronize(s));
+  return PG_OK;
+}
+
 pg_status check_step(const pg_gpt2_model* m, const pg_kv_cache* c) {
   // rust.rs:957-962
   if (c->seq_len >= c->cfg.P)
@@ -781,6 +844,12 @@ pg_status pg_gpt2_prefill_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   if ((s = select_device(m->device))) return s;
   c->seq_len = 0;  // cache.clear() (rust.rs:918)
   c->logits_valid = false;
+  if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) {
+    for (size_t b = 0; b < c->B; ++b)
+      if ((s = run_sequence_gemm(m, c, b, ids + b * n, n, nullptr))) return s;
+    c->seq_len = n;
+    return finish_logits(c, out);
+  }
   if (use_persistent(m, c)) {
     PG_HIP(hipMemcpyAsync(c->d_force, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice,
                           c->stream));
@@ -850,6 +919,7 @@ pg_status pg_gpt2_forward(const pg_gpt2_model* m, const uint32_t* ids, size_t n,
   pg_kv_cache* c = nullptr;
   if ((s = pg_kv_cache_create(m, 1, &c))) return s;
   std::unique_ptr<pg_kv_cache, void (*)(pg_kv_cache*)> holder(c, pg_kv_cache_destroy);
+  if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) return run_sequence_gemm(m, c, 0, ids, n, dst);
   for (size_t i = 0; i < n; ++i) {
     if (use_persistent(m, c)) {
       if ((s = run_persistent(m, c, nullptr, false, false, ids[i], i, 1, false, -1, nullptr,
@@ -1138,11 +1208,20 @@ pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in
   PG_HIP(hipMemcpy(dx.p, x, rows * in_f * 4, hipMemcpyHostToDevice));
   PG_HIP(hipMemcpy(dw.p, weight, in_f * out_f * 4, hipMemcpyHostToDevice));
   PG_HIP(hipMemcpy(db.p, bias, out_f * 4, hipMemcpyHostToDevice));
-  for (uint64_t r = 0; r < rows; ++r) {
-    pgk::GemvArgs a{};
-    a.W = dw.p; a.bias = db.p; a.x = dx.p + r * in_f; a.y = dy.p + r * out_f;
-    a.K = (int)in_f; a.nout = (int)out_f;
-    PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_BIAS, nullptr));
+  pgk::GemmArgs ga{};
+  ga.A = dx.p; ga.W = dw.p; ga.bias = db.p; ga.resid = nullptr; ga.C = dy.p;
+  ga.M = (int)rows; ga.N = (int)out_f; ga.K = (int)in_f; ga.lda = (int)in_f; ga.ldc = (int)out_f;
+  if (rows >= kGemmMinRows && rows <= (1u << 20) && pgk::gemm_supported(ga)) {
+    hipDeviceProp_t prop;
+    PG_HIP(hipGetDeviceProperties(&prop, device));
+    PG_HIP(pgk::launch_gemm(ga, pgk::GEMM_BIAS, prop.multiProcessorCount, nullptr));
+  } else {
+    for (uint64_t r = 0; r < rows; ++r) {
+      pgk::GemvArgs a{};
+      a.W = dw.p; a.bias = db.p; a.x = dx.p + r * in_f; a.y = dy.p + r * out_f;
+      a.K = (int)in_f; a.nout = (int)out_f;
+      PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_BIAS, nullptr));
+    }
   }
   PG_HIP(hipStreamSynchronize(nullptr));
   PG_HIP(hipMemcpy(out, dy.p, rows * out_f * 4, hipMemcpyDeviceToHost));

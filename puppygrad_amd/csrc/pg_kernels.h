@@ -78,6 +78,31 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
                               int H, int head_dim, int nsplit, float* out, hipStream_t s);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
 
+// ---- full-sequence kernels (pg_prefill.hip) ----------------------------------------
+enum GemmEpilogue : int { GEMM_BIAS = 0, GEMM_GELU = 1, GEMM_RESID = 2 };
+// C[M,N] = epilogue(A[M,K] . W[N,K]^T + bias): A rows lda floats apart, C (and resid)
+// rows ldc apart, W dense [N][K]; bias may be nullptr.
+struct GemmArgs {
+  const float* A;
+  const float* W;
+  const float* bias;
+  const float* resid;
+  float* C;
+  int M, N, K;
+  int lda, ldc;
+};
+bool gemm_supported(const GemmArgs& a);
+hipError_t launch_gemm(const GemmArgs& a, int epilogue, int num_cus, hipStream_t s);
+// Causal attention over qkv[T][3C] -> out[T][C]; also appends K, V to the cache panels.
+// scratch ([T*H][T] floats) is only used when head_dim != 64.
+hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
+                               float* kcache, float* vcache, float* out, float* scratch,
+                               hipStream_t s);
+hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                             int T, int C, hipStream_t s);
+hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
+                                  const float* b, float eps, hipStream_t s);
+
 // ---- persistent batch-1 decode (pg_decode.hip) --------------------------------
 struct DecodeParams {
   const LayerW* layers;

@@ -1,0 +1,398 @@
+// Full-sequence (prefill) kernels for gfx950: fp32 MFMA GEMM with LDS staging and
+// causal attention with LDS-staged K/V tiles.
+//
+// They cover Gpt2Model::forward / block_forward / causal_self_attention
+// (src/models/gpt2/rust.rs:831-882, 1053-1134, 1580-1659): the same arithmetic as
+// the reference's token-by-token prefill (rust.rs:910-927), which the reference
+// itself checks against forward() at 1e-5 (rust.rs:1900-1913).
+#include "pg_kernels.h"
+
+#include <math.h>
+
+namespace pgk {
+
+namespace {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  return 0.5f * x * (1.0f + tanhf(0.7978846f * (x + 0.044715f * x * x * x)));
+}
+
+// ---------------------------------------------------------------------------
+// C[M,N] = epilogue(A[M,K] . W[N,K]^T + bias)   (transposed_dense_projection_into,
+// src/models/cpu.rs:58-75, for many rows at once)
+//
+// 256 threads = 4 wavefronts in a 2x2 arrangement; the block owns a BM x BN tile
+// of C, each wavefront a (BM/2) x (BN/2) part made of 32x32 MFMA blocks
+// (v_mfma_f32_32x32x2_f32: A operand lane l -> A[l%32][l/32], B operand lane l ->
+// B[l/32][l%32], D lane l, register v -> D[8*(v/4) + 4*(l/32) + v%4][l%32]).
+// A and W tiles of BK = 16 columns are staged in LDS transposed ([k][row]) so that
+// the operand reads of a wavefront are 32 consecutive floats (no bank conflicts);
+// the next tile's global loads are in flight while the current one is multiplied.
+// Rows past M or N are clamped on load and masked on store; K must be a multiple
+// of 16.
+// ---------------------------------------------------------------------------
+constexpr int BK = 16;
+
+template <int BM, int BN, int EPI>
+__global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
+  constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
+  constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
+  constexpr int LDA = BM + 4, LDB = BN + 4;
+  constexpr int ALD = BM / 64, BLD = BN / 64;  // float4 global loads per thread per tile
+  __shared__ float As[2][BK][LDA];
+  __shared__ float Bs[2][BK][LDB];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // XCD-aware tile order: consecutive workgroup ids go round the 8 XCDs, so give
+  // each XCD a contiguous run of tiles (neighbouring tiles share A rows / W rows in
+  // that XCD's L2).
+  const int nblocks = gridDim.x;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int per_xcd = (nblocks + 7) >> 3;
+  const int tile = xcd * per_xcd + slot;
+  const int tiles_n = (a.N + BN - 1) / BN;
+  if (tile >= ((a.M + BM - 1) / BM) * tiles_n) return;
+  const int tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // global load mapping: 4 lanes cover 16 consecutive k of one row
+  const int lr = tid >> 2, lk = (tid & 3) * 4;
+  const float* Ag[ALD];
+  const float* Wg[BLD];
+#pragma unroll
+  for (int i = 0; i < ALD; ++i)
+    Ag[i] = a.A + (size_t)min(m0 + lr + 64 * i, a.M - 1) * a.lda + lk;
+#pragma unroll
+  for (int i = 0; i < BLD; ++i)
+    Wg[i] = a.W + (size_t)min(n0 + lr + 64 * i, a.N - 1) * a.K + lk;
+
+  f16v acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  f4 ra[ALD], rb[BLD];
+#pragma unroll
+  for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i]);
+#pragma unroll
+  for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const f4*>(Wg[i]);
+
+  const int ktiles = a.K / BK;
+  const int half = lane >> 5, l32 = lane & 31;
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int buf = kt & 1;
+    // registers -> LDS (transposed)
+#pragma unroll
+    for (int i = 0; i < ALD; ++i) {
+      As[buf][lk + 0][lr + 64 * i] = ra[i].x;
+      As[buf][lk + 1][lr + 64 * i] = ra[i].y;
+      As[buf][lk + 2][lr + 64 * i] = ra[i].z;
+      As[buf][lk + 3][lr + 64 * i] = ra[i].w;
+    }
+#pragma unroll
+    for (int i = 0; i < BLD; ++i) {
+      Bs[buf][lk + 0][lr + 64 * i] = rb[i].x;
+      Bs[buf][lk + 1][lr + 64 * i] = rb[i].y;
+      Bs[buf][lk + 2][lr + 64 * i] = rb[i].z;
+      Bs[buf][lk + 3][lr + 64 * i] = rb[i].w;
+    }
+    __syncthreads();
+    if (kt + 1 < ktiles) {
+#pragma unroll
+      for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + (size_t)(kt + 1) * BK);
+#pragma unroll
+      for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const f4*>(Wg[i] + (size_t)(kt + 1) * BK);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float av[MB], bv[NB];
+#pragma unroll
+      for (int i = 0; i < MB; ++i) av[i] = As[buf][kk + half][wm * WM + 32 * i + l32];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) bv[j] = Bs[buf][kk + half][wn * WN + 32 * j + l32];
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+    // the other buffer is free once every wavefront has left it: the barrier at the
+    // top of the next iteration's store is preceded by this iteration's compute
+  }
+
+  // epilogue
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int n = n0 + wn * WN + 32 * j + l32;
+      if (n >= a.N) continue;
+      const float bias = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (m >= a.M) continue;
+        float c = bias + acc[i][j][v];
+        if (EPI == GEMM_GELU) c = gelu_tanh(c);
+        if (EPI == GEMM_RESID) c = a.resid[(size_t)m * a.ldc + n] + c;
+        a.C[(size_t)m * a.ldc + n] = c;
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// causal_self_attention (src/models/gpt2/rust.rs:1580-1659) for head_dim 64 over an
+// interleaved qkv[T][3C] buffer.  One wavefront owns 32 queries of one head and
+// walks the key tiles 0..diagonal, 32 keys at a time, staged in LDS:
+//   S^T (keys x queries) = K . Q^T        32 MFMA steps over d
+//   online softmax per query (a lane holds 16 keys of one query; one xor-32 swap)
+//   O^T (d x queries)   += V^T . P^T      16 MFMA steps over the 32 keys, twice (d halves)
+// Scores are scaled by 1/8 after the dot product, as the reference does
+// (rust.rs:1590, 1634).  It also appends K and V to the cache panels
+// ([head][position][64], kv_index at rust.rs:1851-1855).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(128) void k_attn_prefill64(const float* __restrict__ qkv, int T,
+                                                        int C, int P, float* __restrict__ kcache,
+                                                        float* __restrict__ vcache,
+                                                        float* __restrict__ out) {
+  constexpr int KT = 32;  // keys per tile
+  __shared__ float Kt[2][64][KT + 1];   // per wavefront: [d][key]
+  __shared__ float Vs[2][KT][64 + 4];   // per wavefront: [key][d]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int h = blockIdx.y;
+  const int qb = blockIdx.x * 2 + wave;  // block of 32 queries
+  const int q0 = qb * 32;
+  if (q0 >= T) return;
+  const int C3 = 3 * C;
+  const float* qbase = qkv + h * 64;
+  const float* kbase = qkv + C + h * 64;
+  const float* vbase = qkv + 2 * C + h * 64;
+
+  // Q^T operand: lane (query l32, half) holds Q[query][2s + half] for s = 0..31
+  float qr[32];
+  {
+    const int q = min(q0 + l32, T - 1);
+#pragma unroll
+    for (int s = 0; s < 32; ++s) qr[s] = qbase[(size_t)q * C3 + 2 * s + half];
+  }
+  f16v o0, o1;  // O^T rows d 0..31 and 32..63, column = query l32
+#pragma unroll
+  for (int v = 0; v < 16; ++v) { o0[v] = 0.0f; o1[v] = 0.0f; }
+  float m_run = -INFINITY, l_run = 0.0f;  // per query (replicated in both halves)
+  const int qi = q0 + l32;                // this lane's query
+
+  float (*kt)[KT + 1] = Kt[wave];
+  float (*vs)[64 + 4] = Vs[wave];
+  const int last_tile = min(q0 + 31, T - 1) / KT;
+  for (int tile = 0; tile <= last_tile; ++tile) {
+    const int k0 = tile * KT;
+    // stage K (transposed) and V of 32 keys; also append them to the cache once
+    // (by the wavefront whose query block starts at this tile: q0 == k0)
+    for (int i = lane; i < KT * 16; i += 64) {
+      const int key = i >> 4, d4 = (i & 15) * 4;
+      const int kk = min(k0 + key, T - 1);
+      const f4 kv4 = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + d4);
+      const f4 vv4 = *reinterpret_cast<const f4*>(vbase + (size_t)kk * C3 + d4);
+      kt[d4 + 0][key] = kv4.x; kt[d4 + 1][key] = kv4.y; kt[d4 + 2][key] = kv4.z; kt[d4 + 3][key] = kv4.w;
+      *reinterpret_cast<f4*>(&vs[key][d4]) = vv4;
+      if (q0 == k0 && k0 + key < T) {
+        *reinterpret_cast<f4*>(kcache + ((size_t)h * P + k0 + key) * 64 + d4) = kv4;
+        *reinterpret_cast<f4*>(vcache + ((size_t)h * P + k0 + key) * 64 + d4) = vv4;
+      }
+    }
+    // each wavefront has its own LDS tiles and LDS executes a wavefront's accesses in
+    // order, so only the compiler has to be kept from reordering
+    __builtin_amdgcn_wave_barrier();
+
+    // S^T = K . Q^T : A operand lane -> K[key l32][d = 2s + half]
+    f16v sacc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sacc[v] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 32; ++s)
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kt[2 * s + half][l32], qr[s], sacc, 0, 0, 0);
+    // lane holds keys k0 + 8*(v/4) + 4*half + v%4 of query qi
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+      const float sv = (key <= qi && key < T) ? sacc[v] * 0.125f : -INFINITY;
+      sacc[v] = sv;
+      mx = fmaxf(mx, sv);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    // a fully masked tile cannot occur for a valid query (key 0 <= qi); for lanes
+    // past T (clamped duplicates) qi >= T is still >= key 0
+    const float corr = expf(m_run - m_new);
+    float psum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float pv = expf(sacc[v] - m_new);
+      sacc[v] = pv;
+      psum += pv;
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * corr + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { o0[v] *= corr; o1[v] *= corr; }
+    // O^T += V^T . P^T : step v pairs key (8*(v/4) + v%4) of half 0 with key
+    // (8*(v/4) + 4 + v%4) of half 1; the B operand is this lane's own P value.
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = 8 * (v >> 2) + 4 * half + (v & 3);
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key][l32], sacc[v], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key][32 + l32], sacc[v], o1, 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // normalise and write: lane holds d = 8*(v/4) + 4*half + v%4 (+32) of query qi
+  if (qi < T) {
+    const float inv = 1.0f / l_run;
+    float* dst = out + (size_t)qi * C + h * 64;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int d = 8 * (v >> 2) + 4 * half + (v & 3);
+      dst[d] = o0[v] * inv;
+      dst[32 + d] = o1[v] * inv;
+    }
+  }
+}
+
+// Any head_dim: one thread per (query, head), plain loops (test-sized models).
+__global__ void k_attn_prefill_any(const float* qkv, int T, int C, int H, int hd, int P,
+                                   float* kcache, float* vcache, float* out, float* scratch) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * H) return;
+  const int q = idx / H, h = idx - q * H;
+  const int C3 = 3 * C;
+  const float scale = 1.0f / sqrtf((float)hd);
+  const float* qv = qkv + (size_t)q * C3 + h * hd;
+  float* sc = scratch + (size_t)idx * T;
+  float mx = -INFINITY;
+  for (int k = 0; k <= q; ++k) {
+    const float* kv = qkv + (size_t)k * C3 + C + h * hd;
+    float s = 0.0f;
+    for (int d = 0; d < hd; ++d) s += qv[d] * kv[d];
+    s *= scale;
+    sc[k] = s;
+    mx = fmaxf(mx, s);
+  }
+  float sum = 0.0f;
+  for (int k = 0; k <= q; ++k) {
+    sc[k] = expf(sc[k] - mx);
+    sum += sc[k];
+  }
+  for (int d = 0; d < hd; ++d) {
+    float o = 0.0f;
+    for (int k = 0; k <= q; ++k) o += (sc[k] / sum) * qkv[(size_t)k * C3 + 2 * C + h * hd + d];
+    out[(size_t)q * C + h * hd + d] = o;
+    kcache[((size_t)h * P + q) * hd + d] = qkv[(size_t)q * C3 + C + h * hd + d];
+    vcache[((size_t)h * P + q) * hd + d] = qkv[(size_t)q * C3 + 2 * C + h * hd + d];
+  }
+}
+
+// x[t] = wte[ids[t]] + wpe[t]   (rust.rs:839-846)
+__global__ void k_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                             int T, int C) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < T && i < C) x[(size_t)t * C + i] = wte[(size_t)ids[t] * C + i] + wpe[(size_t)t * C + i];
+}
+
+// dst[r] = LayerNorm(src[r])  (layer_norm_in_place, cpu.rs:119-143), one block per row
+__global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float* dst, int cols,
+                                                         const float* g, const float* b,
+                                                         float eps) {
+  __shared__ float red[4];
+  const float* row = src + (size_t)blockIdx.x * cols;
+  float* orow = dst + (size_t)blockIdx.x * cols;
+  auto bsum = [&](float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+  };
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += 256) s += row[i];
+  const float mean = bsum(s) / (float)cols;
+  float v = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += 256) {
+    const float d = row[i] - mean;
+    v += d * d;
+  }
+  const float var = bsum(v) / (float)cols;
+  const float inv = 1.0f / sqrtf(var + eps);
+  for (int i = threadIdx.x; i < cols; i += 256) orow[i] = (row[i] - mean) * inv * g[i] + b[i];
+}
+
+template <int BM, int BN>
+hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  const int grid = (tiles + 7) / 8 * 8;  // whole rounds over the 8 XCDs
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID>), dim3(grid), dim3(256), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool gemm_supported(const GemmArgs& a) {
+  return a.K % BK == 0 && a.M >= 1 && a.N >= 1 && a.lda % 4 == 0 &&
+         (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.W) & 15) == 0;
+}
+
+hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
+  if (!gemm_supported(a)) return hipErrorInvalidValue;
+  // 128x128 tiles once they fill the chip about twice over, 64x64 tiles otherwise
+  const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
+  if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128>(a, epi, s);
+  return launch_gemm_tile<64, 64>(a, epi, s);
+}
+
+hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
+                               float* kcache, float* vcache, float* out, float* scratch,
+                               hipStream_t s) {
+  if (head_dim == 64) {
+    const int qblocks = (T + 31) / 32;
+    hipLaunchKernelGGL(k_attn_prefill64, dim3((qblocks + 1) / 2, H), dim3(128), 0, s, qkv, T, C, P,
+                       kcache, vcache, out);
+  } else {
+    const int n = T * H;
+    hipLaunchKernelGGL(k_attn_prefill_any, dim3((n + 127) / 128), dim3(128), 0, s, qkv, T, C, H,
+                       head_dim, P, kcache, vcache, out, scratch);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                             int T, int C, hipStream_t s) {
+  hipLaunchKernelGGL(k_embed_rows, dim3((C + 255) / 256, T), dim3(256), 0, s, x, wte, wpe, ids, T,
+                     C);
+  return hipGetLastError();
+}
+
+hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
+                                  const float* b, float eps, hipStream_t s) {
+  hipLaunchKernelGGL(k_layer_norm_rows, dim3(rows), dim3(256), 0, s, src, dst, cols, g, b, eps);
+  return hipGetLastError();
+}
+
+}  // namespace pgk

@@ -124,9 +124,11 @@ class Gpt2HipConfig:
     device: int = 0
     weight_storage: int = _lib.PG_STORE_F32
     decode_path: int = _lib.PG_DECODE_AUTO
+    prefill_path: int = 0  # 0: GEMM prefill for prompts of 16+ tokens, 1: token by token
 
     def to_c(self) -> _lib.pg_hip_options:
-        return _lib.pg_hip_options(self.device, self.weight_storage, self.decode_path, 0)
+        return _lib.pg_hip_options(self.device, self.weight_storage, self.decode_path,
+                                   self.prefill_path)
 
 
 @dataclass

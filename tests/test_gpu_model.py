@@ -146,6 +146,44 @@ def test_logits_match_hf_golden(name):
     assert_logits_close(got, z["logits"])
 
 
+def long_cases():
+    """Prompts long enough (>= 16 tokens) to take the GEMM prefill / forward path."""
+    out = []
+    cfg = synth.Gpt2Config(vocab_size=211, n_positions=96, n_embd=128, n_layer=2, n_head=2)
+    out.append(("c128_T67", cfg, synth.random_weights(cfg, 0x5EED0211, perturb=True),
+                list(synth.token_ids(67, 0x70C00211, 211))))
+    cfg = synth.Gpt2Config(vocab_size=300, n_positions=64, n_embd=48, n_layer=2, n_head=3, n_inner=112)
+    out.append(("hd16_T40", cfg, synth.random_weights(cfg, 0x5EED0212, std=0.08, perturb=True),
+                list(synth.token_ids(40, 0x70C00212, 300))))
+    cfg = synth.Gpt2Config(vocab_size=97, n_positions=160, n_embd=192, n_layer=1, n_head=3)
+    out.append(("c192_T160", cfg, synth.random_weights(cfg, 0x5EED0213, perturb=True),
+                list(synth.token_ids(160, 0x70C00213, 97))))
+    return out
+
+
+@pytest.mark.parametrize("case", long_cases(), ids=lambda c: c[0])
+def test_gemm_prefill_and_forward_match_oracle(case):
+    from puppygrad_amd import Gpt2HipConfig
+    _, cfg, w, ids = case
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
+    want_all = ref.forward(ids)
+    assert_logits_close(model.forward(ids).logits, want_all)
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    assert cache.seq_len == len(ids)
+    for layer in range(cfg.n_layer):  # the GEMM path fills the cache in the reference's layout
+        for which in (0, 1):
+            np.testing.assert_allclose(cache.read_layer(layer, which)[:, :len(ids)],
+                                       rcache.read_layer(layer, which)[:, :len(ids)],
+                                       atol=2e-5, rtol=1e-4)
+    if cache.seq_len < cfg.n_positions:  # decode continues from a GEMM-filled cache
+        assert_logits_close(model.forward_one(3, cache).to_host(), ref.forward_one(3, rcache))
+    # token-by-token prefill (the reference's own order) gives the same logits
+    tok_model = Gpt2Model.new(cfg, w, Gpt2HipConfig(prefill_path=1))
+    c2 = tok_model.new_kv_cache()
+    assert_logits_close(tok_model.prefill(ids, c2).to_host(), want_all[-1])
+
+
 def test_sampler_on_device_logits_matches_oracle():
     _, cfg, w, ids = small_cases()[1]
     model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)

@@ -38,6 +38,20 @@ def test_dense_matches_oracle(rows, k, n):
     np.testing.assert_allclose(got, want, atol=2e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("rows,k,n", [(16, 768, 2304), (1024, 768, 768), (100, 3072, 768), (128, 1600, 4800),
+                                      (37, 64, 50), (1000, 1024, 4096), (33, 16, 129), (64, 6400, 1600),
+                                      (20, 768, 50257)])
+def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
+    # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised
+    rng = np.random.default_rng(rows * 7 + n)
+    x = rng.standard_normal(rows * k).astype(np.float32)
+    w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    got = hip_dense(x, rows, k, n, w, b)
+    want = oracle.transposed_dense(x, rows, k, n, w, b)
+    np.testing.assert_allclose(got, want, atol=3e-5, rtol=1e-5)
+
+
 def test_dense_reference_unit_vector():
     # src/models/cpu.rs:312-327
     x, weight = patterned(6, 0.2), patterned(12, 0.1)
