@@ -83,6 +83,7 @@ struct pg_kv_cache {
   // per-sequence activation scratch, [B][...]
   float *x = nullptr, *q = nullptr, *hbuf = nullptr, *part_acc = nullptr, *part_m = nullptr,
         *part_l = nullptr, *logits_buf = nullptr;
+  float *qkv_b = nullptr, *xn_b = nullptr, *att_b = nullptr;  // batched step: [B][3C], [B][C], [B][C]
   uint32_t* d_tok = nullptr;      // [B] token the next step embeds
   uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
   uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
@@ -437,6 +438,56 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   return PG_OK;
 }
 
+// One cached decoder step for ALL sequences of the cache at their common position
+// (the per-sequence forward_one of src/models/gpt2/rust.rs:943-1006 run for B rows):
+// every weight matrix is read once for the whole batch by the MFMA GEMM (M = B),
+// attention runs per (sequence, head, key split).  Token ids come from d_ids[B]
+// (device).  Needs n_embd and n_inner to be multiples of 16.
+pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* d_ids,
+                                size_t pos) {
+  const Cfg& g = m->cfg;
+  const int B = (int)c->B, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(),
+            P = (int)g.P;
+  hipStream_t s = c->stream;
+  const int nsplit = hd == pgk::kHeadDim
+                         ? pgk::choose_nsplit((int)pos + 1, H * B, m->num_cus) : 1;
+  pgk::BatchStrides bs;
+  bs.q = 3 * g.C;
+  bs.kv = g.H * g.P * g.hd();
+  bs.part = (size_t)H * pgk::kMaxSplits;
+  bs.out = g.C;
+  auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
+                  int ldc, int N, int K, int epi) -> hipError_t {
+    pgk::GemmArgs a{};
+    a.A = A; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
+    a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    return pgk::launch_gemm(a, epi, m->num_cus, s);
+  };
+  PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s));
+  for (size_t l = 0; l < g.L; ++l) {
+    const pgk::LayerW& w = m->layers[l];
+    PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, w.ln_1_g, w.ln_1_b, g.eps, s));
+    PG_HIP(gemm(c->xn_b, C, w.c_attn_w, w.c_attn_b, c->qkv_b, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
+    PG_HIP(pgk::launch_kv_append(c->qkv_b, B, C, hd, P, (int)pos, c->k_panel(l, 0),
+                                 c->v_panel(l, 0), bs.kv, s));
+    PG_HIP(pgk::launch_attn_decode(c->qkv_b, c->k_panel(l, 0), c->v_panel(l, 0), (int)pos, P, H,
+                                   hd, nsplit, c->part_acc, c->part_m, c->part_l, s, B, bs));
+    PG_HIP(pgk::launch_attn_finish(c->part_acc, c->part_m, c->part_l, H, hd, nsplit, c->att_b, s,
+                                   B, bs));
+    PG_HIP(gemm(c->att_b, C, w.c_proj_w, w.c_proj_b, c->x, C, C, C, pgk::GEMM_RESID));
+    PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, w.ln_2_g, w.ln_2_b, g.eps, s));
+    PG_HIP(gemm(c->xn_b, C, w.c_fc_w, w.c_fc_b, c->hbuf, I, I, C, pgk::GEMM_GELU));
+    PG_HIP(gemm(c->hbuf, I, w.c_proj_mlp_w, w.c_proj_mlp_b, c->x, C, C, I, pgk::GEMM_RESID));
+  }
+  PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, m->ln_f_g, m->ln_f_b, g.eps, s));
+  PG_HIP(gemm(c->xn_b, C, m->wte, nullptr, c->logits_buf, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
+  return PG_OK;
+}
+
+bool use_batched_step(const pg_gpt2_model* m, const pg_kv_cache* c) {
+  return c->B > 1 && m->cfg.C % 16 == 0 && m->cfg.I % 16 == 0;
+}
+
 pg_status check_step(const pg_gpt2_model* m, const pg_kv_cache* c) {
   // rust.rs:957-962
   if (c->seq_len >= c->cfg.P)
@@ -748,6 +799,9 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->part_m, parts * sizeof(float)));
   PG_HIP(hipMalloc(&raw->part_l, parts * sizeof(float)));
   PG_HIP(hipMalloc(&raw->logits_buf, B * g.V * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->qkv_b, B * 3 * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->xn_b, B * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->att_b, B * g.C * sizeof(float)));
   PG_HIP(hipMalloc(&raw->d_tok, B * sizeof(uint32_t)));
   PG_HIP(hipMalloc(&raw->d_out_ids, g.P * B * sizeof(uint32_t)));
   PG_HIP(hipHostMalloc(&raw->h_ids, g.P * B * sizeof(uint32_t), hipHostMallocDefault));
@@ -787,6 +841,9 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->part_m);
     (void)hipFree(c->part_l);
     (void)hipFree(c->logits_buf);
+    (void)hipFree(c->qkv_b);
+    (void)hipFree(c->xn_b);
+    (void)hipFree(c->att_b);
     (void)hipFree(c->d_tok);
     (void)hipFree(c->d_out_ids);
     if (c->h_ids) (void)hipHostFree(c->h_ids);
@@ -893,8 +950,15 @@ pg_status pg_gpt2_forward_one_batch(const pg_gpt2_model* m, pg_kv_cache* c, cons
     c->seq_len += 1;
     return finish_logits(c, out);
   }
-  for (size_t b = 0; b < c->B; ++b)
-    if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b], c->seq_len, true))) return s;
+  if (use_batched_step(m, c)) {
+    PG_HIP(hipMemcpyAsync(c->d_tok, ids, c->B * sizeof(uint32_t), hipMemcpyHostToDevice,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));  // ids is the caller's pageable memory
+    if ((s = enqueue_forward_batch(m, c, c->d_tok, c->seq_len))) return s;
+  } else {
+    for (size_t b = 0; b < c->B; ++b)
+      if ((s = enqueue_forward_one(m, c, b, nullptr, ids[b], c->seq_len, true))) return s;
+  }
   PG_HIP(hipStreamSynchronize(c->stream));
   c->seq_len += 1;  // rust.rs:1004
   return finish_logits(c, out);
@@ -944,9 +1008,7 @@ pg_status pg_logits_argmax(pg_logits* l, uint32_t* out) {
   if (!c->logits_valid) return fail(PG_INVALID_INPUT, "logits handle is stale");
   pg_status s;
   if ((s = select_device(c->device))) return s;
-  for (uint32_t r = 0; r < l->rows; ++r)
-    PG_HIP(pgk::launch_argmax(l->data + (size_t)r * l->vocab, (int)l->vocab, c->d_tok + r,
-                              c->stream));
+  PG_HIP(pgk::launch_argmax(l->data, (int)l->vocab, c->d_tok, c->stream, (int)l->rows));
   PG_HIP(hipMemcpyAsync(c->h_ids, c->d_tok, l->rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
                         c->stream));
   PG_HIP(hipStreamSynchronize(c->stream));
@@ -1068,13 +1130,16 @@ static pg_status decode_core(const pg_gpt2_model* m, pg_kv_cache* c, size_t step
   } else {
     PG_HIP(hipEventRecord(c->ev0, c->stream));
     for (size_t i = 0; i < n_steps; ++i) {
-      for (size_t b = 0; b < B; ++b)
-        PG_HIP(pgk::launch_argmax(c->logits_buf + b * V, (int)V, c->d_tok + b, c->stream));
+      PG_HIP(pgk::launch_argmax(c->logits_buf, (int)V, c->d_tok, c->stream, (int)B));
       PG_HIP(hipMemcpyAsync(c->d_out_ids + i * B, c->d_tok, B * sizeof(uint32_t),
                             hipMemcpyDeviceToDevice, c->stream));
       if (i + 1 < n_steps) {
-        for (size_t b = 0; b < B; ++b)
-          if ((s = enqueue_forward_one(m, c, b, c->d_tok + b, 0, c->seq_len, true))) return s;
+        if (use_batched_step(m, c)) {
+          if ((s = enqueue_forward_batch(m, c, c->d_tok, c->seq_len))) return s;
+        } else {
+          for (size_t b = 0; b < B; ++b)
+            if ((s = enqueue_forward_one(m, c, b, c->d_tok + b, 0, c->seq_len, true))) return s;
+        }
         c->seq_len += 1;
       }
     }

@@ -56,14 +56,28 @@ hipError_t launch_gemv(const GemvArgs& a, int prologue, int epilogue, hipStream_
 hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
                         uint32_t tok, int pos, int C, hipStream_t s);
 
-// Split-key decode attention for one query over keys [0, pos].
+// Element strides from one sequence of a batch to the next.
+struct BatchStrides {
+  size_t q = 0;     // query vectors (floats)
+  size_t kv = 0;    // K (and V) panels (floats)
+  size_t part = 0;  // (head, split) partial slots
+  size_t out = 0;   // attention output vectors (floats)
+};
+// Split-key decode attention for one query per sequence over keys [0, pos].
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
-                              float* part_m, float* part_l, hipStream_t s);
+                              float* part_m, float* part_l, hipStream_t s, int batch = 1,
+                              BatchStrides bs = BatchStrides{});
 int choose_nsplit(int n_keys, int H, int num_cus);
 
-// out[0] = argmax with the reference's tie/NaN rules.
-hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s);
+// out[r] = argmax of row r of v[rows][n] with the reference's tie/NaN rules.
+hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, int rows = 1);
+// x[b] = wte[ids[b]] + wpe[pos]
+hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                              int batch, int pos, int C, hipStream_t s);
+// Appends row b of qkv[B][3C] to position pos of sequence b's K and V panels.
+hipError_t launch_kv_append(const float* qkv, int batch, int C, int head_dim, int P, int pos,
+                            float* kcache, float* vcache, size_t kv_stride, hipStream_t s);
 
 // Stand-alone forms of the cpu.rs ops (rows handled one block each).
 hipError_t launch_layer_norm(float* x, int rows, int cols, const float* g, const float* b,
@@ -75,7 +89,8 @@ hipError_t launch_add(float* dst, const float* src, size_t n, hipStream_t s);
 hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, hipStream_t s);
 // Attention output from a single split's (acc, m, l): out = acc / l per head.
 hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
-                              int H, int head_dim, int nsplit, float* out, hipStream_t s);
+                              int H, int head_dim, int nsplit, float* out, hipStream_t s,
+                              int batch = 1, BatchStrides bs = BatchStrides{});
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
 
 // ---- full-sequence kernels (pg_prefill.hip) ----------------------------------------

@@ -192,12 +192,21 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
                                                           const float* __restrict__ vcache,
                                                           int pos, int P, int nsplit,
                                                           float* part_acc, float* part_m,
-                                                          float* part_l) {
+                                                          float* part_l, BatchStrides bs) {
   extern __shared__ float sc[];  // scores of this split
   __shared__ float red[kWaves];
   __shared__ float accs[kWaves][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int split = blockIdx.x, h = blockIdx.y;
+  {  // sequence blockIdx.z of a batch
+    const size_t b = blockIdx.z;
+    q += b * bs.q;
+    kcache += b * bs.kv;
+    vcache += b * bs.kv;
+    part_acc += b * bs.part * 64;
+    part_m += b * bs.part;
+    part_l += b * bs.part;
+  }
   const int n = pos + 1;
   const int per = (n + nsplit - 1) / nsplit;
   const int k0 = split * per;
@@ -273,10 +282,19 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
 __global__ __launch_bounds__(kBlock) void k_attn_decode_any(const float* q, const float* kcache,
                                                             const float* vcache, int pos, int P,
                                                             int hd, float* part_acc, float* part_m,
-                                                            float* part_l) {
+                                                            float* part_l, BatchStrides bs) {
   extern __shared__ float sc[];
   __shared__ float red[kWaves];
   const int tid = threadIdx.x, h = blockIdx.y;
+  {
+    const size_t b = blockIdx.z;
+    q += b * bs.q;
+    kcache += b * bs.kv;
+    vcache += b * bs.kv;
+    part_acc += b * bs.part * hd;
+    part_m += b * bs.part;
+    part_l += b * bs.part;
+  }
   const int n = pos + 1;
   const float scale = 1.0f / sqrtf((float)hd);
   const float* Kh = kcache + (size_t)h * P * hd;
@@ -309,7 +327,14 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode_any(const float* q, cons
 }
 
 __global__ void k_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
-                              int C, int hd, int nsplit, float* out) {
+                              int C, int hd, int nsplit, float* out, BatchStrides bs) {
+  {
+    const size_t b = blockIdx.y;
+    part_acc += b * bs.part * hd;
+    part_m += b * bs.part;
+    part_l += b * bs.part;
+    out += b * bs.out;
+  }
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < C) out[i] = attn_combine_elem(part_acc, part_m, part_l, nsplit, hd, i);
 }
@@ -325,6 +350,8 @@ __device__ __forceinline__ Best better(Best a, Best b) {
   return a;
 }
 __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t* out) {
+  v += (size_t)blockIdx.x * n;  // one block per row
+  out += blockIdx.x;
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   Best b{-INFINITY, 0xffffffffu};
@@ -351,6 +378,27 @@ __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t
     for (int w = 1; w < 16; ++w) r = better(r, Best{sv[w], si[w]});
     out[0] = (r.i == 0xffffffffu) ? 0u : r.i;
   }
+}
+
+// Embedding of one token per sequence at a common position (rust.rs:966-974).
+__global__ void k_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                              int pos, int C) {
+  const int b = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < C) x[(size_t)b * C + i] = wte[(size_t)ids[b] * C + i] + wpe[(size_t)pos * C + i];
+}
+
+// K/V append of cached_self_attention_into (rust.rs:1677-1683) for a batch: row b of
+// qkv[B][3C] goes to position pos of sequence b's panels ([head][P][hd]).
+__global__ void k_kv_append(const float* qkv, int C, int hd, int P, int pos, float* kcache,
+                            float* vcache, size_t kv_stride) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int h = c / hd, d = c - h * hd;
+  const size_t dst = (size_t)b * kv_stride + ((size_t)h * P + pos) * hd + d;
+  kcache[dst] = qkv[(size_t)b * 3 * C + C + c];
+  vcache[dst] = qkv[(size_t)b * 3 * C + 2 * C + c];
 }
 
 // ---- stand-alone cpu.rs ops -------------------------------------------------
@@ -470,28 +518,45 @@ int choose_nsplit(int n_keys, int H, int num_cus) {
 
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
-                              float* part_m, float* part_l, hipStream_t s) {
+                              float* part_m, float* part_l, hipStream_t s, int batch,
+                              BatchStrides bs) {
   if (head_dim == kHeadDim) {
     int per = (pos + 1 + nsplit - 1) / nsplit;
-    hipLaunchKernelGGL(k_attn_decode64, dim3(nsplit, H), dim3(kBlock), per * sizeof(float), s, q,
-                       kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l);
+    hipLaunchKernelGGL(k_attn_decode64, dim3(nsplit, H, batch), dim3(kBlock), per * sizeof(float),
+                       s, q, kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l, bs);
   } else {
-    hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H), dim3(kBlock), (pos + 1) * sizeof(float), s,
-                       q, kcache, vcache, pos, P, head_dim, part_acc, part_m, part_l);
+    hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H, batch), dim3(kBlock),
+                       (pos + 1) * sizeof(float), s, q, kcache, vcache, pos, P, head_dim, part_acc,
+                       part_m, part_l, bs);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
-                              int H, int head_dim, int nsplit, float* out, hipStream_t s) {
+                              int H, int head_dim, int nsplit, float* out, hipStream_t s,
+                              int batch, BatchStrides bs) {
   int C = H * head_dim;
-  hipLaunchKernelGGL(k_attn_finish, dim3((C + 255) / 256), dim3(256), 0, s, part_acc, part_m,
-                     part_l, C, head_dim, nsplit, out);
+  hipLaunchKernelGGL(k_attn_finish, dim3((C + 255) / 256, batch), dim3(256), 0, s, part_acc,
+                     part_m, part_l, C, head_dim, nsplit, out, bs);
   return hipGetLastError();
 }
 
-hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s) {
-  hipLaunchKernelGGL(k_argmax, dim3(1), dim3(1024), 0, s, v, n, out);
+hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
+                              int batch, int pos, int C, hipStream_t s) {
+  hipLaunchKernelGGL(k_embed_batch, dim3((C + 255) / 256, batch), dim3(256), 0, s, x, wte, wpe,
+                     ids, pos, C);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_append(const float* qkv, int batch, int C, int head_dim, int P, int pos,
+                            float* kcache, float* vcache, size_t kv_stride, hipStream_t s) {
+  hipLaunchKernelGGL(k_kv_append, dim3((C + 255) / 256, batch), dim3(256), 0, s, qkv, C, head_dim,
+                     P, pos, kcache, vcache, kv_stride);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, int rows) {
+  hipLaunchKernelGGL(k_argmax, dim3(rows), dim3(1024), 0, s, v, n, out);
   return hipGetLastError();
 }
 
