@@ -64,6 +64,7 @@ struct pg_gpt2_model {
   bool persistent = false;          // batch-1 decode runs as one persistent launch
   int persistent_grid = 0;          // workgroups of that launch (one per CU)
   int attn_splits = 1;              // key splits per head in the persistent kernel
+  int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
 };
 
 struct pg_logits {
@@ -252,12 +253,12 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
   float* pl = c->part_l + b * part_stride;
   const int nsplit = hd == pgk::kHeadDim ? pgk::choose_nsplit((int)pos + 1, H, m->num_cus) : 1;
 
-  PG_HIP(pgk::launch_embed(x, m->wte, m->wpe, tok_ptr, tok, (int)pos, C, s));
+  PG_HIP(pgk::launch_embed(x, m->wte, m->wpe, tok_ptr, tok, (int)pos, C, s, m->w_bf16));
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
     pgk::GemvArgs a{};
     // LN1 + c_attn + K/V append
-    a.W = w.c_attn_w; a.bias = w.c_attn_b; a.x = x; a.y = q; a.K = C; a.nout = 3 * C;
+    a.w_bf16 = m->w_bf16; a.W = w.c_attn_w; a.bias = w.c_attn_b; a.x = x; a.y = q; a.K = C; a.nout = 3 * C;
     a.ln_g = w.ln_1_g; a.ln_b = w.ln_1_b; a.eps = g.eps;
     a.kcache = c->k_panel(l, b); a.vcache = c->v_panel(l, b);
     a.pos = (int)pos; a.P = P; a.C = C; a.head_dim = hd;
@@ -267,23 +268,23 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
                                    nsplit, pa, pm, pl, s));
     // merge splits + c_proj + residual
     a = pgk::GemvArgs{};
-    a.W = w.c_proj_w; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
+    a.w_bf16 = m->w_bf16; a.W = w.c_proj_w; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
     a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
     // LN2 + c_fc + GELU
     a = pgk::GemvArgs{};
-    a.W = w.c_fc_w; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
+    a.w_bf16 = m->w_bf16; a.W = w.c_fc_w; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
     a.ln_g = w.ln_2_g; a.ln_b = w.ln_2_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_GELU, s));
     // mlp c_proj + residual
     a = pgk::GemvArgs{};
-    a.W = w.c_proj_mlp_w; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
+    a.w_bf16 = m->w_bf16; a.W = w.c_proj_mlp_w; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
     a.nout = C;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
   }
   if (want_logits) {
     pgk::GemvArgs a{};
-    a.W = m->wte; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
+    a.w_bf16 = m->w_bf16; a.W = m->wte; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
     a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   }
@@ -404,11 +405,11 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
   PG_HIP(hipMemcpyAsync(d_ids, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
   PG_HIP(hipStreamSynchronize(s));  // ids is the caller's pageable memory
-  PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s));
+  PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s, m->w_bf16));
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
                   int ldc, int N, int K, int epi) -> hipError_t {
     pgk::GemmArgs a{};
-    a.A = A; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
+    a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = T; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
@@ -431,7 +432,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   }
   // last position -> the cache's logits row (LN_f + lm_head, rust.rs:982-1002)
   pgk::GemvArgs a{};
-  a.W = m->wte; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
+  a.w_bf16 = m->w_bf16; a.W = m->wte; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
   a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
   PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   PG_HIP(hipStreamSynchronize(s));
@@ -459,11 +460,11 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
                   int ldc, int N, int K, int epi) -> hipError_t {
     pgk::GemmArgs a{};
-    a.A = A; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
+    a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
-  PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s));
+  PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
     PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, w.ln_1_g, w.ln_1_b, g.eps, s));
@@ -610,8 +611,12 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   if ((s = validate_weights(g, *weights))) return s;
   pg_hip_options opts{};
   if (options) opts = *options;
-  if (opts.weight_storage != PG_STORE_F32)
-    return fail(PG_INVALID_CONFIG, "hip backend weight_storage: only f32 is implemented");
+  if (opts.weight_storage != PG_STORE_F32 && opts.weight_storage != PG_STORE_BF16)
+    return fail(PG_INVALID_CONFIG, "hip backend weight_storage must be f32 or bf16");
+  const bool bf = opts.weight_storage == PG_STORE_BF16;
+  if (bf && opts.decode_path == PG_DECODE_PERSISTENT)
+    return fail(PG_INVALID_CONFIG,
+                "hip backend decode_path=persistent reads f32 weights; use weight_storage=f32");
   if (opts.decode_path > PG_DECODE_PERSISTENT)
     return fail(PG_INVALID_CONFIG, "hip backend decode_path out of range");
   if ((s = select_device(opts.device))) return s;
@@ -620,16 +625,21 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   m->cfg = g;
   m->device = opts.device;
   m->opts = opts;
+  m->w_bf16 = bf ? 1 : 0;
   hipDeviceProp_t prop;
   PG_HIP(hipGetDeviceProperties(&prop, opts.device));
   m->num_cus = prop.multiProcessorCount;
 
   // One arena; every tensor starts on a 256-byte boundary.
+  // With bf16 storage the token embedding and the four matrices of every block hold
+  // 2-byte values (wel() floats of arena for n elements); LayerNorm parameters,
+  // biases and the position embedding stay f32.
   const size_t A = 64;
-  size_t total = round_up(g.V * g.C, A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A);
-  const size_t per_layer = 6 * round_up(g.C, A) + round_up(3 * g.C * g.C, A) +
-                           round_up(3 * g.C, A) + round_up(g.C * g.C, A) +
-                           2 * round_up(g.C * g.I, A) + round_up(g.I, A);
+  auto wel = [&](size_t n) { return bf ? (n + 1) / 2 : n; };
+  size_t total = round_up(wel(g.V * g.C), A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A);
+  const size_t per_layer = 6 * round_up(g.C, A) + round_up(wel(3 * g.C * g.C), A) +
+                           round_up(3 * g.C, A) + round_up(wel(g.C * g.C), A) +
+                           2 * round_up(wel(g.C * g.I), A) + round_up(g.I, A);
   total += g.L * per_layer;
   PG_HIP(hipMalloc(&m->arena, total * sizeof(float)));
   m->arena_floats = total;
@@ -651,21 +661,33 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     PG_HIP(hipMemcpy(dst, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
     return PG_OK;
   };
-  DevBuf staging;
-  if ((s = staging.alloc(std::max(3 * g.C * g.C, g.C * g.I)))) return s;
-  // transpose_dense_weights (src/models/gpt2/rust.rs:1345-1352): [in,out] -> [out,in].
+  DevBuf staging, staging_t;
+  const size_t mat_max = std::max(3 * g.C * g.C, g.C * g.I);
+  if ((s = staging.alloc(bf ? std::max(mat_max, g.V * g.C) : mat_max))) return s;
+  if (bf && (s = staging_t.alloc(mat_max))) return s;
+  // transpose_dense_weights (src/models/gpt2/rust.rs:1345-1352): [in,out] -> [out,in],
+  // then rounded to bf16 (nearest even) when that is the storage type.
   auto upload_t = [&](float* dst, const pg_tensor& t, size_t in_f, size_t out_f) -> pg_status {
     PG_HIP(hipMemcpy(staging.p, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
-    PG_HIP(pgk::launch_transpose(staging.p, dst, (int)in_f, (int)out_f, nullptr));
+    PG_HIP(pgk::launch_transpose(staging.p, bf ? staging_t.p : dst, (int)in_f, (int)out_f,
+                                 nullptr));
+    if (bf) PG_HIP(pgk::launch_f32_to_bf16(staging_t.p, dst, t.len, nullptr));
+    PG_HIP(hipStreamSynchronize(nullptr));
+    return PG_OK;
+  };
+  auto upload_w = [&](float* dst, const pg_tensor& t) -> pg_status {
+    if (!bf) return upload(dst, t);
+    PG_HIP(hipMemcpy(staging.p, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
+    PG_HIP(pgk::launch_f32_to_bf16(staging.p, dst, t.len, nullptr));
     PG_HIP(hipStreamSynchronize(nullptr));
     return PG_OK;
   };
 
-  m->wte = place(g.V * g.C);
+  m->wte = place(wel(g.V * g.C));
   m->wpe = place(g.P * g.C);
   m->ln_f_g = place(g.C);
   m->ln_f_b = place(g.C);
-  if ((s = upload(m->wte, weights->wte))) return s;
+  if ((s = upload_w(m->wte, weights->wte))) return s;
   if ((s = upload(m->wpe, weights->wpe))) return s;
   if ((s = upload(m->ln_f_g, weights->ln_f_g))) return s;
   if ((s = upload(m->ln_f_b, weights->ln_f_b))) return s;
@@ -674,15 +696,15 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     const pg_gpt2_block_view& b = weights->blocks[l];
     float* ln_1_g = place(g.C);
     float* ln_1_b = place(g.C);
-    float* c_attn_w = place(3 * g.C * g.C);
+    float* c_attn_w = place(wel(3 * g.C * g.C));
     float* c_attn_b = place(3 * g.C);
-    float* c_proj_w = place(g.C * g.C);
+    float* c_proj_w = place(wel(g.C * g.C));
     float* c_proj_b = place(g.C);
     float* ln_2_g = place(g.C);
     float* ln_2_b = place(g.C);
-    float* c_fc_w = place(g.C * g.I);
+    float* c_fc_w = place(wel(g.C * g.I));
     float* c_fc_b = place(g.I);
-    float* c_proj_mlp_w = place(g.I * g.C);
+    float* c_proj_mlp_w = place(wel(g.I * g.C));
     float* c_proj_mlp_b = place(g.C);
     if ((s = upload(ln_1_g, b.ln_1_g))) return s;
     if ((s = upload(ln_1_b, b.ln_1_b))) return s;
@@ -716,7 +738,7 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   {
     const int grid = pgk::persistent_grid();
     int blocks_per_cu = 0;
-    bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
+    bool shape_ok = !bf && g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
                     g.P <= 4096 && g.V >= (size_t)grid;
     if (shape_ok) {
       PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu));
@@ -759,8 +781,8 @@ pg_status pg_gpt2_get_config(const pg_gpt2_model* m, pg_gpt2_config* out) {
 
 pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
   if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
-  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=f32, decode=%s)", m->device,
-                m->num_cus, m->persistent ? "persistent" : "kernels");
+  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=%s, decode=%s)", m->device,
+                m->num_cus, m->w_bf16 ? "bf16" : "f32", m->persistent ? "persistent" : "kernels");
   return PG_OK;
 }
 

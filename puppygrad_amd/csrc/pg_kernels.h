@@ -24,6 +24,7 @@ enum Epilogue : int { EPI_BIAS = 0, EPI_GELU = 1, EPI_RESID = 2, EPI_QKV = 3 };
 
 // y = epilogue(bias + W . prologue(x)) for one input vector.
 struct GemvArgs {
+  int w_bf16 = 0;      // W holds bf16 values (2 bytes each) instead of f32
   const float* W;      // [nout][K]
   const float* bias;   // [nout] or nullptr (treated as 0)
   const float* x;      // [K] input (PRO_NONE / PRO_LN)
@@ -54,7 +55,7 @@ hipError_t launch_gemv(const GemvArgs& a, int prologue, int epilogue, hipStream_
 
 // x = wte[tok] + wpe[pos]; tok comes from tok_ptr[0] when tok_ptr != nullptr.
 hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
-                        uint32_t tok, int pos, int C, hipStream_t s);
+                        uint32_t tok, int pos, int C, hipStream_t s, int w_bf16 = 0);
 
 // Element strides from one sequence of a batch to the next.
 struct BatchStrides {
@@ -74,7 +75,7 @@ int choose_nsplit(int n_keys, int H, int num_cus);
 hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, int rows = 1);
 // x[b] = wte[ids[b]] + wpe[pos]
 hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                              int batch, int pos, int C, hipStream_t s);
+                              int batch, int pos, int C, hipStream_t s, int w_bf16 = 0);
 // Appends row b of qkv[B][3C] to position pos of sequence b's K and V panels.
 hipError_t launch_kv_append(const float* qkv, int batch, int C, int head_dim, int P, int pos,
                             float* kcache, float* vcache, size_t kv_stride, hipStream_t s);
@@ -92,12 +93,15 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
                               int H, int head_dim, int nsplit, float* out, hipStream_t s,
                               int batch = 1, BatchStrides bs = BatchStrides{});
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
+// dst[i] = bf16(src[i]), round to nearest even
+hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s);
 
 // ---- full-sequence kernels (pg_prefill.hip) ----------------------------------------
 enum GemmEpilogue : int { GEMM_BIAS = 0, GEMM_GELU = 1, GEMM_RESID = 2 };
 // C[M,N] = epilogue(A[M,K] . W[N,K]^T + bias): A rows lda floats apart, C (and resid)
 // rows ldc apart, W dense [N][K]; bias may be nullptr.
 struct GemmArgs {
+  int w_bf16 = 0;  // W holds bf16 values
   const float* A;
   const float* W;
   const float* bias;
@@ -114,7 +118,7 @@ hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_d
                                float* kcache, float* vcache, float* out, float* scratch,
                                hipStream_t s);
 hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C, hipStream_t s);
+                             int T, int C, hipStream_t s, int w_bf16 = 0);
 hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
                                   const float* b, float eps, hipStream_t s);
 

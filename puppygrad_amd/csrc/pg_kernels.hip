@@ -97,7 +97,13 @@ __device__ __forceinline__ float attn_combine_elem(const float* part_acc, const 
 // producer of x (LayerNorm or the attention merge) and the consumer of y
 // (GELU, residual add, K/V cache append) folded in.  One wavefront owns RPW
 // weight rows; lanes stride over the row in float4 and reduce at the end.
-template <int PRO, int EPI, int RPW, bool VEC4>
+// Weight access modes of k_gemv: f32 scalar / f32 float4 / bf16 x8 / bf16 scalar.
+enum : int { WM_F32 = 0, WM_F32X4 = 1, WM_BF16X8 = 2, WM_BF16 = 3 };
+
+__device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned u) { return __uint_as_float(u & 0xffff0000u); }
+
+template <int PRO, int EPI, int RPW, int WM>
 __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
   extern __shared__ float sx[];  // K floats
   __shared__ float red[kWaves];
@@ -119,7 +125,37 @@ __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
 #pragma unroll
   for (int r = 0; r < RPW; ++r) acc[r] = 0.0f;
 
-  if (VEC4) {
+  if (WM == WM_BF16X8) {
+    // weights stored as bf16 (exactly representable in f32): 8 per 16-byte load
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const int K8 = K >> 3;
+    const float4* sx4 = reinterpret_cast<const float4*>(sx);
+    const u4* W8 = reinterpret_cast<const u4*>(a.W);
+#pragma unroll 2
+    for (int j = lane; j < K8; j += 64) {
+      float4 x0 = sx4[2 * j], x1 = sx4[2 * j + 1];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) {
+          u4 w = __builtin_nontemporal_load(&W8[(size_t)row * K8 + j]);
+          acc[r] += bf16_lo(w.x) * x0.x + bf16_hi(w.x) * x0.y + bf16_lo(w.y) * x0.z +
+                    bf16_hi(w.y) * x0.w + bf16_lo(w.z) * x1.x + bf16_hi(w.z) * x1.y +
+                    bf16_lo(w.w) * x1.z + bf16_hi(w.w) * x1.w;
+        }
+      }
+    }
+  } else if (WM == WM_BF16) {
+    const unsigned short* Wh = reinterpret_cast<const unsigned short*>(a.W);
+    for (int j = lane; j < K; j += 64) {
+      float xv = sx[j];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) acc[r] += bf16_lo(Wh[(size_t)row * K + j]) * xv;
+      }
+    }
+  } else if (WM == WM_F32X4) {
     const int K4 = K >> 2;
     const float4* sx4 = reinterpret_cast<const float4*>(sx);
     const f4* W4 = reinterpret_cast<const f4*>(a.W);
@@ -176,11 +212,15 @@ __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
 }
 
 // Embedding of one token (rust.rs:966-974).
+// wte may be stored as bf16 (w_bf16 != 0); wpe is always f32.
+__device__ __forceinline__ float wte_at(const float* wte, int w_bf16, size_t idx) {
+  return w_bf16 ? bf16_lo(reinterpret_cast<const unsigned short*>(wte)[idx]) : wte[idx];
+}
 __global__ void k_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
-                        uint32_t tok, int pos, int C) {
+                        uint32_t tok, int pos, int C, int w_bf16) {
   uint32_t t = tok_ptr ? tok_ptr[0] : tok;
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < C) x[i] = wte[(size_t)t * C + i] + wpe[(size_t)pos * C + i];
+  if (i < C) x[i] = wte_at(wte, w_bf16, (size_t)t * C + i) + wpe[(size_t)pos * C + i];
 }
 
 // cached_self_attention_into (rust.rs:1721-1740) for head_dim 64, keys split
@@ -382,10 +422,11 @@ __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t
 
 // Embedding of one token per sequence at a common position (rust.rs:966-974).
 __global__ void k_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                              int pos, int C) {
+                              int pos, int C, int w_bf16) {
   const int b = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < C) x[(size_t)b * C + i] = wte[(size_t)ids[b] * C + i] + wpe[(size_t)pos * C + i];
+  if (i < C)
+    x[(size_t)b * C + i] = wte_at(wte, w_bf16, (size_t)ids[b] * C + i) + wpe[(size_t)pos * C + i];
 }
 
 // K/V append of cached_self_attention_into (rust.rs:1677-1683) for a batch: row b of
@@ -440,6 +481,21 @@ __global__ void k_add(float* dst, const float* src, size_t n) {
   if (i < n) dst[i] += src[i];
 }
 
+// f32 -> bf16, round to nearest even (NaN keeps a quiet-NaN payload).
+__global__ void k_f32_to_bf16(const float* src, unsigned short* dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    unsigned u = __float_as_uint(src[i]);
+    unsigned r;
+    if ((u & 0x7fffffffu) > 0x7f800000u)
+      r = (u >> 16) | 0x40u;
+    else
+      r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    dst[i] = (unsigned short)r;
+  }
+}
+
 __global__ void k_fill_zero(float* p, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -464,21 +520,30 @@ __global__ void k_transpose(const float* src, float* dst, int in_f, int out_f) {
 
 template <int PRO, int EPI>
 hipError_t launch_gemv_pe(const GemvArgs& a, hipStream_t s) {
-  const bool vec4 = (a.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.W) & 15) == 0);
+  const bool aligned = (reinterpret_cast<uintptr_t>(a.W) & 15) == 0;
   const size_t lds = (size_t)a.K * sizeof(float);
   // Two rows per wavefront once there are enough rows to fill the chip with
   // 8-row blocks; otherwise one row per wavefront.
   const bool two = a.nout >= 4096;
   const int rpw = two ? 2 : 1;
   const int blocks = (a.nout + kWaves * rpw - 1) / (kWaves * rpw);
-  if (vec4) {
+  const int blocks1 = (a.nout + kWaves - 1) / kWaves;
+  if (a.w_bf16) {
+    if (aligned && a.K % 8 == 0) {
+      if (two)
+        hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, WM_BF16X8>), dim3(blocks), dim3(kBlock), lds, s, a);
+      else
+        hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_BF16X8>), dim3(blocks), dim3(kBlock), lds, s, a);
+    } else {
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_BF16>), dim3(blocks1), dim3(kBlock), lds, s, a);
+    }
+  } else if (aligned && a.K % 4 == 0) {
     if (two)
-      hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, true>), dim3(blocks), dim3(kBlock), lds, s, a);
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, WM_F32X4>), dim3(blocks), dim3(kBlock), lds, s, a);
     else
-      hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, true>), dim3(blocks), dim3(kBlock), lds, s, a);
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_F32X4>), dim3(blocks), dim3(kBlock), lds, s, a);
   } else {
-    hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, false>), dim3((a.nout + kWaves - 1) / kWaves),
-                       dim3(kBlock), lds, s, a);
+    hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_F32>), dim3(blocks1), dim3(kBlock), lds, s, a);
   }
   return hipGetLastError();
 }
@@ -500,9 +565,9 @@ hipError_t launch_gemv(const GemvArgs& a, int prologue, int epilogue, hipStream_
 }
 
 hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint32_t* tok_ptr,
-                        uint32_t tok, int pos, int C, hipStream_t s) {
+                        uint32_t tok, int pos, int C, hipStream_t s, int w_bf16) {
   hipLaunchKernelGGL(k_embed, dim3((C + 255) / 256), dim3(256), 0, s, x, wte, wpe, tok_ptr, tok,
-                     pos, C);
+                     pos, C, w_bf16);
   return hipGetLastError();
 }
 
@@ -542,9 +607,9 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
 }
 
 hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                              int batch, int pos, int C, hipStream_t s) {
+                              int batch, int pos, int C, hipStream_t s, int w_bf16) {
   hipLaunchKernelGGL(k_embed_batch, dim3((C + 255) / 256, batch), dim3(256), 0, s, x, wte, wpe,
-                     ids, pos, C);
+                     ids, pos, C, w_bf16);
   return hipGetLastError();
 }
 
@@ -583,6 +648,15 @@ hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, h
                      dst, in_f, out_f);
   return hipGetLastError();
 }
+hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s) {
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks == 0) blocks = 1;
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)blocks), dim3(256), 0, s, src,
+                     reinterpret_cast<unsigned short*>(dst), n);
+  return hipGetLastError();
+}
+
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s) {
   size_t blocks = (n + 255) / 256;
   if (blocks > 65536) blocks = 65536;

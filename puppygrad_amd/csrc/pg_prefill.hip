@@ -36,7 +36,24 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 // ---------------------------------------------------------------------------
 constexpr int BK = 16;
 
-template <int BM, int BN, int EPI>
+// W tile load: 4 consecutive k of one row as f32 (16 bytes) or bf16 (8 bytes, widened
+// to f32 exactly by a 16-bit shift).
+template <bool WBF>
+__device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
+  if (WBF) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 w = *reinterpret_cast<const u2*>(reinterpret_cast<const unsigned short*>(W) + idx);
+    f4 r;
+    r.x = __uint_as_float(w.x << 16);
+    r.y = __uint_as_float(w.x & 0xffff0000u);
+    r.z = __uint_as_float(w.y << 16);
+    r.w = __uint_as_float(w.y & 0xffff0000u);
+    return r;
+  }
+  return *reinterpret_cast<const f4*>(W + idx);
+}
+
+template <int BM, int BN, int EPI, bool WBF>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
@@ -62,13 +79,13 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   // global load mapping: 4 lanes cover 16 consecutive k of one row
   const int lr = tid >> 2, lk = (tid & 3) * 4;
   const float* Ag[ALD];
-  const float* Wg[BLD];
+  size_t Wg[BLD];  // element offsets into W
 #pragma unroll
   for (int i = 0; i < ALD; ++i)
     Ag[i] = a.A + (size_t)min(m0 + lr + 64 * i, a.M - 1) * a.lda + lk;
 #pragma unroll
   for (int i = 0; i < BLD; ++i)
-    Wg[i] = a.W + (size_t)min(n0 + lr + 64 * i, a.N - 1) * a.K + lk;
+    Wg[i] = (size_t)min(n0 + lr + 64 * i, a.N - 1) * a.K + lk;
 
   f16v acc[MB][NB];
 #pragma unroll
@@ -82,7 +99,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
   for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i]);
 #pragma unroll
-  for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const f4*>(Wg[i]);
+  for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i]);
 
   const int ktiles = a.K / BK;
   const int half = lane >> 5, l32 = lane & 31;
@@ -108,7 +125,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + (size_t)(kt + 1) * BK);
 #pragma unroll
-      for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const f4*>(Wg[i] + (size_t)(kt + 1) * BK);
+      for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i] + (size_t)(kt + 1) * BK);
     }
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
@@ -303,10 +320,16 @@ __global__ void k_attn_prefill_any(const float* qkv, int T, int C, int H, int hd
 
 // x[t] = wte[ids[t]] + wpe[t]   (rust.rs:839-846)
 __global__ void k_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C) {
+                             int T, int C, int w_bf16) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < T && i < C) x[(size_t)t * C + i] = wte[(size_t)ids[t] * C + i] + wpe[(size_t)t * C + i];
+  if (t < T && i < C) {
+    const size_t idx = (size_t)ids[t] * C + i;
+    const float e =
+        w_bf16 ? __uint_as_float((unsigned)reinterpret_cast<const unsigned short*>(wte)[idx] << 16)
+               : wte[idx];
+    x[(size_t)t * C + i] = e + wpe[(size_t)t * C + i];
+  }
 }
 
 // dst[r] = LayerNorm(src[r])  (layer_norm_in_place, cpu.rs:119-143), one block per row
@@ -337,16 +360,16 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
   for (int i = threadIdx.x; i < cols; i += 256) orow[i] = (row[i] - mean) * inv * g[i] + b[i];
 }
 
-template <int BM, int BN>
+template <int BM, int BN, bool WBF>
 hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = (tiles + 7) / 8 * 8;  // whole rounds over the 8 XCDs
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS, WBF>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU, WBF>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID, WBF>), dim3(grid), dim3(256), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
@@ -363,8 +386,12 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
   // 128x128 tiles once they fill the chip about twice over, 64x64 tiles otherwise
   const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
-  if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128>(a, epi, s);
-  return launch_gemm_tile<64, 64>(a, epi, s);
+  if (a.w_bf16) {
+    if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, true>(a, epi, s);
+    return launch_gemm_tile<64, 64, true>(a, epi, s);
+  }
+  if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, false>(a, epi, s);
+  return launch_gemm_tile<64, 64, false>(a, epi, s);
 }
 
 hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
@@ -383,9 +410,9 @@ hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_d
 }
 
 hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C, hipStream_t s) {
+                             int T, int C, hipStream_t s, int w_bf16) {
   hipLaunchKernelGGL(k_embed_rows, dim3((C + 255) / 256, T), dim3(256), 0, s, x, wte, wpe, ids, T,
-                     C);
+                     C, w_bf16);
   return hipGetLastError();
 }
 

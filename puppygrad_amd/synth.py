@@ -105,3 +105,22 @@ def tiny_weights(cfg: Gpt2Config) -> Gpt2Weights:
             ln_2_g=one(C), ln_2_b=zero(C), c_fc_w=patterned(C * I, 0.01), c_fc_b=zero(I),
             c_proj_mlp_w=patterned(I * C, 0.012), c_proj_mlp_b=zero(C))],
         ln_f_g=one(C), ln_f_b=zero(C))
+
+
+def round_bf16(a: np.ndarray) -> np.ndarray:
+    """f32 -> bf16 (round to nearest even) -> f32, as the bf16 weight storage does."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    r = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) & np.uint32(0xFFFF0000)
+    return r.view(np.float32)
+
+
+def bf16_rounded(w: Gpt2Weights) -> Gpt2Weights:
+    """The weights a bf16-storage model really multiplies with: wte and the four block
+    matrices rounded to bf16; LayerNorm parameters, biases and wpe untouched."""
+    blocks = [Gpt2BlockWeights(
+        ln_1_g=b.ln_1_g, ln_1_b=b.ln_1_b, c_attn_w=round_bf16(b.c_attn_w), c_attn_b=b.c_attn_b,
+        c_proj_w=round_bf16(b.c_proj_w), c_proj_b=b.c_proj_b, ln_2_g=b.ln_2_g, ln_2_b=b.ln_2_b,
+        c_fc_w=round_bf16(b.c_fc_w), c_fc_b=b.c_fc_b, c_proj_mlp_w=round_bf16(b.c_proj_mlp_w),
+        c_proj_mlp_b=b.c_proj_mlp_b) for b in w.blocks]
+    return Gpt2Weights(wte=round_bf16(w.wte), wpe=w.wpe, blocks=blocks, ln_f_g=w.ln_f_g,
+                       ln_f_b=w.ln_f_b)
