@@ -99,6 +99,7 @@ def main() -> int:
     wall = gpu = 0.0
     tokens = 0
     kv_total = 0
+    launches = 0
     while steps_left > 0:
         n = min(steps_left, room - 1)
         start = cache.seq_len
@@ -109,14 +110,25 @@ def main() -> int:
         tokens += n + 1
         kv_total += sum(kv_bytes(cfg, p) for p in range(start, start + n))
         steps_left -= n
+        launches += 1
         if steps_left > 0:
             rewind()
     K = args.steps
     ms_per_step = wall / K * 1e3
     gpu_ms_per_step = gpu / K * 1e3
     tok_s = K / wall  # forwards per second; the reference's tokens/sec adds the free last token
-    algo_bytes = weight_bytes(cfg) + kv_total / K
-    achieved = algo_bytes / (gpu / K) / 1e9
+    # Roofline of the dominant kernel.  On the persistent path one launch of
+    # k_decode_persistent<n_embd> runs every forward of a pass (embedding, all blocks,
+    # lm_head, argmax); its duration is the HIP-event time the library takes on the
+    # launch stream (gpu_decode_time).  Algorithmic bytes: the parameters once per
+    # forward plus the K/V rows of positions [0, pos] that forward attends over.
+    algo_bytes = weight_bytes(cfg) + kv_total / K            # per forward
+    bytes_per_launch = algo_bytes * K / launches
+    launch_s = gpu / launches
+    achieved = bytes_per_launch / launch_s / 1e9
+    persistent = "decode=persistent" in model.describe()
+    kernel = (f"k_decode_persistent<{cfg.n_embd}>" if persistent
+              else "all launches of one decode step (k_gemv dominant)")
 
     info = _lib.pg_device_info()
     _lib.load().pg_device_query(0, C.byref(info))
@@ -138,15 +150,19 @@ def main() -> int:
         "config": {"workload": f"GPT-2 {args.model} fp32 B=1 greedy decode, KV cache prefilled to "
                                f"{n_prefill} tokens, positions {n_prefill}..{n_prefill + min(K, room - 1) - 1}",
                    "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
-                   "device": info.name.decode(), "compute_units": info.compute_units,
+                   "device": info.name.decode() or info.arch.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "backend": model.describe()},
         "reference_metric_tokens_per_s": round(tokens / wall, 2),
         "gpu_ms_per_step": round(gpu_ms_per_step, 4),
         "prefill_s": round(prefill_s, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "one decode step (all launches of one token)",
-                     "algorithmic_bytes_per_step": int(algo_bytes)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(args, n_prefill, persistent, launches),
+                     "kernel": kernel, "launches": launches,
+                     "forwards_per_launch": K // launches,
+                     "launch_ms": round(launch_s * 1e3, 3),
+                     "algorithmic_bytes_per_launch": int(bytes_per_launch),
+                     "algorithmic_bytes_per_forward": int(algo_bytes)},
     }
 
     if not args.no_cpu_baseline:
@@ -154,6 +170,20 @@ def main() -> int:
 
     print(json.dumps(result), flush=True)
     return 0
+
+
+# HBM bytes one launch of k_decode_persistent<1600> moves on the default workload
+# (127 forwards from cache length 896), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this file (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the
+# counters and the copy-kernel scale factors).  None for any other workload.
+TRAFFIC_XL_DEFAULT = 931.4e9
+
+
+def measured_traffic(args, n_prefill, persistent, launches):
+    if (args.model == "xl" and n_prefill == 896 and args.steps == 127 and persistent
+            and launches == 1):
+        return TRAFFIC_XL_DEFAULT
+    return None
 
 
 def cpu_baseline(cfg, weights, ids, n_prefill):
@@ -176,7 +206,12 @@ def cpu_baseline(cfg, weights, ids, n_prefill):
         s, _ = ref.timed_forward_steps(rcache, n_prefill, step_ids[:max(1, n // 3)])
         runs.append(max(1, n // 3) / s)
     runs.sort()
+    one = oracle.Model(cfg, weights, oracle.rust_config(1))
+    c1 = one.new_kv_cache()
+    one.timed_forward_steps(c1, n_prefill, step_ids[:1])
+    s1, _ = one.timed_forward_steps(c1, n_prefill, step_ids[:3])
     return {"value": round(runs[1], 3), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "single_thread_value": round(3 / s1, 3),
             "sample": f"median of 3 runs of {max(1, n // 3)} forward_one steps starting at cache length "
                       f"{n_prefill} (KV values zero-filled; timing does not depend on them), "
                       f"default Gpt2RustConfig thresholds"}
