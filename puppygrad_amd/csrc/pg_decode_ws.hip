@@ -1,0 +1,1211 @@
+// Wave-specialised persistent batch-1 decode kernel for gfx950: one launch runs whole
+// cached decoder steps (forward_one_profiled_with_scratch,
+// src/models/gpt2/rust.rs:943-1006, block at 1136-1250, attention at 1662-1741) for
+// one or many greedy tokens.
+//
+// 256 workgroups of 8 wavefronts, one workgroup per CU, never a grid barrier.  Every
+// activation that crosses workgroups is a 64-bit word {epoch, f32 bits} written with
+// one agent-scope store; a reader polls until the word carries the epoch of the
+// producing (token, layer, phase).
+//
+// Vector memory loads of one wavefront return in issue order, so a wavefront that
+// polls global memory behind a prefetch of weights sees the answer only after the
+// weights have landed, and a wavefront that holds prefetched weights must not poll.
+// The roles are therefore split:
+//
+//   * wavefronts 0..6 ("streamers") own the rows of every weight matrix of this
+//     workgroup's band.  They only ever wait on flags in LDS, keep up to two weight
+//     bands in flight in their registers (the band in use and the next one or two,
+//     requested in consumption order as soon as registers free up), multiply and
+//     publish their rows.
+//   * wavefront 7 ("service") owns the dependency chain: it polls the tagged words,
+//     applies LayerNorm, stages the input vector of the next matrix in LDS and raises
+//     the LDS flag; it also runs this workgroup's (head, key-split) attention item,
+//     the per-head merge, the embedding and the argmax merge.
+//
+// Per layer:  A  LN1 + c_attn rows            -> qkv_t   (tagged)
+//             B  split-key attention per head -> part_t  (tagged partial acc, m, l)
+//             B2 per-head merge of the splits -> attn_t  (tagged)
+//             D  c_proj rows + residual       -> xa_t    (tagged)
+//             E  LN2 + c_fc rows + GELU       -> h_t     (tagged)
+//             F  mlp c_proj rows + residual   -> xm_t    (tagged)
+// then LN_f + lm_head rows -> logits (plain) and per-workgroup argmax -> best_t.
+//
+// Every wait is bounded: a poll that does not complete within its spin limit sets
+// the abort word (global) and the halt word (LDS); every other wait observes one of
+// them and all wavefronts leave the kernel.
+#include "pg_kernels.h"
+
+#include <math.h>
+
+#include <type_traits>
+
+namespace pgk {
+
+namespace {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+typedef unsigned long long u64;
+
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+constexpr int kThreads = 512;
+constexpr int kSW = 7;      // streamer wavefronts (0..6); wavefront 7 is the service wavefront
+constexpr int kGrid = 256;  // workgroups; row bands are computed for exactly this many
+constexpr unsigned kSpinLimit = 1u << 21;
+constexpr int kMaxItemKeys = 128;  // keys per (head, split) attention item
+constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
+
+// Tagged words and the abort word live in global memory; saying so in the pointer type
+// gets global_ instead of flat_ instructions (a flat access also counts as an LDS one).
+#define PG_G64(p) ((__attribute__((address_space(1))) unsigned long long*)(p))
+#define PG_G32(p) ((__attribute__((address_space(1))) unsigned*)(p))
+#define PG_LD64(p) __hip_atomic_load(PG_G64(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_ST64(p, v) __hip_atomic_store(PG_G64(p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_LD32(p) __hip_atomic_load(PG_G32(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_ST32(p, v) __hip_atomic_store(PG_G32(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+__device__ __forceinline__ u64 pack(unsigned epoch, float v) {
+  return ((u64)epoch << 32) | (u64)__float_as_uint(v);
+}
+__device__ __forceinline__ u64 pack_u(unsigned epoch, unsigned v) { return ((u64)epoch << 32) | v; }
+__device__ __forceinline__ unsigned tag_of(u64 w) { return (unsigned)(w >> 32); }
+__device__ __forceinline__ float val_of(u64 w) { return __uint_as_float((unsigned)w); }
+
+// Cross-lane adds through DPP (no LDS traffic).  All 64 lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// Sum over each row of 16 lanes; every lane of the row receives it.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_get<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_get<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_get<0x141>(v);  // row_half_mirror
+  v += dpp_get<0x140>(v);  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float lane_get(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+// Sum over the wavefront; the result is wave-uniform.
+__device__ __forceinline__ float wsum(float v) {
+  v = row16_sum(v);
+  return (lane_get(v, 0) + lane_get(v, 16)) + (lane_get(v, 32) + lane_get(v, 48));
+}
+__device__ __forceinline__ float wmax(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  return 0.5f * x * (1.0f + tanhf(0.7978846f * (x + 0.044715f * x * x * x)));
+}
+
+// Control block in LDS.
+struct Ctl {
+  unsigned flag[8];    // [0] A, [1] D, [2] E, [3] F, [4] lm_head: epoch whose input is staged;
+                       // [5], [6]: credits of the two attention hops
+  unsigned halt;       // 0 run, 1 a wait gave up, 2 stopped at the EOS token
+  unsigned lmdone[8];  // per streamer: epoch of its finished lm_head band
+  float bestv[8];
+  unsigned besti[8];
+  float qs[64];
+  float sc[kMaxItemKeys];
+};
+typedef __attribute__((address_space(3))) Ctl* ctlp;
+
+// Orders this wavefront's LDS accesses (and keeps the compiler from moving memory
+// accesses across): LDS executes a wavefront's operations in order, so a flag
+// written after this point is seen no earlier than the data written before it.
+__device__ __forceinline__ void lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void vm_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// The lane and wave index behind an empty asm: index arithmetic built on them is
+// recomputed where it is used instead of being hoisted out of the token/layer loops
+// (dozens of loop-invariant 64-bit addresses would otherwise be kept alive).
+__device__ __forceinline__ int opaque(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// Weight pointers come out of a table in memory; telling the compiler they are
+// global (not generic) addresses gets global_load instead of flat_load.
+typedef const f4 __attribute__((address_space(1)))* gf4p;
+__device__ __forceinline__ gf4p as_global(const f4* p) { return (gf4p)p; }
+__device__ __forceinline__ float gld(const float* p) {
+  return *(const float __attribute__((address_space(1)))*)p;
+}
+// Read-only tables written by the host before the launch (layer table, biases) are
+// read through the constant address space: wave-uniform addresses then become scalar
+// loads, which do not queue behind the vector loads of the weight rows.
+__device__ __forceinline__ float cld(const float* p) {
+  return *(const float __attribute__((address_space(4)))*)p;
+}
+__device__ __forceinline__ LayerW layer_of(const LayerW* table, int l) {
+  typedef const unsigned long long __attribute__((address_space(4)))* cq;
+  constexpr int NQ = sizeof(LayerW) / 8;
+  static_assert(sizeof(LayerW) % 8 == 0, "a table of pointers");
+  const cq src = (cq)(table + l);
+  union {
+    LayerW w;
+    unsigned long long q[NQ];
+  } u;
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) u.q[i] = src[i];
+  return u.w;
+}
+__device__ __forceinline__ void gst(float* p, float v) {
+  *(float __attribute__((address_space(1)))*)p = v;
+}
+__device__ __forceinline__ void gst_u(unsigned* p, unsigned v) {
+  *(unsigned __attribute__((address_space(1)))*)p = v;
+}
+__device__ __forceinline__ void gst_u64(u64* p, u64 v) {
+  *(u64 __attribute__((address_space(1)))*)p = v;
+}
+// LDS pointers keep their address space in the type: every access is a ds_ instruction
+// and never a flat one that would count as a vector memory operation.
+typedef __attribute__((address_space(3))) float* lfp;
+typedef __attribute__((address_space(3))) f4* lf4p;
+typedef volatile __attribute__((address_space(3))) unsigned* lvup;
+typedef __attribute__((address_space(3))) unsigned long long* lu64p;
+
+// One tile = one weight row (or a run of 64*J float4 of one), 64 lanes wide, J deep.
+template <int J>
+struct Tile {
+  f4 w[J];
+};
+// Loads are unconditional (columns past the row re-read its last float4 and meet a
+// zero in x): a load under a branch would make the compiler lose count of the loads
+// in flight and wait for all of them at the next use of an older one.
+// The row address is wave-uniform (scalar registers); the lane's part is a 32-bit byte
+// offset, so that the loads take the "scalar base + vector offset" form and no 64-bit
+// per-lane addresses have to be kept.
+__device__ __forceinline__ f4 ld_row(const f4* row, unsigned byte_off) {
+  typedef const char __attribute__((address_space(1)))* gcp;
+  return __builtin_nontemporal_load((gf4p)((gcp)row + byte_off));
+}
+template <int J>
+__device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const unsigned c = (64 * (j + 1) <= K4s) ? (unsigned)lane + 64u * j
+                                              : (unsigned)min(lane + 64 * j, K4s - 1);
+    t.w[j] = ld_row(p, c * 16u);
+  }
+}
+template <int J, int LO, int HI>
+__device__ __forceinline__ void load_tile_part(Tile<J>& t, const f4* p, int lane) {
+#pragma unroll
+  for (int j = LO; j < HI; ++j) t.w[j] = ld_row(p, ((unsigned)lane + 64u * j) * 16u);
+}
+template <int J>
+__device__ __forceinline__ void load_x(f4* xr, lfp xs, int K4s, int lane) {
+  lf4p x4 = (lf4p)xs;
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    int c = lane + 64 * j;
+    xr[j] = (64 * (j + 1) <= K4s || c < K4s) ? x4[min(c, K4s - 1)] : f4{0.f, 0.f, 0.f, 0.f};
+  }
+}
+template <int J>
+__device__ __forceinline__ float dot_tile(const Tile<J>& t, const f4* xr) {
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    a0 += t.w[j].x * xr[j].x;
+    a1 += t.w[j].y * xr[j].y;
+    a2 += t.w[j].z * xr[j].z;
+    a3 += t.w[j].w * xr[j].w;
+  }
+  return wsum((a0 + a1) + (a2 + a3));
+}
+
+struct Best {
+  float v;
+  unsigned i;
+};
+// argmax_logits order (src/models/generation.rs:269-279): greater value wins,
+// equal values keep the lower index; i == 0xffffffff means "no candidate yet".
+__device__ __forceinline__ Best better(Best a, Best b) {
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+// Best over the wavefront (every lane receives it).
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(b.v, off, 64), (unsigned)__shfl_xor((int)b.i, off, 64)};
+    b = better(b, o);
+  }
+  return b;
+}
+
+__device__ __forceinline__ unsigned epoch_of(const DecodeParams& p, int t, int layer, int phase) {
+  return p.epoch0 + (unsigned)((t * (p.L + 1) + layer) * 8 + phase);
+}
+
+// ---- streamer side: wait for an LDS flag ---------------------------------------------
+__device__ __forceinline__ bool wait_flag(ctlp ctl, int which, unsigned epoch, unsigned* abort_word) {
+  lvup f = (lvup)&ctl->flag[which];
+  lvup h = (lvup)&ctl->halt;
+  unsigned spins = 0;
+  bool ok = true;
+  for (;;) {
+    if (*f == epoch) break;
+    if (*h != 0) {
+      ok = false;
+      break;
+    }
+    if (++spins > kSpinLimit) {
+      ok = false;
+      PG_ST32(abort_word, 1u);
+      *h = 1u;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  asm volatile("" ::: "memory");
+  return ok;
+}
+
+// ---- service side: poll tagged words ---------------------------------------------------
+// One tagged word at a wave-uniform base plus a 32-bit byte offset ("scalar base +
+// vector offset" addressing: no 64-bit per-lane addresses are kept across the retries).
+__device__ __forceinline__ u64 ld_tagged(const u64* base, unsigned byte_off) {
+  typedef char __attribute__((address_space(1)))* gcp;
+  return __hip_atomic_load((__attribute__((address_space(1))) u64*)((gcp)base + byte_off),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Spins until run `run` (words 64 run .. 64 run + 63) carries `epoch`.  Cheap: one
+// 512-byte request per attempt.  Wave-uniform; false on timeout or abort.
+__device__ __forceinline__ bool probe_run(const u64* src, int run, unsigned epoch,
+                                          unsigned* abort_word, unsigned& spins) {
+  const int lane = opaque((int)threadIdx.x) & 63;
+  const unsigned off = (unsigned)(run * 64 + lane) * 8u;
+  for (;;) {
+    u64 v = ld_tagged(src, off);
+    if (__all(tag_of(v) == epoch)) return true;
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+    if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) return false;
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+// The run to probe after a bulk read that found stale words: one that holds a stale
+// word (`run_of_bad` is this lane's, meaningful where `bad`).  The expensive bulk read
+// is then only repeated once that laggard has arrived; the waiting is done by the
+// cheap probe and does not flood the CU's memory pipeline.
+__device__ __forceinline__ int next_probe_run(bool bad, int run_of_bad) {
+  const unsigned long long m = __ballot(bad);
+  const int first = __builtin_ctzll(m);
+  return __builtin_amdgcn_readlane(run_of_bad, first);
+}
+// Waits until src[i] carries `epoch` for every i in [0, 64 NE) and leaves the payloads
+// in dst (LDS): the cheap probe of one run (runs differ per workgroup at first, so that
+// the probes spread over memory channels), then a bulk read of lane + 64 e; while that
+// finds stale words, the probe moves to a stale word's run and the bulk read repeats.
+// Nothing but the probe run lives across a repeat: the payloads go to LDS at once.
+template <int NE>
+__device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp dst,
+                                          unsigned* abort_word, int probe, lu64p dbg = nullptr) {
+  const int lane = opaque((int)threadIdx.x) & 63;
+  unsigned spins = 0;
+  int run = probe % NE;
+  for (;;) {
+    if (!probe_run(src, run, epoch, abort_word, spins)) return false;
+    if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
+    bool bad = false;
+    int bad_e = 0;
+    u64 v[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) v[e] = ld_tagged(src, ((unsigned)lane + 64u * e) * 8u);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      if (tag_of(v[e]) != epoch) {
+        bad = true;
+        bad_e = e;
+      }
+      dst[lane + 64 * e] = val_of(v[e]);
+    }
+    if (!__any(bad)) return true;
+    run = next_probe_run(bad, bad_e);
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+  }
+}
+
+// Same wait for a long vector (N words, a multiple of 128): after the probe the tagged
+// words are copied global -> LDS without passing through registers (1 KiB per
+// request), then this wavefront checks the tags in LDS and writes the payloads to dst.
+// raw needs N * 8 bytes.
+template <int N>
+__device__ __forceinline__ bool dma_poll(const u64* src, unsigned epoch, lfp raw, lfp dst,
+                                         unsigned* abort_word, int probe, lu64p dbg = nullptr) {
+  static_assert(N % 128 == 0, "whole 1 KiB requests");
+  constexpr int NCH = N / 128;
+  const int lane = opaque((int)threadIdx.x) & 63;
+  unsigned spins = 0;
+  int run = probe % (N / 64);
+  typedef const f4 __attribute__((address_space(1)))* g4;
+  const g4 g = (g4)src;
+  unsigned attempts = 0;
+  for (;;) {
+    if (!probe_run(src, run, epoch, abort_word, spins)) return false;
+    if (dbg && lane == 0) {
+      if (attempts == 0) dbg[11] = __builtin_amdgcn_s_memtime();
+      dbg[14] = ++attempts;
+    }
+#pragma unroll 1
+    for (int c = 0; c < NCH; ++c)
+      __builtin_amdgcn_global_load_lds(g + 64 * c + lane,
+                                       (__attribute__((address_space(3))) void*)(raw + 256 * c), 16,
+                                       0, 16 /* sc1: agent scope */);
+    vm_drain();
+    if (dbg && lane == 0) dbg[15] = __builtin_amdgcn_s_memtime();
+    bool bad = false;
+    int bad_run = 0;
+    lf4p r4 = (lf4p)raw;
+    typedef __attribute__((address_space(3))) f2* lf2p;
+    lf2p d2 = (lf2p)dst;
+#pragma unroll 5
+    for (int c = 0; c < NCH; ++c) {
+      const f4 w = r4[64 * c + lane];  // {value, tag, value, tag}: words 2 (64 c + lane), + 1
+      if (__float_as_uint(w.y) != epoch || __float_as_uint(w.w) != epoch) {
+        bad = true;
+        bad_run = 2 * c + (lane >> 5);
+      }
+      d2[64 * c + lane] = f2{w.x, w.z};
+    }
+    if (!__any(bad)) return true;
+    run = next_probe_run(bad, bad_run);
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+  }
+}
+
+// layer_norm_in_place (src/models/cpu.rs:119-143) of the C = 64 NW values in raw (LDS;
+// this lane's are lane + 64 j), two-pass mean / biased variance, eps inside the sqrt;
+// writes the result to xs (LDS).
+template <int NW>
+__device__ __forceinline__ void wave_layer_norm(lfp raw, const float (&g)[NW], const float (&b)[NW],
+                                                float eps, lfp xs, int lane) {
+  constexpr int C = NW * 64;
+  float x[NW];
+#pragma unroll
+  for (int j = 0; j < NW; ++j) x[j] = raw[lane + 64 * j];
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) s += x[j];
+  const float mean = wsum(s) / (float)C;
+  float v = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    const float d = x[j] - mean;
+    v += d * d;
+  }
+  const float var = wsum(v) / (float)C;
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < NW; ++j) xs[lane + 64 * j] = (x[j] - mean) * inv * g[j] + b[j];
+}
+
+// Development timestamps (only when the launch carries a buffer for them): the shader
+// clock of the moment, kept in LDS and copied out once when the kernel ends, so that a
+// stamp costs a counter read and an LDS write and nothing in the vector memory path.
+#define PG_STAMP(layer, phase)                                                          \
+  do {                                                                                  \
+    if (p.prof && lane == 0 && t + 1 == p.n_fwd)                                        \
+      lds.ts[(layer) * 16 + (phase)] = __builtin_amdgcn_s_memtime();                    \
+  } while (0)
+
+struct Lds {
+  lfp xsA, xsD, xsE, xraw1, xraw2, xsF, kbuf, vbuf;
+  lu64p ts;  // development timestamps of the launch's last token: [layer 0..L][16]
+};
+constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
+
+// ===================================================================================
+// Service wavefront
+// ===================================================================================
+template <int C_>
+__device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
+  constexpr int C = C_, I = 4 * C_, NW = C_ / 64, NWI = I / 64;
+  constexpr int G = kGrid;
+  static_assert(C_ % 64 == 0, "vectors are spread over 64 lanes");
+  const int lane = opaque((int)threadIdx.x) & 63;
+  const int wg = blockIdx.x;
+  unsigned* abort_word = p.status;
+  lvup halt = (lvup)&ctl->halt;
+  const int H = p.H, P = p.P, ns = p.ns;
+
+  int t = 0;
+  int stopped = 0;
+  unsigned tok = 0;
+  // a wait gave up: tell the streamers and leave
+#define PG_SERVICE_FAIL()        \
+  do {                           \
+    if (lane == 0) *halt = 1u;   \
+    return;                      \
+  } while (0)
+
+  // merges the per-workgroup (value, index) pairs published with `ep`
+  auto merged_token = [&](unsigned ep, unsigned& out) -> bool {
+    // staged in xsF (idle between the last mlp projection and the next one)
+    if (!wave_poll<(2 * G) / 64>(p.best_t, ep, lds.xsF, abort_word, wg)) return false;
+    lds_fence();
+    // word 2g is the value, 2g+1 the index of workgroup g
+    Best b{-INFINITY, 0xffffffffu};
+#pragma unroll
+    for (int e = 0; e < G / 64; ++e) {
+      const int g = lane + 64 * e;
+      b = better(b, Best{lds.xsF[2 * g], __float_as_uint(lds.xsF[2 * g + 1])});
+    }
+    b = wave_best(b);
+    out = b.i == 0xffffffffu ? 0u : b.i;
+    return true;
+  };
+
+#pragma unroll 1
+  for (; t < p.n_fwd; ++t) {
+    const int pos = p.pos0 + t;
+    PG_STAMP(p.L, 7);
+    if (p.prof && lane == 0 && t + 1 == p.n_fwd) lds.ts[p.L * 16 + 13] = wall_clock64();
+    // ---- token to embed: given, or the argmax of the previous step's logits ----
+    if (p.force_ids) {
+      tok = p.force_ids[t];
+    } else if (t == 0) {
+      tok = p.tok_from_ptr ? p.d_tok[0] : p.tok_val;
+    } else {
+      if (!merged_token(epoch_of(p, t - 1, p.L, 6), tok)) {
+          PG_SERVICE_FAIL();
+        }
+    }
+    if (wg == 0 && lane == 0 && p.out_ids) gst_u(p.out_ids + t, tok);
+    if (p.eos >= 0 && tok == (unsigned)p.eos) {
+      stopped = 1;
+      break;
+    }
+
+#pragma unroll 1
+    for (int l = 0; l < p.L; ++l) {
+      const LayerW w = layer_of(p.layers, l);
+      float* kc = p.kv + (size_t)l * p.kv_layer_stride;
+      float* vc = kc + p.kv_v_offset;
+
+      // ================= A: block input -> LN1 -> xsA =================
+      {
+        float g[NW], b[NW];
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+          g[j] = gld(w.ln_1_g + lane + 64 * j);
+          b[j] = gld(w.ln_1_b + lane + 64 * j);
+        }
+        if (l == 0) {
+          // embedding (rust.rs:966-974)
+#pragma unroll
+          for (int j = 0; j < NW; ++j)
+            lds.xraw1[lane + 64 * j] = gld(p.wte + (size_t)tok * C + lane + 64 * j) +
+                                       gld(p.wpe + (size_t)pos * C + lane + 64 * j);
+        } else {
+          if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, l - 1, 5), lds.xraw1, abort_word, wg))
+            PG_SERVICE_FAIL();
+        }
+        lds_fence();
+        wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsA, lane);
+        lds_fence();
+        if (lane == 0) ctl->flag[0] = epoch_of(p, t, l, 0);
+      }
+      PG_STAMP(l, 0);
+
+      // ================= B: this workgroup's (head, split) items =================
+      const int items = H * ns, n = pos + 1;
+      const int per = (n + ns - 1) / ns;
+      const int sub = lane >> 4, d4 = lane & 15;
+      const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
+#pragma unroll 1
+      for (int item = wg; item < items; item += G) {
+        const int h = item / ns, s = item - h * ns;
+        const int k0 = s * per, k1 = min(n, k0 + per);
+        u64* dst = p.part_t + (size_t)item * 66;
+        if (k0 >= k1) {  // empty split: neutral element of the merge
+          PG_ST64(dst + lane, pack(epp, 0.0f));
+          if (lane == 0) PG_ST64(dst + 64, pack(epp, -INFINITY));
+          if (lane == 1) PG_ST64(dst + 65, pack(epp, 0.0f));
+          continue;
+        }
+        const int nk = k1 - k0;  // <= kMaxItemKeys (the host picks ns >= P / 128)
+        const int groups = (nk + 3) >> 2;
+        const bool owns_new = (k1 == n);
+        // K and V rows of the item straight into LDS, four keys per request.  The row
+        // of `pos` is not in the cache yet: it (and rows past the split) re-read an
+        // older row and are replaced / masked below.
+        {
+          gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
+          gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
+#pragma unroll 1
+          for (int i = 0; i < groups; ++i) {
+            const int key = min(k0 + 4 * i + sub, max(pos - 1, 0));
+            __builtin_amdgcn_global_load_lds(
+                Kh + (size_t)key * 16 + d4,
+                (__attribute__((address_space(3))) void*)(lds.kbuf + 256 * i), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(
+                Vh + (size_t)key * 16 + d4,
+                (__attribute__((address_space(3))) void*)(lds.vbuf + 256 * i), 16, 0, 0);
+          }
+        }
+        // q of this head, and this token's own K/V rows if the split holds pos
+        float qn[3];
+        {
+          bool ok = true;
+          unsigned spins = 0;
+          const unsigned off = (unsigned)(h * 64 + lane) * 8u;
+          for (;;) {
+            // without the new row, the K and V words are not waited for (q is re-read)
+            const u64 v0 = ld_tagged(p.qkv_t, off);
+            const u64 v1 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 8u : 0u));
+            const u64 v2 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 16u : 0u));
+            const bool bad = tag_of(v0) != epq || tag_of(v1) != epq || tag_of(v2) != epq;
+            qn[0] = val_of(v0);
+            qn[1] = val_of(v1);
+            qn[2] = val_of(v2);
+            if (!__any(bad)) break;
+            if (++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
+              ok = false;
+              break;
+            }
+            if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          if (!ok) PG_SERVICE_FAIL();
+        }
+        vm_drain();  // the K/V rows have landed in LDS
+        // first credit: the streamers may request their next slice behind this poll
+        if (lane == 0) ctl->flag[5] = epp;
+        ctl->qs[lane] = qn[0];
+        if (owns_new) {
+          // K/V append (rust.rs:1677-1683); written through to memory so that a later
+          // token's reader on another XCD cannot miss it in a remote L2
+          lds.kbuf[(pos - k0) * 64 + lane] = qn[1];
+          lds.vbuf[(pos - k0) * 64 + lane] = qn[2];
+          PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[1]));
+          PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[2]));
+        }
+        lds_fence();
+        const f4 qv = ((lf4p)&ctl->qs[0])[d4];
+        lf4p k4 = (lf4p)lds.kbuf;
+        lf4p v4 = (lf4p)lds.vbuf;
+        float mx = -INFINITY;
+#pragma unroll 1
+        for (int i = 0; i < groups; ++i) {
+          const f4 kr = k4[64 * i + lane];
+          float sv = (qv.x * kr.x + qv.y * kr.y) + (qv.z * kr.z + qv.w * kr.w);
+          sv = row16_sum(sv);
+          sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
+          const int key = k0 + 4 * i + sub;
+          sv = (key < k1) ? sv : -INFINITY;
+          if (d4 == 0) ctl->sc[4 * i + sub] = sv;
+          mx = fmaxf(mx, sv);
+        }
+        mx = wmax(mx);
+        lds_fence();
+        float lsum = 0.0f;
+        f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+        for (int i = 0; i < groups; ++i) {
+          const float pr = expf(ctl->sc[4 * i + sub] - mx);  // exp(-inf) = 0 for absent keys
+          lsum += pr;
+          acc += pr * v4[64 * i + lane];
+        }
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+          acc.x += __shfl_xor(acc.x, off, 64);
+          acc.y += __shfl_xor(acc.y, off, 64);
+          acc.z += __shfl_xor(acc.z, off, 64);
+          acc.w += __shfl_xor(acc.w, off, 64);
+        }
+        // every lane of a 16-lane row holds the same lsum: the wave sum is 16 x the total
+        lsum = wsum(lsum) * 0.0625f;
+        if (lane < 16) {
+          PG_ST64(dst + 4 * lane + 0, pack(epp, acc.x));
+          PG_ST64(dst + 4 * lane + 1, pack(epp, acc.y));
+          PG_ST64(dst + 4 * lane + 2, pack(epp, acc.z));
+          PG_ST64(dst + 4 * lane + 3, pack(epp, acc.w));
+        }
+        if (lane == 16) PG_ST64(dst + 64, pack(epp, mx));
+        if (lane == 17) PG_ST64(dst + 65, pack(epp, lsum));
+      }
+      // both credits stand from here on (a workgroup without an item raises them now)
+      if (lane == 0) {
+        ctl->flag[5] = epp;
+        ctl->flag[6] = epp;
+      }
+      PG_STAMP(l, 1);
+
+      // ================= B2: the workgroup that took split 0 of a head merges it ====
+      const unsigned epa = epoch_of(p, t, l, 2);
+#pragma unroll 1
+      for (int item = wg; item < items; item += G) {
+        const int h = item / ns, s = item - h * ns;
+        if (s != 0) continue;
+        const u64* src = p.part_t + (size_t)h * ns * 66;
+        float M = -INFINITY, num = 0.0f, den = 0.0f;
+        constexpr int CH = 16;
+#pragma unroll 1
+        for (int q0 = 0; q0 < ns; q0 += CH) {
+          u64 wa[CH], wm[CH], wl[CH];
+          unsigned spins = 0;
+          bool ok = true;
+          for (;;) {
+            bool bad = false;
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+              const unsigned qq = (unsigned)min(q0 + q, ns - 1) * 66u;
+              wa[q] = ld_tagged(src, (qq + (unsigned)lane) * 8u);
+              wm[q] = ld_tagged(src, (qq + 64u) * 8u);
+              wl[q] = ld_tagged(src, (qq + 65u) * 8u);
+            }
+#pragma unroll
+            for (int q = 0; q < CH; ++q)
+              bad = bad || tag_of(wa[q]) != epp || tag_of(wm[q]) != epp || tag_of(wl[q]) != epp;
+            if (!__any(bad)) break;
+            if (++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
+              ok = false;
+              break;
+            }
+            if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          if (!ok) PG_SERVICE_FAIL();
+          // online merge of this chunk of splits (neutral: m = -inf, l = 0, acc = 0)
+          float Mc = M;
+#pragma unroll
+          for (int q = 0; q < CH; ++q)
+            if (q0 + q < ns) Mc = fmaxf(Mc, val_of(wm[q]));
+          const float scale = (M == -INFINITY) ? 0.0f : expf(M - Mc);
+          num *= scale;
+          den *= scale;
+#pragma unroll
+          for (int q = 0; q < CH; ++q) {
+            if (q0 + q < ns) {
+              const float wq = expf(val_of(wm[q]) - Mc);
+              den += wq * val_of(wl[q]);
+              num += wq * val_of(wa[q]);
+            }
+          }
+          M = Mc;
+        }
+          PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
+      }
+
+      // ================= D: attention output -> xsD =================
+      {
+        if (!wave_poll<NW>(p.attn_t, epa, lds.xsD, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        lds_fence();
+        if (lane == 0) ctl->flag[1] = epa;
+      }
+      PG_STAMP(l, 2);
+
+      // ================= E: xa -> xraw2, LN2 -> xsE =================
+      {
+        float g[NW], b[NW];
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+          g[j] = gld(w.ln_2_g + lane + 64 * j);
+          b[j] = gld(w.ln_2_b + lane + 64 * j);
+        }
+        const unsigned ep = epoch_of(p, t, l, 3);
+        if (!wave_poll<NW>(p.xa_t, ep, lds.xraw2, abort_word, wg + 2,
+                           (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 + 13 : (lu64p) nullptr))
+          PG_SERVICE_FAIL();
+        lds_fence();
+        wave_layer_norm<NW>(lds.xraw2, g, b, p.eps, lds.xsE, lane);
+        lds_fence();
+        if (lane == 0) ctl->flag[2] = ep;
+      }
+      PG_STAMP(l, 3);
+
+      // ================= F: h -> xsF =================
+      // 4C tagged words are too many for one wavefront's registers: they are copied
+      // straight into LDS (the K/V staging area, idle now), then checked and compacted.
+      {
+        const unsigned ep = epoch_of(p, t, l, 4);
+        if (!dma_poll<I>(p.h_t, ep, lds.kbuf, lds.xsF, abort_word, wg + 3,
+                         (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 : (lu64p) nullptr)) {
+          PG_SERVICE_FAIL();
+        }
+        lds_fence();
+        if (lane == 0) ctl->flag[3] = ep;
+      }
+      PG_STAMP(l, 4);
+    }  // layers
+
+    // ================= LN_f -> xsD, then this workgroup's argmax =================
+    if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      float g[NW], b[NW];
+#pragma unroll
+      for (int j = 0; j < NW; ++j) {
+        g[j] = gld(p.ln_f_g + lane + 64 * j);
+        b[j] = gld(p.ln_f_b + lane + 64 * j);
+      }
+      const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
+      // staged in xraw1 (the next user is the next token's embedding)
+      if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, p.L - 1, 5), lds.xraw1, abort_word, wg))
+        PG_SERVICE_FAIL();
+      lds_fence();
+      wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsD, lane);
+      lds_fence();
+      if (lane == 0) ctl->flag[4] = epl;
+      PG_STAMP(p.L, 5);
+      // wait for the streamers' bands
+      {
+        lvup done = (lvup)&ctl->lmdone[min(lane, kSW - 1)];
+        unsigned spins = 0;
+        bool ok = true;
+        for (;;) {
+          if (__all(*done == epl)) break;
+          if (*halt != 0) {
+            ok = false;
+            break;
+          }
+          if (++spins > kSpinLimit) {
+            PG_ST32(abort_word, 1u);
+            ok = false;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");
+        if (!ok) {
+          PG_SERVICE_FAIL();
+        }
+      }
+      Best bb{ctl->bestv[min(lane, kSW - 1)], ctl->besti[min(lane, kSW - 1)]};
+      bb = wave_best(bb);
+      if (lane == 0) PG_ST64(p.best_t + 2 * wg, pack(ep_best, bb.v));
+      if (lane == 1) PG_ST64(p.best_t + 2 * wg + 1, pack_u(ep_best, bb.i));
+      PG_STAMP(p.L, 6);
+    }
+  }  // tokens
+
+  if (p.prof) {
+    // calibration pair (wall clock, shader clock), then the copy to global memory
+    if (lane == 0) {
+      lds.ts[p.L * 16 + 14] = wall_clock64();
+      lds.ts[p.L * 16 + 15] = __builtin_amdgcn_s_memtime();
+    }
+    lds_fence();
+    for (int i = lane; i < (p.L + 1) * 16; i += 64)
+      gst_u64(p.prof + (size_t)wg * (p.L + 1) * 16 + i, lds.ts[i]);
+  }
+  if (stopped) {
+    if (lane == 0) *halt = 2u;
+  } else if (p.select_last && p.n_fwd > 0) {
+    unsigned tk = 0;
+    if (!merged_token(epoch_of(p, p.n_fwd - 1, p.L, 6), tk)) {
+      PG_SERVICE_FAIL();
+    }
+    if (wg == 0 && lane == 0) {
+      if (p.out_ids) gst_u(p.out_ids + p.n_fwd, tk);
+      gst_u(p.d_tok, tk);
+    }
+  }
+  if (wg == 0 && lane == 0) {
+    gst_u(p.status + 1, (unsigned)t);
+    gst_u(p.status + 2, (unsigned)stopped);
+  }
+}
+
+#undef PG_SERVICE_FAIL
+
+// ===================================================================================
+// Streamer wavefronts
+// ===================================================================================
+// Wavefront w owns row r0 + w + 7 i of a band (i < T) for the C-wide matrices and row
+// d0 + w of the 4C-wide mlp projection.  A row is J float4 per lane; the input
+// vector's matching float4 come out of LDS once per phase.
+//
+// The vector memory path of a CU returns data in issue order across ALL of its
+// wavefronts, so every byte the streamers have in flight delays the service
+// wavefront's next poll by the time it takes to drain (about 1 us per 32 KiB).  The
+// layer's weights are therefore requested as one fixed stream
+//     c_proj row | c_fc rows | mlp projection row | next layer's c_attn rows
+// cut into six equal slices, and a slice is only requested at a moment when the
+// service wavefront has just completed a poll (one per phase: after the A, D, E and F
+// products, and on the two "credits" it raises during the attention phases).  Each
+// slice drains while the dependency chain makes its next hop; each is requested at
+// least one phase before its rows are used.
+template <int C_>
+struct StreamPlan {
+  static constexpr int C = C_, I = 4 * C_, K4 = C_ / 4, G = kGrid;
+  static constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
+  static constexpr int TA = cdiv(RA, kSW), TE = cdiv(RE, kSW);
+  static constexpr int J = cdiv(K4, 64);
+  static constexpr int JF = C_ / 64;  // float4 per lane of one 4C-wide row
+  // loads per layer and wavefront, in stream order
+  static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
+  // Equal cuts where the registers allow it.  The widest model cannot hold the c_fc rows
+  // next to much of the mlp projection row: its first four slices are shorter and the
+  // last two longer (those two phases then run at the speed of the stream).
+  static constexpr bool kTight = (ND + NE + NF) * 4 > 200;
+  static constexpr int cut(int k) {
+    if (!kTight || k == 0 || k == 6) return k * NL / 6;
+    const int c4 = ND + NE + 4;
+    if (k <= 4) return k * c4 / 4;
+    return (c4 + NL) / 2 > ND + NE + NF ? (c4 + NL) / 2 : ND + NE + NF;
+  }
+  // slice k is requested: 0 after A, 1 and 2 on the attention credits, 3 after D,
+  // 4 after E, 5 after F.  D is used after slice 2, E after 3, F after 4, A' after 5.
+  static_assert(ND <= cut(3), "c_proj row is requested before it is used");
+  static_assert(ND + NE <= cut(4), "c_fc rows are requested before they are used");
+  static_assert(ND + NE + NF <= cut(5), "mlp projection row is requested before it is used");
+  static_assert(RD <= kSW, "one mlp projection row per streamer");
+  static_assert(C_ % 64 == 0, "4C-wide rows are whole runs of 64 float4");
+};
+
+template <int C_>
+__device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
+  typedef StreamPlan<C_> SP;
+  constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
+  constexpr int G = kGrid;
+  constexpr int TA = SP::TA, TE = SP::TE, J = SP::J, JF = SP::JF;
+
+  const int lane = opaque((int)threadIdx.x) & 63;
+  const int wg = blockIdx.x;
+  const int V = p.V;
+  unsigned* abort_word = p.status;
+
+  // row bands of this workgroup
+  const int a0 = (int)(((long long)wg * (3 * C)) / G), a1 = (int)(((long long)(wg + 1) * (3 * C)) / G);
+  const int d0 = (int)(((long long)wg * C) / G), d1 = (int)(((long long)(wg + 1) * C) / G);
+  const int e0 = (int)(((long long)wg * I) / G), e1 = (int)(((long long)(wg + 1) * I) / G);
+  const int v0 = (int)(((long long)wg * V) / G), v1 = (int)(((long long)(wg + 1) * V) / G);
+
+  // the wavefront index as a scalar: rows, row addresses and biases are wave-uniform
+  auto wave_id = [&]() { return __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6); };
+  // Row i of this wavefront in a band [r0, r1), clamped into the band (rows past the
+  // end re-read the last row; their results are dropped).
+  auto row_of = [&](int r0, int r1, int i) { return min(r0 + wave_id() + kSW * i, r1 - 1); };
+
+  Tile<J> WA[TA];  // c_attn rows of the layer about to run
+  Tile<J> WD;      // c_proj row
+  Tile<J> WE[TE];  // c_fc rows
+  Tile<JF> WF;     // mlp projection row
+
+  // One float4 of a C-wide row: column block j (columns past the row re-read its last
+  // float4 and meet a zero in x).  Unconditional, like every load here: a load under a
+  // branch would make the compiler lose count of the loads in flight.
+  auto ld_c = [&](const float* W, int row, int j) -> f4 {
+    const unsigned c = (64 * (j + 1) <= K4) ? (unsigned)lane + 64u * j
+                                            : (unsigned)min(lane + 64 * j, K4 - 1);
+    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * K4, c * 16u);
+  };
+  // Requests loads [N0, N1) of the layer stream: `w` is the layer whose c_proj, c_fc and
+  // mlp projection rows are meant, `wn` the one whose c_attn rows follow.
+  auto issue = [&](auto n0_, auto n1_, const LayerW& w, const LayerW& wn) {
+    constexpr int N0 = decltype(n0_)::value, N1 = decltype(n1_)::value;
+#pragma unroll
+    for (int n = N0; n < N1; ++n) {
+      if (n < SP::ND) {
+        WD.w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n);
+      } else if (n < SP::ND + SP::NE) {
+        const int i = (n - SP::ND) / J, j = (n - SP::ND) % J;
+        WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j);
+      } else if (n < SP::ND + SP::NE + SP::NF) {
+        const int j = n - SP::ND - SP::NE;
+        WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
+                         ((unsigned)lane + 64u * j) * 16u);
+      } else {
+        const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
+        WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j);
+      }
+    }
+  };
+#define PG_SLICE(k, w, wn)                                              \
+  issue(std::integral_constant<int, SP::cut(k)>{},                      \
+        std::integral_constant<int, SP::cut((k) + 1)>{}, (w), (wn))
+
+  // before the first layer: its c_attn rows
+  {
+    const LayerW w0 = layer_of(p.layers, 0);
+    issue(std::integral_constant<int, SP::ND + SP::NE + SP::NF>{},
+          std::integral_constant<int, SP::NL>{}, w0, w0);
+  }
+
+  // development timestamps of streamer 0 (slots 5.. of the layer's 16)
+#define SSTAMP(slot)                                                                   \
+  do {                                                                                 \
+    if (p.prof && lane == 0 && wave == 0 && t + 1 == p.n_fwd)                          \
+      lds.ts[l * 16 + (slot)] = __builtin_amdgcn_s_memtime();                          \
+  } while (0)
+  bool ok = true;
+  for (int t = 0; t < p.n_fwd && ok; ++t) {
+    for (int l = 0; l < p.L; ++l) {
+      const LayerW w = layer_of(p.layers, l);
+      const LayerW wn = layer_of(p.layers, (l + 1 < p.L) ? l + 1 : 0);
+      const int wave = wave_id();
+
+      // ================= A: c_attn rows =================
+      // (biases are scalar loads: requested before each wait, they neither use vector
+      // registers while the rows are in flight nor queue behind them)
+      float biasA[TA];
+#pragma unroll
+      for (int i = 0; i < TA; ++i) biasA[i] = cld(w.c_attn_b + row_of(a0, a1, i));
+      if (!wait_flag(ctl, 0, epoch_of(p, t, l, 0), abort_word)) {
+        ok = false;
+        break;
+      }
+      // (a slice goes out the moment the flag is seen where the registers allow it:
+      // the service wavefront has just completed a poll and its next ones are early)
+      PG_SLICE(0, w, wn);
+      {
+        f4 xr[J];
+        load_x<J>(xr, lds.xsA, K4, lane);
+        const unsigned ep = epoch_of(p, t, l, 0);
+#pragma unroll
+        for (int i = 0; i < TA; ++i) {
+          const int r = a0 + wave + kSW * i;
+          const float v = dot_tile<J>(WA[i], xr);
+          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, biasA[i] + v));
+        }
+      }
+      SSTAMP(5);
+      // ---- the two attention hops: nothing to compute, one slice each ----
+      if (!wait_flag(ctl, 5, epoch_of(p, t, l, 1), abort_word)) {
+        ok = false;
+        break;
+      }
+      PG_SLICE(1, w, wn);
+      if (!wait_flag(ctl, 6, epoch_of(p, t, l, 1), abort_word)) {
+        ok = false;
+        break;
+      }
+      PG_SLICE(2, w, wn);
+
+      // ================= D: c_proj row + residual =================
+      const float biasD = cld(w.c_proj_b + row_of(d0, d1, 0));
+      if (!wait_flag(ctl, 1, epoch_of(p, t, l, 2), abort_word)) {
+        ok = false;
+        break;
+      }
+      {
+        f4 xr[J];
+        load_x<J>(xr, lds.xsD, K4, lane);
+        const int r = d0 + wave;
+        const float v = dot_tile<J>(WD, xr);
+        if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v)));
+      }
+      PG_SLICE(3, w, wn);
+
+      // ================= E: c_fc rows + GELU =================
+      float biasE[TE];
+#pragma unroll
+      for (int i = 0; i < TE; ++i) biasE[i] = cld(w.c_fc_b + row_of(e0, e1, i));
+      if (!wait_flag(ctl, 2, epoch_of(p, t, l, 3), abort_word)) {
+        ok = false;
+        break;
+      }
+      {
+        f4 xr[J];
+        load_x<J>(xr, lds.xsE, K4, lane);
+        const unsigned ep = epoch_of(p, t, l, 4);
+#pragma unroll
+        for (int i = 0; i < TE; ++i) {
+          const int r = e0 + wave + kSW * i;
+          const float v = dot_tile<J>(WE[i], xr);
+          if (lane == 0 && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(biasE[i] + v)));
+        }
+      }
+      SSTAMP(6);
+      PG_SLICE(4, w, wn);
+
+      // ================= F: mlp projection row + residual =================
+      const float biasF = cld(w.c_proj_mlp_b + row_of(d0, d1, 0));
+      if (!wait_flag(ctl, 3, epoch_of(p, t, l, 4), abort_word)) {
+        ok = false;
+        break;
+      }
+      SSTAMP(10);
+      if (p.prof) {  // development: how long the row's last loads are still in flight
+        vm_drain();
+        SSTAMP(12);
+      }
+      {
+        lf4p x4 = (lf4p)lds.xsF;
+        float a0_ = 0.f, a1_ = 0.f, a2_ = 0.f, a3_ = 0.f;
+        constexpr int B = 5;  // LDS reads kept in flight together
+#pragma unroll
+        for (int j0 = 0; j0 < JF; j0 += B) {
+          f4 x[B];
+          // keeps the LDS reads of later groups from being moved up here (they would
+          // all be live at once next to the weight row)
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int b = 0; b < B; ++b)
+#ifdef PG_DBG_F_NOLDS
+            if (j0 + b < JF) x[b] = f4{(float)lane, 1.0f, 2.0f, (float)(j0 + b)};
+#else
+            if (j0 + b < JF) x[b] = x4[lane + 64 * (j0 + b)];
+#endif
+#pragma unroll
+          for (int b = 0; b < B; ++b)
+            if (j0 + b < JF) {
+              a0_ += WF.w[j0 + b].x * x[b].x;
+              a1_ += WF.w[j0 + b].y * x[b].y;
+              a2_ += WF.w[j0 + b].z * x[b].z;
+              a3_ += WF.w[j0 + b].w * x[b].w;
+            }          if (j0 == 0) SSTAMP(8);
+          if (j0 == 2 * B) SSTAMP(9);
+        }
+        const float v = wsum((a0_ + a1_) + (a2_ + a3_));
+        const int r = d0 + wave;
+        if (lane == 0 && r < d1) PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), lds.xraw2[r] + (biasF + v)));
+      }
+      SSTAMP(7);
+      PG_SLICE(5, w, wn);
+    }  // layers
+    if (!ok) break;
+
+    // ================= lm_head rows (rust.rs:982-1002) + band argmax =================
+    if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      const int wave = wave_id();
+      const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
+      float* const logits = p.logits;
+      Tile<J> T[kLmTiles];
+#pragma unroll
+      for (int k = 0; k < kLmTiles; ++k)
+        load_tile<J>(T[k], wte4 + (size_t)min(v0 + wave + kSW * k, v1 - 1) * K4, K4, lane);
+      const unsigned epl = epoch_of(p, t, p.L, 5);
+      if (!wait_flag(ctl, 4, epl, abort_word)) {
+        ok = false;
+        break;
+      }
+      f4 xr[J];
+      load_x<J>(xr, lds.xsD, K4, lane);
+      Best best{-INFINITY, 0xffffffffu};
+      for (int r = v0 + wave; r < v1; r += kSW * kLmTiles) {
+#pragma unroll
+        for (int k = 0; k < kLmTiles; ++k) {
+          const int rk = r + kSW * k;
+          const float v = dot_tile<J>(T[k], xr);
+          load_tile<J>(T[k], wte4 + (size_t)min(rk + kSW * kLmTiles, v1 - 1) * K4, K4, lane);
+          if (rk < v1) {
+            if (lane == 0) gst(logits + rk, v);
+            if (v > best.v) best = Best{v, (unsigned)rk};
+          }
+        }
+      }
+      if (lane == 0) {
+        ctl->bestv[wave] = best.v;
+        ctl->besti[wave] = best.i;
+      }
+      lds_fence();
+      if (lane == 0) ctl->lmdone[wave] = epl;
+    }
+  }  // tokens
+  vm_drain();  // nothing of this wavefront is still in flight when it ends
+#undef SSTAMP
+#undef PG_SLICE
+}
+
+// C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
+template <int C_>
+__global__ __launch_bounds__(kThreads) void k_decode_ws(DecodeParams p) {
+  constexpr int C = C_, I = 4 * C_;
+  // 16-byte LDS accesses run at full speed only on 16-byte boundaries: the dynamic block
+  // starts on one whatever the size of the static control block before it
+  extern __shared__ __attribute__((aligned(256))) float dyn[];
+  __shared__ Ctl ctl_block;
+  ctlp ctl = (ctlp)&ctl_block;
+  Lds lds;
+  lds.xsA = (lfp)dyn;
+  lds.xsD = lds.xsA + C;
+  lds.xsE = lds.xsA + 2 * C;
+  lds.xraw1 = lds.xsA + 3 * C;
+  lds.xraw2 = lds.xsA + 4 * C;
+  lds.xsF = lds.xsA + 5 * C;
+  lds.kbuf = lds.xsA + 5 * C + I;
+  lds.vbuf = lds.kbuf + kMaxItemKeys * 64;
+  lds.ts = (lu64p)(lds.vbuf + kMaxItemKeys * 64);
+  if (p.prof)
+    for (int i = threadIdx.x; i < kTsLayers * 16; i += kThreads) lds.ts[i] = 0;
+
+  if (threadIdx.x < 8) {
+    ctl->flag[threadIdx.x] = 0u;
+    ctl->lmdone[threadIdx.x] = 0u;
+  }
+  if (threadIdx.x == 0) ctl->halt = 0u;
+  __syncthreads();
+
+#ifndef PG_WS_ONLY_STREAMER
+  if ((threadIdx.x >> 6) == kSW)
+    service_wave<C_>(p, ctl, lds);
+#endif
+#ifndef PG_WS_ONLY_SERVICE
+  if ((threadIdx.x >> 6) != kSW)
+    streamer_wave<C_>(p, ctl, lds);
+#endif
+}
+
+}  // namespace
+
+size_t ws_lds_bytes(int C) {
+  return (size_t)(9 * C + 2 * kMaxItemKeys * 64) * sizeof(float) + (size_t)kTsLayers * 16 * 8;
+}
+int ws_grid() { return kGrid; }
+int ws_max_item_keys() { return kMaxItemKeys; }
+
+namespace {
+template <int C_>
+hipError_t launch_ws(const DecodeParams& p, hipStream_t s) {
+  const size_t lds = ws_lds_bytes(C_);
+  // more than the 64 KiB default of dynamic LDS: opt in once per device
+  static thread_local int armed_device = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (armed_device != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_ws<C_>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    armed_device = dev;
+  }
+  hipLaunchKernelGGL(k_decode_ws<C_>, dim3(kGrid), dim3(kThreads), lds, s, p);
+  return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_decode_ws(const DecodeParams& p, hipStream_t s) {
+  if (p.C == 768) return launch_ws<768>(p, s);
+  if (p.C == 1024) return launch_ws<1024>(p, s);
+  if (p.C == 1600) return launch_ws<1600>(p, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t ws_max_blocks_per_cu(int C, int* out) {
+  const size_t lds = ws_lds_bytes(C);
+  if (C == 768) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_ws<768>, kThreads, lds);
+  if (C == 1024) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_ws<1024>, kThreads, lds);
+  if (C == 1600) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_ws<1600>, kThreads, lds);
+  *out = 0;
+  return hipSuccess;
+}
+
+}  // namespace pgk
