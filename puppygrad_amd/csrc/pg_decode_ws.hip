@@ -107,13 +107,19 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 // Control block in LDS.
 struct Ctl {
   unsigned flag[8];    // [0] A, [1] D, [2] E, [3] F, [4] lm_head: epoch whose input is staged;
-                       // [5], [6]: credits of the two attention hops
+                       // [5] attention item staged (running count), [6] credit of the
+                       // second attention hop (epoch), [7] "read your share of h" (running count)
   unsigned halt;       // 0 run, 1 a wait gave up, 2 stopped at the EOS token
   unsigned lmdone[8];  // per streamer: epoch of its finished lm_head band
+  unsigned bdone[8];   // per wavefront: count of the attention item whose partial it has written
+  unsigned hstat[8];   // per wavefront: (count << 8) | (1 + a stale run, or 0) of its share of h
   float bestv[8];
   unsigned besti[8];
-  float qs[64];
-  float sc[kMaxItemKeys];
+  float wm[8], wl[8];  // attention partials of the wavefronts: max, sum of weights ...
+  __attribute__((aligned(16))) float wacc[8][64];  // ... and weighted V rows
+  __attribute__((aligned(16))) float qs[64];       // q, and this token's K and V rows of the head
+  __attribute__((aligned(16))) float kn[64];
+  __attribute__((aligned(16))) float vn[64];
 };
 typedef __attribute__((address_space(3))) Ctl* ctlp;
 
@@ -137,6 +143,12 @@ typedef const f4 __attribute__((address_space(1)))* gf4p;
 __device__ __forceinline__ gf4p as_global(const f4* p) { return (gf4p)p; }
 __device__ __forceinline__ float gld(const float* p) {
   return *(const float __attribute__((address_space(1)))*)p;
+}
+// element i of a wave-uniform array: the base stays scalar, the lane's part is a 32-bit
+// byte offset
+__device__ __forceinline__ float gld_at(const float* base, unsigned i) {
+  typedef const char __attribute__((address_space(1)))* gcp;
+  return *(const float __attribute__((address_space(1)))*)((gcp)base + i * 4u);
 }
 // Read-only tables written by the host before the launch (layer table, biases) are
 // read through the constant address space: wave-uniform addresses then become scalar
@@ -223,6 +235,47 @@ __device__ __forceinline__ float dot_tile(const Tile<J>& t, const f4* xr) {
   }
   return wsum((a0 + a1) + (a2 + a3));
 }
+// The same products for T rows at once with the input vector read from LDS column block
+// by column block (two in flight) instead of being held in registers for the whole
+// phase: same order of additions per row as dot_tile.
+template <int T, int J>
+__device__ __forceinline__ void dot_tiles(const Tile<J> (&W)[T], lfp xs, int K4s, int lane,
+                                          float (&out)[T]) {
+  lf4p x4 = (lf4p)xs;
+  f4 acc[T];
+#pragma unroll
+  for (int i = 0; i < T; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+  constexpr int B = 2;
+#pragma unroll
+  for (int j0 = 0; j0 < J; j0 += B) {
+    f4 x[B];
+    // keeps the LDS reads of later column blocks from being moved up here
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int j = j0 + b;
+      if (j < J) {
+        const int c = lane + 64 * j;
+        x[b] = (64 * (j + 1) <= K4s || c < K4s) ? x4[min(c, K4s - 1)] : f4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int j = j0 + b;
+      if (j < J) {
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+          acc[i].x += W[i].w[j].x * x[b].x;
+          acc[i].y += W[i].w[j].y * x[b].y;
+          acc[i].z += W[i].w[j].z * x[b].z;
+          acc[i].w += W[i].w[j].w * x[b].w;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < T; ++i) out[i] = wsum((acc[i].x + acc[i].y) + (acc[i].z + acc[i].w));
+}
 
 struct Best {
   float v;
@@ -270,6 +323,35 @@ __device__ __forceinline__ bool wait_flag(ctlp ctl, int which, unsigned epoch, u
   }
   asm volatile("" ::: "memory");
   return ok;
+}
+
+// Waits until flag a carries va (returns 1) or flag b carries vb (returns 2); 0 on halt.
+__device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, unsigned vb,
+                                           unsigned* abort_word) {
+  lvup fa = (lvup)&ctl->flag[a];
+  lvup fb = (lvup)&ctl->flag[b];
+  lvup h = (lvup)&ctl->halt;
+  unsigned spins = 0;
+  int r = 0;
+  for (;;) {
+    if (*fa == va) {
+      r = 1;
+      break;
+    }
+    if (*fb == vb) {
+      r = 2;
+      break;
+    }
+    if (*h != 0) break;
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      *h = 1u;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  asm volatile("" ::: "memory");
+  return r;
 }
 
 // ---- service side: poll tagged words ---------------------------------------------------
@@ -342,57 +424,6 @@ __device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp ds
   }
 }
 
-// Same wait for a long vector (N words, a multiple of 128): after the probe the tagged
-// words are copied global -> LDS without passing through registers (1 KiB per
-// request), then this wavefront checks the tags in LDS and writes the payloads to dst.
-// raw needs N * 8 bytes.
-template <int N>
-__device__ __forceinline__ bool dma_poll(const u64* src, unsigned epoch, lfp raw, lfp dst,
-                                         unsigned* abort_word, int probe, lu64p dbg = nullptr) {
-  static_assert(N % 128 == 0, "whole 1 KiB requests");
-  constexpr int NCH = N / 128;
-  const int lane = opaque((int)threadIdx.x) & 63;
-  unsigned spins = 0;
-  int run = probe % (N / 64);
-  typedef const f4 __attribute__((address_space(1)))* g4;
-  const g4 g = (g4)src;
-  unsigned attempts = 0;
-  for (;;) {
-    if (!probe_run(src, run, epoch, abort_word, spins)) return false;
-    if (dbg && lane == 0) {
-      if (attempts == 0) dbg[11] = __builtin_amdgcn_s_memtime();
-      dbg[14] = ++attempts;
-    }
-#pragma unroll 1
-    for (int c = 0; c < NCH; ++c)
-      __builtin_amdgcn_global_load_lds(g + 64 * c + lane,
-                                       (__attribute__((address_space(3))) void*)(raw + 256 * c), 16,
-                                       0, 16 /* sc1: agent scope */);
-    vm_drain();
-    if (dbg && lane == 0) dbg[15] = __builtin_amdgcn_s_memtime();
-    bool bad = false;
-    int bad_run = 0;
-    lf4p r4 = (lf4p)raw;
-    typedef __attribute__((address_space(3))) f2* lf2p;
-    lf2p d2 = (lf2p)dst;
-#pragma unroll 5
-    for (int c = 0; c < NCH; ++c) {
-      const f4 w = r4[64 * c + lane];  // {value, tag, value, tag}: words 2 (64 c + lane), + 1
-      if (__float_as_uint(w.y) != epoch || __float_as_uint(w.w) != epoch) {
-        bad = true;
-        bad_run = 2 * c + (lane >> 5);
-      }
-      d2[64 * c + lane] = f2{w.x, w.z};
-    }
-    if (!__any(bad)) return true;
-    run = next_probe_run(bad, bad_run);
-    if (++spins > kSpinLimit) {
-      PG_ST32(abort_word, 1u);
-      return false;
-    }
-  }
-}
-
 // layer_norm_in_place (src/models/cpu.rs:119-143) of the C = 64 NW values in raw (LDS;
 // this lane's are lane + 64 j), two-pass mean / biased variance, eps inside the sqrt;
 // writes the result to xs (LDS).
@@ -434,6 +465,97 @@ struct Lds {
 };
 constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
 
+// ---- attention item: shared by all eight wavefronts ----------------------------------
+// An item is the keys [k0, k1) of one head (at most 128).  Key k0 + slot + 32 i belongs
+// to slot = 4 wave + (lane >> 4), step i < 4; the 16 lanes of a slot hold 4 dims each.
+constexpr int kAttnSteps = kMaxItemKeys / 32;
+struct KvRegs {
+  f4 k[kAttnSteps], v[kAttnSteps];
+};
+// Requests this wavefront's K and V rows.  Unconditional: keys past the split, and the
+// key `pos` that is not in the cache yet, re-read an older row and are masked / replaced.
+__device__ __forceinline__ void attn_load_kv(KvRegs& r, const float* kc, const float* vc, int h, int P,
+                                             int k0, int pos, int slot, int d4) {
+  gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
+  gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int key = min(k0 + slot + 32 * i, max(pos - 1, 0));
+    r.k[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
+    r.v[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
+  }
+}
+// This wavefront's part of cached_self_attention_into (src/models/gpt2/rust.rs:1662-1741)
+// once q (and the new K/V rows) are in LDS: max, sum of exp and weighted V rows over its
+// keys, written to the control block.  A wavefront without keys writes the neutral element.
+__device__ __forceinline__ void attn_wave_partial(KvRegs& r, ctlp ctl, int k0, int k1, int pos,
+                                                  int wave, int lane) {
+  const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
+  const f4 qv = ((lf4p)&ctl->qs[0])[d4];
+  float sc[kAttnSteps];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int key = k0 + slot + 32 * i;
+    if (key == pos && key < k1) {
+      r.k[i] = ((lf4p)&ctl->kn[0])[d4];
+      r.v[i] = ((lf4p)&ctl->vn[0])[d4];
+    }
+    float sv = (qv.x * r.k[i].x + qv.y * r.k[i].y) + (qv.z * r.k[i].z + qv.w * r.k[i].w);
+    sv = row16_sum(sv);
+    sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
+    sc[i] = (key < k1) ? sv : -INFINITY;
+    mx = fmaxf(mx, sc[i]);
+  }
+  // every lane of a 16-lane row holds the same values: the wave maximum is that of rows
+  mx = fmaxf(fmaxf(lane_get(mx, 0), lane_get(mx, 16)), fmaxf(lane_get(mx, 32), lane_get(mx, 48)));
+  float lsum = 0.0f;
+  f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const float pr = (sc[i] == -INFINITY) ? 0.0f : expf(sc[i] - mx);
+    lsum += pr;
+    acc += pr * r.v[i];
+  }
+#pragma unroll
+  for (int off = 16; off <= 32; off <<= 1) {
+    acc.x += __shfl_xor(acc.x, off, 64);
+    acc.y += __shfl_xor(acc.y, off, 64);
+    acc.z += __shfl_xor(acc.z, off, 64);
+    acc.w += __shfl_xor(acc.w, off, 64);
+  }
+  lsum = (lane_get(lsum, 0) + lane_get(lsum, 16)) + (lane_get(lsum, 32) + lane_get(lsum, 48));
+  if (lane < 16) ((lf4p)&ctl->wacc[wave][0])[lane] = acc;
+  if (lane == 0) {
+    ctl->wm[wave] = mx;
+    ctl->wl[wave] = lsum;
+  }
+}
+
+// ---- this wavefront's share of the 4C tagged words of h ---------------------------------
+// Runs wave + 8 e (64 words each).  Payloads go to dst (LDS); returns 0, or 1 + a run
+// that held a stale word.
+template <int RUNS>
+__device__ __forceinline__ unsigned h_share(const u64* src, unsigned epoch, lfp dst, int wave, int lane) {
+  constexpr int RPW = cdiv(RUNS, 8);
+  u64 v[RPW];
+#pragma unroll
+  for (int e = 0; e < RPW; ++e) {
+    const int run = min(wave + 8 * e, RUNS - 1);
+    v[e] = ld_tagged(src, (unsigned)(run * 64 + lane) * 8u);
+  }
+  unsigned code = 0;
+#pragma unroll
+  for (int e = 0; e < RPW; ++e) {
+    const int run = min(wave + 8 * e, RUNS - 1);
+    if (tag_of(v[e]) != epoch) code = 1u + (unsigned)run;
+    dst[run * 64 + lane] = val_of(v[e]);
+  }
+  // wave-uniform: any lane's stale run will do
+  const unsigned long long m = __ballot(code != 0);
+  return m ? (unsigned)__builtin_amdgcn_readlane((int)code, __builtin_ctzll(m)) : 0u;
+}
+
 // ===================================================================================
 // Service wavefront
 // ===================================================================================
@@ -451,6 +573,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
   int t = 0;
   int stopped = 0;
   unsigned tok = 0;
+  unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
   // a wait gave up: tell the streamers and leave
 #define PG_SERVICE_FAIL()        \
   do {                           \
@@ -504,18 +627,19 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 
       // ================= A: block input -> LN1 -> xsA =================
       {
+        const int ln = opaque(lane);  // per-lane addresses are built here, not hoisted
         float g[NW], b[NW];
 #pragma unroll
         for (int j = 0; j < NW; ++j) {
-          g[j] = gld(w.ln_1_g + lane + 64 * j);
-          b[j] = gld(w.ln_1_b + lane + 64 * j);
+          g[j] = gld_at(w.ln_1_g, (unsigned)ln + 64u * j);
+          b[j] = gld_at(w.ln_1_b, (unsigned)ln + 64u * j);
         }
         if (l == 0) {
           // embedding (rust.rs:966-974)
 #pragma unroll
           for (int j = 0; j < NW; ++j)
-            lds.xraw1[lane + 64 * j] = gld(p.wte + (size_t)tok * C + lane + 64 * j) +
-                                       gld(p.wpe + (size_t)pos * C + lane + 64 * j);
+            lds.xraw1[lane + 64 * j] = gld_at(p.wte + (size_t)tok * C, (unsigned)ln + 64u * j) +
+                                       gld_at(p.wpe + (size_t)pos * C, (unsigned)ln + 64u * j);
         } else {
           if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, l - 1, 5), lds.xraw1, abort_word, wg))
             PG_SERVICE_FAIL();
@@ -528,41 +652,27 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       PG_STAMP(l, 0);
 
       // ================= B: this workgroup's (head, split) items =================
+      // All eight wavefronts work on an item: each loads the K/V rows of its slots as
+      // soon as the item is known; this wavefront waits for q, stages it in LDS, counts
+      // the item in flag[5], and merges the eight partial results.
       const int items = H * ns, n = pos + 1;
       const int per = (n + ns - 1) / ns;
-      const int sub = lane >> 4, d4 = lane & 15;
       const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
 #pragma unroll 1
       for (int item = wg; item < items; item += G) {
         const int h = item / ns, s = item - h * ns;
         const int k0 = s * per, k1 = min(n, k0 + per);
         u64* dst = p.part_t + (size_t)item * 66;
-        if (k0 >= k1) {  // empty split: neutral element of the merge
+        ++bseq;
+        if (k0 >= k1) {  // empty split: neutral element of the merge (the streamers skip it too)
           PG_ST64(dst + lane, pack(epp, 0.0f));
           if (lane == 0) PG_ST64(dst + 64, pack(epp, -INFINITY));
           if (lane == 1) PG_ST64(dst + 65, pack(epp, 0.0f));
           continue;
         }
-        const int nk = k1 - k0;  // <= kMaxItemKeys (the host picks ns >= P / 128)
-        const int groups = (nk + 3) >> 2;
         const bool owns_new = (k1 == n);
-        // K and V rows of the item straight into LDS, four keys per request.  The row
-        // of `pos` is not in the cache yet: it (and rows past the split) re-read an
-        // older row and are replaced / masked below.
-        {
-          gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
-          gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
-#pragma unroll 1
-          for (int i = 0; i < groups; ++i) {
-            const int key = min(k0 + 4 * i + sub, max(pos - 1, 0));
-            __builtin_amdgcn_global_load_lds(
-                Kh + (size_t)key * 16 + d4,
-                (__attribute__((address_space(3))) void*)(lds.kbuf + 256 * i), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(
-                Vh + (size_t)key * 16 + d4,
-                (__attribute__((address_space(3))) void*)(lds.vbuf + 256 * i), 16, 0, 0);
-          }
-        }
+        KvRegs kv;
+        attn_load_kv(kv, kc, vc, h, P, k0, pos, kSW * 4 + (lane >> 4), lane & 15);
         // q of this head, and this token's own K/V rows if the split holds pos
         float qn[3];
         {
@@ -588,71 +698,59 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
               ok = false;
               break;
             }
-            __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_s_sleep(2);
           }
           if (!ok) PG_SERVICE_FAIL();
         }
-        vm_drain();  // the K/V rows have landed in LDS
-        // first credit: the streamers may request their next slice behind this poll
-        if (lane == 0) ctl->flag[5] = epp;
         ctl->qs[lane] = qn[0];
         if (owns_new) {
           // K/V append (rust.rs:1677-1683); written through to memory so that a later
           // token's reader on another XCD cannot miss it in a remote L2
-          lds.kbuf[(pos - k0) * 64 + lane] = qn[1];
-          lds.vbuf[(pos - k0) * 64 + lane] = qn[2];
+          ctl->kn[lane] = qn[1];
+          ctl->vn[lane] = qn[2];
           PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[1]));
           PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[2]));
         }
         lds_fence();
-        const f4 qv = ((lf4p)&ctl->qs[0])[d4];
-        lf4p k4 = (lf4p)lds.kbuf;
-        lf4p v4 = (lf4p)lds.vbuf;
-        float mx = -INFINITY;
-#pragma unroll 1
-        for (int i = 0; i < groups; ++i) {
-          const f4 kr = k4[64 * i + lane];
-          float sv = (qv.x * kr.x + qv.y * kr.y) + (qv.z * kr.z + qv.w * kr.w);
-          sv = row16_sum(sv);
-          sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
-          const int key = k0 + 4 * i + sub;
-          sv = (key < k1) ? sv : -INFINITY;
-          if (d4 == 0) ctl->sc[4 * i + sub] = sv;
-          mx = fmaxf(mx, sv);
+        if (lane == 0) ctl->flag[5] = bseq;
+        attn_wave_partial(kv, ctl, k0, k1, pos, kSW, lane);
+        // the streamers' partials
+        {
+          lvup done = (lvup)&ctl->bdone[min(lane, kSW - 1)];
+          unsigned spins = 0;
+          bool ok = true;
+          for (;;) {
+            if (__all(*done == bseq)) break;
+            if (*halt != 0 || ++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          asm volatile("" ::: "memory");
+          if (!ok) PG_SERVICE_FAIL();
         }
-        mx = wmax(mx);
         lds_fence();
-        float lsum = 0.0f;
-        f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-        for (int i = 0; i < groups; ++i) {
-          const float pr = expf(ctl->sc[4 * i + sub] - mx);  // exp(-inf) = 0 for absent keys
-          lsum += pr;
-          acc += pr * v4[64 * i + lane];
-        }
+        {
+          float M = ctl->wm[0];
 #pragma unroll
-        for (int off = 16; off <= 32; off <<= 1) {
-          acc.x += __shfl_xor(acc.x, off, 64);
-          acc.y += __shfl_xor(acc.y, off, 64);
-          acc.z += __shfl_xor(acc.z, off, 64);
-          acc.w += __shfl_xor(acc.w, off, 64);
+          for (int wv = 1; wv < 8; ++wv) M = fmaxf(M, ctl->wm[wv]);
+          float num = 0.0f, den = 0.0f;
+#pragma unroll
+          for (int wv = 0; wv < 8; ++wv) {
+            const float mw = ctl->wm[wv];
+            const float wq = (mw == -INFINITY) ? 0.0f : expf(mw - M);
+            den += wq * ctl->wl[wv];
+            num += wq * ctl->wacc[wv][lane];
+          }
+          PG_ST64(dst + lane, pack(epp, num));
+          if (lane == 0) PG_ST64(dst + 64, pack(epp, M));
+          if (lane == 1) PG_ST64(dst + 65, pack(epp, den));
         }
-        // every lane of a 16-lane row holds the same lsum: the wave sum is 16 x the total
-        lsum = wsum(lsum) * 0.0625f;
-        if (lane < 16) {
-          PG_ST64(dst + 4 * lane + 0, pack(epp, acc.x));
-          PG_ST64(dst + 4 * lane + 1, pack(epp, acc.y));
-          PG_ST64(dst + 4 * lane + 2, pack(epp, acc.z));
-          PG_ST64(dst + 4 * lane + 3, pack(epp, acc.w));
-        }
-        if (lane == 16) PG_ST64(dst + 64, pack(epp, mx));
-        if (lane == 17) PG_ST64(dst + 65, pack(epp, lsum));
       }
-      // both credits stand from here on (a workgroup without an item raises them now)
-      if (lane == 0) {
-        ctl->flag[5] = epp;
-        ctl->flag[6] = epp;
-      }
+      // the credit of the second attention hop (the streamers request a slice on it)
+      if (lane == 0) ctl->flag[6] = epp;
       PG_STAMP(l, 1);
 
       // ================= B2: the workgroup that took split 0 of a head merges it ====
@@ -661,58 +759,66 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       for (int item = wg; item < items; item += G) {
         const int h = item / ns, s = item - h * ns;
         if (s != 0) continue;
+        // the head's ns partials (66 words each) are one run of tagged words: probe the
+        // last word of every partial, then read them all into LDS (the staging area of
+        // the long vector, idle now) and merge from there
         const u64* src = p.part_t + (size_t)h * ns * 66;
-        float M = -INFINITY, num = 0.0f, den = 0.0f;
-        constexpr int CH = 16;
+        const int nw = ns * 66;
+        lfp stage = lds.xsF;
+        unsigned spins = 0;
+        for (;;) {
+          {
+            const unsigned off = (unsigned)(min(lane, ns - 1) * 66 + 65) * 8u;
+            bool ok = true;
+            for (;;) {
+              const u64 v = ld_tagged(src, off);
+              if (__all(tag_of(v) == epp)) break;
+              if (++spins > kSpinLimit) {
+                PG_ST32(abort_word, 1u);
+                ok = false;
+                break;
+              }
+              if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+                ok = false;
+                break;
+              }
+              __builtin_amdgcn_s_sleep(2);
+            }
+            if (!ok) PG_SERVICE_FAIL();
+          }
+          bool bad = false;
+          constexpr int CH = 12;
 #pragma unroll 1
-        for (int q0 = 0; q0 < ns; q0 += CH) {
-          u64 wa[CH], wm[CH], wl[CH];
-          unsigned spins = 0;
-          bool ok = true;
-          for (;;) {
-            bool bad = false;
+          for (int e0 = 0; e0 * 64 < nw; e0 += CH) {
+            u64 v[CH];
 #pragma unroll
-            for (int q = 0; q < CH; ++q) {
-              const unsigned qq = (unsigned)min(q0 + q, ns - 1) * 66u;
-              wa[q] = ld_tagged(src, (qq + (unsigned)lane) * 8u);
-              wm[q] = ld_tagged(src, (qq + 64u) * 8u);
-              wl[q] = ld_tagged(src, (qq + 65u) * 8u);
-            }
+            for (int e = 0; e < CH; ++e)
+              v[e] = ld_tagged(src, (unsigned)min(lane + 64 * (e0 + e), nw - 1) * 8u);
 #pragma unroll
-            for (int q = 0; q < CH; ++q)
-              bad = bad || tag_of(wa[q]) != epp || tag_of(wm[q]) != epp || tag_of(wl[q]) != epp;
-            if (!__any(bad)) break;
-            if (++spins > kSpinLimit) {
-              PG_ST32(abort_word, 1u);
-              ok = false;
-              break;
-            }
-            if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
-              ok = false;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-          }
-          if (!ok) PG_SERVICE_FAIL();
-          // online merge of this chunk of splits (neutral: m = -inf, l = 0, acc = 0)
-          float Mc = M;
-#pragma unroll
-          for (int q = 0; q < CH; ++q)
-            if (q0 + q < ns) Mc = fmaxf(Mc, val_of(wm[q]));
-          const float scale = (M == -INFINITY) ? 0.0f : expf(M - Mc);
-          num *= scale;
-          den *= scale;
-#pragma unroll
-          for (int q = 0; q < CH; ++q) {
-            if (q0 + q < ns) {
-              const float wq = expf(val_of(wm[q]) - Mc);
-              den += wq * val_of(wl[q]);
-              num += wq * val_of(wa[q]);
+            for (int e = 0; e < CH; ++e) {
+              bad = bad || (tag_of(v[e]) != epp);
+              stage[min(lane + 64 * (e0 + e), nw - 1)] = val_of(v[e]);
             }
           }
-          M = Mc;
+          if (!__any(bad)) break;
+          if (++spins > kSpinLimit) {
+            PG_ST32(abort_word, 1u);
+            PG_SERVICE_FAIL();
+          }
         }
-          PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
+        lds_fence();
+        float M = -INFINITY;
+#pragma unroll 1
+        for (int q = 0; q < ns; ++q) M = fmaxf(M, stage[q * 66 + 64]);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll 1
+        for (int q = 0; q < ns; ++q) {
+          const float mq = stage[q * 66 + 64];
+          const float wq = (mq == -INFINITY) ? 0.0f : expf(mq - M);
+          den += wq * stage[q * 66 + 65];
+          num += wq * stage[q * 66 + lane];
+        }
+        PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
       }
 
       // ================= D: attention output -> xsD =================
@@ -725,11 +831,12 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 
       // ================= E: xa -> xraw2, LN2 -> xsE =================
       {
+        const int ln = opaque(lane);
         float g[NW], b[NW];
 #pragma unroll
         for (int j = 0; j < NW; ++j) {
-          g[j] = gld(w.ln_2_g + lane + 64 * j);
-          b[j] = gld(w.ln_2_b + lane + 64 * j);
+          g[j] = gld_at(w.ln_2_g, (unsigned)ln + 64u * j);
+          b[j] = gld_at(w.ln_2_b, (unsigned)ln + 64u * j);
         }
         const unsigned ep = epoch_of(p, t, l, 3);
         if (!wave_poll<NW>(p.xa_t, ep, lds.xraw2, abort_word, wg + 2,
@@ -743,13 +850,38 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       PG_STAMP(l, 3);
 
       // ================= F: h -> xsF =================
-      // 4C tagged words are too many for one wavefront's registers: they are copied
-      // straight into LDS (the K/V staging area, idle now), then checked and compacted.
+      // 4C tagged words: after the cheap probe all eight wavefronts read a share each
+      // (flag[7] counts the rounds); a stale word sends the probe to its run and the
+      // round is repeated.
       {
+        constexpr int RUNS = I / 64;
         const unsigned ep = epoch_of(p, t, l, 4);
-        if (!dma_poll<I>(p.h_t, ep, lds.kbuf, lds.xsF, abort_word, wg + 3,
-                         (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 : (lu64p) nullptr)) {
-          PG_SERVICE_FAIL();
+        int run = (wg + 3) % RUNS;
+        unsigned spins = 0;
+        for (;;) {
+          if (!probe_run(p.h_t, run, ep, abort_word, spins)) PG_SERVICE_FAIL();
+          ++hseq;
+          if (lane == 0) ctl->flag[7] = hseq;
+          unsigned code = h_share<RUNS>(p.h_t, ep, lds.xsF, kSW, lane);
+          lvup st = (lvup)&ctl->hstat[min(lane, kSW - 1)];
+          bool ok = true;
+          unsigned v = 0;
+          for (;;) {
+            v = *st;
+            if (__all((v >> 8) == hseq)) break;
+            if (*halt != 0 || ++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          asm volatile("" ::: "memory");
+          if (!ok) PG_SERVICE_FAIL();
+          const unsigned mine = (lane < kSW) ? (v & 0xffu) : code;
+          const unsigned long long m = __ballot(mine != 0);
+          if (m == 0) break;
+          run = __builtin_amdgcn_readlane((int)mine, __builtin_ctzll(m)) - 1;
         }
         lds_fence();
         if (lane == 0) ctl->flag[3] = ep;
@@ -759,11 +891,12 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 
     // ================= LN_f -> xsD, then this workgroup's argmax =================
     if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      const int ln = opaque(lane);
       float g[NW], b[NW];
 #pragma unroll
       for (int j = 0; j < NW; ++j) {
-        g[j] = gld(p.ln_f_g + lane + 64 * j);
-        b[j] = gld(p.ln_f_b + lane + 64 * j);
+        g[j] = gld_at(p.ln_f_g, (unsigned)ln + 64u * j);
+        b[j] = gld_at(p.ln_f_b, (unsigned)ln + 64u * j);
       }
       const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
       // staged in xraw1 (the next user is the next token's embedding)
@@ -905,36 +1038,39 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
   auto row_of = [&](int r0, int r1, int i) { return min(r0 + wave_id() + kSW * i, r1 - 1); };
 
   Tile<J> WA[TA];  // c_attn rows of the layer about to run
-  Tile<J> WD;      // c_proj row
+  Tile<J> WD[1];   // c_proj row
   Tile<J> WE[TE];  // c_fc rows
   Tile<JF> WF;     // mlp projection row
 
   // One float4 of a C-wide row: column block j (columns past the row re-read its last
   // float4 and meet a zero in x).  Unconditional, like every load here: a load under a
   // branch would make the compiler lose count of the loads in flight.
-  auto ld_c = [&](const float* W, int row, int j) -> f4 {
-    const unsigned c = (64 * (j + 1) <= K4) ? (unsigned)lane + 64u * j
-                                            : (unsigned)min(lane + 64 * j, K4 - 1);
+  auto ld_c = [&](const float* W, int row, int j, int ln) -> f4 {
+    const unsigned c = (64 * (j + 1) <= K4) ? (unsigned)ln + 64u * j
+                                            : (unsigned)min(ln + 64 * j, K4 - 1);
     return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * K4, c * 16u);
   };
   // Requests loads [N0, N1) of the layer stream: `w` is the layer whose c_proj, c_fc and
   // mlp projection rows are meant, `wn` the one whose c_attn rows follow.
   auto issue = [&](auto n0_, auto n1_, const LayerW& w, const LayerW& wn) {
     constexpr int N0 = decltype(n0_)::value, N1 = decltype(n1_)::value;
+    // the lane index behind an empty asm again: the per-lane parts of the addresses are
+    // rebuilt for each slice instead of being kept (and spilled) across the whole layer
+    const int ln = opaque(lane);
 #pragma unroll
     for (int n = N0; n < N1; ++n) {
       if (n < SP::ND) {
-        WD.w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n);
+        WD[0].w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n, ln);
       } else if (n < SP::ND + SP::NE) {
         const int i = (n - SP::ND) / J, j = (n - SP::ND) % J;
-        WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j);
+        WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
       } else if (n < SP::ND + SP::NE + SP::NF) {
         const int j = n - SP::ND - SP::NE;
         WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
-                         ((unsigned)lane + 64u * j) * 16u);
+                         ((unsigned)ln + 64u * j) * 16u);
       } else {
         const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
-        WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j);
+        WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
       }
     }
   };
@@ -956,6 +1092,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       lds.ts[l * 16 + (slot)] = __builtin_amdgcn_s_memtime();                          \
   } while (0)
   bool ok = true;
+  unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
   for (int t = 0; t < p.n_fwd && ok; ++t) {
     for (int l = 0; l < p.L; ++l) {
       const LayerW w = layer_of(p.layers, l);
@@ -976,21 +1113,39 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       // the service wavefront has just completed a poll and its next ones are early)
       PG_SLICE(0, w, wn);
       {
-        f4 xr[J];
-        load_x<J>(xr, lds.xsA, K4, lane);
+        float v[TA];
+        dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 0);
 #pragma unroll
         for (int i = 0; i < TA; ++i) {
           const int r = a0 + wave + kSW * i;
-          const float v = dot_tile<J>(WA[i], xr);
-          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, biasA[i] + v));
+          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, biasA[i] + v[i]));
         }
       }
       SSTAMP(5);
-      // ---- the two attention hops: nothing to compute, one slice each ----
-      if (!wait_flag(ctl, 5, epoch_of(p, t, l, 1), abort_word)) {
-        ok = false;
-        break;
+      // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
+      {
+        const int H = p.H, P = p.P, ns = p.ns, pos = p.pos0 + t;
+        const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
+        const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
+        const float* vc = kc + p.kv_v_offset;
+#pragma unroll 1
+        for (int item = wg; item < items; item += G) {
+          const int h = item / ns, sp = item - h * ns;
+          const int k0 = sp * per, k1 = min(n, k0 + per);
+          ++bseq;
+          if (k0 >= k1) continue;
+          KvRegs kv;
+          attn_load_kv(kv, kc, vc, h, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
+          if (!wait_flag(ctl, 5, bseq, abort_word)) {
+            ok = false;
+            break;
+          }
+          attn_wave_partial(kv, ctl, k0, k1, pos, wave, lane);
+          lds_fence();
+          if (lane == 0) ctl->bdone[wave] = bseq;
+        }
+        if (!ok) break;
       }
       PG_SLICE(1, w, wn);
       if (!wait_flag(ctl, 6, epoch_of(p, t, l, 1), abort_word)) {
@@ -1006,11 +1161,10 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         break;
       }
       {
-        f4 xr[J];
-        load_x<J>(xr, lds.xsD, K4, lane);
+        float v[1];
+        dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
         const int r = d0 + wave;
-        const float v = dot_tile<J>(WD, xr);
-        if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v)));
+        if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v[0])));
       }
       PG_SLICE(3, w, wn);
 
@@ -1023,25 +1177,37 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         break;
       }
       {
-        f4 xr[J];
-        load_x<J>(xr, lds.xsE, K4, lane);
+        float v[TE];
+        dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 4);
+        // lane i finishes row i: one GELU and one store for all of the wavefront's rows
+        float mine = 0.0f;
+        int r = e1;
 #pragma unroll
-        for (int i = 0; i < TE; ++i) {
-          const int r = e0 + wave + kSW * i;
-          const float v = dot_tile<J>(WE[i], xr);
-          if (lane == 0 && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(biasE[i] + v)));
-        }
+        for (int i = 0; i < TE; ++i)
+          if (lane == i) {
+            mine = biasE[i] + v[i];
+            r = e0 + wave + kSW * i;
+          }
+        if (lane < TE && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(mine)));
       }
       SSTAMP(6);
       PG_SLICE(4, w, wn);
 
       // ================= F: mlp projection row + residual =================
       const float biasF = cld(w.c_proj_mlp_b + row_of(d0, d1, 0));
-      if (!wait_flag(ctl, 3, epoch_of(p, t, l, 4), abort_word)) {
-        ok = false;
-        break;
+      // rounds of reading this wavefront's share of h, until the service wavefront has
+      // seen a complete one
+      for (;;) {
+        const int r = wait_either(ctl, 3, epoch_of(p, t, l, 4), 7, hseq + 1, abort_word);
+        if (r == 0) ok = false;
+        if (r != 2) break;
+        ++hseq;
+        const unsigned code = h_share<I / 64>(p.h_t, epoch_of(p, t, l, 4), lds.xsF, wave, lane);
+        lds_fence();
+        if (lane == 0) ctl->hstat[wave] = (hseq << 8) | code;
       }
+      if (!ok) break;
       SSTAMP(10);
       if (p.prof) {  // development: how long the row's last loads are still in flight
         vm_drain();
@@ -1150,6 +1316,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_ws(DecodeParams p) {
   if (threadIdx.x < 8) {
     ctl->flag[threadIdx.x] = 0u;
     ctl->lmdone[threadIdx.x] = 0u;
+    ctl->bdone[threadIdx.x] = 0u;
+    ctl->hstat[threadIdx.x] = 0u;
   }
   if (threadIdx.x == 0) ctl->halt = 0u;
   __syncthreads();
