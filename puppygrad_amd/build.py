@@ -9,7 +9,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libpuppygrad_hip.so"
-SOURCES = ["pg_kernels.hip", "pg_decode.hip", "pg_decode_ws.hip", "pg_prefill.hip", "pg_host.cpp"]
+SOURCES = ["pg_kernels.hip", "pg_decode.hip", "pg_prefill.hip", "pg_host.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-FP32 instruction selection is switched off for every device pass.
@@ -26,7 +26,7 @@ def build_library(verbose: bool = True) -> Path:
             continue
         obj = CSRC / (path.stem + ".o")
         cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
-               *DEVICE_FLAGS, *os.environ.get("PG_EXTRA_FLAGS", "").split(), "-Wno-unused-command-line-argument", "-c", str(path), "-o", str(obj)]
+               *DEVICE_FLAGS, "-Wno-unused-command-line-argument", "-c", str(path), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))

@@ -1,20 +1,27 @@
-// Persistent batch-1 decode kernel for gfx950: one launch runs whole cached
-// decoder steps (forward_one_profiled_with_scratch, src/models/gpt2/rust.rs:943-1006,
-// block at 1136-1250, attention at 1662-1741) for one or many greedy tokens.
+// Wave-specialised persistent batch-1 decode kernel for gfx950: one launch runs whole
+// cached decoder steps (forward_one_profiled_with_scratch,
+// src/models/gpt2/rust.rs:943-1006, block at 1136-1250, attention at 1662-1741) for
+// one or many greedy tokens.
 //
-// Design.  256 workgroups (one per CU) each own a contiguous band of rows of every
-// weight matrix and stream it exactly once per token with nontemporal 16-byte
-// loads.  Workgroups never meet at a grid barrier.  Every activation that crosses
-// workgroups is stored as a 64-bit word {epoch, f32 bits} with one agent-scope
-// atomic store; a consumer polls the words it needs until they carry the epoch of
-// the producing (token, layer, phase).  Weight addresses do not depend on data, so
-// the whole band of the NEXT matrix is requested into registers before the current
-// phase starts waiting: HBM keeps streaming while the dependency chain catches up.
+// 256 workgroups of 8 wavefronts, one workgroup per CU, never a grid barrier.  Every
+// activation that crosses workgroups is a 64-bit word {epoch, f32 bits} written with
+// one agent-scope store; a reader polls until the word carries the epoch of the
+// producing (token, layer, phase).
 //
-// A band is treated as a flat array of float4: thread t holds elements
-// t, t+512, t+1024, ...  A wavefront's 64 consecutive float4 lie in at most two
-// rows, so one (or two) DPP wave reductions per 1 KiB give per-chunk partial sums,
-// which are added per row in a fixed order (results do not depend on timing).
+// Vector memory loads of one wavefront return in issue order, so a wavefront that
+// polls global memory behind a prefetch of weights sees the answer only after the
+// weights have landed, and a wavefront that holds prefetched weights must not poll.
+// The roles are therefore split:
+//
+//   * wavefronts 0..6 ("streamers") own the rows of every weight matrix of this
+//     workgroup's band.  They only ever wait on flags in LDS, keep up to two weight
+//     bands in flight in their registers (the band in use and the next one or two,
+//     requested in consumption order as soon as registers free up), multiply and
+//     publish their rows.
+//   * wavefront 7 ("service") owns the dependency chain: it polls the tagged words,
+//     applies LayerNorm, stages the input vector of the next matrix in LDS and raises
+//     the LDS flag; it also runs this workgroup's (head, key-split) attention item,
+//     the per-head merge, the embedding and the argmax merge.
 //
 // Per layer:  A  LN1 + c_attn rows            -> qkv_t   (tagged)
 //             B  split-key attention per head -> part_t  (tagged partial acc, m, l)
@@ -24,31 +31,40 @@
 //             F  mlp c_proj rows + residual   -> xm_t    (tagged)
 // then LN_f + lm_head rows -> logits (plain) and per-workgroup argmax -> best_t.
 //
-// Every wait is bounded: a poll that does not complete within kSpinLimit sets
-// the abort word, which every other poll observes, and all waves leave the kernel.
+// Every wait is bounded: a poll that does not complete within its spin limit sets
+// the abort word (global) and the halt word (LDS); every other wait observes one of
+// them and all wavefronts leave the kernel.
 #include "pg_kernels.h"
 
 #include <math.h>
+
+#include <type_traits>
 
 namespace pgk {
 
 namespace {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
 typedef unsigned long long u64;
 
 constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 
 constexpr int kThreads = 512;
-constexpr int kWavesP = kThreads / 64;
+constexpr int kSW = 7;      // streamer wavefronts (0..6); wavefront 7 is the service wavefront
 constexpr int kGrid = 256;  // workgroups; row bands are computed for exactly this many
 constexpr unsigned kSpinLimit = 1u << 21;
-constexpr int kAttnSteps = 4;  // up to 4*32 = 128 keys per (head, split) item
+constexpr int kMaxItemKeys = 128;  // keys per (head, split) attention item
+constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
 
-#define PG_LD64(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define PG_ST64(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define PG_LD32(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define PG_ST32(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+// Tagged words and the abort word live in global memory; saying so in the pointer type
+// gets global_ instead of flat_ instructions (a flat access also counts as an LDS one).
+#define PG_G64(p) ((__attribute__((address_space(1))) unsigned long long*)(p))
+#define PG_G32(p) ((__attribute__((address_space(1))) unsigned*)(p))
+#define PG_LD64(p) __hip_atomic_load(PG_G64(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_ST64(p, v) __hip_atomic_store(PG_G64(p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_LD32(p) __hip_atomic_load(PG_G32(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define PG_ST32(p, v) __hip_atomic_store(PG_G32(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
 __device__ __forceinline__ u64 pack(unsigned epoch, float v) {
   return ((u64)epoch << 32) | (u64)__float_as_uint(v);
@@ -70,14 +86,13 @@ __device__ __forceinline__ float row16_sum(float v) {
   v += dpp_get<0x140>(v);  // row_mirror
   return v;
 }
+__device__ __forceinline__ float lane_get(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
 // Sum over the wavefront; the result is wave-uniform.
 __device__ __forceinline__ float wsum(float v) {
   v = row16_sum(v);
-  float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-  float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-  float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-  float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-  return (r0 + r1) + (r2 + r3);
+  return (lane_get(v, 0) + lane_get(v, 16)) + (lane_get(v, 32) + lane_get(v, 48));
 }
 __device__ __forceinline__ float wmax(float v) {
 #pragma unroll
@@ -85,255 +100,127 @@ __device__ __forceinline__ float wmax(float v) {
   return v;
 }
 
-struct Smem {
-  float red[2][kWavesP];  // alternating buffers: consecutive reductions need one barrier each
-  float accs[kWavesP][64];
-  float qs[64], kn[64], vn[64];
-  float psum[64];  // phase F: partial sums of the (row, quarter) tiles
-  float bestv[kWavesP];
-  unsigned besti[kWavesP];
-  int ok;
-  unsigned tok;
-};
-
-// Block reductions with ONE barrier each.  Two calls in a row must use different
-// buffers (B = 0, 1); a buffer may be reused once another barrier has passed.
-template <int B>
-__device__ __forceinline__ float bsum(float v, Smem& sm) {
-  v = wsum(v);
-  if ((threadIdx.x & 63) == 0) sm.red[B][threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = 0.0f;
-#pragma unroll
-  for (int w = 0; w < kWavesP; ++w) t += sm.red[B][w];
-  return t;
-}
-template <int B>
-__device__ __forceinline__ float bmax(float v, Smem& sm) {
-  v = wmax(v);
-  if ((threadIdx.x & 63) == 0) sm.red[B][threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = sm.red[B][0];
-#pragma unroll
-  for (int w = 1; w < kWavesP; ++w) t = fmaxf(t, sm.red[B][w]);
-  return t;
-}
-
 __device__ __forceinline__ float gelu_tanh(float x) {
   return 0.5f * x * (1.0f + tanhf(0.7978846f * (x + 0.044715f * x * x * x)));
 }
 
-// threadIdx.x behind an empty asm: index arithmetic built on it is recomputed where
-// it is used instead of being hoisted out of the token/layer loops (dozens of
-// loop-invariant 64-bit addresses would otherwise be kept alive and spilled).
-__device__ __forceinline__ int local_tid() {
-  int t = (int)threadIdx.x;
-  asm volatile("" : "+v"(t));
-  return t;
-}
-
-// Waits until src[i] carries `epoch` for every i in [0, n) that this thread owns
-// (i = tid + 512*e), then writes the payloads to dst (LDS).  NE bounds the
-// elements per thread.  Returns false on timeout or external abort.  All loads of
-// a round are issued before any is checked.
-template <int NE>
-__device__ __forceinline__ bool poll_vec(const u64* src, int n, unsigned epoch, float* dst,
-                                         unsigned* abort_word) {
-  u64 v[NE];
-  const int tid = local_tid();
-#pragma unroll
-  for (int e = 0; e < NE; ++e) {
-    // out-of-range slots re-read the last word: every load is unconditional, so the
-    // compiler can count outstanding loads exactly and never waits for younger ones
-    int i = min(tid + kThreads * e, n - 1);
-    v[e] = PG_LD64(src + i);
-  }
-  unsigned spins = 0;
-  bool good = true;
-  for (;;) {
-    bool bad = false;
-#pragma unroll
-    for (int e = 0; e < NE; ++e) {
-      if (tag_of(v[e]) != epoch) {
-        v[e] = PG_LD64(src + min(tid + kThreads * e, n - 1));
-        bad = bad || (tag_of(v[e]) != epoch);
-      }
-    }
-    if (!bad) break;
-    if (++spins > kSpinLimit) {
-      good = false;
-      PG_ST32(abort_word, 1u);
-      break;
-    }
-    if ((spins & 63) == 0 && PG_LD32(abort_word) != 0) {
-      good = false;
-      break;
-    }
-    __builtin_amdgcn_s_sleep(1);
-  }
-#pragma unroll
-  for (int e = 0; e < NE; ++e) {
-    int i = tid + kThreads * e;
-    if (i < n) dst[i] = val_of(v[e]);
-  }
-  return good;
-}
-
-// Makes a per-thread success flag uniform over the workgroup (also a barrier
-// that publishes LDS written by poll_vec).
-// sm.ok starts at 1 and is only ever cleared, so one barrier suffices.
-__device__ __forceinline__ bool all_ok(bool mine, Smem& sm) {
-  if (!mine) sm.ok = 0;
-  __syncthreads();
-  return sm.ok != 0;
-}
-
-// LayerNorm scale/shift of this thread's elements (i = tid + 512*e), fetched ahead
-// of time: a load issued after a weight band would only return behind the band.
-template <int NE>
-struct LnParams {
-  float g[NE], b[NE];
+// Control block in LDS.
+struct Ctl {
+  unsigned flag[8];    // [0] A, [1] D, [2] E, [3] F, [4] lm_head: epoch whose input is staged;
+                       // [5] attention item staged (running count), [6] credit of the
+                       // second attention hop (epoch), [7] "read your share of h" (running count)
+  unsigned halt;       // 0 run, 1 a wait gave up, 2 stopped at the EOS token
+  unsigned lmdone[8];  // per streamer: epoch of its finished lm_head band
+  unsigned bdone[8];   // per wavefront: count of the attention item whose partial it has written
+  unsigned hstat[8];   // per wavefront: (count << 8) | (1 + a stale run, or 0) of its share of h
+  float bestv[8];
+  unsigned besti[8];
+  float wm[8], wl[8];  // attention partials of the wavefronts: max, sum of weights ...
+  __attribute__((aligned(16))) float wacc[8][64];  // ... and weighted V rows
+  __attribute__((aligned(16))) float qs[64];       // q, and this token's K and V rows of the head
+  __attribute__((aligned(16))) float kn[64];
+  __attribute__((aligned(16))) float vn[64];
 };
-template <int NE>
-__device__ __forceinline__ void ln_fetch(LnParams<NE>& q, const float* g, const float* b, int C) {
-  const int tid = local_tid();
-#pragma unroll
-  for (int e = 0; e < NE; ++e) {
-    int i = min(tid + kThreads * e, C - 1);  // unconditional loads (see poll_vec)
-    q.g[e] = g[i];
-    q.b[e] = b[i];
-  }
-}
-// layer_norm_in_place (src/models/cpu.rs:119-143): raw -> xs, both in LDS; two-pass
-// mean / biased variance, eps inside the sqrt.  Every wavefront reduces the whole
-// vector on its own (C/64 LDS reads per lane, DPP sums): no block barrier is
-// needed for the statistics, only one at the end to publish xs.
-template <int NE, int C>
-__device__ __forceinline__ void ln_lds(const float* raw, float* xs, const LnParams<NE>& q,
-                                       float eps) {
-  constexpr int NW = cdiv(C, 64);
-  const int tid = local_tid();
-  const int lane = tid & 63;
-  float x[NW];
-  float s = 0.0f;
-#pragma unroll
-  for (int j = 0; j < NW; ++j) {
-    const int i = lane + 64 * j;
-    x[j] = raw[min(i, C - 1)];
-    if (i >= C) x[j] = 0.0f;
-    s += x[j];
-  }
-  const float mean = wsum(s) / (float)C;
-  float v = 0.0f;
-#pragma unroll
-  for (int j = 0; j < NW; ++j) {
-    const float d = (lane + 64 * j < C) ? x[j] - mean : 0.0f;
-    v += d * d;
-  }
-  const float var = wsum(v) / (float)C;
-  const float inv = 1.0f / sqrtf(var + eps);
-#pragma unroll
-  for (int e = 0; e < NE; ++e) {
-    const int i = tid + kThreads * e;
-    if (i < C) xs[i] = (raw[i] - mean) * inv * q.g[e] + q.b[e];
-  }
-  __syncthreads();
+typedef __attribute__((address_space(3))) Ctl* ctlp;
+
+// Orders this wavefront's LDS accesses (and keeps the compiler from moving memory
+// accesses across): LDS executes a wavefront's operations in order, so a flag
+// written after this point is seen no earlier than the data written before it.
+__device__ __forceinline__ void lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void vm_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// The lane and wave index behind an empty asm: index arithmetic built on them is
+// recomputed where it is used instead of being hoisted out of the token/layer loops
+// (dozens of loop-invariant 64-bit addresses would otherwise be kept alive).
+__device__ __forceinline__ int opaque(int v) {
+  asm volatile("" : "+v"(v));
+  return v;
 }
 
 // Weight pointers come out of a table in memory; telling the compiler they are
 // global (not generic) addresses gets global_load instead of flat_load.
 typedef const f4 __attribute__((address_space(1)))* gf4p;
 __device__ __forceinline__ gf4p as_global(const f4* p) { return (gf4p)p; }
-
-// ---- flat band streaming -------------------------------------------------------
-
-// Requests this thread's share of a band of n4 >= 1 float4 starting at base:
-// elements tid + 512*u.  Loads are unconditional (indices past the end re-read the
-// last element and are never summed): a load under a branch would make the
-// compiler lose count of outstanding loads and wait for ALL of them at the next
-// use of any older one, which serialises the phase behind the band just requested.
-template <int U, int LO = 0, int HI = U>
-__device__ __forceinline__ void band_load(f4 (&w)[U], const f4* base, int n4) {
-  gf4p g = as_global(base);
-  const int tid = local_tid();
-#pragma unroll
-  for (int u = LO; u < HI; ++u) {
-    int f = min(tid + kThreads * u, n4 - 1);
-    w[u] = __builtin_nontemporal_load(g + f);
-  }
+__device__ __forceinline__ float gld(const float* p) {
+  return *(const float __attribute__((address_space(1)))*)p;
 }
-
-// Stage 1 of a band product: every thread multiplies its float4 of the band with
-// the matching float4 of the vector xs (LDS; rows are K4 float4 long) and leaves
-// the scalar product of flat element f in prod[f] (LDS).  About ten instructions
-// per float4: the per-CU instruction issue rate, not HBM, bounds this part.
-template <int U, int K4>
-__device__ __forceinline__ void band_mul(const f4 (&w)[U], const float* xs, float* prod) {
-  const f4* x4 = reinterpret_cast<const f4*>(xs);
-  const int tid = local_tid();
-  constexpr int B = 5;  // LDS reads kept in flight together
-#pragma unroll
-  for (int u0 = 0; u0 < U; u0 += B) {
-    f4 x[B];
-#pragma unroll
-    for (int b = 0; b < B; ++b)
-      if (u0 + b < U) x[b] = x4[(tid + kThreads * (u0 + b)) % K4];
-#pragma unroll
-    for (int b = 0; b < B; ++b)
-      if (u0 + b < U) {
-        const int u = u0 + b;
-        prod[tid + kThreads * u] =
-            (w[u].x * x[b].x + w[u].y * x[b].y) + (w[u].z * x[b].z + w[u].w * x[b].w);
-      }
-  }
+// element i of a wave-uniform array: the base stays scalar, the lane's part is a 32-bit
+// byte offset
+__device__ __forceinline__ float gld_at(const float* base, unsigned i) {
+  typedef const char __attribute__((address_space(1)))* gcp;
+  return *(const float __attribute__((address_space(1)))*)((gcp)base + i * 4u);
 }
-
-// Stage 2: LPR lanes add up the K4 products of one row in a fixed order (lane s
-// takes s, s+LPR, ...; then a DPP tree), so the result does not depend on timing.
-// Returns the row sum on every lane of the group; `row` must be < rows for the
-// value to be meaningful.  All lanes execute it (the DPP tree needs them active).
-template <int K4, int LPR>
-__device__ __forceinline__ float band_row(const float* prod, int row, int rows) {
-  static_assert(LPR == 16 || LPR == 64, "a row is summed by a DPP row or a whole wavefront");
-  constexpr int N = cdiv(K4, LPR);
-  const int sub = local_tid() & (LPR - 1);
-  const float* src = prod + (size_t)min(row, rows - 1) * K4;
-  float v[N];
-#pragma unroll
-  for (int j = 0; j < N; ++j) {
-    const int k = sub + LPR * j;
-    v[j] = src[min(k, K4 - 1)];
-    if (k >= K4) v[j] = 0.0f;
-  }
-  float s = 0.0f;
-#pragma unroll
-  for (int j = 0; j < N; ++j) s += v[j];
-  return LPR == 16 ? row16_sum(s) : wsum(s);
+// Read-only tables written by the host before the launch (layer table, biases) are
+// read through the constant address space: wave-uniform addresses then become scalar
+// loads, which do not queue behind the vector loads of the weight rows.
+__device__ __forceinline__ float cld(const float* p) {
+  return *(const float __attribute__((address_space(4)))*)p;
 }
+__device__ __forceinline__ LayerW layer_of(const LayerW* table, int l) {
+  typedef const unsigned long long __attribute__((address_space(4)))* cq;
+  constexpr int NQ = sizeof(LayerW) / 8;
+  static_assert(sizeof(LayerW) % 8 == 0, "a table of pointers");
+  const cq src = (cq)(table + l);
+  union {
+    LayerW w;
+    unsigned long long q[NQ];
+  } u;
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) u.q[i] = src[i];
+  return u.w;
+}
+__device__ __forceinline__ void gst(float* p, float v) {
+  *(float __attribute__((address_space(1)))*)p = v;
+}
+__device__ __forceinline__ void gst_u(unsigned* p, unsigned v) {
+  *(unsigned __attribute__((address_space(1)))*)p = v;
+}
+__device__ __forceinline__ void gst_u64(u64* p, u64 v) {
+  *(u64 __attribute__((address_space(1)))*)p = v;
+}
+// LDS pointers keep their address space in the type: every access is a ds_ instruction
+// and never a flat one that would count as a vector memory operation.
+typedef __attribute__((address_space(3))) float* lfp;
+typedef __attribute__((address_space(3))) f4* lf4p;
+typedef volatile __attribute__((address_space(3))) unsigned* lvup;
+typedef __attribute__((address_space(3))) unsigned long long* lu64p;
 
-// ---- row tiles for the long lm_head band -----------------------------------------
-
+// One tile = one weight row (or a run of 64*J float4 of one), 64 lanes wide, J deep.
 template <int J>
 struct Tile {
   f4 w[J];
 };
-// One tile = one weight row, 64 lanes wide, J deep; defined on every path.
-template <int J>
-__device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
-  gf4p g = as_global(p);
-#pragma unroll
-  for (int j = 0; j < J; ++j) {
-    int c = min(lane + 64 * j, K4s - 1);  // unconditional; load_x zeroes the matching x
-    t.w[j] = __builtin_nontemporal_load(g + c);
-  }
+// Loads are unconditional (columns past the row re-read its last float4 and meet a
+// zero in x): a load under a branch would make the compiler lose count of the loads
+// in flight and wait for all of them at the next use of an older one.
+// The row address is wave-uniform (scalar registers); the lane's part is a 32-bit byte
+// offset, so that the loads take the "scalar base + vector offset" form and no 64-bit
+// per-lane addresses have to be kept.
+__device__ __forceinline__ f4 ld_row(const f4* row, unsigned byte_off) {
+  typedef const char __attribute__((address_space(1)))* gcp;
+  return __builtin_nontemporal_load((gf4p)((gcp)row + byte_off));
 }
 template <int J>
-__device__ __forceinline__ void load_x(f4* xr, const float* xs, int K4s, int lane) {
-  const f4* x4 = reinterpret_cast<const f4*>(xs);
+__device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const unsigned c = (64 * (j + 1) <= K4s) ? (unsigned)lane + 64u * j
+                                              : (unsigned)min(lane + 64 * j, K4s - 1);
+    t.w[j] = ld_row(p, c * 16u);
+  }
+}
+template <int J, int LO, int HI>
+__device__ __forceinline__ void load_tile_part(Tile<J>& t, const f4* p, int lane) {
+#pragma unroll
+  for (int j = LO; j < HI; ++j) t.w[j] = ld_row(p, ((unsigned)lane + 64u * j) * 16u);
+}
+template <int J>
+__device__ __forceinline__ void load_x(f4* xr, lfp xs, int K4s, int lane) {
+  lf4p x4 = (lf4p)xs;
 #pragma unroll
   for (int j = 0; j < J; ++j) {
     int c = lane + 64 * j;
-    xr[j] = (j < J - 1 || c < K4s) ? x4[c] : f4{0.f, 0.f, 0.f, 0.f};
+    xr[j] = (64 * (j + 1) <= K4s || c < K4s) ? x4[min(c, K4s - 1)] : f4{0.f, 0.f, 0.f, 0.f};
   }
 }
 template <int J>
@@ -348,6 +235,47 @@ __device__ __forceinline__ float dot_tile(const Tile<J>& t, const f4* xr) {
   }
   return wsum((a0 + a1) + (a2 + a3));
 }
+// The same products for T rows at once with the input vector read from LDS column block
+// by column block (two in flight) instead of being held in registers for the whole
+// phase: same order of additions per row as dot_tile.
+template <int T, int J>
+__device__ __forceinline__ void dot_tiles(const Tile<J> (&W)[T], lfp xs, int K4s, int lane,
+                                          float (&out)[T]) {
+  lf4p x4 = (lf4p)xs;
+  f4 acc[T];
+#pragma unroll
+  for (int i = 0; i < T; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+  constexpr int B = 2;
+#pragma unroll
+  for (int j0 = 0; j0 < J; j0 += B) {
+    f4 x[B];
+    // keeps the LDS reads of later column blocks from being moved up here
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int j = j0 + b;
+      if (j < J) {
+        const int c = lane + 64 * j;
+        x[b] = (64 * (j + 1) <= K4s || c < K4s) ? x4[min(c, K4s - 1)] : f4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int j = j0 + b;
+      if (j < J) {
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+          acc[i].x += W[i].w[j].x * x[b].x;
+          acc[i].y += W[i].w[j].y * x[b].y;
+          acc[i].z += W[i].w[j].z * x[b].z;
+          acc[i].w += W[i].w[j].w * x[b].w;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < T; ++i) out[i] = wsum((acc[i].x + acc[i].y) + (acc[i].z + acc[i].w));
+}
 
 struct Best {
   float v;
@@ -359,241 +287,740 @@ __device__ __forceinline__ Best better(Best a, Best b) {
   if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
   return a;
 }
+// Best over the wavefront (every lane receives it).
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(b.v, off, 64), (unsigned)__shfl_xor((int)b.i, off, 64)};
+    b = better(b, o);
+  }
+  return b;
+}
 
 __device__ __forceinline__ unsigned epoch_of(const DecodeParams& p, int t, int layer, int phase) {
   return p.epoch0 + (unsigned)((t * (p.L + 1) + layer) * 8 + phase);
 }
 
-// Phases B and B2 of one layer: split-key attention of cached_self_attention_into
-// (src/models/gpt2/rust.rs:1662-1741) for the (head, split) items of this
-// workgroup, then the per-head merge by the workgroup that took split 0.  Out of
-// line so that its registers are allocated apart from the weight bands.
-__device__ __attribute__((noinline)) bool attention_phase(const DecodeParams& p, Smem& sm,
-                                                          float* xs, int t, int l, int pos,
-                                                          float* kc, float* vc) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wg = blockIdx.x;
-  const int G = kGrid, H = p.H, P = p.P, C = p.C;
-  unsigned* abort_word = p.status;
-  {
-    const int ns = p.ns, items = H * ns, n = pos + 1;
-    const int per = (n + ns - 1) / ns;
-    const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
-    const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
-    for (int item = wg; item < items; item += G) {
-      const int h = item / ns, s = item - h * ns;
-      const int k0 = s * per, k1 = min(n, k0 + per);
-      u64* dst = p.part_t + (size_t)item * 66;
-      if (k0 >= k1) {  // empty split: neutral element of the merge
-        if (tid < 64) PG_ST64(dst + tid, pack(epp, 0.0f));
-        if (tid == 64) PG_ST64(dst + 64, pack(epp, -INFINITY));
-        if (tid == 65) PG_ST64(dst + 65, pack(epp, 0.0f));
-        continue;
-      }
-      const bool owns_new = (pos >= k0 && pos < k1);
-      gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
-      gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
-      f4 kr[kAttnSteps], vr[kAttnSteps];
+// ---- streamer side: wait for an LDS flag ---------------------------------------------
+__device__ __forceinline__ bool wait_flag(ctlp ctl, int which, unsigned epoch, unsigned* abort_word) {
+  lvup f = (lvup)&ctl->flag[which];
+  lvup h = (lvup)&ctl->halt;
+  unsigned spins = 0;
+  bool ok = true;
+  for (;;) {
+    if (*f == epoch) break;
+    if (*h != 0) {
+      ok = false;
+      break;
+    }
+    if (++spins > kSpinLimit) {
+      ok = false;
+      PG_ST32(abort_word, 1u);
+      *h = 1u;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  asm volatile("" ::: "memory");
+  return ok;
+}
+
+// Waits until flag a carries va (returns 1) or flag b carries vb (returns 2); 0 on halt.
+__device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, unsigned vb,
+                                           unsigned* abort_word) {
+  lvup fa = (lvup)&ctl->flag[a];
+  lvup fb = (lvup)&ctl->flag[b];
+  lvup h = (lvup)&ctl->halt;
+  unsigned spins = 0;
+  int r = 0;
+  for (;;) {
+    if (*fa == va) {
+      r = 1;
+      break;
+    }
+    if (*fb == vb) {
+      r = 2;
+      break;
+    }
+    if (*h != 0) break;
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      *h = 1u;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  asm volatile("" ::: "memory");
+  return r;
+}
+
+// ---- service side: poll tagged words ---------------------------------------------------
+// One tagged word at a wave-uniform base plus a 32-bit byte offset ("scalar base +
+// vector offset" addressing: no 64-bit per-lane addresses are kept across the retries).
+__device__ __forceinline__ u64 ld_tagged(const u64* base, unsigned byte_off) {
+  typedef char __attribute__((address_space(1)))* gcp;
+  return __hip_atomic_load((__attribute__((address_space(1))) u64*)((gcp)base + byte_off),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Spins until run `run` (words 64 run .. 64 run + 63) carries `epoch`.  Cheap: one
+// 512-byte request per attempt.  Wave-uniform; false on timeout or abort.
+__device__ __forceinline__ bool probe_run(const u64* src, int run, unsigned epoch,
+                                          unsigned* abort_word, unsigned& spins) {
+  const int lane = opaque((int)threadIdx.x) & 63;
+  const unsigned off = (unsigned)(run * 64 + lane) * 8u;
+  for (;;) {
+    u64 v = ld_tagged(src, off);
+    if (__all(tag_of(v) == epoch)) return true;
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+    if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) return false;
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+// The run to probe after a bulk read that found stale words: one that holds a stale
+// word (`run_of_bad` is this lane's, meaningful where `bad`).  The expensive bulk read
+// is then only repeated once that laggard has arrived; the waiting is done by the
+// cheap probe and does not flood the CU's memory pipeline.
+__device__ __forceinline__ int next_probe_run(bool bad, int run_of_bad) {
+  const unsigned long long m = __ballot(bad);
+  const int first = __builtin_ctzll(m);
+  return __builtin_amdgcn_readlane(run_of_bad, first);
+}
+// Waits until src[i] carries `epoch` for every i in [0, 64 NE) and leaves the payloads
+// in dst (LDS): the cheap probe of one run (runs differ per workgroup at first, so that
+// the probes spread over memory channels), then a bulk read of lane + 64 e; while that
+// finds stale words, the probe moves to a stale word's run and the bulk read repeats.
+// Nothing but the probe run lives across a repeat: the payloads go to LDS at once.
+template <int NE>
+__device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp dst,
+                                          unsigned* abort_word, int probe, lu64p dbg = nullptr) {
+  const int lane = opaque((int)threadIdx.x) & 63;
+  unsigned spins = 0;
+  int run = probe % NE;
+  for (;;) {
+    if (!probe_run(src, run, epoch, abort_word, spins)) return false;
+    if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
+    bool bad = false;
+    int bad_e = 0;
+    u64 v[NE];
 #pragma unroll
-      for (int i = 0; i < kAttnSteps; ++i) {
-        // unconditional: keys past the split re-read a cached row (position 0 when
-        // nothing is cached yet; the cache is zero-filled at creation) and get weight 0
-        int key = min(k0 + slot + 32 * i, max(pos - 1, 0));
-        kr[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
-        vr[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
+    for (int e = 0; e < NE; ++e) v[e] = ld_tagged(src, ((unsigned)lane + 64u * e) * 8u);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      if (tag_of(v[e]) != epoch) {
+        bad = true;
+        bad_e = e;
       }
-      // q of this head, and this token's own K/V rows if the split holds pos
-      bool ok = true;
+      dst[lane + 64 * e] = val_of(v[e]);
+    }
+    if (!__any(bad)) return true;
+    run = next_probe_run(bad, bad_e);
+    if (++spins > kSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+  }
+}
+
+// layer_norm_in_place (src/models/cpu.rs:119-143) of the C = 64 NW values in raw (LDS;
+// this lane's are lane + 64 j), two-pass mean / biased variance, eps inside the sqrt;
+// writes the result to xs (LDS).
+template <int NW>
+__device__ __forceinline__ void wave_layer_norm(lfp raw, const float (&g)[NW], const float (&b)[NW],
+                                                float eps, lfp xs, int lane) {
+  constexpr int C = NW * 64;
+  float x[NW];
+#pragma unroll
+  for (int j = 0; j < NW; ++j) x[j] = raw[lane + 64 * j];
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) s += x[j];
+  const float mean = wsum(s) / (float)C;
+  float v = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    const float d = x[j] - mean;
+    v += d * d;
+  }
+  const float var = wsum(v) / (float)C;
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < NW; ++j) xs[lane + 64 * j] = (x[j] - mean) * inv * g[j] + b[j];
+}
+
+// Development timestamps (only when the launch carries a buffer for them): the shader
+// clock of the moment, kept in LDS and copied out once when the kernel ends, so that a
+// stamp costs a counter read and an LDS write and nothing in the vector memory path.
+#define PG_STAMP(layer, phase)                                                          \
+  do {                                                                                  \
+    if (p.prof && lane == 0 && t + 1 == p.n_fwd)                                        \
+      lds.ts[(layer) * 16 + (phase)] = __builtin_amdgcn_s_memtime();                    \
+  } while (0)
+
+struct Lds {
+  lfp xsA, xsD, xsE, xraw1, xraw2, xsF;
+  lu64p ts;  // development timestamps of the launch's last token: [layer 0..L][16]
+};
+constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
+
+// ---- attention item: shared by all eight wavefronts ----------------------------------
+// An item is the keys [k0, k1) of one head (at most 128).  Key k0 + slot + 32 i belongs
+// to slot = 4 wave + (lane >> 4), step i < 4; the 16 lanes of a slot hold 4 dims each.
+constexpr int kAttnSteps = kMaxItemKeys / 32;
+struct KvRegs {
+  f4 k[kAttnSteps], v[kAttnSteps];
+};
+// Requests this wavefront's K and V rows.  Unconditional: keys past the split, and the
+// key `pos` that is not in the cache yet, re-read an older row and are masked / replaced.
+__device__ __forceinline__ void attn_load_kv(KvRegs& r, const float* kc, const float* vc, int h, int P,
+                                             int k0, int pos, int slot, int d4) {
+  gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
+  gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int key = min(k0 + slot + 32 * i, max(pos - 1, 0));
+    r.k[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
+    r.v[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
+  }
+}
+// This wavefront's part of cached_self_attention_into (src/models/gpt2/rust.rs:1662-1741)
+// once q (and the new K/V rows) are in LDS: max, sum of exp and weighted V rows over its
+// keys, written to the control block.  A wavefront without keys writes the neutral element.
+__device__ __forceinline__ void attn_wave_partial(KvRegs& r, ctlp ctl, int k0, int k1, int pos,
+                                                  int wave, int lane) {
+  const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
+  const f4 qv = ((lf4p)&ctl->qs[0])[d4];
+  float sc[kAttnSteps];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int key = k0 + slot + 32 * i;
+    if (key == pos && key < k1) {
+      r.k[i] = ((lf4p)&ctl->kn[0])[d4];
+      r.v[i] = ((lf4p)&ctl->vn[0])[d4];
+    }
+    float sv = (qv.x * r.k[i].x + qv.y * r.k[i].y) + (qv.z * r.k[i].z + qv.w * r.k[i].w);
+    sv = row16_sum(sv);
+    sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
+    sc[i] = (key < k1) ? sv : -INFINITY;
+    mx = fmaxf(mx, sc[i]);
+  }
+  // every lane of a 16-lane row holds the same values: the wave maximum is that of rows
+  mx = fmaxf(fmaxf(lane_get(mx, 0), lane_get(mx, 16)), fmaxf(lane_get(mx, 32), lane_get(mx, 48)));
+  float lsum = 0.0f;
+  f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const float pr = (sc[i] == -INFINITY) ? 0.0f : expf(sc[i] - mx);
+    lsum += pr;
+    acc += pr * r.v[i];
+  }
+#pragma unroll
+  for (int off = 16; off <= 32; off <<= 1) {
+    acc.x += __shfl_xor(acc.x, off, 64);
+    acc.y += __shfl_xor(acc.y, off, 64);
+    acc.z += __shfl_xor(acc.z, off, 64);
+    acc.w += __shfl_xor(acc.w, off, 64);
+  }
+  lsum = (lane_get(lsum, 0) + lane_get(lsum, 16)) + (lane_get(lsum, 32) + lane_get(lsum, 48));
+  if (lane < 16) ((lf4p)&ctl->wacc[wave][0])[lane] = acc;
+  if (lane == 0) {
+    ctl->wm[wave] = mx;
+    ctl->wl[wave] = lsum;
+  }
+}
+
+// ---- this wavefront's share of the 4C tagged words of h ---------------------------------
+// Runs wave + 8 e (64 words each).  Payloads go to dst (LDS); returns 0, or 1 + a run
+// that held a stale word.
+template <int RUNS>
+__device__ __forceinline__ unsigned h_share(const u64* src, unsigned epoch, lfp dst, int wave, int lane) {
+  constexpr int RPW = cdiv(RUNS, 8);
+  u64 v[RPW];
+#pragma unroll
+  for (int e = 0; e < RPW; ++e) {
+    const int run = min(wave + 8 * e, RUNS - 1);
+    v[e] = ld_tagged(src, (unsigned)(run * 64 + lane) * 8u);
+  }
+  unsigned code = 0;
+#pragma unroll
+  for (int e = 0; e < RPW; ++e) {
+    const int run = min(wave + 8 * e, RUNS - 1);
+    if (tag_of(v[e]) != epoch) code = 1u + (unsigned)run;
+    dst[run * 64 + lane] = val_of(v[e]);
+  }
+  // wave-uniform: any lane's stale run will do
+  const unsigned long long m = __ballot(code != 0);
+  return m ? (unsigned)__builtin_amdgcn_readlane((int)code, __builtin_ctzll(m)) : 0u;
+}
+
+// ===================================================================================
+// Service wavefront
+// ===================================================================================
+template <int C_>
+__device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
+  constexpr int C = C_, I = 4 * C_, NW = C_ / 64, NWI = I / 64;
+  constexpr int G = kGrid;
+  static_assert(C_ % 64 == 0, "vectors are spread over 64 lanes");
+  const int lane = opaque((int)threadIdx.x) & 63;
+  const int wg = blockIdx.x;
+  unsigned* abort_word = p.status;
+  lvup halt = (lvup)&ctl->halt;
+  const int H = p.H, P = p.P, ns = p.ns;
+
+  int t = 0;
+  int stopped = 0;
+  unsigned tok = 0;
+  unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
+  // a wait gave up: tell the streamers and leave
+#define PG_SERVICE_FAIL()        \
+  do {                           \
+    if (lane == 0) *halt = 1u;   \
+    return;                      \
+  } while (0)
+
+  // merges the per-workgroup (value, index) pairs published with `ep`
+  auto merged_token = [&](unsigned ep, unsigned& out) -> bool {
+    // staged in xsF (idle between the last mlp projection and the next one)
+    if (!wave_poll<(2 * G) / 64>(p.best_t, ep, lds.xsF, abort_word, wg)) return false;
+    lds_fence();
+    // word 2g is the value, 2g+1 the index of workgroup g
+    Best b{-INFINITY, 0xffffffffu};
+#pragma unroll
+    for (int e = 0; e < G / 64; ++e) {
+      const int g = lane + 64 * e;
+      b = better(b, Best{lds.xsF[2 * g], __float_as_uint(lds.xsF[2 * g + 1])});
+    }
+    b = wave_best(b);
+    out = b.i == 0xffffffffu ? 0u : b.i;
+    return true;
+  };
+
+#pragma unroll 1
+  for (; t < p.n_fwd; ++t) {
+    const int pos = p.pos0 + t;
+    PG_STAMP(p.L, 7);
+    if (p.prof && lane == 0 && t + 1 == p.n_fwd) lds.ts[p.L * 16 + 13] = wall_clock64();
+    // ---- token to embed: given, or the argmax of the previous step's logits ----
+    if (p.force_ids) {
+      tok = p.force_ids[t];
+    } else if (t == 0) {
+      tok = p.tok_from_ptr ? p.d_tok[0] : p.tok_val;
+    } else {
+      if (!merged_token(epoch_of(p, t - 1, p.L, 6), tok)) {
+          PG_SERVICE_FAIL();
+        }
+    }
+    if (wg == 0 && lane == 0 && p.out_ids) gst_u(p.out_ids + t, tok);
+    if (p.eos >= 0 && tok == (unsigned)p.eos) {
+      stopped = 1;
+      break;
+    }
+
+#pragma unroll 1
+    for (int l = 0; l < p.L; ++l) {
+      const LayerW w = layer_of(p.layers, l);
+      float* kc = p.kv + (size_t)l * p.kv_layer_stride;
+      float* vc = kc + p.kv_v_offset;
+
+      // ================= A: block input -> LN1 -> xsA =================
       {
-        const int part = tid >> 6;  // 0: q, 1: k_new, 2: v_new
-        if (part == 0 || (owns_new && part < 3)) {
-          const u64* src = p.qkv_t + (size_t)part * C + h * 64 + lane;
-          u64 v = PG_LD64(src);
+        const int ln = opaque(lane);  // per-lane addresses are built here, not hoisted
+        float g[NW], b[NW];
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+          g[j] = gld_at(w.ln_1_g, (unsigned)ln + 64u * j);
+          b[j] = gld_at(w.ln_1_b, (unsigned)ln + 64u * j);
+        }
+        if (l == 0) {
+          // embedding (rust.rs:966-974)
+#pragma unroll
+          for (int j = 0; j < NW; ++j)
+            lds.xraw1[lane + 64 * j] = gld_at(p.wte + (size_t)tok * C, (unsigned)ln + 64u * j) +
+                                       gld_at(p.wpe + (size_t)pos * C, (unsigned)ln + 64u * j);
+        } else {
+          if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, l - 1, 5), lds.xraw1, abort_word, wg))
+            PG_SERVICE_FAIL();
+        }
+        lds_fence();
+        wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsA, lane);
+        lds_fence();
+        if (lane == 0) ctl->flag[0] = epoch_of(p, t, l, 0);
+      }
+      PG_STAMP(l, 0);
+
+      // ================= B: this workgroup's (head, split) items =================
+      // All eight wavefronts work on an item: each loads the K/V rows of its slots as
+      // soon as the item is known; this wavefront waits for q, stages it in LDS, counts
+      // the item in flag[5], and merges the eight partial results.
+      const int items = H * ns, n = pos + 1;
+      const int per = (n + ns - 1) / ns;
+      const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
+#pragma unroll 1
+      for (int item = wg; item < items; item += G) {
+        const int h = item / ns, s = item - h * ns;
+        const int k0 = s * per, k1 = min(n, k0 + per);
+        u64* dst = p.part_t + (size_t)item * 66;
+        ++bseq;
+        if (k0 >= k1) {  // empty split: neutral element of the merge (the streamers skip it too)
+          PG_ST64(dst + lane, pack(epp, 0.0f));
+          if (lane == 0) PG_ST64(dst + 64, pack(epp, -INFINITY));
+          if (lane == 1) PG_ST64(dst + 65, pack(epp, 0.0f));
+          continue;
+        }
+        const bool owns_new = (k1 == n);
+        KvRegs kv;
+        attn_load_kv(kv, kc, vc, h, P, k0, pos, kSW * 4 + (lane >> 4), lane & 15);
+        // q of this head, and this token's own K/V rows if the split holds pos
+        float qn[3];
+        {
+          bool ok = true;
           unsigned spins = 0;
-          while (tag_of(v) != epq) {
+          const unsigned off = (unsigned)(h * 64 + lane) * 8u;
+          for (;;) {
+            // without the new row, the K and V words are not waited for (q is re-read)
+            const u64 v0 = ld_tagged(p.qkv_t, off);
+            const u64 v1 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 8u : 0u));
+            const u64 v2 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 16u : 0u));
+            const bool bad = tag_of(v0) != epq || tag_of(v1) != epq || tag_of(v2) != epq;
+            qn[0] = val_of(v0);
+            qn[1] = val_of(v1);
+            qn[2] = val_of(v2);
+            if (!__any(bad)) break;
             if (++spins > kSpinLimit) {
-              ok = false;
               PG_ST32(abort_word, 1u);
+              ok = false;
               break;
             }
-            if ((spins & 63) == 0 && PG_LD32(abort_word) != 0) {
+            if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+          }
+          if (!ok) PG_SERVICE_FAIL();
+        }
+        ctl->qs[lane] = qn[0];
+        if (owns_new) {
+          // K/V append (rust.rs:1677-1683); written through to memory so that a later
+          // token's reader on another XCD cannot miss it in a remote L2
+          ctl->kn[lane] = qn[1];
+          ctl->vn[lane] = qn[2];
+          PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[1]));
+          PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, __float_as_uint(qn[2]));
+        }
+        lds_fence();
+        if (lane == 0) ctl->flag[5] = bseq;
+        attn_wave_partial(kv, ctl, k0, k1, pos, kSW, lane);
+        // the streamers' partials
+        {
+          lvup done = (lvup)&ctl->bdone[min(lane, kSW - 1)];
+          unsigned spins = 0;
+          bool ok = true;
+          for (;;) {
+            if (__all(*done == bseq)) break;
+            if (*halt != 0 || ++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
               ok = false;
               break;
             }
             __builtin_amdgcn_s_sleep(1);
-            v = PG_LD64(src);
           }
-          float f = val_of(v);
-          if (part == 0) sm.qs[lane] = f;
-          if (part == 1) {
-            sm.kn[lane] = f;
-            // K append (rust.rs:1677-1683); written through to memory so that a
-            // later token's reader on another XCD cannot miss it in a remote L2
-            PG_ST32(kc + ((size_t)h * P + pos) * 64 + lane, f);
+          asm volatile("" ::: "memory");
+          if (!ok) PG_SERVICE_FAIL();
+        }
+        lds_fence();
+        {
+          float M = ctl->wm[0];
+#pragma unroll
+          for (int wv = 1; wv < 8; ++wv) M = fmaxf(M, ctl->wm[wv]);
+          float num = 0.0f, den = 0.0f;
+#pragma unroll
+          for (int wv = 0; wv < 8; ++wv) {
+            const float mw = ctl->wm[wv];
+            const float wq = (mw == -INFINITY) ? 0.0f : expf(mw - M);
+            den += wq * ctl->wl[wv];
+            num += wq * ctl->wacc[wv][lane];
           }
-          if (part == 2) {
-            sm.vn[lane] = f;
-            PG_ST32(vc + ((size_t)h * P + pos) * 64 + lane, f);  // V append
-          }
+          PG_ST64(dst + lane, pack(epp, num));
+          if (lane == 0) PG_ST64(dst + 64, pack(epp, M));
+          if (lane == 1) PG_ST64(dst + 65, pack(epp, den));
         }
       }
-      if (!all_ok(ok, sm)) return false;
-      const f4 qv = reinterpret_cast<const f4*>(sm.qs)[d4];
-      float sc[kAttnSteps];
-      float mx = -INFINITY;
+      // the credit of the second attention hop (the streamers request a slice on it)
+      if (lane == 0) ctl->flag[6] = epp;
+      PG_STAMP(l, 1);
+
+      // ================= B2: the workgroup that took split 0 of a head merges it ====
+      const unsigned epa = epoch_of(p, t, l, 2);
+#pragma unroll 1
+      for (int item = wg; item < items; item += G) {
+        const int h = item / ns, s = item - h * ns;
+        if (s != 0) continue;
+        // the head's ns partials (66 words each) are one run of tagged words: probe the
+        // last word of every partial, then read them all into LDS (the staging area of
+        // the long vector, idle now) and merge from there
+        const u64* src = p.part_t + (size_t)h * ns * 66;
+        const int nw = ns * 66;
+        lfp stage = lds.xsF;
+        unsigned spins = 0;
+        for (;;) {
+          {
+            const unsigned off = (unsigned)(min(lane, ns - 1) * 66 + 65) * 8u;
+            bool ok = true;
+            for (;;) {
+              const u64 v = ld_tagged(src, off);
+              if (__all(tag_of(v) == epp)) break;
+              if (++spins > kSpinLimit) {
+                PG_ST32(abort_word, 1u);
+                ok = false;
+                break;
+              }
+              if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+                ok = false;
+                break;
+              }
+              __builtin_amdgcn_s_sleep(2);
+            }
+            if (!ok) PG_SERVICE_FAIL();
+          }
+          bool bad = false;
+          constexpr int CH = 12;
+#pragma unroll 1
+          for (int e0 = 0; e0 * 64 < nw; e0 += CH) {
+            u64 v[CH];
 #pragma unroll
-      for (int i = 0; i < kAttnSteps; ++i) {
-        int key = k0 + slot + 32 * i;
-        if (key == pos && key < k1) {
-          kr[i] = reinterpret_cast<const f4*>(sm.kn)[d4];
-          vr[i] = reinterpret_cast<const f4*>(sm.vn)[d4];
+            for (int e = 0; e < CH; ++e)
+              v[e] = ld_tagged(src, (unsigned)min(lane + 64 * (e0 + e), nw - 1) * 8u);
+#pragma unroll
+            for (int e = 0; e < CH; ++e) {
+              bad = bad || (tag_of(v[e]) != epp);
+              stage[min(lane + 64 * (e0 + e), nw - 1)] = val_of(v[e]);
+            }
+          }
+          if (!__any(bad)) break;
+          if (++spins > kSpinLimit) {
+            PG_ST32(abort_word, 1u);
+            PG_SERVICE_FAIL();
+          }
         }
-        float sv = (qv.x * kr[i].x + qv.y * kr[i].y) + (qv.z * kr[i].z + qv.w * kr[i].w);
-        sv = row16_sum(sv);
-        sv *= 0.125f;  // 1/sqrt(64), applied after the sum (rust.rs:1675, 1699)
-        sc[i] = (key < k1) ? sv : -INFINITY;
-        mx = fmaxf(mx, sc[i]);
-      }
-      mx = bmax<0>(mx, sm);
-      float lsum = 0.0f;
-      f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int i = 0; i < kAttnSteps; ++i) {
-        float pr = expf(sc[i] - mx);  // exp(-inf) = 0 for absent keys
-        if (d4 == 0) lsum += pr;
-        acc += pr * vr[i];
-      }
-      lsum = bsum<1>(lsum, sm);
-#pragma unroll
-      for (int off = 16; off <= 32; off <<= 1) {
-        acc.x += __shfl_xor(acc.x, off, 64);
-        acc.y += __shfl_xor(acc.y, off, 64);
-        acc.z += __shfl_xor(acc.z, off, 64);
-        acc.w += __shfl_xor(acc.w, off, 64);
-      }
-      if (sub == 0) reinterpret_cast<f4*>(sm.accs[wave])[d4] = acc;
-      __syncthreads();
-      if (tid < 64) {
-        float tsum = 0.0f;
-#pragma unroll
-        for (int wv = 0; wv < kWavesP; ++wv) tsum += sm.accs[wv][tid];
-        PG_ST64(dst + tid, pack(epp, tsum));
-      }
-      if (tid == 64) PG_ST64(dst + 64, pack(epp, mx));
-      if (tid == 65) PG_ST64(dst + 65, pack(epp, lsum));
-      __syncthreads();
-    }
-    // ---- B2: the workgroup that took split 0 of a head merges that head ----
-    const unsigned epa = epoch_of(p, t, l, 2);
-    for (int item = wg; item < items; item += G) {
-      const int h = item / ns, s = item - h * ns;
-      if (s != 0) continue;
-      float* stage = xs;  // ns*66 floats
-      bool ok = poll_vec<cdiv(kMaxSplits * 66, kThreads)>(p.part_t + (size_t)h * ns * 66,
-                                                          ns * 66, epp, stage, abort_word);
-      if (!all_ok(ok, sm)) return false;
-      if (tid < 64) {
-        float M = stage[64];
-        for (int q = 1; q < ns; ++q) M = fmaxf(M, stage[q * 66 + 64]);
+        lds_fence();
+        float M = -INFINITY;
+#pragma unroll 1
+        for (int q = 0; q < ns; ++q) M = fmaxf(M, stage[q * 66 + 64]);
         float num = 0.0f, den = 0.0f;
+#pragma unroll 1
         for (int q = 0; q < ns; ++q) {
-          float wq = expf(stage[q * 66 + 64] - M);
+          const float mq = stage[q * 66 + 64];
+          const float wq = (mq == -INFINITY) ? 0.0f : expf(mq - M);
           den += wq * stage[q * 66 + 65];
-          num += wq * stage[q * 66 + tid];
+          num += wq * stage[q * 66 + lane];
         }
-        PG_ST64(p.attn_t + h * 64 + tid, pack(epa, num / den));
+        PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
       }
-      __syncthreads();
+
+      // ================= D: attention output -> xsD =================
+      {
+        if (!wave_poll<NW>(p.attn_t, epa, lds.xsD, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        lds_fence();
+        if (lane == 0) ctl->flag[1] = epa;
+      }
+      PG_STAMP(l, 2);
+
+      // ================= E: xa -> xraw2, LN2 -> xsE =================
+      {
+        const int ln = opaque(lane);
+        float g[NW], b[NW];
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+          g[j] = gld_at(w.ln_2_g, (unsigned)ln + 64u * j);
+          b[j] = gld_at(w.ln_2_b, (unsigned)ln + 64u * j);
+        }
+        const unsigned ep = epoch_of(p, t, l, 3);
+        if (!wave_poll<NW>(p.xa_t, ep, lds.xraw2, abort_word, wg + 2,
+                           (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 + 13 : (lu64p) nullptr))
+          PG_SERVICE_FAIL();
+        lds_fence();
+        wave_layer_norm<NW>(lds.xraw2, g, b, p.eps, lds.xsE, lane);
+        lds_fence();
+        if (lane == 0) ctl->flag[2] = ep;
+      }
+      PG_STAMP(l, 3);
+
+      // ================= F: h -> xsF =================
+      // 4C tagged words: after the cheap probe all eight wavefronts read a share each
+      // (flag[7] counts the rounds); a stale word sends the probe to its run and the
+      // round is repeated.
+      {
+        constexpr int RUNS = I / 64;
+        const unsigned ep = epoch_of(p, t, l, 4);
+        int run = (wg + 3) % RUNS;
+        unsigned spins = 0;
+        for (;;) {
+          if (!probe_run(p.h_t, run, ep, abort_word, spins)) PG_SERVICE_FAIL();
+          ++hseq;
+          if (lane == 0) ctl->flag[7] = hseq;
+          unsigned code = h_share<RUNS>(p.h_t, ep, lds.xsF, kSW, lane);
+          lvup st = (lvup)&ctl->hstat[min(lane, kSW - 1)];
+          bool ok = true;
+          unsigned v = 0;
+          for (;;) {
+            v = *st;
+            if (__all((v >> 8) == hseq)) break;
+            if (*halt != 0 || ++spins > kSpinLimit) {
+              PG_ST32(abort_word, 1u);
+              ok = false;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          asm volatile("" ::: "memory");
+          if (!ok) PG_SERVICE_FAIL();
+          const unsigned mine = (lane < kSW) ? (v & 0xffu) : code;
+          const unsigned long long m = __ballot(mine != 0);
+          if (m == 0) break;
+          run = __builtin_amdgcn_readlane((int)mine, __builtin_ctzll(m)) - 1;
+        }
+        lds_fence();
+        if (lane == 0) ctl->flag[3] = ep;
+      }
+      PG_STAMP(l, 4);
+    }  // layers
+
+    // ================= LN_f -> xsD, then this workgroup's argmax =================
+    if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      const int ln = opaque(lane);
+      float g[NW], b[NW];
+#pragma unroll
+      for (int j = 0; j < NW; ++j) {
+        g[j] = gld_at(p.ln_f_g, (unsigned)ln + 64u * j);
+        b[j] = gld_at(p.ln_f_b, (unsigned)ln + 64u * j);
+      }
+      const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
+      // staged in xraw1 (the next user is the next token's embedding)
+      if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, p.L - 1, 5), lds.xraw1, abort_word, wg))
+        PG_SERVICE_FAIL();
+      lds_fence();
+      wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsD, lane);
+      lds_fence();
+      if (lane == 0) ctl->flag[4] = epl;
+      PG_STAMP(p.L, 5);
+      // wait for the streamers' bands
+      {
+        lvup done = (lvup)&ctl->lmdone[min(lane, kSW - 1)];
+        unsigned spins = 0;
+        bool ok = true;
+        for (;;) {
+          if (__all(*done == epl)) break;
+          if (*halt != 0) {
+            ok = false;
+            break;
+          }
+          if (++spins > kSpinLimit) {
+            PG_ST32(abort_word, 1u);
+            ok = false;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");
+        if (!ok) {
+          PG_SERVICE_FAIL();
+        }
+      }
+      Best bb{ctl->bestv[min(lane, kSW - 1)], ctl->besti[min(lane, kSW - 1)]};
+      bb = wave_best(bb);
+      if (lane == 0) PG_ST64(p.best_t + 2 * wg, pack(ep_best, bb.v));
+      if (lane == 1) PG_ST64(p.best_t + 2 * wg + 1, pack_u(ep_best, bb.i));
+      PG_STAMP(p.L, 6);
+    }
+  }  // tokens
+
+  if (p.prof) {
+    // calibration pair (wall clock, shader clock), then the copy to global memory
+    if (lane == 0) {
+      lds.ts[p.L * 16 + 14] = wall_clock64();
+      lds.ts[p.L * 16 + 15] = __builtin_amdgcn_s_memtime();
+    }
+    lds_fence();
+    for (int i = lane; i < (p.L + 1) * 16; i += 64)
+      gst_u64(p.prof + (size_t)wg * (p.L + 1) * 16 + i, lds.ts[i]);
+  }
+  if (stopped) {
+    if (lane == 0) *halt = 2u;
+  } else if (p.select_last && p.n_fwd > 0) {
+    unsigned tk = 0;
+    if (!merged_token(epoch_of(p, p.n_fwd - 1, p.L, 6), tk)) {
+      PG_SERVICE_FAIL();
+    }
+    if (wg == 0 && lane == 0) {
+      if (p.out_ids) gst_u(p.out_ids + p.n_fwd, tk);
+      gst_u(p.d_tok, tk);
     }
   }
-  return true;
+  if (wg == 0 && lane == 0) {
+    gst_u(p.status + 1, (unsigned)t);
+    gst_u(p.status + 2, (unsigned)stopped);
+  }
 }
 
-// LN_f + lm_head for this workgroup's band of vocabulary rows, one weight row per
-// wavefront at a time with two rows in flight (the band is ~200 rows deep), plus
-// the band's argmax.  Kept out of line so that its registers are allocated apart
-// from the layer loop's.  Returns false if the wait for its input gave up.
-template <int C_>
-__device__ __attribute__((noinline)) bool lm_head_phase(const DecodeParams& p, Smem& sm, float* xs,
-                                                        float* xraw, int t, int v0, int v1) {
-  constexpr int C = C_, K4 = C_ / 4, J = cdiv(K4, 64), NEC = cdiv(C, kThreads);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wg = blockIdx.x;
-  // parameter fields are read once, before any weight row is requested
-  const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
-  float* const logits = p.logits;
-  u64* const best_t = p.best_t;
-  const float eps = p.eps;
-  const unsigned ep_best = epoch_of(p, t, p.L, 6);
-  LnParams<NEC> lp;
-  ln_fetch<NEC>(lp, p.ln_f_g, p.ln_f_b, C);
-  bool ok = poll_vec<NEC>(p.xm_t, C, epoch_of(p, t, p.L - 1, 5), xraw, p.status);
-  if (!all_ok(ok, sm)) return false;
-  Tile<J> ta, tb;
-  int r = v0 + wave;
-  // rows past the band are clamped to its last row and their products discarded
-  load_tile<J>(ta, wte4 + (size_t)min(r, v1 - 1) * K4, K4, lane);
-  load_tile<J>(tb, wte4 + (size_t)min(r + kWavesP, v1 - 1) * K4, K4, lane);
-  ln_lds<NEC, C>(xraw, xs, lp, eps);
-  f4 xr[J];
-  load_x<J>(xr, xs, K4, lane);
-  Best best{-INFINITY, 0xffffffffu};
-  for (; r < v1; r += 2 * kWavesP) {
-    float va = dot_tile<J>(ta, xr);
-    load_tile<J>(ta, wte4 + (size_t)min(r + 2 * kWavesP, v1 - 1) * K4, K4, lane);
-    if (lane == 0) logits[r] = va;
-    if (va > best.v) best = Best{va, (unsigned)r};
-    int r2 = r + kWavesP;
-    if (r2 < v1) {
-      float vb = dot_tile<J>(tb, xr);
-      load_tile<J>(tb, wte4 + (size_t)min(r2 + 2 * kWavesP, v1 - 1) * K4, K4, lane);
-      if (lane == 0) logits[r2] = vb;
-      if (vb > best.v) best = Best{vb, (unsigned)r2};
-    }
-  }
-  if (lane == 0) {
-    sm.bestv[wave] = best.v;
-    sm.besti[wave] = best.i;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    Best b{sm.bestv[0], sm.besti[0]};
-    for (int wv = 1; wv < kWavesP; ++wv) b = better(b, Best{sm.bestv[wv], sm.besti[wv]});
-    PG_ST64(best_t + 2 * wg, pack(ep_best, b.v));
-    PG_ST64(best_t + 2 * wg + 1, pack_u(ep_best, b.i));
-  }
-  __syncthreads();
-  return true;
-}
+#undef PG_SERVICE_FAIL
 
-#define PG_STAMP(layer, phase)                                                          \
-  do {                                                                                  \
-    if (p.prof && tid == 0 && t + 1 == p.n_fwd)                                         \
-      p.prof[((size_t)wg * (p.L + 1) + (layer)) * 8 + (phase)] = wall_clock64();        \
-  } while (0)
-
-// C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
+// ===================================================================================
+// Streamer wavefronts
+// ===================================================================================
+// Wavefront w owns row r0 + w + 7 i of a band (i < T) for the C-wide matrices and row
+// d0 + w of the 4C-wide mlp projection.  A row is J float4 per lane; the input
+// vector's matching float4 come out of LDS once per phase.
 //
-// Each wavefront owns whole weight rows (row-phases A, D, E) or quarter rows of
-// K = 4C (phase F): row r0 + wave + 8*i for i < T.  A row is J float4 per lane; the
-// input vector's matching J float4 sit in registers for the whole phase, so a row
-// costs J loads, 4J multiply-adds and one DPP tree.  All T rows of the NEXT matrix
-// are requested as soon as the current phase's input has arrived.
+// The vector memory path of a CU returns data in issue order across ALL of its
+// wavefronts, so every byte the streamers have in flight delays the service
+// wavefront's next poll by the time it takes to drain (about 1 us per 32 KiB).  The
+// layer's weights are therefore requested as one fixed stream
+//     c_proj row | c_fc rows | mlp projection row | next layer's c_attn rows
+// cut into six equal slices, and a slice is only requested at a moment when the
+// service wavefront has just completed a poll (one per phase: after the A, D, E and F
+// products, and on the two "credits" it raises during the attention phases).  Each
+// slice drains while the dependency chain makes its next hop; each is requested at
+// least one phase before its rows are used.
 template <int C_>
-__global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
+struct StreamPlan {
+  static constexpr int C = C_, I = 4 * C_, K4 = C_ / 4, G = kGrid;
+  static constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
+  static constexpr int TA = cdiv(RA, kSW), TE = cdiv(RE, kSW);
+  static constexpr int J = cdiv(K4, 64);
+  static constexpr int JF = C_ / 64;  // float4 per lane of one 4C-wide row
+  // loads per layer and wavefront, in stream order
+  static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
+  // Equal cuts where the registers allow it.  The widest model cannot hold the c_fc rows
+  // next to much of the mlp projection row: its first four slices are shorter and the
+  // last two longer (those two phases then run at the speed of the stream).
+  static constexpr bool kTight = (ND + NE + NF) * 4 > 200;
+  static constexpr int cut(int k) {
+    if (!kTight || k == 0 || k == 6) return k * NL / 6;
+    const int c4 = ND + NE + 4;
+    if (k <= 4) return k * c4 / 4;
+    return (c4 + NL) / 2 > ND + NE + NF ? (c4 + NL) / 2 : ND + NE + NF;
+  }
+  // slice k is requested: 0 after A, 1 and 2 on the attention credits, 3 after D,
+  // 4 after E, 5 after F.  D is used after slice 2, E after 3, F after 4, A' after 5.
+  static_assert(ND <= cut(3), "c_proj row is requested before it is used");
+  static_assert(ND + NE <= cut(4), "c_fc rows are requested before they are used");
+  static_assert(ND + NE + NF <= cut(5), "mlp projection row is requested before it is used");
+  static_assert(RD <= kSW, "one mlp projection row per streamer");
+  static_assert(C_ % 64 == 0, "4C-wide rows are whole runs of 64 float4");
+};
+
+template <int C_>
+__device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
+  typedef StreamPlan<C_> SP;
   constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
   constexpr int G = kGrid;
-  constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
-  constexpr int TA = cdiv(RA, kWavesP), TD = cdiv(RD, kWavesP), TE = cdiv(RE, kWavesP),
-                TF = cdiv(4 * RD, kWavesP);  // rows (quarter rows for F) per wavefront
-  constexpr int J = cdiv(K4, 64);
-  constexpr int NEC = cdiv(C, kThreads), NEI = cdiv(I, kThreads);
-  static_assert(4 * RD <= 64, "phase F partial sums");
+  constexpr int TA = SP::TA, TE = SP::TE, J = SP::J, JF = SP::JF;
 
-  extern __shared__ float dyn[];
-  __shared__ Smem sm;
-  float* xs = dyn;        // [I] normalised / staged input of the current matrix
-  float* xraw = dyn + I;  // [C] residual stream entering the current half-block
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = opaque((int)threadIdx.x) & 63;
   const int wg = blockIdx.x;
   const int V = p.V;
   unsigned* abort_word = p.status;
@@ -603,238 +1030,307 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
   const int d0 = (int)(((long long)wg * C) / G), d1 = (int)(((long long)(wg + 1) * C) / G);
   const int e0 = (int)(((long long)wg * I) / G), e1 = (int)(((long long)(wg + 1) * I) / G);
   const int v0 = (int)(((long long)wg * V) / G), v1 = (int)(((long long)(wg + 1) * V) / G);
-  const int nF = (d1 - d0) * 4;  // (row, quarter) tiles of phase F
 
-  if (tid == 0) sm.ok = 1;
-  __syncthreads();
-
-  // The out-of-line phases get their own copy of the parameters.  Taking the address
-  // of `p` itself would move it to scratch memory, and every later read of a field
-  // would be a memory load that has to wait for the weight rows in flight.
-  const DecodeParams pc = p;
-
+  // the wavefront index as a scalar: rows, row addresses and biases are wave-uniform
+  auto wave_id = [&]() { return __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6); };
   // Row i of this wavefront in a band [r0, r1), clamped into the band (rows past the
   // end re-read the last row; their results are dropped).
-  // (the wave index goes through local_tid() so that row addresses are recomputed at
-  // each use instead of being kept alive across the layer loop)
-  auto row_of = [&](int r0, int r1, int i) {
-    return min(r0 + (local_tid() >> 6) + kWavesP * i, r1 - 1);
-  };
+  auto row_of = [&](int r0, int r1, int i) { return min(r0 + wave_id() + kSW * i, r1 - 1); };
 
-  int t = 0;
-  int stopped = 0;
-  unsigned tok = 0;
   Tile<J> WA[TA];  // c_attn rows of the layer about to run
-  for (; t < p.n_fwd; ++t) {
-    const int pos = p.pos0 + t;
-    PG_STAMP(p.L, 7);
-    {
-      const f4* W4 = reinterpret_cast<const f4*>(p.layers[0].c_attn_w);
+  Tile<J> WD[1];   // c_proj row
+  Tile<J> WE[TE];  // c_fc rows
+  Tile<JF> WF;     // mlp projection row
+
+  // One float4 of a C-wide row: column block j (columns past the row re-read its last
+  // float4 and meet a zero in x).  Unconditional, like every load here: a load under a
+  // branch would make the compiler lose count of the loads in flight.
+  auto ld_c = [&](const float* W, int row, int j, int ln) -> f4 {
+    const unsigned c = (64 * (j + 1) <= K4) ? (unsigned)ln + 64u * j
+                                            : (unsigned)min(ln + 64 * j, K4 - 1);
+    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * K4, c * 16u);
+  };
+  // Requests loads [N0, N1) of the layer stream: `w` is the layer whose c_proj, c_fc and
+  // mlp projection rows are meant, `wn` the one whose c_attn rows follow.
+  auto issue = [&](auto n0_, auto n1_, const LayerW& w, const LayerW& wn) {
+    constexpr int N0 = decltype(n0_)::value, N1 = decltype(n1_)::value;
+    // the lane index behind an empty asm again: the per-lane parts of the addresses are
+    // rebuilt for each slice instead of being kept (and spilled) across the whole layer
+    const int ln = opaque(lane);
 #pragma unroll
-      for (int i = 0; i < TA; ++i) load_tile<J>(WA[i], W4 + (size_t)row_of(a0, a1, i) * K4, K4, lane);
-    }
-    // ---- token to embed: given, or the argmax of the previous step's logits ----
-    if (p.force_ids) {
-      tok = p.force_ids[t];
-    } else if (t == 0) {
-      tok = p.tok_from_ptr ? p.d_tok[0] : p.tok_val;
-    } else {
-      // merge the per-workgroup (value, index) pairs in workgroup order
-      float* bv = xs;  // 2*G floats of staging
-      bool ok = poll_vec<1>(p.best_t, 2 * G, epoch_of(p, t - 1, p.L, 6), bv, abort_word);
-      if (!all_ok(ok, sm)) return;
-      if (tid == 0) {
-        Best b{-INFINITY, 0xffffffffu};
-        for (int g = 0; g < G; ++g) b = better(b, Best{bv[2 * g], __float_as_uint(bv[2 * g + 1])});
-        sm.tok = b.i == 0xffffffffu ? 0u : b.i;
+    for (int n = N0; n < N1; ++n) {
+      if (n < SP::ND) {
+        WD[0].w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n, ln);
+      } else if (n < SP::ND + SP::NE) {
+        const int i = (n - SP::ND) / J, j = (n - SP::ND) % J;
+        WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
+      } else if (n < SP::ND + SP::NE + SP::NF) {
+        const int j = n - SP::ND - SP::NE;
+        WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
+                         ((unsigned)ln + 64u * j) * 16u);
+      } else {
+        const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
+        WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
       }
-      __syncthreads();
-      tok = sm.tok;
-      __syncthreads();
     }
-    if (wg == 0 && tid == 0 && p.out_ids) p.out_ids[t] = tok;
-    if (p.eos >= 0 && tok == (unsigned)p.eos) {
-      stopped = 1;
-      break;
-    }
+  };
+#define PG_SLICE(k, w, wn)                                              \
+  issue(std::integral_constant<int, SP::cut(k)>{},                      \
+        std::integral_constant<int, SP::cut((k) + 1)>{}, (w), (wn))
 
+  // before the first layer: its c_attn rows
+  {
+    const LayerW w0 = layer_of(p.layers, 0);
+    issue(std::integral_constant<int, SP::ND + SP::NE + SP::NF>{},
+          std::integral_constant<int, SP::NL>{}, w0, w0);
+  }
+
+  // development timestamps of streamer 0 (slots 5.. of the layer's 16)
+#define SSTAMP(slot)                                                                   \
+  do {                                                                                 \
+    if (p.prof && lane == 0 && wave == 0 && t + 1 == p.n_fwd)                          \
+      lds.ts[l * 16 + (slot)] = __builtin_amdgcn_s_memtime();                          \
+  } while (0)
+  bool ok = true;
+  unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
+  for (int t = 0; t < p.n_fwd && ok; ++t) {
     for (int l = 0; l < p.L; ++l) {
-      const LayerW w = p.layers[l];
-      float* kc = p.kv + (size_t)l * p.kv_layer_stride;
-      float* vc = kc + p.kv_v_offset;
+      const LayerW w = layer_of(p.layers, l);
+      const LayerW wn = layer_of(p.layers, (l + 1 < p.L) ? l + 1 : 0);
+      const int wave = wave_id();
 
-      // ================= A: LN1 + c_attn =================
-      {
-        LnParams<NEC> lp;
-        ln_fetch<NEC>(lp, w.ln_1_g, w.ln_1_b, C);
-        float bias[TA];
+      // ================= A: c_attn rows =================
+      // (biases are scalar loads: requested before each wait, they neither use vector
+      // registers while the rows are in flight nor queue behind them)
+      float biasA[TA];
 #pragma unroll
-        for (int i = 0; i < TA; ++i) bias[i] = w.c_attn_b[row_of(a0, a1, i)];
-        __syncthreads();  // every wave is done with xs / xraw of the previous phase
-        if (l == 0) {
-          // embedding (rust.rs:966-974)
-          for (int i = tid; i < C; i += kThreads)
-            xraw[i] = p.wte[(size_t)tok * C + i] + p.wpe[(size_t)pos * C + i];
-          __syncthreads();
-        } else {
-          bool ok = poll_vec<NEC>(p.xm_t, C, epoch_of(p, t, l - 1, 5), xraw, abort_word);
-          if (!all_ok(ok, sm)) return;
-        }
-        ln_lds<NEC, C>(xraw, xs, lp, p.eps);
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
+      for (int i = 0; i < TA; ++i) biasA[i] = cld(w.c_attn_b + row_of(a0, a1, i));
+      if (!wait_flag(ctl, 0, epoch_of(p, t, l, 0), abort_word)) {
+        ok = false;
+        break;
+      }
+      // (a slice goes out the moment the flag is seen where the registers allow it:
+      // the service wavefront has just completed a poll and its next ones are early)
+      PG_SLICE(0, w, wn);
+      {
+        float v[TA];
+        dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 0);
 #pragma unroll
         for (int i = 0; i < TA; ++i) {
-          const int r = a0 + wave + kWavesP * i;
-          const float v = dot_tile<J>(WA[i], xr);
-          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, bias[i] + v));
+          const int r = a0 + wave + kSW * i;
+          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, biasA[i] + v[i]));
         }
       }
-      PG_STAMP(l, 0);
-
-      // ================= B, B2: attention over keys [0, pos] =================
-      if (!attention_phase(pc, sm, xs, t, l, pos, kc, vc)) return;
-      PG_STAMP(l, 2);
-
-      // ================= D: c_proj + residual =================
-      Tile<J> WE[TE];  // c_fc rows, requested as soon as D's input has arrived
+      SSTAMP(5);
+      // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
       {
-        float bias[TD];
-#pragma unroll
-        for (int i = 0; i < TD; ++i) bias[i] = w.c_proj_b[row_of(d0, d1, i)];
-        Tile<J> WD[TD];  // c_proj rows: few, requested right before D waits for its input
-        {
-          const f4* W4 = reinterpret_cast<const f4*>(w.c_proj_w);
-#pragma unroll
-          for (int i = 0; i < TD; ++i)
-            load_tile<J>(WD[i], W4 + (size_t)row_of(d0, d1, i) * K4, K4, lane);
+        const int H = p.H, P = p.P, ns = p.ns, pos = p.pos0 + t;
+        const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
+        const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
+        const float* vc = kc + p.kv_v_offset;
+#pragma unroll 1
+        for (int item = wg; item < items; item += G) {
+          const int h = item / ns, sp = item - h * ns;
+          const int k0 = sp * per, k1 = min(n, k0 + per);
+          ++bseq;
+          if (k0 >= k1) continue;
+          KvRegs kv;
+          attn_load_kv(kv, kc, vc, h, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
+          if (!wait_flag(ctl, 5, bseq, abort_word)) {
+            ok = false;
+            break;
+          }
+          attn_wave_partial(kv, ctl, k0, k1, pos, wave, lane);
+          lds_fence();
+          if (lane == 0) ctl->bdone[wave] = bseq;
         }
-        __syncthreads();  // every wave is done with xs of the previous phase
-        bool ok = poll_vec<NEC>(p.attn_t, C, epoch_of(p, t, l, 2), xs, abort_word);
-        if (!all_ok(ok, sm)) return;
-        {
-          const f4* W4 = reinterpret_cast<const f4*>(w.c_fc_w);
-#pragma unroll
-          for (int i = 0; i < TE; ++i)
-            load_tile<J>(WE[i], W4 + (size_t)row_of(e0, e1, i) * K4, K4, lane);
-        }
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
-        const unsigned ep = epoch_of(p, t, l, 3);
-#pragma unroll
-        for (int i = 0; i < TD; ++i) {
-          const int r = d0 + wave + kWavesP * i;
-          const float v = dot_tile<J>(WD[i], xr);
-          if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(ep, xraw[r] + (bias[i] + v)));
-        }
+        if (!ok) break;
       }
-      PG_STAMP(l, 3);
+      PG_SLICE(1, w, wn);
+      if (!wait_flag(ctl, 6, epoch_of(p, t, l, 1), abort_word)) {
+        ok = false;
+        break;
+      }
+      PG_SLICE(2, w, wn);
 
-      // ================= E: LN2 + c_fc + GELU =================
-      // mlp c_proj quarter rows: a quarter of them is requested once E's input has
-      // arrived, the rest once E's own rows are consumed and their registers are free
-      Tile<J> WF[TF];
-      const f4* Wf4 = reinterpret_cast<const f4*>(w.c_proj_mlp_w);
-      auto f_tile = [&](int i) {  // quarter row (row d0 + id/4, quarter id%4), clamped
-        const int id = min((local_tid() >> 6) + kWavesP * i, nF - 1);
-        return Wf4 + (size_t)(d0 + (id >> 2)) * C + (size_t)(id & 3) * K4;
-      };
+      // ================= D: c_proj row + residual =================
+      const float biasD = cld(w.c_proj_b + row_of(d0, d1, 0));
+      if (!wait_flag(ctl, 1, epoch_of(p, t, l, 2), abort_word)) {
+        ok = false;
+        break;
+      }
       {
-        LnParams<NEC> lp;
-        ln_fetch<NEC>(lp, w.ln_2_g, w.ln_2_b, C);
-        float bias[TE];
+        float v[1];
+        dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
+        const int r = d0 + wave;
+        if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v[0])));
+      }
+      PG_SLICE(3, w, wn);
+
+      // ================= E: c_fc rows + GELU =================
+      float biasE[TE];
 #pragma unroll
-        for (int i = 0; i < TE; ++i) bias[i] = w.c_fc_b[row_of(e0, e1, i)];
-        __syncthreads();  // every wave is done with xraw (residual of phase D)
-        bool ok = poll_vec<NEC>(p.xa_t, C, epoch_of(p, t, l, 3), xraw, abort_word);
-        if (!all_ok(ok, sm)) return;
-        PG_STAMP(l, 6);
-#pragma unroll
-        for (int i = 0; i < TF / 4; ++i) load_tile<J>(WF[i], f_tile(i), K4, lane);
-        ln_lds<NEC, C>(xraw, xs, lp, p.eps);
-        f4 xr[J];
-        load_x<J>(xr, xs, K4, lane);
+      for (int i = 0; i < TE; ++i) biasE[i] = cld(w.c_fc_b + row_of(e0, e1, i));
+      if (!wait_flag(ctl, 2, epoch_of(p, t, l, 3), abort_word)) {
+        ok = false;
+        break;
+      }
+      {
+        float v[TE];
+        dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 4);
+        // lane i finishes row i: one GELU and one store for all of the wavefront's rows
+        float mine = 0.0f;
+        int r = e1;
 #pragma unroll
-        for (int i = 0; i < TE; ++i) {
-          const int r = e0 + wave + kWavesP * i;
-          const float v = dot_tile<J>(WE[i], xr);
-          if (lane == 0 && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(bias[i] + v)));
-        }
-        PG_STAMP(l, 7);
-#pragma unroll
-        for (int i = TF / 4; i < TF; ++i) load_tile<J>(WF[i], f_tile(i), K4, lane);
+        for (int i = 0; i < TE; ++i)
+          if (lane == i) {
+            mine = biasE[i] + v[i];
+            r = e0 + wave + kSW * i;
+          }
+        if (lane < TE && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(mine)));
       }
-      PG_STAMP(l, 4);
+      SSTAMP(6);
+      PG_SLICE(4, w, wn);
 
-      // ================= F: mlp c_proj + residual =================
+      // ================= F: mlp projection row + residual =================
+      const float biasF = cld(w.c_proj_mlp_b + row_of(d0, d1, 0));
+      // rounds of reading this wavefront's share of h, until the service wavefront has
+      // seen a complete one
+      for (;;) {
+        const int r = wait_either(ctl, 3, epoch_of(p, t, l, 4), 7, hseq + 1, abort_word);
+        if (r == 0) ok = false;
+        if (r != 2) break;
+        ++hseq;
+        const unsigned code = h_share<I / 64>(p.h_t, epoch_of(p, t, l, 4), lds.xsF, wave, lane);
+        lds_fence();
+        if (lane == 0) ctl->hstat[wave] = (hseq << 8) | code;
+      }
+      if (!ok) break;
+      SSTAMP(10);
+      if (p.prof) {  // development: how long the row's last loads are still in flight
+        vm_drain();
+        SSTAMP(12);
+      }
       {
-        const float bias = w.c_proj_mlp_b[d0 + min(tid, d1 - d0 - 1)];
-        __syncthreads();  // every wave is done with xs (input of phase E)
-        bool ok = poll_vec<NEI>(p.h_t, I, epoch_of(p, t, l, 4), xs, abort_word);
-        if (!all_ok(ok, sm)) return;
-        // The next layer's c_attn rows (after the last layer this re-reads its own
-        // rows: an unconditional request keeps the load count exact; unused).  One row
-        // per wavefront now, the rest once F's own tiles are consumed.
-        const f4* Wn4 = reinterpret_cast<const f4*>(p.layers[min(l + 1, p.L - 1)].c_attn_w);
-        load_tile<J>(WA[0], Wn4 + (size_t)row_of(a0, a1, 0) * K4, K4, lane);
+        lf4p x4 = (lf4p)lds.xsF;
+        float a0_ = 0.f, a1_ = 0.f, a2_ = 0.f, a3_ = 0.f;
+        constexpr int B = 5;  // LDS reads kept in flight together
 #pragma unroll
-        for (int i = 0; i < TF; ++i) {
-          const int id = wave + kWavesP * i;
-          f4 xr[J];
-          load_x<J>(xr, xs + (size_t)(min(id, nF - 1) & 3) * C, K4, lane);
-          const float v = dot_tile<J>(WF[i], xr);
-          if (lane == 0 && id < nF) sm.psum[id] = v;
+        for (int j0 = 0; j0 < JF; j0 += B) {
+          f4 x[B];
+          // keeps the LDS reads of later groups from being moved up here (they would
+          // all be live at once next to the weight row)
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int b = 0; b < B; ++b)
+            if (j0 + b < JF) x[b] = x4[lane + 64 * (j0 + b)];
+#pragma unroll
+          for (int b = 0; b < B; ++b)
+            if (j0 + b < JF) {
+              a0_ += WF.w[j0 + b].x * x[b].x;
+              a1_ += WF.w[j0 + b].y * x[b].y;
+              a2_ += WF.w[j0 + b].z * x[b].z;
+              a3_ += WF.w[j0 + b].w * x[b].w;
+            }          if (j0 == 0) SSTAMP(8);
+          if (j0 == 2 * B) SSTAMP(9);
         }
+        const float v = wsum((a0_ + a1_) + (a2_ + a3_));
+        const int r = d0 + wave;
+        if (lane == 0 && r < d1) PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), lds.xraw2[r] + (biasF + v)));
+      }
+      SSTAMP(7);
+      PG_SLICE(5, w, wn);
+    }  // layers
+    if (!ok) break;
+
+    // ================= lm_head rows (rust.rs:982-1002) + band argmax =================
+    if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
+      const int wave = wave_id();
+      const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
+      float* const logits = p.logits;
+      Tile<J> T[kLmTiles];
 #pragma unroll
-        for (int i = 1; i < TA; ++i)
-          load_tile<J>(WA[i], Wn4 + (size_t)row_of(a0, a1, i) * K4, K4, lane);
-        __syncthreads();
-        if (tid < d1 - d0) {
-          const int r = d0 + tid;
-          const float s4 = (sm.psum[4 * tid] + sm.psum[4 * tid + 1]) +
-                           (sm.psum[4 * tid + 2] + sm.psum[4 * tid + 3]);
-          PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), xraw[r] + (bias + s4)));
+      for (int k = 0; k < kLmTiles; ++k)
+        load_tile<J>(T[k], wte4 + (size_t)min(v0 + wave + kSW * k, v1 - 1) * K4, K4, lane);
+      const unsigned epl = epoch_of(p, t, p.L, 5);
+      if (!wait_flag(ctl, 4, epl, abort_word)) {
+        ok = false;
+        break;
+      }
+      f4 xr[J];
+      load_x<J>(xr, lds.xsD, K4, lane);
+      Best best{-INFINITY, 0xffffffffu};
+      for (int r = v0 + wave; r < v1; r += kSW * kLmTiles) {
+#pragma unroll
+        for (int k = 0; k < kLmTiles; ++k) {
+          const int rk = r + kSW * k;
+          const float v = dot_tile<J>(T[k], xr);
+          load_tile<J>(T[k], wte4 + (size_t)min(rk + kSW * kLmTiles, v1 - 1) * K4, K4, lane);
+          if (rk < v1) {
+            if (lane == 0) gst(logits + rk, v);
+            if (v > best.v) best = Best{v, (unsigned)rk};
+          }
         }
       }
-      PG_STAMP(l, 5);
-    }  // layers
-
-    // ================= LN_f + lm_head (rust.rs:982-1002) =================
-    if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
-      __syncthreads();
-      if (!lm_head_phase<C_>(pc, sm, xs, xraw, t, v0, v1)) return;
-      PG_STAMP(p.L, 6);
+      if (lane == 0) {
+        ctl->bestv[wave] = best.v;
+        ctl->besti[wave] = best.i;
+      }
+      lds_fence();
+      if (lane == 0) ctl->lmdone[wave] = epl;
     }
   }  // tokens
+  vm_drain();  // nothing of this wavefront is still in flight when it ends
+#undef SSTAMP
+#undef PG_SLICE
+}
 
-  if (!stopped && p.select_last && p.n_fwd > 0) {
-    float* bv = xs;
-    __syncthreads();
-    bool ok = poll_vec<1>(p.best_t, 2 * G, epoch_of(p, p.n_fwd - 1, p.L, 6), bv, abort_word);
-    if (!all_ok(ok, sm)) return;
-    if (wg == 0 && tid == 0) {
-      Best b{-INFINITY, 0xffffffffu};
-      for (int g = 0; g < G; ++g) b = better(b, Best{bv[2 * g], __float_as_uint(bv[2 * g + 1])});
-      unsigned tk = b.i == 0xffffffffu ? 0u : b.i;
-      if (p.out_ids) p.out_ids[p.n_fwd] = tk;
-      p.d_tok[0] = tk;
-    }
+// C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
+template <int C_>
+__global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
+  constexpr int C = C_, I = 4 * C_;
+  // 16-byte LDS accesses run at full speed only on 16-byte boundaries: the dynamic block
+  // starts on one whatever the size of the static control block before it
+  extern __shared__ __attribute__((aligned(256))) float dyn[];
+  __shared__ Ctl ctl_block;
+  ctlp ctl = (ctlp)&ctl_block;
+  Lds lds;
+  lds.xsA = (lfp)dyn;
+  lds.xsD = lds.xsA + C;
+  lds.xsE = lds.xsA + 2 * C;
+  lds.xraw1 = lds.xsA + 3 * C;
+  lds.xraw2 = lds.xsA + 4 * C;
+  lds.xsF = lds.xsA + 5 * C;
+  lds.ts = (lu64p)(lds.xsA + 5 * C + I);
+  if (p.prof)
+    for (int i = threadIdx.x; i < kTsLayers * 16; i += kThreads) lds.ts[i] = 0;
+
+  if (threadIdx.x < 8) {
+    ctl->flag[threadIdx.x] = 0u;
+    ctl->lmdone[threadIdx.x] = 0u;
+    ctl->bdone[threadIdx.x] = 0u;
+    ctl->hstat[threadIdx.x] = 0u;
   }
-  if (wg == 0 && tid == 0) {
-    p.status[1] = (unsigned)t;
-    p.status[2] = (unsigned)stopped;
-  }
+  if (threadIdx.x == 0) ctl->halt = 0u;
+  __syncthreads();
+
+  if ((threadIdx.x >> 6) == kSW)
+    service_wave<C_>(p, ctl, lds);
+  else
+    streamer_wave<C_>(p, ctl, lds);
 }
 
 }  // namespace
 
-// n_embd values the persistent kernel is instantiated for (GPT-2 small, medium, XL).
+size_t persistent_lds_bytes(int C) {
+  return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8;
+}
+// n_embd values the kernel is instantiated for (GPT-2 small, medium, XL).
 bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }
 int persistent_grid() { return kGrid; }
-
-size_t persistent_lds_bytes(int C) { return (size_t)(5 * C) * sizeof(float); }  // xs [4C] + xraw [C]
+int persistent_max_item_keys() { return kMaxItemKeys; }
 
 namespace {
 template <int C_>
@@ -865,12 +1361,9 @@ hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
 
 hipError_t persistent_max_blocks_per_cu(int C, int* out) {
   const size_t lds = persistent_lds_bytes(C);
-  if (C == 768)
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<768>, kThreads, lds);
-  if (C == 1024)
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1024>, kThreads, lds);
-  if (C == 1600)
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1600>, kThreads, lds);
+  if (C == 768) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<768>, kThreads, lds);
+  if (C == 1024) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1024>, kThreads, lds);
+  if (C == 1600) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1600>, kThreads, lds);
   *out = 0;
   return hipSuccess;
 }

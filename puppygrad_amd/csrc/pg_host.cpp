@@ -62,7 +62,6 @@ struct pg_gpt2_model {
   std::vector<pgk::LayerW> layers;
   pgk::LayerW* d_layers = nullptr;  // the same table in device memory
   bool persistent = false;          // batch-1 decode runs as one persistent launch
-  bool ws = false;                  // ... of the wave-specialised kernel
   int persistent_grid = 0;          // workgroups of that launch (one per CU)
   int attn_splits = 1;              // key splits per head in the persistent kernel
   int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
@@ -357,7 +356,7 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   std::lock_guard<std::mutex> lk(g_persistent_mu);
   PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
   if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
-  PG_HIP(m->ws ? pgk::launch_decode_ws(p, c->stream) : pgk::launch_decode_persistent(p, c->stream));
+  PG_HIP(pgk::launch_decode_persistent(p, c->stream));
   if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
   PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
                         c->stream));
@@ -742,14 +741,8 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     int blocks_per_cu = 0;
     bool shape_ok = !bf && g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
                     g.P <= 4096 && g.V >= (size_t)grid;
-    // Development aid: PG_DECODE_KERNEL=v1 selects the older all-waves-poll kernel.
-    const char* which = std::getenv("PG_DECODE_KERNEL");
-    m->ws = !(which && std::strcmp(which, "v1") == 0);
     if (shape_ok) {
-      if (m->ws)
-        PG_HIP(pgk::ws_max_blocks_per_cu((int)g.C, &blocks_per_cu));
-      else
-        PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu));
+      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu));
       shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
     }
     if (shape_ok) {

@@ -154,15 +154,8 @@ struct DecodeParams {
 bool persistent_supports(int C);
 int persistent_grid();
 size_t persistent_lds_bytes(int C);
+int persistent_max_item_keys();
 hipError_t persistent_max_blocks_per_cu(int C, int* out);
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
-
-// Wave-specialised form of the same kernel (pg_decode_ws.hip): same parameters, tagged
-// buffers and results; seven wavefronts stream weights, one runs the dependency chain.
-int ws_grid();
-size_t ws_lds_bytes(int C);
-int ws_max_item_keys();
-hipError_t ws_max_blocks_per_cu(int C, int* out);
-hipError_t launch_decode_ws(const DecodeParams& p, hipStream_t s);
 
 }  // namespace pgk
