@@ -82,6 +82,8 @@ struct pg_kv_cache {
   size_t seq_len = 0;
   float* kv = nullptr;  // [L][2][B][H][P][hd]
   // per-sequence activation scratch, [B][...]
+  float* gemm_ws = nullptr;      // split-K partial tiles of the batched decode step
+  size_t gemm_ws_floats = 0;
   float *x = nullptr, *q = nullptr, *hbuf = nullptr, *part_acc = nullptr, *part_m = nullptr,
         *part_l = nullptr, *logits_buf = nullptr;
   float *qkv_b = nullptr, *xn_b = nullptr, *att_b = nullptr;  // batched step: [B][3C], [B][C], [B][C]
@@ -397,10 +399,13 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   const int T = (int)n, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
   hipStream_t s = c->stream;
   pg_status st;
-  DevBuf X, XN, QKV, ATT, HB, IDS, SCR, LOG;
+  DevBuf X, XN, QKV, ATT, HB, IDS, SCR, LOG, WS;
   if ((st = X.alloc(n * g.C)) || (st = XN.alloc(n * g.C)) || (st = QKV.alloc(n * 3 * g.C)) ||
       (st = ATT.alloc(n * g.C)) || (st = HB.alloc(n * g.I)) || (st = IDS.alloc(n)))
     return st;
+  // split-K partial tiles of the projections back to n_embd columns (up to 8 parts)
+  const size_t ws_floats = 8 * n * g.C;
+  if ((st = WS.alloc(ws_floats))) return st;
   if (hd != 64 && (st = SCR.alloc(n * g.H * n))) return st;
   if (all_logits_dst && (st = LOG.alloc(n * g.V))) return st;
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
@@ -412,6 +417,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = T; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    a.ws = WS.p; a.ws_floats = ws_floats;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   for (size_t l = 0; l < g.L; ++l) {
@@ -463,6 +469,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    a.ws = c->gemm_ws; a.ws_floats = c->gemm_ws_floats;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
@@ -818,6 +825,10 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->x, B * g.C * sizeof(float)));
   PG_HIP(hipMalloc(&raw->q, B * g.C * sizeof(float)));
   PG_HIP(hipMalloc(&raw->hbuf, B * g.I * sizeof(float)));
+  if (B > 1) {
+    raw->gemm_ws_floats = 8 * B * std::max<size_t>(3 * g.C, g.I);
+    PG_HIP(hipMalloc(&raw->gemm_ws, raw->gemm_ws_floats * sizeof(float)));
+  }
   PG_HIP(hipMalloc(&raw->part_acc, parts * hd * sizeof(float)));
   PG_HIP(hipMalloc(&raw->part_m, parts * sizeof(float)));
   PG_HIP(hipMalloc(&raw->part_l, parts * sizeof(float)));
@@ -860,6 +871,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->x);
     (void)hipFree(c->q);
     (void)hipFree(c->hbuf);
+    if (c->gemm_ws) (void)hipFree(c->gemm_ws);
     (void)hipFree(c->part_acc);
     (void)hipFree(c->part_m);
     (void)hipFree(c->part_l);

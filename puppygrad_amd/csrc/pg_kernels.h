@@ -109,8 +109,11 @@ struct GemmArgs {
   float* C;
   int M, N, K;
   int lda, ldc;
+  float* ws = nullptr;    // optional workspace for the split-K form (may be nullptr)
+  size_t ws_floats = 0;   // its size
 };
 bool gemm_supported(const GemmArgs& a);
+int gemm_split_parts(const GemmArgs& a, int num_cus);
 hipError_t launch_gemm(const GemmArgs& a, int epilogue, int num_cus, hipStream_t s);
 // Causal attention over qkv[T][3C] -> out[T][C]; also appends K, V to the cache panels.
 // scratch ([T*H][T] floats) is only used when head_dim != 64.

@@ -9,6 +9,8 @@
 
 #include <math.h>
 
+#include <algorithm>
+
 namespace pgk {
 
 namespace {
@@ -53,7 +55,11 @@ __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
   return *reinterpret_cast<const f4*>(W + idx);
 }
 
-template <int BM, int BN, int EPI, bool WBF>
+// With SPLIT the K range is cut into gridDim.y parts: part blockIdx.y multiplies its
+// k-tiles and writes the raw partial tile to a.ws[part][M][N]; k_splitk_reduce adds the
+// parts in order and applies bias and epilogue (a fixed order: results do not depend on
+// timing).  It fills the chip when M x N alone gives fewer tiles than there are CUs.
+template <int BM, int BN, int EPI, bool WBF, bool SPLIT = false>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
@@ -96,15 +102,18 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   f4 ra[ALD], rb[BLD];
+  const size_t kfirst = SPLIT ? (size_t)(((long)blockIdx.y * (a.K / BK)) / gridDim.y) * BK : 0;
 #pragma unroll
-  for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i]);
+  for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + kfirst);
 #pragma unroll
-  for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i]);
+  for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i] + kfirst);
 
-  const int ktiles = a.K / BK;
+  const int ktiles_all = a.K / BK;
+  const int kt0 = SPLIT ? (int)(((long)blockIdx.y * ktiles_all) / gridDim.y) : 0;
+  const int kt1 = SPLIT ? (int)(((long)(blockIdx.y + 1) * ktiles_all) / gridDim.y) : ktiles_all;
   const int half = lane >> 5, l32 = lane & 31;
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int buf = kt & 1;
+  for (int kt = kt0; kt < kt1; ++kt) {
+    const int buf = (kt - kt0) & 1;
     // registers -> LDS (transposed)
 #pragma unroll
     for (int i = 0; i < ALD; ++i) {
@@ -121,7 +130,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
       Bs[buf][lk + 3][lr + 64 * i] = rb[i].w;
     }
     __syncthreads();
-    if (kt + 1 < ktiles) {
+    if (kt + 1 < kt1) {
 #pragma unroll
       for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + (size_t)(kt + 1) * BK);
 #pragma unroll
@@ -151,6 +160,15 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     for (int j = 0; j < NB; ++j) {
       const int n = n0 + wn * WN + 32 * j + l32;
       if (n >= a.N) continue;
+      if (SPLIT) {
+        float* part = a.ws + (size_t)blockIdx.y * a.M * a.N;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+          if (m < a.M) part[(size_t)m * a.N + n] = acc[i][j][v];
+        }
+        continue;
+      }
       const float bias = a.bias ? a.bias[n] : 0.0f;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -164,6 +182,28 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     }
 }
 
+// C = epilogue(bias + part[0] + part[1] + ...) for the split-K form of k_gemm; one
+// float4 of a row per thread (N is a multiple of 4 whenever the split is used).
+template <int EPI>
+__global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
+  const size_t i4 = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t n4 = (size_t)a.N / 4;
+  if (i4 >= (size_t)a.M * n4) return;
+  const size_t m = i4 / n4, n = (i4 - m * n4) * 4;
+  const size_t stride = (size_t)a.M * a.N;
+  f4 s = *reinterpret_cast<const f4*>(a.ws + m * a.N + n);
+  for (int p = 1; p < parts; ++p) s += *reinterpret_cast<const f4*>(a.ws + p * stride + m * a.N + n);
+  f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
+  float c[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
+  float* dst = a.C + m * a.ldc + n;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (EPI == GEMM_GELU) c[k] = gelu_tanh(c[k]);
+    if (EPI == GEMM_RESID) c[k] = a.resid[m * a.ldc + n + k] + c[k];
+    dst[k] = c[k];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // causal_self_attention (src/models/gpt2/rust.rs:1580-1659) for head_dim 64 over an
 // interleaved qkv[T][3C] buffer.  One wavefront owns 32 queries of one head and
@@ -175,19 +215,23 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 // (rust.rs:1590, 1634).  It also appends K and V to the cache panels
 // ([head][position][64], kv_index at rust.rs:1851-1855).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(128) void k_attn_prefill64(const float* __restrict__ qkv, int T,
+__global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict__ qkv, int T,
                                                         int C, int P, float* __restrict__ kcache,
                                                         float* __restrict__ vcache,
                                                         float* __restrict__ out) {
-  constexpr int KT = 32;  // keys per tile
-  __shared__ float Kt[2][64][KT + 1];   // per wavefront: [d][key]
-  __shared__ float Vs[2][KT][64 + 4];   // per wavefront: [key][d]
+  constexpr int KT = 32;   // keys per tile
+  constexpr int NWV = 4;   // wavefronts per block: they share one block of 32 queries and
+                           // take the key tiles round-robin, each with its own running
+                           // (max, sum, O) that are merged through LDS at the end
+  __shared__ float Kt[NWV][64][KT + 1];   // per wavefront: [d][key]
+  __shared__ float Vs[NWV][KT][64 + 4];   // per wavefront: [key][d]
+  __shared__ float Ms[NWV][32], Ls[NWV][32];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
   const int h = blockIdx.y;
-  const int qb = blockIdx.x * 2 + wave;  // block of 32 queries
+  const int nqb = (T + 31) / 32;
+  const int qb = nqb - 1 - (int)blockIdx.x;  // the longest rows first
   const int q0 = qb * 32;
-  if (q0 >= T) return;
   const int C3 = 3 * C;
   const float* qbase = qkv + h * 64;
   const float* kbase = qkv + C + h * 64;
@@ -209,10 +253,10 @@ __global__ __launch_bounds__(128) void k_attn_prefill64(const float* __restrict_
   float (*kt)[KT + 1] = Kt[wave];
   float (*vs)[64 + 4] = Vs[wave];
   const int last_tile = min(q0 + 31, T - 1) / KT;
-  for (int tile = 0; tile <= last_tile; ++tile) {
+  for (int tile = wave; tile <= last_tile; tile += NWV) {
     const int k0 = tile * KT;
     // stage K (transposed) and V of 32 keys; also append them to the cache once
-    // (by the wavefront whose query block starts at this tile: q0 == k0)
+    // (by the wavefront that meets the tile on the diagonal: q0 == k0)
     for (int i = lane; i < KT * 16; i += 64) {
       const int key = i >> 4, d4 = (i & 15) * 4;
       const int kk = min(k0 + key, T - 1);
@@ -247,13 +291,15 @@ __global__ __launch_bounds__(128) void k_attn_prefill64(const float* __restrict_
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
-    // a fully masked tile cannot occur for a valid query (key 0 <= qi); for lanes
-    // past T (clamped duplicates) qi >= T is still >= key 0
-    const float corr = expf(m_run - m_new);
+    // a tile can be fully masked for a query only on the diagonal tile's upper part,
+    // and there key k0 <= qi always holds for the first key: m_new is finite from the
+    // first tile a wavefront sees (tile 0 .. 3 hold keys <= q0 for every later block;
+    // a wavefront that never gets a tile keeps the neutral (-inf, 0, 0))
+    const float corr = (m_run == -INFINITY) ? 0.0f : expf(m_run - m_new);
     float psum = 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const float pv = expf(sacc[v] - m_new);
+      const float pv = (m_new == -INFINITY) ? 0.0f : expf(sacc[v] - m_new);
       sacc[v] = pv;
       psum += pv;
     }
@@ -272,15 +318,40 @@ __global__ __launch_bounds__(128) void k_attn_prefill64(const float* __restrict_
     }
     __builtin_amdgcn_wave_barrier();
   }
-  // normalise and write: lane holds d = 8*(v/4) + 4*half + v%4 (+32) of query qi
+  // ---- merge the wavefronts' results (in wavefront order: results do not depend on timing)
+  if (half == 0) {
+    Ms[wave][l32] = m_run;
+    Ls[wave][l32] = l_run;
+  }
+  __syncthreads();  // every wavefront is done with its K/V tiles too
+  float M = Ms[0][l32];
+#pragma unroll
+  for (int w = 1; w < NWV; ++w) M = fmaxf(M, Ms[w][l32]);
+  const float mine = (m_run == -INFINITY) ? 0.0f : expf(m_run - M);
+  float L = 0.0f;
+#pragma unroll
+  for (int w = 0; w < NWV; ++w) {
+    const float mw = Ms[w][l32];
+    L += ((mw == -INFINITY) ? 0.0f : expf(mw - M)) * Ls[w][l32];
+  }
+  // O^T of the four wavefronts through LDS (the K tiles' space: [wave][d 0..63][query])
+  float (*ob)[KT + 1] = Kt[wave];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int d = 8 * (v >> 2) + 4 * half + (v & 3);
+    ob[d][l32] = o0[v] * mine;
+    ob[32 + d][l32] = o1[v] * mine;
+  }
+  __syncthreads();
+  // wavefront w writes d in [16 w, 16 w + 16): lane -> (query l32, 8 d values by half)
   if (qi < T) {
-    const float inv = 1.0f / l_run;
+    const float inv = 1.0f / L;
     float* dst = out + (size_t)qi * C + h * 64;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int d = 8 * (v >> 2) + 4 * half + (v & 3);
-      dst[d] = o0[v] * inv;
-      dst[32 + d] = o1[v] * inv;
+    for (int j = 0; j < 8; ++j) {
+      const int d = 16 * wave + 8 * half + j;
+      const float sum = (Kt[0][d][l32] + Kt[1][d][l32]) + (Kt[2][d][l32] + Kt[3][d][l32]);
+      dst[d] = sum * inv;
     }
   }
 }
@@ -382,8 +453,45 @@ bool gemm_supported(const GemmArgs& a) {
          (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.W) & 15) == 0;
 }
 
+namespace {
+template <bool WBF>
+hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s) {
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int grid = (tiles + 7) / 8 * 8;
+  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, true>), dim3(grid, parts), dim3(256), 0, s, a);
+  const unsigned rblocks = (unsigned)(((size_t)a.M * (a.N / 4) + 255) / 256);
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL(k_splitk_reduce<GEMM_BIAS>, dim3(rblocks), dim3(256), 0, s, a, parts);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL(k_splitk_reduce<GEMM_GELU>, dim3(rblocks), dim3(256), 0, s, a, parts);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL(k_splitk_reduce<GEMM_RESID>, dim3(rblocks), dim3(256), 0, s, a, parts);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+}  // namespace
+
+// Parts the K range is cut into (1 = no split): when the 64x64 tiles of C are fewer than
+// about 1.5 per CU, enough parts for about three work items per CU.  A part is at least
+// 512 deep for tall operands; for a batch of a few rows (decode), where the job is to
+// stream W at the speed of HBM, 128.  Needs the workspace a.ws of parts x M x N floats.
+int gemm_split_parts(const GemmArgs& a, int num_cus) {
+  const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
+  if (!a.ws || a.N % 4 != 0 || tiles * 2 >= 3L * num_cus) return 1;
+  const int depth = a.M < 64 ? 128 : 512;
+  int parts = (int)((3L * num_cus) / tiles);
+  parts = std::min(parts, a.K / depth);
+  parts = std::min(parts, 8);
+  while (parts > 1 && (size_t)parts * a.M * a.N > a.ws_floats) --parts;
+  return std::max(parts, 1);
+}
+
 hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
+  const int parts = gemm_split_parts(a, num_cus);
+  if (parts > 1)
+    return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s) : launch_gemm_split<false>(a, epi, parts, s);
   // 128x128 tiles once they fill the chip about twice over, 64x64 tiles otherwise
   const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
   if (a.w_bf16) {
@@ -399,8 +507,8 @@ hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_d
                                hipStream_t s) {
   if (head_dim == 64) {
     const int qblocks = (T + 31) / 32;
-    hipLaunchKernelGGL(k_attn_prefill64, dim3((qblocks + 1) / 2, H), dim3(128), 0, s, qkv, T, C, P,
-                       kcache, vcache, out);
+    hipLaunchKernelGGL(k_attn_prefill64, dim3(qblocks, H), dim3(256), 0, s, qkv, T, C, P, kcache,
+                       vcache, out);
   } else {
     const int n = T * H;
     hipLaunchKernelGGL(k_attn_prefill_any, dim3((n + 127) / 128), dim3(128), 0, s, qkv, T, C, H,
