@@ -55,6 +55,7 @@ constexpr int kSW = 7;      // streamer wavefronts (0..6); wavefront 7 is the se
 constexpr int kGrid = 256;  // workgroups; row bands are computed for exactly this many
 constexpr unsigned kSpinLimit = 1u << 21;
 constexpr int kMaxItemKeys = 128;  // keys per (head, split) attention item
+constexpr int kPace = 4;           // loads per pacing group of a slice
 constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
 
 // Tagged words and the abort word live in global memory; saying so in the pointer type
@@ -1059,6 +1060,11 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
     const int ln = opaque(lane);
 #pragma unroll
     for (int n = N0; n < N1; ++n) {
+      // Pacing: a long slice goes out in groups of kPace loads, the next group only once
+      // at most kPace of this wavefront's loads are still in flight.  What the streamers
+      // have in flight delays the service wavefront's polls (in-order return per CU), so
+      // this bounds that delay by the time of about two groups instead of a whole slice.
+      if (n > N0 && (n - N0) % kPace == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
       if (n < SP::ND) {
         WD[0].w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n, ln);
       } else if (n < SP::ND + SP::NE) {
