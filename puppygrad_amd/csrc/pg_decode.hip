@@ -201,6 +201,14 @@ __device__ __forceinline__ f4 ld_row(const f4* row, unsigned byte_off) {
   typedef const char __attribute__((address_space(1)))* gcp;
   return __builtin_nontemporal_load((gf4p)((gcp)row + byte_off));
 }
+// The same load with LDS as its destination: lane i's 16 bytes land at dst + 16 i (dst
+// is wave-uniform).  It is counted with the vector loads and completes in order with
+// them.
+__device__ __forceinline__ void ld_row_lds(const f4* row, unsigned byte_off, lfp dst) {
+  typedef const char __attribute__((address_space(1)))* gcp;
+  __builtin_amdgcn_global_load_lds((gf4p)((gcp)row + byte_off), (__attribute__((address_space(3))) void*)dst, 16, 0,
+                                   2 /* nt */);
+}
 template <int J>
 __device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
 #pragma unroll
@@ -462,6 +470,7 @@ __device__ __forceinline__ void wave_layer_norm(lfp raw, const float (&g)[NW], c
 
 struct Lds {
   lfp xsA, xsD, xsE, xraw1, xraw2, xsF;
+  lfp stage;  // [streamer][FS][64] float4: the staged part of the mlp projection rows
   lu64p ts;  // development timestamps of the launch's last token: [layer 0..L][16]
 };
 constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
@@ -995,16 +1004,32 @@ struct StreamPlan {
   static constexpr int JF = C_ / 64;  // float4 per lane of one 4C-wide row
   // loads per layer and wavefront, in stream order
   static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
-  // Equal cuts where the registers allow it.  The widest model cannot hold the c_fc rows
-  // next to much of the mlp projection row: its first four slices are shorter and the
-  // last two longer (those two phases then run at the speed of the stream).
+  // Six equal cuts.  The widest model cannot hold the c_fc rows next to much of the mlp
+  // projection row in registers: the first FS float4 per lane of that row are copied
+  // straight into LDS instead (the same loads, in the same order, with LDS as their
+  // destination) and read from there by the product.
   static constexpr bool kTight = (ND + NE + NF) * 4 > 200;
+  static constexpr int FS = kTight ? 12 : 0;
+  // (the first slice goes out next to the c_attn rows and their product: it is the one
+  // cut short where those leave fewer registers)
+  static constexpr int kRegsA = 31, kRegs = 36;  // float4 per lane a product can sit next to
+  static constexpr int c1 = NL / 6 < kRegsA - NA ? NL / 6 : kRegsA - NA;
+#ifndef PG_CUTS
+#define PG_CUTS 0, 9, 20, 31, 48, 66, 81
+#endif
   static constexpr int cut(int k) {
-    if (!kTight || k == 0 || k == 6) return k * NL / 6;
-    const int c4 = ND + NE + 4;
-    if (k <= 4) return k * c4 / 4;
-    return (c4 + NL) / 2 > ND + NE + NF ? (c4 + NL) / 2 : ND + NE + NF;
+    if (!kTight) return k == 0 ? 0 : c1 + (k - 1) * (NL - c1) / 5;
+    constexpr int c[7] = {PG_CUTS};
+    return c[k];
   }
+  // float4 per lane resident in registers at the three products that run next to rows
+  // of later phases (after slices 2, 3 and 0)
+  static constexpr int in_regs(int n) {  // of the loads [0, n): those held in registers
+    const int f = n - ND - NE;
+    return n - (f <= 0 ? 0 : (f < FS ? f : FS));
+  }
+  static_assert(in_regs(cut(3)) <= kRegs && in_regs(cut(4)) - ND <= kRegs && NA + in_regs(cut(1)) <= kRegsA,
+                "weight rows resident next to a product fit the register file");
   // slice k is requested: 0 after A, 1 and 2 on the attention credits, 3 after D,
   // 4 after E, 5 after F.  D is used after slice 2, E after 3, F after 4, A' after 5.
   static_assert(ND <= cut(3), "c_proj row is requested before it is used");
@@ -1072,8 +1097,11 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
       } else if (n < SP::ND + SP::NE + SP::NF) {
         const int j = n - SP::ND - SP::NE;
-        WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
-                         ((unsigned)ln + 64u * j) * 16u);
+        const f4* row = reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C;
+        if (j < SP::FS)
+          ld_row_lds(row, ((unsigned)ln + 64u * j) * 16u, lds.stage + (wave_id() * SP::FS + j) * 256);
+        else
+          WF.w[j] = ld_row(row, ((unsigned)ln + 64u * j) * 16u);
       } else {
         const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
         WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
@@ -1220,7 +1248,10 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         SSTAMP(12);
       }
       {
-        lf4p x4 = (lf4p)lds.xsF;
+        // (the lane's LDS addresses are rebuilt here, not kept in registers across the layer)
+        const int ln = opaque(lane);
+        lf4p x4 = (lf4p)lds.xsF + ln;
+        lf4p ws4 = (lf4p)(lds.stage + wave * SP::FS * 256) + ln;
         float a0_ = 0.f, a1_ = 0.f, a2_ = 0.f, a3_ = 0.f;
         constexpr int B = 5;  // LDS reads kept in flight together
 #pragma unroll
@@ -1231,14 +1262,15 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
           asm volatile("" ::: "memory");
 #pragma unroll
           for (int b = 0; b < B; ++b)
-            if (j0 + b < JF) x[b] = x4[lane + 64 * (j0 + b)];
+            if (j0 + b < JF) x[b] = x4[64 * (j0 + b)];
 #pragma unroll
           for (int b = 0; b < B; ++b)
             if (j0 + b < JF) {
-              a0_ += WF.w[j0 + b].x * x[b].x;
-              a1_ += WF.w[j0 + b].y * x[b].y;
-              a2_ += WF.w[j0 + b].z * x[b].z;
-              a3_ += WF.w[j0 + b].w * x[b].w;
+              const f4 wv = (j0 + b < SP::FS) ? ws4[64 * (j0 + b)] : WF.w[j0 + b];
+              a0_ += wv.x * x[b].x;
+              a1_ += wv.y * x[b].y;
+              a2_ += wv.z * x[b].z;
+              a3_ += wv.w * x[b].w;
             }          if (j0 == 0) SSTAMP(8);
           if (j0 == 2 * B) SSTAMP(9);
         }
@@ -1310,6 +1342,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
   lds.xraw2 = lds.xsA + 4 * C;
   lds.xsF = lds.xsA + 5 * C;
   lds.ts = (lu64p)(lds.xsA + 5 * C + I);
+  lds.stage = lds.xsA + 9 * C + kTsLayers * 32;
   if (p.prof)
     for (int i = threadIdx.x; i < kTsLayers * 16; i += kThreads) lds.ts[i] = 0;
 
@@ -1331,7 +1364,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 }  // namespace
 
 size_t persistent_lds_bytes(int C) {
-  return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8;
+  const int fs = C == 1600 ? StreamPlan<1600>::FS : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
+  return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8 + (size_t)kSW * fs * 1024;
 }
 // n_embd values the kernel is instantiated for (GPT-2 small, medium, XL).
 bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }

@@ -98,6 +98,7 @@ struct pg_kv_cache {
   unsigned long long *qkv_t = nullptr, *part_t = nullptr, *attn_t = nullptr, *xa_t = nullptr,
                      *h_t = nullptr, *xm_t = nullptr, *best_t = nullptr;
   size_t tagged_words = 0;  // total words in the allocation that starts at qkv_t
+  size_t tagged_bytes = 0;  // size of that allocation as the exchange pool counts it
   unsigned* status = nullptr;
   unsigned* h_status = nullptr;  // pinned
   uint32_t* d_force = nullptr;   // [P] prompt ids for a one-launch prefill
@@ -291,6 +292,48 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   }
   return PG_OK;
+}
+
+// The tagged activation words live in uncached device memory: a word written by one
+// workgroup is read by workgroups on other dies, and without a cache level that has to be
+// written through and missed on purpose the hand-over is about a third faster.  Such
+// memory is never given back to the driver once a kernel has read it (tensors allocated
+// after such a free have held wrong values): a destroyed cache returns its block to this
+// pool, and the next cache on that device with room in it takes it over.
+struct ExchangeBlock {
+  int device;
+  size_t bytes;
+  void* p;
+};
+std::mutex g_exchange_mu;
+std::vector<ExchangeBlock> g_exchange_free;
+
+hipError_t exchange_acquire(int device, size_t bytes, void** out, size_t* got_bytes) {
+  bytes = (bytes + 65535) / 65536 * 65536;
+  {
+    std::lock_guard<std::mutex> lk(g_exchange_mu);
+    size_t best = g_exchange_free.size();
+    for (size_t i = 0; i < g_exchange_free.size(); ++i) {
+      const ExchangeBlock& b = g_exchange_free[i];
+      if (b.device == device && b.bytes >= bytes &&
+          (best == g_exchange_free.size() || b.bytes < g_exchange_free[best].bytes))
+        best = i;
+    }
+    if (best != g_exchange_free.size()) {
+      *out = g_exchange_free[best].p;
+      *got_bytes = g_exchange_free[best].bytes;
+      g_exchange_free.erase(g_exchange_free.begin() + (long)best);
+      return hipSuccess;
+    }
+  }
+  *got_bytes = bytes;
+  return hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
+}
+
+void exchange_release(int device, size_t bytes, void* p) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lk(g_exchange_mu);
+  g_exchange_free.push_back(ExchangeBlock{device, bytes, p});
 }
 
 // Persistent launches are serialised process-wide: two of them resident at once
@@ -842,7 +885,8 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   if (m->persistent && batch == 1) {
     const size_t n_part = g.H * pgk::kMaxSplits * 66;
     const size_t words = 3 * g.C + n_part + g.C + g.C + g.I + g.C + 2 * (size_t)m->persistent_grid;
-    PG_HIP(hipMalloc(&raw->qkv_t, words * sizeof(unsigned long long)));
+    PG_HIP(exchange_acquire(raw->device, words * sizeof(unsigned long long),
+                            reinterpret_cast<void**>(&raw->qkv_t), &raw->tagged_bytes));
     raw->tagged_words = words;
     raw->part_t = raw->qkv_t + 3 * g.C;
     raw->attn_t = raw->part_t + n_part;
@@ -882,7 +926,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->d_tok);
     (void)hipFree(c->d_out_ids);
     if (c->h_ids) (void)hipHostFree(c->h_ids);
-    (void)hipFree(c->qkv_t);
+    exchange_release(c->device, c->tagged_bytes, c->qkv_t);
     (void)hipFree(c->status);
     (void)hipFree(c->d_force);
     if (c->h_status) (void)hipHostFree(c->h_status);
