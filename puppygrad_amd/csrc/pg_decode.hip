@@ -203,11 +203,29 @@ __device__ __forceinline__ f4 ld_row(const f4* row, unsigned byte_off) {
 }
 // The same load with LDS as its destination: lane i's 16 bytes land at dst + 16 i (dst
 // is wave-uniform).  It is counted with the vector loads and completes in order with
-// them.
+// them.  Written as assembly on purpose: the compiler treats the instruction as one that
+// may touch both memories and from then on waits for ALL loads in flight at every use of
+// a loaded register or of LDS.  It therefore does not know of these loads: its own counts
+// stay exact for every load requested after them (those return later anyway), and the
+// reader of the staged data waits by hand (stage_wait).  A register load requested BEFORE
+// them and waited for after them is waited for too long, by as many loads as were staged:
+// the staged group goes where that does not matter.
 __device__ __forceinline__ void ld_row_lds(const f4* row, unsigned byte_off, lfp dst) {
-  typedef const char __attribute__((address_space(1)))* gcp;
-  __builtin_amdgcn_global_load_lds((gf4p)((gcp)row + byte_off), (__attribute__((address_space(3))) void*)dst, 16, 0,
-                                   2 /* nt */);
+  unsigned keep;  // m0 holds the LDS address for the instruction and is put back after it
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %2, %3 nt\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(keep)
+      : "s"((unsigned)(size_t)dst), "v"(byte_off), "s"(row)
+      : "memory");
+}
+// All staged loads have landed once at most N younger loads are in flight.
+template <int N>
+__device__ __forceinline__ void stage_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N < 63 ? N : 63) : "memory");
 }
 template <int J>
 __device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int lane) {
@@ -371,6 +389,61 @@ __device__ __forceinline__ u64 ld_tagged(const u64* base, unsigned byte_off) {
   return __hip_atomic_load((__attribute__((address_space(1))) u64*)((gcp)base + byte_off),
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// ---- probes through the scalar data path ------------------------------------------------
+// Vector loads of a CU return in the order they were issued, whichever wavefront issued
+// them, so a vector poll waits behind every weight byte the streamers have in flight.
+// Scalar loads take another path with its own (out-of-order) return, and their round
+// trip stays at about a tenth of a microsecond whatever is being streamed.  "Has it
+// arrived yet" is therefore asked with scalar loads that go past the scalar cache (glc;
+// the words live in uncached memory, so nothing else can hold an old copy); only the
+// one read of the payloads that follows a positive answer is a vector load.  (The scalar
+// path is narrow: reading whole rows of payloads through it was measured slower than the
+// vector read it replaced.)
+typedef unsigned u16x __attribute__((ext_vector_type(16)));
+constexpr unsigned kProbeSpinLimit = 1u << 24;  // a few seconds of scalar probes
+constexpr int kProbeSleep = 4;  // units of 64 clocks between two probes of a wavefront
+// Three lines of eight tagged words each: zero iff all 24 carry `epoch`.
+__device__ __forceinline__ unsigned lines3_diff(const u64* a, const u64* b, const u64* c, unsigned epoch) {
+  u16x va, vb, vc;
+  asm volatile(
+      "s_load_dwordx16 %0, %3, 0x0 glc\n\t"
+      "s_load_dwordx16 %1, %4, 0x0 glc\n\t"
+      "s_load_dwordx16 %2, %5, 0x0 glc\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(va), "=&s"(vb), "=&s"(vc)
+      : "s"(a), "s"(b), "s"(c)
+      : "memory");
+  unsigned d = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) d |= (va[2 * i + 1] ^ epoch) | (vb[2 * i + 1] ^ epoch) | (vc[2 * i + 1] ^ epoch);
+  return d;
+}
+// Spins until lines la, lb, lc (of eight words each) of src carry `epoch`.  Wave-uniform;
+// false on timeout or abort.
+__device__ __forceinline__ bool probe_lines(const u64* src, int la, int lb, int lc, unsigned epoch,
+                                            unsigned* abort_word) {
+  const u64* a = src + 8 * __builtin_amdgcn_readfirstlane(la);
+  const u64* b = src + 8 * __builtin_amdgcn_readfirstlane(lb);
+  const u64* c = src + 8 * __builtin_amdgcn_readfirstlane(lc);
+  unsigned spins = 0;
+  for (;;) {
+    if (lines3_diff(a, b, c, epoch) == 0) return true;
+    if (++spins > kProbeSpinLimit) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+    if ((spins & 127) == 0 && PG_LD32(abort_word) != 0) return false;
+    __builtin_amdgcn_s_sleep(kProbeSleep);
+  }
+}
+// The same over a vector of LINES lines: the line `first` and two more a third of the
+// vector apart (different rows of a vector come from different workgroups).
+template <int LINES>
+__device__ __forceinline__ bool probe_spread(const u64* src, int first, unsigned epoch, unsigned* abort_word) {
+  const int l0 = first % LINES;
+  return probe_lines(src, l0, (l0 + LINES / 3) % LINES, (l0 + 2 * (LINES / 3)) % LINES, epoch, abort_word);
+}
+
 // Spins until run `run` (words 64 run .. 64 run + 63) carries `epoch`.  Cheap: one
 // 512-byte request per attempt.  Wave-uniform; false on timeout or abort.
 __device__ __forceinline__ bool probe_run(const u64* src, int run, unsigned epoch,
@@ -398,18 +471,18 @@ __device__ __forceinline__ int next_probe_run(bool bad, int run_of_bad) {
   return __builtin_amdgcn_readlane(run_of_bad, first);
 }
 // Waits until src[i] carries `epoch` for every i in [0, 64 NE) and leaves the payloads
-// in dst (LDS): the cheap probe of one run (runs differ per workgroup at first, so that
-// the probes spread over memory channels), then a bulk read of lane + 64 e; while that
-// finds stale words, the probe moves to a stale word's run and the bulk read repeats.
-// Nothing but the probe run lives across a repeat: the payloads go to LDS at once.
+// in dst (LDS): scalar probes of three lines (they differ per workgroup), then a bulk read
+// of lane + 64 e; while that finds stale words, the probe moves to a stale word's line
+// and the bulk read repeats.  Nothing but the probe line lives across a repeat: the
+// payloads go to LDS at once.
 template <int NE>
 __device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp dst,
                                           unsigned* abort_word, int probe, lu64p dbg = nullptr) {
   const int lane = opaque((int)threadIdx.x) & 63;
-  unsigned spins = 0;
-  int run = probe % NE;
+  unsigned rounds = 0;
+  int line = probe * 3;
   for (;;) {
-    if (!probe_run(src, run, epoch, abort_word, spins)) return false;
+    if (!probe_spread<8 * NE>(src, line, epoch, abort_word)) return false;
     if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
     bool bad = false;
     int bad_e = 0;
@@ -424,9 +497,11 @@ __device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp ds
       }
       dst[lane + 64 * e] = val_of(v[e]);
     }
-    if (!__any(bad)) return true;
-    run = next_probe_run(bad, bad_e);
-    if (++spins > kSpinLimit) {
+    const unsigned long long m = __ballot(bad);
+    if (m == 0) return true;
+    const int first = __builtin_ctzll(m);
+    line = 8 * __builtin_amdgcn_readlane(bad_e, first) + (first >> 3);
+    if (++rounds > 4096u) {
       PG_ST32(abort_word, 1u);
       return false;
     }
@@ -866,10 +941,12 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       {
         constexpr int RUNS = I / 64;
         const unsigned ep = epoch_of(p, t, l, 4);
-        int run = (wg + 3) % RUNS;
+        int run = -1;  // the run a stale word was seen in
         unsigned spins = 0;
         for (;;) {
-          if (!probe_run(p.h_t, run, ep, abort_word, spins)) PG_SERVICE_FAIL();
+          if (run < 0 ? !probe_spread<8 * RUNS>(p.h_t, (wg + 3) * 5, ep, abort_word)
+                      : !probe_lines(p.h_t, 8 * run, 8 * run + 3, 8 * run + 7, ep, abort_word))
+            PG_SERVICE_FAIL();
           ++hseq;
           if (lane == 0) ctl->flag[7] = hseq;
           unsigned code = h_share<RUNS>(p.h_t, ep, lds.xsF, kSW, lane);
@@ -1004,15 +1081,22 @@ struct StreamPlan {
   static constexpr int JF = C_ / 64;  // float4 per lane of one 4C-wide row
   // loads per layer and wavefront, in stream order
   static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
-  // Six equal cuts.  The widest model cannot hold the c_fc rows next to much of the mlp
-  // projection row in registers: the first FS float4 per lane of that row are copied
-  // straight into LDS instead (the same loads, in the same order, with LDS as their
-  // destination) and read from there by the product.
+  // Loads into registers, in stream order:
+  //     c_proj row | c_fc rows | mlp projection row | next layer's c_attn rows
+  // The widest model cannot hold the c_fc rows next to much of the mlp projection row in
+  // registers: the first FS float4 per lane of that row are copied straight into LDS
+  // instead (the same kind of load, with LDS as its destination) and read from there by
+  // the product.  They take no registers and are requested as one group, in front of
+  // load PS of the stream above.
   static constexpr bool kTight = (ND + NE + NF) * 4 > 200;
   static constexpr int FS = kTight ? 12 : 0;
+#ifndef PG_PS
+#define PG_PS 31
+#endif
+  static constexpr int PS = kTight ? PG_PS : 0;
   // (the first slice goes out next to the c_attn rows and their product: it is the one
   // cut short where those leave fewer registers)
-  static constexpr int kRegsA = 31, kRegs = 36;  // float4 per lane a product can sit next to
+  static constexpr int kRegsA = 31, kRegs = 33;  // float4 per lane a product can sit next to
   static constexpr int c1 = NL / 6 < kRegsA - NA ? NL / 6 : kRegsA - NA;
 #ifndef PG_CUTS
 #define PG_CUTS 0, 9, 20, 31, 48, 66, 81
@@ -1022,18 +1106,17 @@ struct StreamPlan {
     constexpr int c[7] = {PG_CUTS};
     return c[k];
   }
-  // float4 per lane resident in registers at the three products that run next to rows
-  // of later phases (after slices 2, 3 and 0)
-  static constexpr int in_regs(int n) {  // of the loads [0, n): those held in registers
-    const int f = n - ND - NE;
-    return n - (f <= 0 ? 0 : (f < FS ? f : FS));
-  }
+  // of the loads [0, n): those held in registers
+  static constexpr int in_regs(int n) { return n - (n <= PS ? 0 : (n - PS < FS ? n - PS : FS)); }
   static_assert(in_regs(cut(3)) <= kRegs && in_regs(cut(4)) - ND <= kRegs && NA + in_regs(cut(1)) <= kRegsA,
                 "weight rows resident next to a product fit the register file");
+  // the staged group is never cut by a slice boundary, and is requested after the last
+  // product that reads the staging area and before the one that needs it
+  static_assert(PS + FS <= cut(5), "staged part of the mlp projection row is requested before it is used");
   // slice k is requested: 0 after A, 1 and 2 on the attention credits, 3 after D,
   // 4 after E, 5 after F.  D is used after slice 2, E after 3, F after 4, A' after 5.
-  static_assert(ND <= cut(3), "c_proj row is requested before it is used");
-  static_assert(ND + NE <= cut(4), "c_fc rows are requested before they are used");
+  static_assert(in_regs(cut(3)) >= ND, "c_proj row is requested before it is used");
+  static_assert(in_regs(cut(4)) >= ND + NE, "c_fc rows are requested before they are used");
   static_assert(ND + NE + NF <= cut(5), "mlp projection row is requested before it is used");
   static_assert(RD <= kSW, "one mlp projection row per streamer");
   static_assert(C_ % 64 == 0, "4C-wide rows are whole runs of 64 float4");
@@ -1078,8 +1161,9 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
   };
   // Requests loads [N0, N1) of the layer stream: `w` is the layer whose c_proj, c_fc and
   // mlp projection rows are meant, `wn` the one whose c_attn rows follow.
-  auto issue = [&](auto n0_, auto n1_, const LayerW& w, const LayerW& wn) {
+  auto issue = [&](auto n0_, auto n1_, const LayerW& w, const LayerW& wn, auto paced_) {
     constexpr int N0 = decltype(n0_)::value, N1 = decltype(n1_)::value;
+    constexpr bool kPaced = decltype(paced_)::value;
     // the lane index behind an empty asm again: the per-lane parts of the addresses are
     // rebuilt for each slice instead of being kept (and spilled) across the whole layer
     const int ln = opaque(lane);
@@ -1089,34 +1173,38 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       // at most kPace of this wavefront's loads are still in flight.  What the streamers
       // have in flight delays the service wavefront's polls (in-order return per CU), so
       // this bounds that delay by the time of about two groups instead of a whole slice.
-      if (n > N0 && (n - N0) % kPace == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
-      if (n < SP::ND) {
-        WD[0].w[n] = ld_c(w.c_proj_w, row_of(d0, d1, 0), n, ln);
-      } else if (n < SP::ND + SP::NE) {
-        const int i = (n - SP::ND) / J, j = (n - SP::ND) % J;
+      if (kPaced && n > N0 && (n - N0) % kPace == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
+      const int m = n < SP::PS ? n : n - SP::FS;  // index among the loads into registers
+      if (n >= SP::PS && n < SP::PS + SP::FS) {
+        const int j = n - SP::PS;
+        ld_row_lds(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
+                   ((unsigned)ln + 64u * j) * 16u, lds.stage + (wave_id() * SP::FS + j) * 256);
+      } else if (m < SP::ND) {
+        WD[0].w[m] = ld_c(w.c_proj_w, row_of(d0, d1, 0), m, ln);
+      } else if (m < SP::ND + SP::NE) {
+        const int i = (m - SP::ND) / J, j = (m - SP::ND) % J;
         WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
-      } else if (n < SP::ND + SP::NE + SP::NF) {
-        const int j = n - SP::ND - SP::NE;
-        const f4* row = reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C;
-        if (j < SP::FS)
-          ld_row_lds(row, ((unsigned)ln + 64u * j) * 16u, lds.stage + (wave_id() * SP::FS + j) * 256);
-        else
-          WF.w[j] = ld_row(row, ((unsigned)ln + 64u * j) * 16u);
+      } else if (m < SP::ND + SP::NE + SP::NF - SP::FS) {
+        const int j = m - SP::ND - SP::NE + SP::FS;  // FS <= j < NF
+        WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
+                         ((unsigned)ln + 64u * j) * 16u);
       } else {
         const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
         WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
       }
     }
   };
+  // (slice 0 goes out in one piece: it stands before a product, which must not wait)
 #define PG_SLICE(k, w, wn)                                              \
   issue(std::integral_constant<int, SP::cut(k)>{},                      \
-        std::integral_constant<int, SP::cut((k) + 1)>{}, (w), (wn))
+        std::integral_constant<int, SP::cut((k) + 1)>{}, (w), (wn),     \
+        std::integral_constant<bool, (k) != 0>{})
 
   // before the first layer: its c_attn rows
   {
     const LayerW w0 = layer_of(p.layers, 0);
     issue(std::integral_constant<int, SP::ND + SP::NE + SP::NF>{},
-          std::integral_constant<int, SP::NL>{}, w0, w0);
+          std::integral_constant<int, SP::NL>{}, w0, w0, std::true_type{});
   }
 
   // development timestamps of streamer 0 (slots 5.. of the layer's 16)
@@ -1248,6 +1336,9 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         SSTAMP(12);
       }
       {
+        // the staged part of the row: complete once only the c_attn rows requested after
+        // the row's last registers are still in flight
+        if (SP::FS) stage_wait<SP::cut(5) - (SP::ND + SP::NE + SP::NF)>();
         // (the lane's LDS addresses are rebuilt here, not kept in registers across the layer)
         const int ln = opaque(lane);
         lf4p x4 = (lf4p)lds.xsF + ln;
