@@ -51,6 +51,8 @@ def main() -> int:
     ap.add_argument("--prefill", type=int, default=None, help="tokens in the cache before decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
+                    help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this path runs on ONE GPU (batch-1 decode does not shard usefully; see "
@@ -74,6 +76,9 @@ def main() -> int:
             "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
     model = Gpt2Model.new(cfg, weights, Gpt2HipConfig(device=0, decode_path=path))
     log(f"[bench] upload: {time.time() - t0:.1f}s; backend: {model.describe()}")
+
+    if args.workload == "prefill":
+        return bench_prefill(args, cfg, model, ids, n_prefill)
 
     cache = model.new_kv_cache()
     t0 = time.time()
@@ -170,6 +175,60 @@ def main() -> int:
 
     print(json.dumps(result), flush=True)
     return 0
+
+
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+
+
+def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
+    """Secondary workload (BASELINE.json configs[1]-style prompt processing): a step is one
+    prefill of n_prefill tokens into an empty cache through the GEMM path.  Algorithmic
+    flops: the four projections of every layer over all tokens, causal attention
+    (QK^T and PV over the lower triangle), and the lm_head row of the last token."""
+    C_, I, L, V, T = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size, n_prefill
+    gemm_flops = 2.0 * T * L * (3 * C_ * C_ + C_ * C_ + 2 * C_ * I)
+    attn_flops = 4.0 * C_ * (T * (T + 1) / 2) * L
+    flops = gemm_flops + attn_flops + 2.0 * V * C_
+    cache = model.new_kv_cache()
+
+    def one():
+        cache.seq_len = 0
+        return model.prefill(ids, cache)
+
+    for _ in range(max(1, args.warmup)):
+        one().argmax()
+    t0 = time.time()
+    for _ in range(args.steps):
+        lg = one()
+    lg.argmax()  # waits for the last prefill
+    wall = time.time() - t0
+    sec = wall / args.steps
+    info = _devinfo()
+    achieved = flops / sec / 1e12
+    result = {
+        "metric": f"prefill tokens/sec, GPT-2 {args.model} fp32 bs=1, {T}-token prompt",
+        "value": round(T / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": max(1, args.warmup), "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"GPT-2 {args.model} fp32 B=1 prefill of {T} tokens into an empty KV cache",
+                   "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
+                   "device": info.name.decode() or info.arch.decode(), "compute_units": info.compute_units,
+                   "backend": model.describe()},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
+                     "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
+    }
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def _devinfo():
+    from puppygrad_amd import _lib
+    info = _lib.pg_device_info()
+    _lib.load().pg_device_query(0, C.byref(info))
+    return info
 
 
 # HBM bytes one launch of k_decode_persistent<1600> moves on the default workload

@@ -111,9 +111,12 @@ struct GemmArgs {
   int lda, ldc;
   float* ws = nullptr;    // optional workspace for the split-K form (may be nullptr)
   size_t ws_floats = 0;   // its size
+  int tail_first = 0;     // filled by gemm_tail_plan: first tile of the tail that is cut along K,
+  int tail_parts = 1;     // and the number of parts
 };
 bool gemm_supported(const GemmArgs& a);
 int gemm_split_parts(const GemmArgs& a, int num_cus);
+bool gemm_tail_plan(GemmArgs& a, int num_cus);
 hipError_t launch_gemm(const GemmArgs& a, int epilogue, int num_cus, hipStream_t s);
 // Causal attention over qkv[T][3C] -> out[T][C]; also appends K, V to the cache panels.
 // scratch ([T*H][T] floats) is only used when head_dim != 64.

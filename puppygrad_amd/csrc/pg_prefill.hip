@@ -55,11 +55,16 @@ __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
   return *reinterpret_cast<const f4*>(W + idx);
 }
 
-// With SPLIT the K range is cut into gridDim.y parts: part blockIdx.y multiplies its
+// SPLIT = 1: the K range is cut into gridDim.y parts: part blockIdx.y multiplies its
 // k-tiles and writes the raw partial tile to a.ws[part][M][N]; k_splitk_reduce adds the
 // parts in order and applies bias and epilogue (a fixed order: results do not depend on
 // timing).  It fills the chip when M x N alone gives fewer tiles than there are CUs.
-template <int BM, int BN, int EPI, bool WBF, bool SPLIT = false>
+// SPLIT = 2: only the tail is cut.  The tiles [0, a.tail_first) are whole rounds over the
+// CUs and are computed as usual; each of the remaining tiles (a partial round that would
+// keep a few CUs busy and the others idle) is cut into a.tail_parts parts along K, so that
+// the tail is one short item for every CU.  Their raw partial tiles go to
+// a.ws[(tile - tail_first) * parts + part][BM][BN] and k_tail_reduce finishes them.
+template <int BM, int BN, int EPI, bool WBF, int SPLIT = 0>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
@@ -73,12 +78,22 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   // XCD-aware tile order: consecutive workgroup ids go round the 8 XCDs, so give
   // each XCD a contiguous run of tiles (neighbouring tiles share A rows / W rows in
   // that XCD's L2).
-  const int nblocks = gridDim.x;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int per_xcd = (nblocks + 7) >> 3;
-  const int tile = xcd * per_xcd + slot;
   const int tiles_n = (a.N + BN - 1) / BN;
-  if (tile >= ((a.M + BM - 1) / BM) * tiles_n) return;
+  const int tiles_all = ((a.M + BM - 1) / BM) * tiles_n;
+  int tile, tail_part = 0;
+  bool in_tail = false;
+  if (SPLIT == 2 && (int)blockIdx.x >= a.tail_first) {
+    const int q = (int)blockIdx.x - a.tail_first;
+    tile = a.tail_first + q / a.tail_parts;
+    tail_part = q - (q / a.tail_parts) * a.tail_parts;
+    in_tail = true;
+  } else {
+    const int nblocks = SPLIT == 2 ? a.tail_first : (int)gridDim.x;  // a multiple of 8
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int per_xcd = (nblocks + 7) >> 3;
+    tile = xcd * per_xcd + slot;
+  }
+  if (tile >= tiles_all) return;
   const int tm = tile / tiles_n, tn = tile - tm * tiles_n;
   const int m0 = tm * BM, n0 = tn * BN;
 
@@ -102,15 +117,18 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   f4 ra[ALD], rb[BLD];
-  const size_t kfirst = SPLIT ? (size_t)(((long)blockIdx.y * (a.K / BK)) / gridDim.y) * BK : 0;
+  const int ktiles_all = a.K / BK;
+  // this block's k-tiles [kt0, kt1)
+  const int kpart = SPLIT == 1 ? (int)blockIdx.y : tail_part;
+  const int kparts = SPLIT == 1 ? (int)gridDim.y : (in_tail ? a.tail_parts : 1);
+  const int kt0 = (int)(((long)kpart * ktiles_all) / kparts);
+  const int kt1 = (int)(((long)(kpart + 1) * ktiles_all) / kparts);
+  const size_t kfirst = (size_t)kt0 * BK;
 #pragma unroll
   for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + kfirst);
 #pragma unroll
   for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i] + kfirst);
 
-  const int ktiles_all = a.K / BK;
-  const int kt0 = SPLIT ? (int)(((long)blockIdx.y * ktiles_all) / gridDim.y) : 0;
-  const int kt1 = SPLIT ? (int)(((long)(blockIdx.y + 1) * ktiles_all) / gridDim.y) : ktiles_all;
   const int half = lane >> 5, l32 = lane & 31;
   for (int kt = kt0; kt < kt1; ++kt) {
     const int buf = (kt - kt0) & 1;
@@ -160,7 +178,16 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     for (int j = 0; j < NB; ++j) {
       const int n = n0 + wn * WN + 32 * j + l32;
       if (n >= a.N) continue;
-      if (SPLIT) {
+      if (SPLIT == 2 && in_tail) {
+        float* part = a.ws + ((size_t)(tile - a.tail_first) * a.tail_parts + tail_part) * (BM * BN);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int lm = wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+          part[lm * BN + wn * WN + 32 * j + l32] = acc[i][j][v];
+        }
+        continue;
+      }
+      if (SPLIT == 1) {
         float* part = a.ws + (size_t)blockIdx.y * a.M * a.N;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -200,6 +227,31 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
   for (int k = 0; k < 4; ++k) {
     if (EPI == GEMM_GELU) c[k] = gelu_tanh(c[k]);
     if (EPI == GEMM_RESID) c[k] = a.resid[m * a.ldc + n + k] + c[k];
+    dst[k] = c[k];
+  }
+}
+
+// The same for the tail tiles of the SPLIT = 2 form: block (x, y) finishes a quarter of
+// tail tile y (tile-local partials, BM = BN = 64).
+template <int EPI>
+__global__ __launch_bounds__(256) void k_tail_reduce(GemmArgs a) {
+  const int tile = a.tail_first + (int)blockIdx.y;
+  const int tiles_n = (a.N + 63) / 64;
+  const int tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  const int e4 = (int)blockIdx.x * 256 + (int)threadIdx.x;  // float4 index in the tile
+  const int lm = e4 >> 4, ln = (e4 & 15) * 4;
+  const int m = tm * 64 + lm, n = tn * 64 + ln;
+  if (m >= a.M || n >= a.N) return;
+  const float* part = a.ws + (size_t)blockIdx.y * a.tail_parts * 4096 + lm * 64 + ln;
+  f4 s = *reinterpret_cast<const f4*>(part);
+  for (int p = 1; p < a.tail_parts; ++p) s += *reinterpret_cast<const f4*>(part + (size_t)p * 4096);
+  f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
+  float c[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
+  float* dst = a.C + (size_t)m * a.ldc + n;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (EPI == GEMM_GELU) c[k] = gelu_tanh(c[k]);
+    if (EPI == GEMM_RESID) c[k] = a.resid[(size_t)m * a.ldc + n + k] + c[k];
     dst[k] = c[k];
   }
 }
@@ -458,7 +510,7 @@ template <bool WBF>
 hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s) {
   const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
   const int grid = (tiles + 7) / 8 * 8;
-  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, true>), dim3(grid, parts), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 1>), dim3(grid, parts), dim3(256), 0, s, a);
   const unsigned rblocks = (unsigned)(((size_t)a.M * (a.N / 4) + 255) / 256);
   if (epi == GEMM_BIAS)
     hipLaunchKernelGGL(k_splitk_reduce<GEMM_BIAS>, dim3(rblocks), dim3(256), 0, s, a, parts);
@@ -468,6 +520,26 @@ hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t 
     hipLaunchKernelGGL(k_splitk_reduce<GEMM_RESID>, dim3(rblocks), dim3(256), 0, s, a, parts);
   else
     return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+// 64x64 tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
+template <bool WBF>
+hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int grid = a.tail_first + (tiles - a.tail_first) * a.tail_parts;
+  const dim3 rgrid(4, (unsigned)(tiles - a.tail_first));
+  if (epi == GEMM_BIAS) {
+    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_tail_reduce<GEMM_BIAS>, rgrid, dim3(256), 0, s, a);
+  } else if (epi == GEMM_GELU) {
+    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_GELU, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_tail_reduce<GEMM_GELU>, rgrid, dim3(256), 0, s, a);
+  } else if (epi == GEMM_RESID) {
+    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_RESID, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_tail_reduce<GEMM_RESID>, rgrid, dim3(256), 0, s, a);
+  } else {
+    return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }
 }  // namespace
@@ -487,6 +559,23 @@ int gemm_split_parts(const GemmArgs& a, int num_cus) {
   return std::max(parts, 1);
 }
 
+// The tail split of the 64x64 form: with more tiles than CUs and a last round that would
+// occupy at most half of them, that round's tiles are cut into as many K parts as make it
+// one item per CU.  Fills a.tail_first / a.tail_parts; false when it does not apply.
+bool gemm_tail_plan(GemmArgs& a, int num_cus) {
+  const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
+  if (!a.ws || a.N % 4 != 0 || num_cus % 8 != 0 || tiles <= num_cus) return false;
+  const int r = (int)(tiles % num_cus);
+  if (r == 0 || 2 * r > num_cus) return false;
+  int parts = std::min(8, num_cus / r);
+  parts = std::min(parts, a.K / (4 * BK));  // at least four k-tiles per part
+  while (parts > 1 && (size_t)r * parts * 4096 > a.ws_floats) --parts;
+  if (parts < 2) return false;
+  a.tail_first = (int)(tiles - r);
+  a.tail_parts = parts;
+  return true;
+}
+
 hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
   const int parts = gemm_split_parts(a, num_cus);
@@ -496,9 +585,15 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
   if (a.w_bf16) {
     if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, true>(a, epi, s);
+    GemmArgs t = a;
+    if (gemm_tail_plan(t, num_cus)) return launch_gemm_tail<true>(t, epi, s);
     return launch_gemm_tile<64, 64, true>(a, epi, s);
   }
   if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, false>(a, epi, s);
+  {
+    GemmArgs t = a;
+    if (gemm_tail_plan(t, num_cus)) return launch_gemm_tail<false>(t, epi, s);
+  }
   return launch_gemm_tile<64, 64, false>(a, epi, s);
 }
 
