@@ -218,8 +218,15 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
   if (i4 >= (size_t)a.M * n4) return;
   const size_t m = i4 / n4, n = (i4 - m * n4) * 4;
   const size_t stride = (size_t)a.M * a.N;
-  f4 s = *reinterpret_cast<const f4*>(a.ws + m * a.N + n);
-  for (int p = 1; p < parts; ++p) s += *reinterpret_cast<const f4*>(a.ws + p * stride + m * a.N + n);
+  // all parts requested before the first is used (at most 8: gemm_split_parts), added in order
+  f4 v[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p)
+    v[p] = *reinterpret_cast<const f4*>(a.ws + (size_t)min(p, parts - 1) * stride + m * a.N + n);
+  f4 s = v[0];
+#pragma unroll
+  for (int p = 1; p < 8; ++p)
+    if (p < parts) s += v[p];
   f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
   float c[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
   float* dst = a.C + m * a.ldc + n;
@@ -470,6 +477,33 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
     __syncthreads();
     return (red[0] + red[1]) + (red[2] + red[3]);
   };
+  if (cols <= 256 * 8) {
+    // the row is read once and kept in registers (8 values per thread at most)
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = (int)threadIdx.x + 256 * j;
+      x[j] = i < cols ? row[i] : 0.0f;
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += x[j];
+    const float mean = bsum(s) / (float)cols;
+    float v = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float d = ((int)threadIdx.x + 256 * j < cols) ? x[j] - mean : 0.0f;
+      v += d * d;
+    }
+    const float var = bsum(v) / (float)cols;
+    const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = (int)threadIdx.x + 256 * j;
+      if (i < cols) orow[i] = (x[j] - mean) * inv * g[i] + b[i];
+    }
+    return;
+  }
   float s = 0.0f;
   for (int i = threadIdx.x; i < cols; i += 256) s += row[i];
   const float mean = bsum(s) / (float)cols;
