@@ -1355,9 +1355,16 @@ pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in
   pgk::GemmArgs ga{};
   ga.A = dx.p; ga.W = dw.p; ga.bias = db.p; ga.resid = nullptr; ga.C = dy.p;
   ga.M = (int)rows; ga.N = (int)out_f; ga.K = (int)in_f; ga.lda = (int)in_f; ga.ldc = (int)out_f;
+  DevBuf dws;  // workspace for the split-K forms, as the model paths pass it (8 partial outputs)
   if (rows >= kGemmMinRows && rows <= (1u << 20) && pgk::gemm_supported(ga)) {
     hipDeviceProp_t prop;
     PG_HIP(hipGetDeviceProperties(&prop, device));
+    const uint64_t ws_floats = 8 * rows * out_f;
+    if (ws_floats <= (64u << 20)) {
+      if ((s = dws.alloc(ws_floats))) return s;
+      ga.ws = dws.p;
+      ga.ws_floats = ws_floats;
+    }
     PG_HIP(pgk::launch_gemm(ga, pgk::GEMM_BIAS, prop.multiProcessorCount, nullptr));
   } else {
     for (uint64_t r = 0; r < rows; ++r) {

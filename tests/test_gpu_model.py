@@ -249,3 +249,11 @@ def test_config1_gpt2_small_greedy_decode_parity():
     if explained == 0:
         assert got == want[32:]
     assert cache.seq_len == 32 + 127  # the forward after the last token is skipped
+    # A destroyed cache hands its block of tagged activation words back to a pool and the
+    # next cache takes it over, old epochs and all: the result must not depend on that.
+    for _ in range(3):
+        del cache
+        cache = model.new_kv_cache()
+        model.prefill(ids, cache)
+        again, _ = model.decode_greedy(cache, 128)
+        assert again == got
