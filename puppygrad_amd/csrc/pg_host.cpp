@@ -82,6 +82,8 @@ struct pg_kv_cache {
   size_t seq_len = 0;
   float* kv = nullptr;  // [L][2][B][H][P][hd]
   // per-sequence activation scratch, [B][...]
+  float* seq_scratch = nullptr;  // activations of the full-sequence (GEMM) forward, grown on demand
+  size_t seq_scratch_floats = 0;
   float* gemm_ws = nullptr;      // split-K partial tiles of the batched decode step
   size_t gemm_ws_floats = 0;
   float *x = nullptr, *q = nullptr, *hbuf = nullptr, *part_acc = nullptr, *part_m = nullptr,
@@ -442,13 +444,32 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   const int T = (int)n, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
   hipStream_t s = c->stream;
   pg_status st;
-  DevBuf X, XN, QKV, ATT, HB, IDS, SCR, LOG, WS;
-  if ((st = X.alloc(n * g.C)) || (st = XN.alloc(n * g.C)) || (st = QKV.alloc(n * 3 * g.C)) ||
-      (st = ATT.alloc(n * g.C)) || (st = HB.alloc(n * g.I)) || (st = IDS.alloc(n)))
-    return st;
+  // The activations of the sequence live in one block that stays with the cache between
+  // calls (allocating and freeing them cost about 0.4 ms per call): it only ever grows.
+  struct View { float* p; } X, XN, QKV, ATT, HB, IDS, WS;
+  DevBuf SCR, LOG;
   // split-K partial tiles of the projections back to n_embd columns (up to 8 parts)
   const size_t ws_floats = 8 * n * g.C;
-  if ((st = WS.alloc(ws_floats))) return st;
+  {
+    auto up = [](size_t v) { return (v + 63) / 64 * 64; };  // 256-byte boundaries
+    const size_t sizes[7] = {up(n * g.C), up(n * g.C), up(n * 3 * g.C), up(n * g.C),
+                             up(n * g.I), up(n),       up(ws_floats)};
+    size_t total = 0;
+    for (size_t v : sizes) total += v;
+    if (c->seq_scratch_floats < total) {
+      if (c->seq_scratch) (void)hipFree(c->seq_scratch);
+      c->seq_scratch = nullptr;
+      c->seq_scratch_floats = 0;
+      PG_HIP(hipMalloc(&c->seq_scratch, total * sizeof(float)));
+      c->seq_scratch_floats = total;
+    }
+    View* views[7] = {&X, &XN, &QKV, &ATT, &HB, &IDS, &WS};
+    float* at = c->seq_scratch;
+    for (int i = 0; i < 7; ++i) {
+      views[i]->p = at;
+      at += sizes[i];
+    }
+  }
   if (hd != 64 && (st = SCR.alloc(n * g.H * n))) return st;
   if (all_logits_dst && (st = LOG.alloc(n * g.V))) return st;
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
@@ -916,6 +937,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->q);
     (void)hipFree(c->hbuf);
     if (c->gemm_ws) (void)hipFree(c->gemm_ws);
+    if (c->seq_scratch) (void)hipFree(c->seq_scratch);
     (void)hipFree(c->part_acc);
     (void)hipFree(c->part_m);
     (void)hipFree(c->part_l);

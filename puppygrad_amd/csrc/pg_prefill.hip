@@ -312,15 +312,30 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
   float (*kt)[KT + 1] = Kt[wave];
   float (*vs)[64 + 4] = Vs[wave];
   const int last_tile = min(q0 + 31, T - 1) / KT;
+  // K and V rows of a tile as this lane loads them: 8 pieces of (key i/16, 4 dims); the
+  // next tile's are requested while the current one is multiplied
+  f4 kreg[KT * 16 / 64], vreg[KT * 16 / 64];
+  auto fetch = [&](int tile) {
+    const int k0 = tile * KT;
+#pragma unroll
+    for (int j = 0; j < KT * 16 / 64; ++j) {
+      const int i = lane + 64 * j;
+      const int key = i >> 4, d4 = (i & 15) * 4;
+      const int kk = min(k0 + key, T - 1);
+      kreg[j] = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + d4);
+      vreg[j] = *reinterpret_cast<const f4*>(vbase + (size_t)kk * C3 + d4);
+    }
+  };
+  if (wave <= last_tile) fetch(wave);
   for (int tile = wave; tile <= last_tile; tile += NWV) {
     const int k0 = tile * KT;
     // stage K (transposed) and V of 32 keys; also append them to the cache once
     // (by the wavefront that meets the tile on the diagonal: q0 == k0)
-    for (int i = lane; i < KT * 16; i += 64) {
+#pragma unroll
+    for (int j = 0; j < KT * 16 / 64; ++j) {
+      const int i = lane + 64 * j;
       const int key = i >> 4, d4 = (i & 15) * 4;
-      const int kk = min(k0 + key, T - 1);
-      const f4 kv4 = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + d4);
-      const f4 vv4 = *reinterpret_cast<const f4*>(vbase + (size_t)kk * C3 + d4);
+      const f4 kv4 = kreg[j], vv4 = vreg[j];
       kt[d4 + 0][key] = kv4.x; kt[d4 + 1][key] = kv4.y; kt[d4 + 2][key] = kv4.z; kt[d4 + 3][key] = kv4.w;
       *reinterpret_cast<f4*>(&vs[key][d4]) = vv4;
       if (q0 == k0 && k0 + key < T) {
@@ -331,6 +346,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
     // each wavefront has its own LDS tiles and LDS executes a wavefront's accesses in
     // order, so only the compiler has to be kept from reordering
     __builtin_amdgcn_wave_barrier();
+    if (tile + NWV <= last_tile) fetch(tile + NWV);
 
     // S^T = K . Q^T : A operand lane -> K[key l32][d = 2s + half]
     f16v sacc;
