@@ -381,6 +381,13 @@ __device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, 
   return r;
 }
 
+// Key splits per head at position pos: one (and then no merge hop: the item's result is
+// the head's attention output) while all keys fit a single item, the launch's count
+// otherwise.  Every wavefront of the grid derives the same value.
+__device__ __forceinline__ int splits_at(const DecodeParams& p, int pos) {
+  return pos + 1 <= kMaxItemKeys ? 1 : p.ns;
+}
+
 // ---- service side: poll tagged words ---------------------------------------------------
 // One tagged word at a wave-uniform base plus a 32-bit byte offset ("scalar base +
 // vector offset" addressing: no 64-bit per-lane addresses are kept across the retries).
@@ -653,7 +660,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
   const int wg = blockIdx.x;
   unsigned* abort_word = p.status;
   lvup halt = (lvup)&ctl->halt;
-  const int H = p.H, P = p.P, ns = p.ns;
+  const int H = p.H, P = p.P;
 
   int t = 0;
   int stopped = 0;
@@ -686,6 +693,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 #pragma unroll 1
   for (; t < p.n_fwd; ++t) {
     const int pos = p.pos0 + t;
+    const int ns = splits_at(p, pos);
     PG_STAMP(p.L, 7);
     if (p.prof && lane == 0 && t + 1 == p.n_fwd) lds.ts[p.L * 16 + 13] = wall_clock64();
     // ---- token to embed: given, or the argmax of the previous step's logits ----
@@ -829,9 +837,14 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
             den += wq * ctl->wl[wv];
             num += wq * ctl->wacc[wv][lane];
           }
-          PG_ST64(dst + lane, pack(epp, num));
-          if (lane == 0) PG_ST64(dst + 64, pack(epp, M));
-          if (lane == 1) PG_ST64(dst + 65, pack(epp, den));
+          if (ns == 1) {
+            // the head's only split: this is the attention output itself, no merge hop
+            PG_ST64(p.attn_t + h * 64 + lane, pack(epoch_of(p, t, l, 2), num / den));
+          } else {
+            PG_ST64(dst + lane, pack(epp, num));
+            if (lane == 0) PG_ST64(dst + 64, pack(epp, M));
+            if (lane == 1) PG_ST64(dst + 65, pack(epp, den));
+          }
         }
       }
       // the credit of the second attention hop (the streamers request a slice on it)
@@ -841,7 +854,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // ================= B2: the workgroup that took split 0 of a head merges it ====
       const unsigned epa = epoch_of(p, t, l, 2);
 #pragma unroll 1
-      for (int item = wg; item < items; item += G) {
+      for (int item = wg; ns > 1 && item < items; item += G) {
         const int h = item / ns, s = item - h * ns;
         if (s != 0) continue;
         // the head's ns partials (66 words each) are one run of tagged words: probe the
@@ -1247,7 +1260,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       SSTAMP(5);
       // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
       {
-        const int H = p.H, P = p.P, ns = p.ns, pos = p.pos0 + t;
+        const int H = p.H, P = p.P, pos = p.pos0 + t, ns = splits_at(p, pos);
         const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
         const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
         const float* vc = kc + p.kv_v_offset;
