@@ -238,6 +238,105 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// A batch of at most MB rows against W (the projections of a batched decode step).  The
+// job is to stream W once at the speed of HBM, and tiles that stage W through LDS cut it
+// into pieces too short for that.  Here a wavefront owns R whole rows of W (read
+// contiguously, like the batch-1 matrix-vector kernel) and multiplies them with all MB
+// input vectors, which lie in LDS (K in chunks of KC so that they fit).  Each lane ends up
+// with R x MB partial sums over its columns; they are added across the lanes by a
+// butterfly that halves the number of values per lane at every step, after which lane i
+// holds the finished sum number i and applies bias and epilogue.  Sums are formed in a
+// fixed order: results do not depend on timing.
+// acc[0..CUR) per lane -> sums over the wavefront, one per lane: the step over the lane
+// bit DIST keeps half of the values, each now summed over the two lanes that differ in
+// that bit (a lane with the bit set keeps the upper half).  Once a single value is left
+// (CUR = 1) the remaining lane bits hold partial sums of the same value.  At the end lane
+// i holds, in acc[0], the sum of the value whose index is the top log2(CUR) bits of i.
+template <int CUR, int DIST>
+__device__ __forceinline__ void lane_butterfly(float* acc, int lane) {
+  if constexpr (DIST >= 1) {
+    if constexpr (CUR > 1) {
+      constexpr int half = CUR / 2;
+      const bool up = (lane & DIST) != 0;
+#pragma unroll
+      for (int i = 0; i < half; ++i) {
+        const float keep = up ? acc[i + half] : acc[i];
+        const float send = up ? acc[i] : acc[i + half];
+        acc[i] = keep + __shfl_xor(send, DIST, 64);
+      }
+      lane_butterfly<half, DIST / 2>(acc, lane);
+    } else {
+      acc[0] += __shfl_xor(acc[0], DIST, 64);
+      lane_butterfly<1, DIST / 2>(acc, lane);
+    }
+  }
+}
+
+template <int MB, int R, int EPI, bool WBF>
+__global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
+  constexpr int KC = 16384 / MB;      // floats of one input vector per chunk (64 KiB in all)
+  constexpr int J = KC / 256;         // float4 per lane, row and chunk
+  constexpr int NV = R * MB;          // partial sums per lane
+  static_assert(NV <= 64 && (NV & (NV - 1)) == 0, "one finished sum per lane at most");
+  __shared__ __attribute__((aligned(16))) float xs[MB * KC];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = ((int)blockIdx.x * 4 + wave) * R;  // this wavefront's first row
+
+  float acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = 0.0f;
+
+  for (int k0 = 0; k0 < a.K; k0 += KC) {
+    // this chunk of the R rows: requested first, in flight while the inputs are staged
+    f4 w[R][J];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < J; ++j) {
+        const int k = min(k0 + 4 * lane + 256 * j, a.K - 4);  // past the row: re-read, meets 0 in x
+        w[r][j] = load_w4<WBF>(a.W, (size_t)min(n0 + r, a.N - 1) * a.K + k);
+      }
+    __syncthreads();  // the previous chunk has been read by every wavefront
+    {
+      // (all of this thread's pieces are requested before the first is stored)
+      constexpr int NP = MB * (KC / 4) / 256;
+      f4 v[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        const int i = tid + 256 * q;
+        const int b = i / (KC / 4), k = k0 + (i - b * (KC / 4)) * 4;
+        v[q] = f4{0.f, 0.f, 0.f, 0.f};
+        if (b < a.M && k < a.K) v[q] = *reinterpret_cast<const f4*>(a.A + (size_t)b * a.lda + k);
+      }
+#pragma unroll
+      for (int q = 0; q < NP; ++q) *reinterpret_cast<f4*>(&xs[(tid + 256 * q) * 4]) = v[q];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int j = 0; j < J; ++j) {
+        const f4 xv = *reinterpret_cast<const f4*>(&xs[b * KC + 4 * lane + 256 * j]);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          acc[r * MB + b] += (w[r][j].x * xv.x + w[r][j].y * xv.y) + (w[r][j].z * xv.z + w[r][j].w * xv.w);
+      }
+  }
+
+  lane_butterfly<NV, 32>(acc, lane);
+  // lane -> value index: its top log2(NV) bits
+  constexpr int kShift = NV == 64 ? 0 : NV == 32 ? 1 : NV == 16 ? 2 : NV == 8 ? 3 : NV == 4 ? 4 : NV == 2 ? 5 : 6;
+  if ((lane & ((1 << kShift) - 1)) != 0) return;
+  const int idx = lane >> kShift;
+  const int r = idx / MB, b = idx - r * MB, n = n0 + r;
+  if (b >= a.M || n >= a.N) return;
+  float c = (a.bias ? a.bias[n] : 0.0f) + acc[0];
+  if (EPI == GEMM_GELU) c = gelu_tanh(c);
+  if (EPI == GEMM_RESID) c = a.resid[(size_t)b * a.ldc + n] + c;
+  a.C[(size_t)b * a.ldc + n] = c;
+}
+
 // The same for the tail tiles of the SPLIT = 2 form: block (x, y) finishes a quarter of
 // tail tile y (tile-local partials, BM = BN = 64).
 template <int EPI>
@@ -572,6 +671,32 @@ hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t 
     return hipErrorInvalidValue;
   return hipGetLastError();
 }
+template <int MB, int R, bool WBF>
+hipError_t launch_gemv_rows_r(const GemmArgs& a, int epi, hipStream_t s) {
+  const dim3 grid((unsigned)((a.N + 4 * R - 1) / (4 * R)));
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemv_rows<MB, R, GEMM_BIAS, WBF>), grid, dim3(256), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemv_rows<MB, R, GEMM_GELU, WBF>), grid, dim3(256), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemv_rows<MB, R, GEMM_RESID, WBF>), grid, dim3(256), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+// Rows per wavefront: as many as leave about two blocks per CU (and one sum per lane).
+template <bool WBF>
+hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
+  const long want = 2L * num_cus;
+  if (a.M <= 16) {
+    if ((a.N + 15) / 16 >= want) return launch_gemv_rows_r<16, 4, WBF>(a, epi, s);
+    if ((a.N + 7) / 8 >= want) return launch_gemv_rows_r<16, 2, WBF>(a, epi, s);
+    return launch_gemv_rows_r<16, 1, WBF>(a, epi, s);
+  }
+  if ((a.N + 7) / 8 >= want) return launch_gemv_rows_r<32, 2, WBF>(a, epi, s);
+  return launch_gemv_rows_r<32, 1, WBF>(a, epi, s);
+}
+
 // 64x64 tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
 template <bool WBF>
 hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
@@ -628,6 +753,11 @@ bool gemm_tail_plan(GemmArgs& a, int num_cus) {
 
 hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
+  // A small decode batch over a short K: whole rows of W per wavefront (HBM-bound), no MFMA
+  // tiles.  (Every block stages all input vectors; beyond 16 x 1024 values that costs more
+  // than the tiles' short pieces of W.)
+  if (a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 4096)
+    return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);
   const int parts = gemm_split_parts(a, num_cus);
   if (parts > 1)
     return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s) : launch_gemm_split<false>(a, epi, parts, s);

@@ -41,12 +41,15 @@ def test_dense_matches_oracle(rows, k, n):
 @pytest.mark.parametrize("rows,k,n", [(16, 768, 2304), (1024, 768, 768), (100, 3072, 768), (128, 1600, 4800),
                                       (37, 64, 50), (1000, 1024, 4096), (33, 16, 129), (64, 6400, 1600),
                                       (20, 768, 50257), (512, 768, 2304), (1024, 768, 2304),
-                                      (512, 768, 3072), (16, 1024, 3072), (32, 1600, 6400)])
+                                      (512, 768, 3072), (16, 1024, 3072), (32, 1600, 6400),
+                                      (16, 4096, 1024), (16, 1600, 4800)])
 def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised.
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
     # parts; (512, 768, 2304), (1024, 768, 2304) and (512, 768, 3072) have 288 / 576 / 384
     # tiles of 64x64 on 256 CUs and cut only the tiles of the last partial round.
+    # 16 rows with K <= 4096 take the row-streaming kernel of the decode batch (one, four
+    # and two chunks of K for 1024, 4096 and 1600, the last one partial).
     rng = np.random.default_rng(rows * 7 + n)
     x = rng.standard_normal(rows * k).astype(np.float32)
     w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
