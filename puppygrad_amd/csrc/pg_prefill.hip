@@ -337,6 +337,100 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
   a.C[(size_t)b * a.ldc + n] = c;
 }
 
+// ---------------------------------------------------------------------------
+// A batch of at most 32 rows against W on the matrix cores.  A block owns 32 rows of W;
+// its eight wavefronts cut the block's K range into eight pieces, and each multiplies its
+// piece straight out of registers: lane (l, half) loads 16 bytes of row n0 + l of W and
+// the same columns of input row l, and feeds them to MFMA 32x32x2 as the B and A operands
+// (which columns meet in one MFMA step does not matter for a sum over all of them).  No
+// LDS staging and no barrier in the stream; the eight 32x32 partial tiles are added in
+// wavefront order through LDS at the end.  With gridDim.y > 1 the K range is cut over
+// blocks as well and the raw tile goes to a.ws[part][M][N] for k_splitk_reduce.
+template <int EPI, bool WBF>
+__global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
+  constexpr int U = WBF ? 16 : 8;  // columns per unit: 16 bytes of W per lane, two lane halves
+  constexpr int D = 6;             // units requested together
+  __shared__ float red[8][32][33];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int n0 = (int)blockIdx.x * 32;
+  const int units = a.K / U;
+  const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
+  const int u0 = (int)(((long)piece * units) / pieces), u1 = (int)(((long)(piece + 1) * units) / pieces);
+
+  const size_t wrow = (size_t)min(n0 + l32, a.N - 1) * a.K + (U / 2) * half;
+  const float* xrow = a.A + (size_t)min(l32, a.M - 1) * a.lda + (U / 2) * half;
+
+  f16v acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+  for (int u = u0; u < u1; u += D) {
+    f4 wv[D], xa[D], xb[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      const size_t k = (size_t)min(u + i, u1 - 1) * U;
+      if (WBF) {
+        // 8 bf16 columns: widened below; the matching 8 input columns are two float4
+        wv[i] = *reinterpret_cast<const f4*>(reinterpret_cast<const unsigned short*>(a.W) + wrow + k);
+        xa[i] = *reinterpret_cast<const f4*>(xrow + k);
+        xb[i] = *reinterpret_cast<const f4*>(xrow + k + 4);
+      } else {
+        wv[i] = *reinterpret_cast<const f4*>(a.W + wrow + k);
+        xa[i] = *reinterpret_cast<const f4*>(xrow + k);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      if (u + i < u1) {  // wave-uniform
+        if (WBF) {
+          const unsigned* p = reinterpret_cast<const unsigned*>(&wv[i]);
+          float w8[8];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            w8[2 * q] = __uint_as_float(p[q] << 16);
+            w8[2 * q + 1] = __uint_as_float(p[q] & 0xffff0000u);
+          }
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].x, w8[0], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].y, w8[1], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].z, w8[2], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].w, w8[3], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].x, w8[4], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].y, w8[5], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].z, w8[6], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].w, w8[7], acc, 0, 0, 0);
+        } else {
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].x, wv[i].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].y, wv[i].y, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].z, wv[i].z, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].w, wv[i].w, acc, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // acc[v] is row (batch index) 8 (v / 4) + 4 half + v % 4 of column l32
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[wave][8 * (v >> 2) + 4 * half + (v & 3)][l32] = acc[v];
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int idx = tid + 512 * q, b = idx >> 5, nl = idx & 31, n = n0 + nl;
+    if (b >= a.M || n >= a.N) continue;
+    float sum = red[0][b][nl];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) sum += red[w][b][nl];
+    if (gridDim.y > 1) {
+      a.ws[((size_t)blockIdx.y * a.M + b) * a.N + n] = sum;
+      continue;
+    }
+    float c = (a.bias ? a.bias[n] : 0.0f) + sum;
+    if (EPI == GEMM_GELU) c = gelu_tanh(c);
+    if (EPI == GEMM_RESID) c = a.resid[(size_t)b * a.ldc + n] + c;
+    a.C[(size_t)b * a.ldc + n] = c;
+  }
+}
+
 // The same for the tail tiles of the SPLIT = 2 form: block (x, y) finishes a quarter of
 // tail tile y (tile-local partials, BM = BN = 64).
 template <int EPI>
@@ -697,6 +791,45 @@ hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t
   return launch_gemv_rows_r<32, 1, WBF>(a, epi, s);
 }
 
+// K parts for k_gemm_rows32 (0 = not applicable): up to one block per CU (cutting K further
+// was measured slower: the reduce and the shorter pieces cost more than the idle CUs), at
+// least sixteen units per block and part, bounded by the workspace.
+int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
+  const int U = a.w_bf16 ? 16 : 8;
+  if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
+  const long tiles = (a.N + 31) / 32;
+  long parts = std::max<long>(1, num_cus / tiles);
+  parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 16));
+  parts = std::min<long>(parts, 8);
+  if (parts > 1) {
+    if (!a.ws || a.N % 4 != 0) parts = 1;
+    else parts = std::min<long>(parts, (long)(a.ws_floats / ((size_t)a.M * a.N)));
+  }
+  return (int)std::max<long>(parts, 1);
+}
+template <bool WBF>
+hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s) {
+  const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)parts);
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF>), grid, dim3(512), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF>), grid, dim3(512), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF>), grid, dim3(512), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  if (parts > 1) {
+    const unsigned rblocks = (unsigned)(((size_t)a.M * (a.N / 4) + 255) / 256);
+    if (epi == GEMM_BIAS)
+      hipLaunchKernelGGL(k_splitk_reduce<GEMM_BIAS>, dim3(rblocks), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_GELU)
+      hipLaunchKernelGGL(k_splitk_reduce<GEMM_GELU>, dim3(rblocks), dim3(256), 0, s, a, parts);
+    else
+      hipLaunchKernelGGL(k_splitk_reduce<GEMM_RESID>, dim3(rblocks), dim3(256), 0, s, a, parts);
+  }
+  return hipGetLastError();
+}
+
 // 64x64 tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
 template <bool WBF>
 hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
@@ -753,11 +886,14 @@ bool gemm_tail_plan(GemmArgs& a, int num_cus) {
 
 hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
-  // A small decode batch over a short K: whole rows of W per wavefront (HBM-bound), no MFMA
-  // tiles.  (Every block stages all input vectors; beyond 16 x 1024 values that costs more
-  // than the tiles' short pieces of W.)
-  if (a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 4096)
+  // A small decode batch over a short K: whole rows of W per wavefront, no MFMA tiles.
+  // (Every block stages all input vectors; beyond 16 x 1024 values that costs more than it
+  // saves.)
+  if (a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024)
     return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);
+  // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
+  if (const int rp = gemm_rows32_parts(a, num_cus))
+    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s) : launch_gemm_rows32<false>(a, epi, rp, s);
   const int parts = gemm_split_parts(a, num_cus);
   if (parts > 1)
     return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s) : launch_gemm_split<false>(a, epi, parts, s);

@@ -48,8 +48,8 @@ def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
     # parts; (512, 768, 2304), (1024, 768, 2304) and (512, 768, 3072) have 288 / 576 / 384
     # tiles of 64x64 on 256 CUs and cut only the tiles of the last partial round.
-    # 16 rows with K <= 4096 take the row-streaming kernel of the decode batch (one, four
-    # and two chunks of K for 1024, 4096 and 1600, the last one partial).
+    # 16 rows with K <= 1024 take the row-streaming kernel of the decode batch; other shapes
+    # of up to 32 rows the register-fed MFMA kernel (with and without a cut of K over blocks).
     rng = np.random.default_rng(rows * 7 + n)
     x = rng.standard_normal(rows * k).astype(np.float32)
     w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
