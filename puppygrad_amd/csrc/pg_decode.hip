@@ -236,11 +236,6 @@ __device__ __forceinline__ void load_tile(Tile<J>& t, const f4* p, int K4s, int 
     t.w[j] = ld_row(p, c * 16u);
   }
 }
-template <int J, int LO, int HI>
-__device__ __forceinline__ void load_tile_part(Tile<J>& t, const f4* p, int lane) {
-#pragma unroll
-  for (int j = LO; j < HI; ++j) t.w[j] = ld_row(p, ((unsigned)lane + 64u * j) * 16u);
-}
 template <int J>
 __device__ __forceinline__ void load_x(f4* xr, lfp xs, int K4s, int lane) {
   lf4p x4 = (lf4p)xs;
@@ -451,32 +446,6 @@ __device__ __forceinline__ bool probe_spread(const u64* src, int first, unsigned
   return probe_lines(src, l0, (l0 + LINES / 3) % LINES, (l0 + 2 * (LINES / 3)) % LINES, epoch, abort_word);
 }
 
-// Spins until run `run` (words 64 run .. 64 run + 63) carries `epoch`.  Cheap: one
-// 512-byte request per attempt.  Wave-uniform; false on timeout or abort.
-__device__ __forceinline__ bool probe_run(const u64* src, int run, unsigned epoch,
-                                          unsigned* abort_word, unsigned& spins) {
-  const int lane = opaque((int)threadIdx.x) & 63;
-  const unsigned off = (unsigned)(run * 64 + lane) * 8u;
-  for (;;) {
-    u64 v = ld_tagged(src, off);
-    if (__all(tag_of(v) == epoch)) return true;
-    if (++spins > kSpinLimit) {
-      PG_ST32(abort_word, 1u);
-      return false;
-    }
-    if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) return false;
-    __builtin_amdgcn_s_sleep(2);
-  }
-}
-// The run to probe after a bulk read that found stale words: one that holds a stale
-// word (`run_of_bad` is this lane's, meaningful where `bad`).  The expensive bulk read
-// is then only repeated once that laggard has arrived; the waiting is done by the
-// cheap probe and does not flood the CU's memory pipeline.
-__device__ __forceinline__ int next_probe_run(bool bad, int run_of_bad) {
-  const unsigned long long m = __ballot(bad);
-  const int first = __builtin_ctzll(m);
-  return __builtin_amdgcn_readlane(run_of_bad, first);
-}
 // Waits until src[i] carries `epoch` for every i in [0, 64 NE) and leaves the payloads
 // in dst (LDS): scalar probes of three lines (they differ per workgroup), then a bulk read
 // of lane + 64 e; while that finds stale words, the probe moves to a stale word's line
@@ -1103,20 +1072,16 @@ struct StreamPlan {
   // load PS of the stream above.
   static constexpr bool kTight = (ND + NE + NF) * 4 > 200;
   static constexpr int FS = kTight ? 12 : 0;
-#ifndef PG_PS
-#define PG_PS 31
-#endif
-  static constexpr int PS = kTight ? PG_PS : 0;
+  static constexpr int PS = kTight ? 31 : 0;
   // (the first slice goes out next to the c_attn rows and their product: it is the one
   // cut short where those leave fewer registers)
   static constexpr int kRegsA = 31, kRegs = 33;  // float4 per lane a product can sit next to
   static constexpr int c1 = NL / 6 < kRegsA - NA ? NL / 6 : kRegsA - NA;
-#ifndef PG_CUTS
-#define PG_CUTS 0, 9, 20, 31, 48, 66, 81
-#endif
   static constexpr int cut(int k) {
     if (!kTight) return k == 0 ? 0 : c1 + (k - 1) * (NL - c1) / 5;
-    constexpr int c[7] = {PG_CUTS};
+    // C = 1600 (the only width that stages): found by measurement within what the
+    // registers allow at each product
+    constexpr int c[7] = {0, 9, 20, 31, 48, 66, 81};
     return c[k];
   }
   // of the loads [0, n): those held in registers
