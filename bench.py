@@ -55,8 +55,9 @@ def main() -> int:
                     help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound)")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this path runs on ONE GPU (batch-1 decode does not shard usefully; see "
-            "DESIGN.md); --gpus must be 1")
+        log("bench.py: this path runs on ONE GPU (a batch-1 decode step has one all-reduce of "
+            "n_embd floats after every projection pair to offer to a second GPU: latency-bound); "
+            "--gpus must be 1")
         return 2
 
     from puppygrad_amd import Gpt2Config, Gpt2HipConfig, Gpt2Model, _lib, synth
