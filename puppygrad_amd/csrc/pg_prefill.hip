@@ -458,43 +458,50 @@ __global__ __launch_bounds__(256) void k_tail_reduce(GemmArgs a) {
 
 // ---------------------------------------------------------------------------
 // causal_self_attention (src/models/gpt2/rust.rs:1580-1659) for head_dim 64 over an
-// interleaved qkv[T][3C] buffer.  One wavefront owns 32 queries of one head and
-// walks the key tiles 0..diagonal, 32 keys at a time, staged in LDS:
-//   S^T (keys x queries) = K . Q^T        32 MFMA steps over d
+// interleaved qkv[T][3C] buffer.  A block of eight wavefronts owns 32 queries of one head;
+// the wavefronts take the key tiles 0..diagonal (32 keys each) round-robin, each with its
+// own running (max, sum, O), merged through LDS at the end:
+//   S^T (keys x queries) = K . Q^T        32 MFMA steps; both operands come straight from
+//                                         registers: lane (l, half) holds dims
+//                                         32 half .. 32 half + 31 of key l / query l, and step
+//                                         s pairs dim s with dim 32 + s
 //   online softmax per query (a lane holds 16 keys of one query; one xor-32 swap)
-//   O^T (d x queries)   += V^T . P^T      16 MFMA steps over the 32 keys, twice (d halves)
+//   O^T (d x queries)   += V^T . P^T      16 MFMA steps over the 32 keys, twice (d halves),
+//                                         V rows staged in LDS
+// The next tile's K and V rows are requested while the current tile is multiplied.
 // Scores are scaled by 1/8 after the dot product, as the reference does
 // (rust.rs:1590, 1634).  It also appends K and V to the cache panels
 // ([head][position][64], kv_index at rust.rs:1851-1855).
+// Grid: x = head, y = block of queries, longest rows first (blocks are handed out x
+// fastest: every head's long blocks start before any short one).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict__ qkv, int T,
+__global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict__ qkv, int T,
                                                         int C, int P, float* __restrict__ kcache,
                                                         float* __restrict__ vcache,
                                                         float* __restrict__ out) {
   constexpr int KT = 32;   // keys per tile
-  constexpr int NWV = 4;   // wavefronts per block: they share one block of 32 queries and
-                           // take the key tiles round-robin, each with its own running
-                           // (max, sum, O) that are merged through LDS at the end
-  __shared__ float Kt[NWV][64][KT + 1];   // per wavefront: [d][key]
-  __shared__ float Vs[NWV][KT][64 + 4];   // per wavefront: [key][d]
+  constexpr int NWV = 8;   // wavefronts per block
+  // per wavefront: V rows [key][d] of the current tile; reused as [d][query] for the merge
+  __shared__ __attribute__((aligned(16))) float Vs[NWV][KT * (64 + 4)];
   __shared__ float Ms[NWV][32], Ls[NWV][32];
+  static_assert(KT * (64 + 4) >= 64 * (KT + 1), "the merge tile fits the V tile's space");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
-  const int h = blockIdx.y;
+  const int h = blockIdx.x;
   const int nqb = (T + 31) / 32;
-  const int qb = nqb - 1 - (int)blockIdx.x;  // the longest rows first
+  const int qb = nqb - 1 - (int)blockIdx.y;  // the longest rows first
   const int q0 = qb * 32;
   const int C3 = 3 * C;
   const float* qbase = qkv + h * 64;
   const float* kbase = qkv + C + h * 64;
   const float* vbase = qkv + 2 * C + h * 64;
 
-  // Q^T operand: lane (query l32, half) holds Q[query][2s + half] for s = 0..31
-  float qr[32];
+  // Q^T operand: lane (query l32, half) holds Q[query][32 half + s] for s = 0..31
+  f4 qr[8];
   {
     const int q = min(q0 + l32, T - 1);
 #pragma unroll
-    for (int s = 0; s < 32; ++s) qr[s] = qbase[(size_t)q * C3 + 2 * s + half];
+    for (int j = 0; j < 8; ++j) qr[j] = *reinterpret_cast<const f4*>(qbase + (size_t)q * C3 + 32 * half + 4 * j);
   }
   f16v o0, o1;  // O^T rows d 0..31 and 32..63, column = query l32
 #pragma unroll
@@ -502,52 +509,62 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
   float m_run = -INFINITY, l_run = 0.0f;  // per query (replicated in both halves)
   const int qi = q0 + l32;                // this lane's query
 
-  float (*kt)[KT + 1] = Kt[wave];
-  float (*vs)[64 + 4] = Vs[wave];
+  float (*vs)[64 + 4] = reinterpret_cast<float (*)[64 + 4]>(Vs[wave]);
   const int last_tile = min(q0 + 31, T - 1) / KT;
-  // K and V rows of a tile as this lane loads them: 8 pieces of (key i/16, 4 dims); the
-  // next tile's are requested while the current one is multiplied
-  f4 kreg[KT * 16 / 64], vreg[KT * 16 / 64];
-  auto fetch = [&](int tile) {
-    const int k0 = tile * KT;
+  // K operand: lane (key l32, half) holds K[key][32 half + s]; V rows as this lane loads
+  // them: 8 pieces of (key i / 16, 4 dims)
+  f4 kr[8], vreg[8];
+  auto fetch_k = [&](int tile) {
+    const int kk = min(tile * KT + l32, T - 1);
 #pragma unroll
-    for (int j = 0; j < KT * 16 / 64; ++j) {
+    for (int j = 0; j < 8; ++j) kr[j] = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + 32 * half + 4 * j);
+  };
+  auto fetch_v = [&](int tile) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
       const int i = lane + 64 * j;
-      const int key = i >> 4, d4 = (i & 15) * 4;
-      const int kk = min(k0 + key, T - 1);
-      kreg[j] = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + d4);
-      vreg[j] = *reinterpret_cast<const f4*>(vbase + (size_t)kk * C3 + d4);
+      const int kk = min(tile * KT + (i >> 4), T - 1);
+      vreg[j] = *reinterpret_cast<const f4*>(vbase + (size_t)kk * C3 + (i & 15) * 4);
     }
   };
-  if (wave <= last_tile) fetch(wave);
+  if (wave <= last_tile) {
+    fetch_k(wave);
+    fetch_v(wave);
+  }
   for (int tile = wave; tile <= last_tile; tile += NWV) {
     const int k0 = tile * KT;
-    // stage K (transposed) and V of 32 keys; also append them to the cache once
-    // (by the wavefront that meets the tile on the diagonal: q0 == k0)
+    const bool diag = (q0 == k0);  // this wavefront appends the tile's K and V to the cache
+    // stage V of 32 keys
 #pragma unroll
-    for (int j = 0; j < KT * 16 / 64; ++j) {
+    for (int j = 0; j < 8; ++j) {
       const int i = lane + 64 * j;
       const int key = i >> 4, d4 = (i & 15) * 4;
-      const f4 kv4 = kreg[j], vv4 = vreg[j];
-      kt[d4 + 0][key] = kv4.x; kt[d4 + 1][key] = kv4.y; kt[d4 + 2][key] = kv4.z; kt[d4 + 3][key] = kv4.w;
-      *reinterpret_cast<f4*>(&vs[key][d4]) = vv4;
-      if (q0 == k0 && k0 + key < T) {
-        *reinterpret_cast<f4*>(kcache + ((size_t)h * P + k0 + key) * 64 + d4) = kv4;
-        *reinterpret_cast<f4*>(vcache + ((size_t)h * P + k0 + key) * 64 + d4) = vv4;
-      }
+      *reinterpret_cast<f4*>(&vs[key][d4]) = vreg[j];
+      if (diag && k0 + key < T)
+        *reinterpret_cast<f4*>(vcache + ((size_t)h * P + k0 + key) * 64 + d4) = vreg[j];
     }
-    // each wavefront has its own LDS tiles and LDS executes a wavefront's accesses in
+    if (diag && k0 + l32 < T) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<f4*>(kcache + ((size_t)h * P + k0 + l32) * 64 + 32 * half + 4 * j) = kr[j];
+    }
+    // each wavefront has its own LDS tile and LDS executes a wavefront's accesses in
     // order, so only the compiler has to be kept from reordering
     __builtin_amdgcn_wave_barrier();
-    if (tile + NWV <= last_tile) fetch(tile + NWV);
+    if (tile + NWV <= last_tile) fetch_v(tile + NWV);
 
-    // S^T = K . Q^T : A operand lane -> K[key l32][d = 2s + half]
+    // S^T = K . Q^T
     f16v sacc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) sacc[v] = 0.0f;
 #pragma unroll
-    for (int s = 0; s < 32; ++s)
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kt[2 * s + half][l32], qr[s], sacc, 0, 0, 0);
+    for (int j = 0; j < 8; ++j) {
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].x, qr[j].x, sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].y, qr[j].y, sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].z, qr[j].z, sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].w, qr[j].w, sacc, 0, 0, 0);
+    }
+    if (tile + NWV <= last_tile) fetch_k(tile + NWV);
     // lane holds keys k0 + 8*(v/4) + 4*half + v%4 of query qi
     float mx = -INFINITY;
 #pragma unroll
@@ -559,10 +576,10 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
-    // a tile can be fully masked for a query only on the diagonal tile's upper part,
-    // and there key k0 <= qi always holds for the first key: m_new is finite from the
-    // first tile a wavefront sees (tile 0 .. 3 hold keys <= q0 for every later block;
-    // a wavefront that never gets a tile keeps the neutral (-inf, 0, 0))
+    // Every tile a wavefront sees holds a key <= qi for each of its queries (tiles before
+    // the diagonal hold only such keys, and the diagonal tile's first key is q0 <= qi), so
+    // m_new is finite from its first tile on; a wavefront that never gets a tile keeps the
+    // neutral (-inf, 0, 0).
     const float corr = (m_run == -INFINITY) ? 0.0f : expf(m_run - m_new);
     float psum = 0.0f;
 #pragma unroll
@@ -591,7 +608,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
     Ms[wave][l32] = m_run;
     Ls[wave][l32] = l_run;
   }
-  __syncthreads();  // every wavefront is done with its K/V tiles too
+  __syncthreads();  // every wavefront is done with its V tile too
   float M = Ms[0][l32];
 #pragma unroll
   for (int w = 1; w < NWV; ++w) M = fmaxf(M, Ms[w][l32]);
@@ -602,8 +619,8 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
     const float mw = Ms[w][l32];
     L += ((mw == -INFINITY) ? 0.0f : expf(mw - M)) * Ls[w][l32];
   }
-  // O^T of the four wavefronts through LDS (the K tiles' space: [wave][d 0..63][query])
-  float (*ob)[KT + 1] = Kt[wave];
+  // O^T of the wavefronts through LDS (the V tiles' space: [wave][d 0..63][query])
+  float (*ob)[KT + 1] = reinterpret_cast<float (*)[KT + 1]>(Vs[wave]);
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     const int d = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -611,14 +628,16 @@ __global__ __launch_bounds__(256) void k_attn_prefill64(const float* __restrict_
     ob[32 + d][l32] = o1[v] * mine;
   }
   __syncthreads();
-  // wavefront w writes d in [16 w, 16 w + 16): lane -> (query l32, 8 d values by half)
+  // wavefront w writes d in [8 w, 8 w + 8): lane -> (query l32, 4 d values by half)
   if (qi < T) {
     const float inv = 1.0f / L;
     float* dst = out + (size_t)qi * C + h * 64;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int d = 16 * wave + 8 * half + j;
-      const float sum = (Kt[0][d][l32] + Kt[1][d][l32]) + (Kt[2][d][l32] + Kt[3][d][l32]);
+    for (int j = 0; j < 64 / NWV / 2; ++j) {
+      const int d = (64 / NWV) * wave + (64 / NWV / 2) * half + j;
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NWV; ++w) sum += reinterpret_cast<float (*)[KT + 1]>(Vs[w])[d][l32];
       dst[d] = sum * inv;
     }
   }
@@ -918,7 +937,7 @@ hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_d
                                hipStream_t s) {
   if (head_dim == 64) {
     const int qblocks = (T + 31) / 32;
-    hipLaunchKernelGGL(k_attn_prefill64, dim3(qblocks, H), dim3(256), 0, s, qkv, T, C, P, kcache,
+    hipLaunchKernelGGL(k_attn_prefill64, dim3(H, qblocks), dim3(512), 0, s, qkv, T, C, P, kcache,
                        vcache, out);
   } else {
     const int n = T * H;
