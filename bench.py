@@ -51,8 +51,11 @@ def main() -> int:
     ap.add_argument("--prefill", type=int, default=None, help="tokens in the cache before decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
-                    help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "batch-decode"],
+                    help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound); "
+                         "batch-decode: a step is one greedy step of --batch sequences")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--bf16", action="store_true", help="store the weights as bf16 (fp32 arithmetic)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this path runs on ONE GPU (a batch-1 decode step has one all-reduce of "
@@ -75,11 +78,17 @@ def main() -> int:
     t0 = time.time()
     path = {"auto": _lib.PG_DECODE_AUTO, "kernels": _lib.PG_DECODE_KERNELS,
             "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
-    model = Gpt2Model.new(cfg, weights, Gpt2HipConfig(device=0, decode_path=path))
+    storage = _lib.PG_STORE_BF16 if args.bf16 else _lib.PG_STORE_F32
+    if args.bf16 and args.workload != "batch-decode":
+        log("bench.py: --bf16 is for --workload batch-decode")
+        return 2
+    model = Gpt2Model.new(cfg, weights, Gpt2HipConfig(device=0, weight_storage=storage, decode_path=path))
     log(f"[bench] upload: {time.time() - t0:.1f}s; backend: {model.describe()}")
 
     if args.workload == "prefill":
         return bench_prefill(args, cfg, model, ids, n_prefill)
+    if args.workload == "batch-decode":
+        return bench_batch_decode(args, cfg, model, n_prefill)
 
     cache = model.new_kv_cache()
     t0 = time.time()
@@ -220,6 +229,46 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
                      "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
                      "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
+    }
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def bench_batch_decode(args, cfg, model, n_prefill) -> int:
+    """Secondary workload (BASELINE.json configs[2] / configs[4] style): --batch sequences
+    prefilled to n_prefill tokens each, then --steps greedy steps for all of them.  A step
+    reads every weight once plus the K/V rows of every sequence: HBM-bound."""
+    from puppygrad_amd import synth
+    B = args.batch
+    room = cfg.n_positions - n_prefill
+    steps = min(args.steps, room - 1)
+    ids = np.stack([synth.token_ids(n_prefill, synth.TOKEN_SEED_BASE + 100 + b, cfg.vocab_size) for b in range(B)])
+    cache = model.new_kv_cache(B)
+    t0 = time.time()
+    model.prefill_batch(ids, cache).argmax()
+    prefill_s = time.time() - t0
+    toks, st = model.decode_greedy_batch(cache, steps + 1)  # steps + 1 tokens per sequence, steps forwards
+    n = st.generated_tokens - 1
+    sec = st.gpu_decode_time / n
+    C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    wbytes = (2 if args.bf16 else 4) * (L * (4 * C_ * C_ + 2 * C_ * I) + V * C_)
+    kvb = sum(kv_bytes(cfg, p) for p in range(n_prefill, n_prefill + n)) / n * B
+    achieved = (wbytes + kvb) / sec / 1e9
+    info = _devinfo()
+    result = {
+        "metric": f"batched decode tokens/sec, GPT-2 {args.model} {'bf16-stored' if args.bf16 else 'fp32'} bs={B}",
+        "value": round(B / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": n, "warmup": 0,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"GPT-2 {args.model} B={B} greedy decode, every KV cache prefilled to {n_prefill} "
+                               f"tokens, weights stored as {'bf16' if args.bf16 else 'f32'}",
+                   "device": info.name.decode() or info.arch.decode(), "compute_units": info.compute_units,
+                   "backend": model.describe()},
+        "prefill_s": round(prefill_s, 3),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "all launches of one batched step",
+                     "algorithmic_bytes_per_step": int(wbytes + kvb)},
     }
     print(json.dumps(result), flush=True)
     return 0
