@@ -817,7 +817,7 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 16 : 8;
   if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
   const long tiles = (a.N + 31) / 32;
-  long parts = std::max<long>(1, num_cus / tiles);
+  long parts = std::max<long>(1, (num_cus + tiles / 2) / tiles);
   parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 16));
   parts = std::min<long>(parts, 8);
   if (parts > 1) {
