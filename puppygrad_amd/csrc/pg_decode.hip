@@ -376,11 +376,12 @@ __device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, 
   return r;
 }
 
-// Key splits per head at position pos: one (and then no merge hop: the item's result is
-// the head's attention output) while all keys fit a single item, the launch's count
-// otherwise.  Every wavefront of the grid derives the same value.
+// Key splits per head at position pos: as few as hold the pos + 1 keys in items of at
+// most kMaxItemKeys (never more than the launch's count, which covers the longest context).
+// With one split there is no merge hop: the item's result is the head's attention output.
+// Every wavefront of the grid derives the same value.
 __device__ __forceinline__ int splits_at(const DecodeParams& p, int pos) {
-  return pos + 1 <= kMaxItemKeys ? 1 : p.ns;
+  return min((pos + kMaxItemKeys) / kMaxItemKeys, p.ns);
 }
 
 // ---- service side: poll tagged words ---------------------------------------------------

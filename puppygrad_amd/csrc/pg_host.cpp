@@ -817,9 +817,11 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
       shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
     }
     if (shape_ok) {
-      int ns = std::min<int>(16, grid / (int)g.H);
-      ns = std::max<int>(ns, (int)((g.P + 127) / 128));
-      ns = std::max(ns, 1);
+      // key splits per head at the longest context (the kernel uses as few as the position
+      // at hand needs: fewer splits are fewer partials to merge and fewer workgroups held
+      // up by attention)
+      int ns = std::max<int>(1, (int)((g.P + pgk::persistent_max_item_keys() - 1) /
+                                      pgk::persistent_max_item_keys()));
       shape_ok = ns <= pgk::kMaxSplits && (size_t)ns * 66 <= g.I;
       m->attn_splits = ns;
     }
