@@ -821,12 +821,22 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       if (lane == 0) ctl->flag[6] = epp;
       PG_STAMP(l, 1);
 
-      // ================= B2: the workgroup that took split 0 of a head merges it ====
+      // ================= B2: merge of a head's splits ================================
+      // By a workgroup without an attention item of its own where there are enough of
+      // those (workgroup items + h merges head h: it is polling while the others still
+      // compute), else by the one that took the head's split 0.
       const unsigned epa = epoch_of(p, t, l, 2);
+      const bool spare = items + H <= G;
 #pragma unroll 1
-      for (int item = wg; ns > 1 && item < items; item += G) {
-        const int h = item / ns, s = item - h * ns;
-        if (s != 0) continue;
+      for (int slot = wg; ns > 1 && slot < (spare ? items + H : items); slot += G) {
+        int h;
+        if (spare) {
+          if (slot < items) continue;
+          h = slot - items;
+        } else {
+          h = slot / ns;
+          if (slot - h * ns != 0) continue;
+        }
         // the head's ns partials (66 words each) are one run of tagged words: probe the
         // last word of every partial, then read them all into LDS (the staging area of
         // the long vector, idle now) and merge from there
