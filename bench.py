@@ -285,7 +285,7 @@ def _devinfo():
 # (127 forwards from cache length 896), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this file (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the
 # counters and the copy-kernel scale factors).  None for any other workload.
-TRAFFIC_XL_DEFAULT = 909.7e9
+TRAFFIC_XL_DEFAULT = 891.8e9
 
 
 def measured_traffic(args, n_prefill, persistent, launches):
