@@ -817,8 +817,11 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           }
         }
       }
-      // the credit of the second attention hop (the streamers request a slice on it)
-      if (lane == 0) ctl->flag[6] = epp;
+      // The credit of the second attention hop (the streamers request a slice on it).  A
+      // workgroup that merges a head gives it only after the merge: the partials it is about
+      // to read would otherwise queue behind that slice.
+      const bool merges = ns > 1 && items + H <= G && wg >= items && wg < items + H;
+      if (!merges && lane == 0) ctl->flag[6] = epp;
       PG_STAMP(l, 1);
 
       // ================= B2: merge of a head's splits ================================
@@ -898,6 +901,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         }
         PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
       }
+      if (merges && lane == 0) ctl->flag[6] = epp;
 
       // ================= D: attention output -> xsD =================
       {
