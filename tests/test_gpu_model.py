@@ -158,6 +158,13 @@ def long_cases():
     cfg = synth.Gpt2Config(vocab_size=97, n_positions=160, n_embd=192, n_layer=1, n_head=3)
     out.append(("c192_T160", cfg, synth.random_weights(cfg, 0x5EED0213, perturb=True),
                 list(synth.token_ids(160, 0x70C00213, 97))))
+    # 124M's layer shapes at 512 tokens: more 64x64 tiles than CUs with a partial last round
+    # (c_attn 288, c_fc 384: the tail-split form with BIAS and GELU epilogues), split-K for the
+    # projections back to n_embd, and attention blocks whose eight wavefronts get two key
+    # tiles each
+    cfg = synth.Gpt2Config(vocab_size=97, n_positions=512, n_embd=768, n_layer=1, n_head=12)
+    out.append(("c768_T512", cfg, synth.random_weights(cfg, 0x5EED0214, perturb=True),
+                list(synth.token_ids(512, 0x70C00214, 97))))
     return out
 
 
