@@ -191,6 +191,37 @@ def test_gemm_prefill_and_forward_match_oracle(case):
     assert_logits_close(tok_model.prefill(ids, c2).to_host(), want_all[-1])
 
 
+@pytest.mark.parametrize("n_prompt", [100, 1500, 2750])
+def test_persistent_decode_split_counts_match_oracle(n_prompt):
+    """The persistent decode kernel picks the number of key splits per head from the position:
+    one split and no merge hop up to 128 keys (prompt 100), several with the merge done by
+    workgroups that hold no attention item (prompt 1500: 12 splits, 144 items), and beyond one
+    item per workgroup with the merge by the head's first split (prompt 2750: 22 splits, 264
+    items on 256 workgroups).  One layer keeps the oracle cheap at these lengths."""
+    cfg = synth.Gpt2Config(vocab_size=300, n_positions=4096, n_embd=768, n_layer=1, n_head=12)
+    w = synth.random_weights(cfg, 0x5EED0215, perturb=True)
+    ids = list(synth.token_ids(n_prompt, 0x70C00215, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(8))
+    assert "decode=persistent" in model.describe()
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    rlog = None
+    for tok in (7, 123, 42):  # teacher-forced steps through the persistent kernel
+        rlog = ref.forward_one(tok, rcache)
+        assert_logits_close(model.forward_one(tok, cache).to_host(), rlog)
+    got, _ = model.decode_greedy(cache, 6)  # five forwards in one launch
+    want, clear = [], True
+    for i in range(6):
+        top = np.sort(rlog)[-2:]
+        clear = clear and (top[1] - top[0]) > 2 * (ABS_TOL + REL_TOL * abs(float(top[1])))
+        want.append(oracle.argmax_logits(rlog))
+        if i < 5:
+            rlog = ref.forward_one(want[-1], rcache)
+    assert len(got) == 6
+    if clear:  # no near-tie on the way: the ids are the oracle's
+        assert got == want
+
+
 def test_sampler_on_device_logits_matches_oracle():
     _, cfg, w, ids = small_cases()[1]
     model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
