@@ -531,6 +531,7 @@ constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
 // An item is the keys [k0, k1) of one head (at most 128).  Key k0 + slot + 32 i belongs
 // to slot = 4 wave + (lane >> 4), step i < 4; the 16 lanes of a slot hold 4 dims each.
 constexpr int kAttnSteps = kMaxItemKeys / 32;
+static_assert(kMaxItemKeys % 32 == 0, "an item is whole steps of 32 key slots");
 struct KvRegs {
   f4 k[kAttnSteps], v[kAttnSteps];
 };
