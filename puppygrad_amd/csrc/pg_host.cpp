@@ -329,7 +329,15 @@ hipError_t exchange_acquire(int device, size_t bytes, void** out, size_t* got_by
     }
   }
   *got_bytes = bytes;
-  return hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
+  hipError_t e = hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
+  if (e != hipSuccess) {
+    // no uncached memory to be had: ordinary device memory works too (the kernel's accesses
+    // to these words are agent-scope atomics and cache-bypassing scalar loads), only slower;
+    // it is pooled the same way
+    (void)hipGetLastError();
+    e = hipMalloc(out, bytes);
+  }
+  return e;
 }
 
 void exchange_release(int device, size_t bytes, void* p) {
