@@ -484,24 +484,30 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   PG_HIP(hipMemcpyAsync(d_ids, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
   PG_HIP(hipStreamSynchronize(s));  // ids is the caller's pageable memory
   PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s, m->w_bf16));
+  // (ln_g / ln_b: the LayerNorm that reads this projection's result, written to XN by the
+  // same call: fused into the projection's reduce where it has one)
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
-                  int ldc, int N, int K, int epi) -> hipError_t {
+                  int ldc, int N, int K, int epi, const float* ln_g = nullptr,
+                  const float* ln_b = nullptr) -> hipError_t {
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = T; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
     a.ws = WS.p; a.ws_floats = ws_floats;
+    if (ln_g) { a.ln_out = XN.p; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
+  PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b, g.eps, s));
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
-    PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, w.ln_1_g, w.ln_1_b, g.eps, s));
+    // the LayerNorm after this layer: the next layer's ln_1; ln_f is applied where it is needed
+    const float* next_g = l + 1 < g.L ? m->layers[l + 1].ln_1_g : nullptr;
+    const float* next_b = l + 1 < g.L ? m->layers[l + 1].ln_1_b : nullptr;
     PG_HIP(gemm(XN.p, C, w.c_attn_w, w.c_attn_b, QKV.p, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
     PG_HIP(pgk::launch_attn_prefill(QKV.p, T, C, H, hd, P, c->k_panel(l, b), c->v_panel(l, b),
                                     ATT.p, SCR.p, s));
-    PG_HIP(gemm(ATT.p, C, w.c_proj_w, w.c_proj_b, X.p, C, C, C, pgk::GEMM_RESID));
-    PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, w.ln_2_g, w.ln_2_b, g.eps, s));
+    PG_HIP(gemm(ATT.p, C, w.c_proj_w, w.c_proj_b, X.p, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));
     PG_HIP(gemm(XN.p, C, w.c_fc_w, w.c_fc_b, HB.p, I, I, C, pgk::GEMM_GELU));
-    PG_HIP(gemm(HB.p, I, w.c_proj_mlp_w, w.c_proj_mlp_b, X.p, C, C, I, pgk::GEMM_RESID));
+    PG_HIP(gemm(HB.p, I, w.c_proj_mlp_w, w.c_proj_mlp_b, X.p, C, C, I, pgk::GEMM_RESID, next_g, next_b));
   }
   if (all_logits_dst) {
     PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->ln_f_g, m->ln_f_b, g.eps, s));
@@ -536,18 +542,26 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   bs.kv = g.H * g.P * g.hd();
   bs.part = (size_t)H * pgk::kMaxSplits;
   bs.out = g.C;
+  // (ln_g / ln_b: the LayerNorm that reads this projection's result, written to xn_b by the
+  // same call: fused into the projection's reduce where it has one)
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
-                  int ldc, int N, int K, int epi) -> hipError_t {
+                  int ldc, int N, int K, int epi, const float* ln_g = nullptr,
+                  const float* ln_b = nullptr) -> hipError_t {
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
     a.ws = c->gemm_ws; a.ws_floats = c->gemm_ws_floats;
+    if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
+  PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b,
+                                     g.eps, s));
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
-    PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, w.ln_1_g, w.ln_1_b, g.eps, s));
+    // the LayerNorm after this layer: the next layer's ln_1, or ln_f
+    const float* next_g = l + 1 < g.L ? m->layers[l + 1].ln_1_g : m->ln_f_g;
+    const float* next_b = l + 1 < g.L ? m->layers[l + 1].ln_1_b : m->ln_f_b;
     PG_HIP(gemm(c->xn_b, C, w.c_attn_w, w.c_attn_b, c->qkv_b, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
     PG_HIP(pgk::launch_kv_append(c->qkv_b, B, C, hd, P, (int)pos, c->k_panel(l, 0),
                                  c->v_panel(l, 0), bs.kv, s));
@@ -555,12 +569,10 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
                                    hd, nsplit, c->part_acc, c->part_m, c->part_l, s, B, bs));
     PG_HIP(pgk::launch_attn_finish(c->part_acc, c->part_m, c->part_l, H, hd, nsplit, c->att_b, s,
                                    B, bs));
-    PG_HIP(gemm(c->att_b, C, w.c_proj_w, w.c_proj_b, c->x, C, C, C, pgk::GEMM_RESID));
-    PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, w.ln_2_g, w.ln_2_b, g.eps, s));
+    PG_HIP(gemm(c->att_b, C, w.c_proj_w, w.c_proj_b, c->x, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));
     PG_HIP(gemm(c->xn_b, C, w.c_fc_w, w.c_fc_b, c->hbuf, I, I, C, pgk::GEMM_GELU));
-    PG_HIP(gemm(c->hbuf, I, w.c_proj_mlp_w, w.c_proj_mlp_b, c->x, C, C, I, pgk::GEMM_RESID));
+    PG_HIP(gemm(c->hbuf, I, w.c_proj_mlp_w, w.c_proj_mlp_b, c->x, C, C, I, pgk::GEMM_RESID, next_g, next_b));
   }
-  PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, m->ln_f_g, m->ln_f_b, g.eps, s));
   PG_HIP(gemm(c->xn_b, C, m->wte, nullptr, c->logits_buf, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
   return PG_OK;
 }

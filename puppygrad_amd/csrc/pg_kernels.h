@@ -113,6 +113,12 @@ struct GemmArgs {
   size_t ws_floats = 0;   // its size
   int tail_first = 0;     // filled by gemm_tail_plan: first tile of the tail that is cut along K,
   int tail_parts = 1;     // and the number of parts
+  // Optional: also write LayerNorm(row of C) to ln_out[M][N] (needs ldc == N).  Fused into the
+  // split-K reduce where the chosen form has one, a separate launch otherwise.
+  float* ln_out = nullptr;
+  const float* ln_g = nullptr;
+  const float* ln_b = nullptr;
+  float ln_eps = 0.0f;
 };
 bool gemm_supported(const GemmArgs& a);
 int gemm_split_parts(const GemmArgs& a, int num_cus);

@@ -238,6 +238,79 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
   }
 }
 
+// k_splitk_reduce for one whole row per block, followed by the LayerNorm of that row
+// (layer_norm_in_place, cpu.rs:119-143: mean, biased variance in a second pass, eps inside
+// the root) into a.ln_out: the projection back to n_embd and the LayerNorm that reads its
+// result are one launch.  N <= 4096, a multiple of 4; ldc == N.
+template <int EPI>
+__global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts) {
+  __shared__ float red[4];
+  const size_t m = blockIdx.x;
+  const int n4 = a.N / 4;
+  const size_t stride = (size_t)a.M * a.N;
+  auto bsum = [&](float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+  };
+  f4 c[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int i = (int)threadIdx.x + 256 * q;
+    c[q] = f4{0.f, 0.f, 0.f, 0.f};
+    if (i < n4) {
+      const size_t n = (size_t)i * 4;
+      f4 v[8];
+#pragma unroll
+      for (int p = 0; p < 8; ++p)
+        v[p] = *reinterpret_cast<const f4*>(a.ws + (size_t)min(p, parts - 1) * stride + m * a.N + n);
+      f4 s = v[0];
+#pragma unroll
+      for (int p = 1; p < 8; ++p)
+        if (p < parts) s += v[p];
+      const f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
+      float r[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (EPI == GEMM_GELU) r[k] = gelu_tanh(r[k]);
+        if (EPI == GEMM_RESID) r[k] = a.resid[m * a.ldc + n + k] + r[k];
+      }
+      c[q] = f4{r[0], r[1], r[2], r[3]};
+      *reinterpret_cast<f4*>(a.C + m * a.ldc + n) = c[q];
+    }
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) sum += (c[q].x + c[q].y) + (c[q].z + c[q].w);
+  const float mean = bsum(sum) / (float)a.N;
+  float var = 0.0f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if ((int)threadIdx.x + 256 * q < n4) {
+      const float d0 = c[q].x - mean, d1 = c[q].y - mean, d2 = c[q].z - mean, d3 = c[q].w - mean;
+      var += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    }
+  }
+  const float inv = 1.0f / sqrtf(bsum(var) / (float)a.N + a.ln_eps);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int i = (int)threadIdx.x + 256 * q;
+    if (i < n4) {
+      const size_t n = (size_t)i * 4;
+      const f4 g = *reinterpret_cast<const f4*>(a.ln_g + n), b = *reinterpret_cast<const f4*>(a.ln_b + n);
+      f4 o;
+      o.x = (c[q].x - mean) * inv * g.x + b.x;
+      o.y = (c[q].y - mean) * inv * g.y + b.y;
+      o.z = (c[q].z - mean) * inv * g.z + b.z;
+      o.w = (c[q].w - mean) * inv * g.w + b.w;
+      *reinterpret_cast<f4*>(a.ln_out + m * a.N + n) = o;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // A batch of at most MB rows against W (the projections of a batched decode step).  The
 // job is to stream W once at the speed of HBM, and tiles that stage W through LDS cut it
@@ -768,11 +841,21 @@ bool gemm_supported(const GemmArgs& a) {
 }
 
 namespace {
-template <bool WBF>
-hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s) {
-  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
-  const int grid = (tiles + 7) / 8 * 8;
-  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 1>), dim3(grid, parts), dim3(256), 0, s, a);
+// Finishes a.ws[parts][M][N]: bias, epilogue and, where asked for and possible, the
+// LayerNorm of the result in the same launch (*ln_done tells).
+hipError_t launch_splitk_reduce(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
+  if (a.ln_out && a.N % 4 == 0 && a.N <= 4096 && a.ldc == a.N) {
+    if (epi == GEMM_BIAS)
+      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_BIAS>, dim3(a.M), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_GELU)
+      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_GELU>, dim3(a.M), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_RESID)
+      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_RESID>, dim3(a.M), dim3(256), 0, s, a, parts);
+    else
+      return hipErrorInvalidValue;
+    *ln_done = true;
+    return hipGetLastError();
+  }
   const unsigned rblocks = (unsigned)(((size_t)a.M * (a.N / 4) + 255) / 256);
   if (epi == GEMM_BIAS)
     hipLaunchKernelGGL(k_splitk_reduce<GEMM_BIAS>, dim3(rblocks), dim3(256), 0, s, a, parts);
@@ -783,6 +866,14 @@ hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t 
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
+}
+
+template <bool WBF>
+hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int grid = (tiles + 7) / 8 * 8;
+  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 1>), dim3(grid, parts), dim3(256), 0, s, a);
+  return launch_splitk_reduce(a, epi, parts, s, ln_done);
 }
 template <int MB, int R, bool WBF>
 hipError_t launch_gemv_rows_r(const GemmArgs& a, int epi, hipStream_t s) {
@@ -827,7 +918,7 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   return (int)std::max<long>(parts, 1);
 }
 template <bool WBF>
-hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s) {
+hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
   const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)parts);
   if (epi == GEMM_BIAS)
     hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF>), grid, dim3(512), 0, s, a);
@@ -837,15 +928,7 @@ hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t
     hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF>), grid, dim3(512), 0, s, a);
   else
     return hipErrorInvalidValue;
-  if (parts > 1) {
-    const unsigned rblocks = (unsigned)(((size_t)a.M * (a.N / 4) + 255) / 256);
-    if (epi == GEMM_BIAS)
-      hipLaunchKernelGGL(k_splitk_reduce<GEMM_BIAS>, dim3(rblocks), dim3(256), 0, s, a, parts);
-    else if (epi == GEMM_GELU)
-      hipLaunchKernelGGL(k_splitk_reduce<GEMM_GELU>, dim3(rblocks), dim3(256), 0, s, a, parts);
-    else
-      hipLaunchKernelGGL(k_splitk_reduce<GEMM_RESID>, dim3(rblocks), dim3(256), 0, s, a, parts);
-  }
+  if (parts > 1) return launch_splitk_reduce(a, epi, parts, s, ln_done);
   return hipGetLastError();
 }
 
@@ -903,7 +986,21 @@ bool gemm_tail_plan(GemmArgs& a, int num_cus) {
   return true;
 }
 
+namespace {
+hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t s, bool* ln_done);
+}
+
 hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
+  if (a.ln_out && a.ldc != a.N) return hipErrorInvalidValue;
+  bool ln_done = false;
+  hipError_t e = launch_gemm_form(a, epi, num_cus, s, &ln_done);
+  if (e == hipSuccess && a.ln_out && !ln_done)
+    e = launch_layer_norm_rows(a.C, a.ln_out, a.M, a.N, a.ln_g, a.ln_b, a.ln_eps, s);
+  return e;
+}
+
+namespace {
+hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t s, bool* ln_done) {
   if (!gemm_supported(a)) return hipErrorInvalidValue;
   // A small decode batch over a short K: whole rows of W per wavefront, no MFMA tiles.
   // (Every block stages all input vectors; beyond 16 x 1024 values that costs more than it
@@ -912,10 +1009,12 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
     return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);
   // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
   if (const int rp = gemm_rows32_parts(a, num_cus))
-    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s) : launch_gemm_rows32<false>(a, epi, rp, s);
+    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done)
+                    : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
   const int parts = gemm_split_parts(a, num_cus);
   if (parts > 1)
-    return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s) : launch_gemm_split<false>(a, epi, parts, s);
+    return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s, ln_done)
+                    : launch_gemm_split<false>(a, epi, parts, s, ln_done);
   // 128x128 tiles once they fill the chip about twice over, 64x64 tiles otherwise
   const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
   if (a.w_bf16) {
@@ -931,6 +1030,7 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   }
   return launch_gemm_tile<64, 64, false>(a, epi, s);
 }
+}  // namespace
 
 hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
                                float* kcache, float* vcache, float* out, float* scratch,
