@@ -563,10 +563,14 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     const float* next_g = l + 1 < g.L ? m->layers[l + 1].ln_1_g : m->ln_f_g;
     const float* next_b = l + 1 < g.L ? m->layers[l + 1].ln_1_b : m->ln_f_b;
     PG_HIP(gemm(c->xn_b, C, w.c_attn_w, w.c_attn_b, c->qkv_b, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
-    PG_HIP(pgk::launch_kv_append(c->qkv_b, B, C, hd, P, (int)pos, c->k_panel(l, 0),
-                                 c->v_panel(l, 0), bs.kv, s));
+    // K/V append (rust.rs:1677-1683): by the attention launch itself for head_dim 64
+    const bool fused_append = hd == pgk::kHeadDim;
+    if (!fused_append)
+      PG_HIP(pgk::launch_kv_append(c->qkv_b, B, C, hd, P, (int)pos, c->k_panel(l, 0),
+                                   c->v_panel(l, 0), bs.kv, s));
     PG_HIP(pgk::launch_attn_decode(c->qkv_b, c->k_panel(l, 0), c->v_panel(l, 0), (int)pos, P, H,
-                                   hd, nsplit, c->part_acc, c->part_m, c->part_l, s, B, bs));
+                                   hd, nsplit, c->part_acc, c->part_m, c->part_l, s, B, bs,
+                                   fused_append ? C : 0));
     PG_HIP(pgk::launch_attn_finish(c->part_acc, c->part_m, c->part_l, H, hd, nsplit, c->att_b, s,
                                    B, bs));
     PG_HIP(gemm(c->att_b, C, w.c_proj_w, w.c_proj_b, c->x, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));

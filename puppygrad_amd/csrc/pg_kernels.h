@@ -64,11 +64,14 @@ struct BatchStrides {
   size_t part = 0;  // (head, split) partial slots
   size_t out = 0;   // attention output vectors (floats)
 };
-// Split-key decode attention for one query per sequence over keys [0, pos].
+// Split-key decode attention for one query per sequence over keys [0, pos].  With
+// append_C = n_embd (head_dim 64 only) q is the step's interleaved qkv row and the rows of
+// position pos are taken from it and written to the cache panels by the same launch;
+// with 0 they are in the cache already.
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
                               float* part_m, float* part_l, hipStream_t s, int batch = 1,
-                              BatchStrides bs = BatchStrides{});
+                              BatchStrides bs = BatchStrides{}, int append_C = 0);
 int choose_nsplit(int n_keys, int H, int num_cus);
 
 // out[r] = argmax of row r of v[rows][n] with the reference's tie/NaN rules.

@@ -228,11 +228,15 @@ __global__ void k_embed(float* x, const float* wte, const float* wpe, const uint
 // takes the max-subtracted exponentials (softmax_in_place, cpu.rs:152-165) and
 // accumulates p.V; the per-split (acc, m, l) are merged by the consumer.
 __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restrict__ q,
-                                                          const float* __restrict__ kcache,
-                                                          const float* __restrict__ vcache,
+                                                          const float* kcache, const float* vcache,
                                                           int pos, int P, int nsplit,
                                                           float* part_acc, float* part_m,
-                                                          float* part_l, BatchStrides bs) {
+                                                          float* part_l, BatchStrides bs,
+                                                          int append_C) {
+  // append_C > 0: the rows of position pos are not in the cache yet.  They are the k and v
+  // parts of this step's interleaved qkv row (q + append_C, q + 2 append_C); the block whose
+  // split holds pos uses them from there and writes them to the cache panels
+  // (rust.rs:1677-1683), which saves the launch that would only copy them.
   extern __shared__ float sc[];  // scores of this split
   __shared__ float red[kWaves];
   __shared__ float accs[kWaves][64];
@@ -265,6 +269,18 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
   const float4* K4 = reinterpret_cast<const float4*>(kcache + (size_t)h * P * 64);
   const float4* V4 = reinterpret_cast<const float4*>(vcache + (size_t)h * P * 64);
   const float scale = 1.0f / sqrtf(64.0f);
+  if (append_C > 0 && k1 == n) {
+    // the block whose split holds pos: sixteen lanes copy the two rows, and the block reads
+    // them back from the panels like any other key (same CU: visible after the barrier)
+    if (tid < 16) {
+      const float4 knew = reinterpret_cast<const float4*>(q + append_C + h * 64)[d4];
+      const float4 vnew = reinterpret_cast<const float4*>(q + 2 * append_C + h * 64)[d4];
+      reinterpret_cast<float4*>(const_cast<float*>(kcache) + (size_t)h * P * 64)[(size_t)pos * 16 + d4] = knew;
+      reinterpret_cast<float4*>(const_cast<float*>(vcache) + (size_t)h * P * 64)[(size_t)pos * 16 + d4] = vnew;
+    }
+    __threadfence_block();
+    __syncthreads();
+  }
 
   float mx = -INFINITY;
   for (int k = k0 + wave * 4 + sub; k < k1; k += kWaves * 4) {
@@ -584,11 +600,11 @@ int choose_nsplit(int n_keys, int H, int num_cus) {
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
                               float* part_m, float* part_l, hipStream_t s, int batch,
-                              BatchStrides bs) {
+                              BatchStrides bs, int append_C) {
   if (head_dim == kHeadDim) {
     int per = (pos + 1 + nsplit - 1) / nsplit;
     hipLaunchKernelGGL(k_attn_decode64, dim3(nsplit, H, batch), dim3(kBlock), per * sizeof(float),
-                       s, q, kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l, bs);
+                       s, q, kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l, bs, append_C);
   } else {
     hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H, batch), dim3(kBlock),
                        (pos + 1) * sizeof(float), s, q, kcache, vcache, pos, P, head_dim, part_acc,
