@@ -8,24 +8,28 @@
 // one agent-scope store; a reader polls until the word carries the epoch of the
 // producing (token, layer, phase).
 //
-// Vector memory loads of one wavefront return in issue order, so a wavefront that
-// polls global memory behind a prefetch of weights sees the answer only after the
-// weights have landed, and a wavefront that holds prefetched weights must not poll.
-// The roles are therefore split:
+// Vector memory instructions of a CU complete in issue order, across all of its
+// wavefronts: a poll of global memory sees its answer only after every weight byte the CU
+// requested before it has landed.  Deep weight prefetch and low-latency polling exclude
+// each other on that path, so the roles are split:
 //
 //   * wavefronts 0..6 ("streamers") own the rows of every weight matrix of this
-//     workgroup's band.  They only ever wait on flags in LDS, keep up to two weight
-//     bands in flight in their registers (the band in use and the next one or two,
-//     requested in consumption order as soon as registers free up), multiply and
-//     publish their rows.
-//   * wavefront 7 ("service") owns the dependency chain: it polls the tagged words,
-//     applies LayerNorm, stages the input vector of the next matrix in LDS and raises
-//     the LDS flag; it also runs this workgroup's (head, key-split) attention item,
-//     the per-head merge, the embedding and the argmax merge.
+//     workgroup's band.  They only ever wait on flags in LDS, hold the rows in registers
+//     (part of the widest model's mlp row in LDS), request the layer's weights as one
+//     stream cut into six slices, each at a moment when the chain has just made a hop,
+//     multiply and publish their rows.
+//   * wavefront 7 ("service") owns the dependency chain: it probes the tagged words with
+//     scalar loads (another path, not queued behind the weights), reads a complete vector
+//     once with vector loads, applies LayerNorm, stages the input vector of the next matrix
+//     in LDS and raises the LDS flag; it also runs this workgroup's (head, key-split)
+//     attention item together with the streamers, the per-head merge (workgroups without
+//     an attention item do that where there are enough of them), the embedding and the
+//     argmax merge.
 //
 // Per layer:  A  LN1 + c_attn rows            -> qkv_t   (tagged)
 //             B  split-key attention per head -> part_t  (tagged partial acc, m, l)
-//             B2 per-head merge of the splits -> attn_t  (tagged)
+//             B2 per-head merge of the splits -> attn_t  (tagged; B writes it directly
+//                                                         when one split holds all keys)
 //             D  c_proj rows + residual       -> xa_t    (tagged)
 //             E  LN2 + c_fc rows + GELU       -> h_t     (tagged)
 //             F  mlp c_proj rows + residual   -> xm_t    (tagged)
