@@ -253,6 +253,49 @@ pg_status pg_op_attention_decode(int32_t device, const float* qkv, uint64_t pos,
 /* argmax_logits (src/models/generation.rs:269-279) on a host vector. */
 pg_status pg_op_argmax(int32_t device, const float* values, uint64_t n, uint32_t* out);
 
+/* ---- model assets: safetensors store, config.json, model directory ---- */
+
+/* TensorStore (src/models/safetensors.rs:93-138) over a read-only mapping of one
+ * .safetensors file; read_safetensors_file + TensorStore::from_bytes
+ * (safetensors.rs:79-101).  Failures are PG_ASSET with the reference's wording
+ * ("failed to read safetensors file {path}: ...", "failed to parse safetensors
+ * file {path}: ...", safetensors.rs:40-70). */
+typedef struct pg_tensor_store pg_tensor_store;
+pg_status pg_tensor_store_open(const char* path, pg_tensor_store** out);
+void pg_tensor_store_close(pg_tensor_store* store);
+/* Number of tensors in the file. */
+uint64_t pg_tensor_store_len(const pg_tensor_store* store);
+/* TensorStore::required_f32 (safetensors.rs:125-129): dtype must be F32 (else
+ * PG_ASSET "tensor {name} has dtype {actual}, expected F32"), the shape must equal
+ * shape[0..ndim) (else PG_INVALID_WEIGHTS "tensor {name} shape [..] does not match
+ * expected [..]", the mapping of src/models/gpt2/rust.rs:773-785); a missing tensor
+ * is PG_ASSET "failed to read tensor {name}: ...".  out->data points into the store
+ * (little-endian f32, as f32_data reads it, safetensors.rs:172-185) and is valid
+ * until pg_tensor_store_close. */
+pg_status pg_tensor_store_required_f32(const pg_tensor_store* store, const char* name,
+                                       const uint64_t* shape, size_t ndim, pg_tensor* out);
+/* TensorStore::optional_f32 (safetensors.rs:131-137): a missing tensor is not an
+ * error; *found says whether out was filled. */
+pg_status pg_tensor_store_optional_f32(const pg_tensor_store* store, const char* name,
+                                       const uint64_t* shape, size_t ndim, int32_t* found,
+                                       pg_tensor* out);
+
+/* load_config (src/models/gpt2/rust.rs:684-711): reads a Hugging Face GPT-2
+ * config.json (vocab_size, n_positions or n_ctx, n_embd, n_layer, n_head; optional
+ * n_inner and layer_norm_epsilon; other keys ignored) and validates it.
+ * Unreadable or malformed files are PG_ASSET ("failed to read config {path}: ...",
+ * "failed to parse config {path}: ...", src/models/config.rs:19-29). */
+pg_status pg_gpt2_load_config(const char* path, pg_gpt2_config* out);
+
+/* Gpt2Runtime::from_dir_with_backend without the tokenizer
+ * (src/models/gpt2/rust.rs:382-393): {model_dir}/config.json and
+ * {model_dir}/model.safetensors (src/models/gpt2/assets.rs:20-30), tensor names and
+ * shapes as load_weights with the `transformer.` prefix fallback
+ * (rust.rs:713-771), then pg_gpt2_create.  Tensors are uploaded straight from the
+ * file mapping; no host copy of the weights is made. */
+pg_status pg_gpt2_create_from_dir(const char* model_dir, const pg_hip_options* options,
+                                  pg_gpt2_model** out);
+
 /* Seeded synthetic inputs for benchmarks and tests (no reference counterpart;
  * the draw is the reference's splitmix64, src/models/generation.rs:244-267).
  * Element i of the stream uses draws 2i and 2i+1 of SmallRng::new(seed):

@@ -123,6 +123,15 @@ SIGNATURES = {
     "pg_op_attention_decode": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _f32p, _f32p, C.c_uint64,
                                          C.c_uint64, C.c_uint64, _f32p]),
     "pg_op_argmax": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _u32p]),
+    "pg_tensor_store_open": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
+    "pg_tensor_store_close": (None, [_vp]),
+    "pg_tensor_store_len": (C.c_uint64, [_vp]),
+    "pg_tensor_store_required_f32": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.c_size_t,
+                                               C.POINTER(pg_tensor)]),
+    "pg_tensor_store_optional_f32": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.c_size_t,
+                                               C.POINTER(C.c_int32), C.POINTER(pg_tensor)]),
+    "pg_gpt2_load_config": (C.c_int, [C.c_char_p, C.POINTER(pg_gpt2_config)]),
+    "pg_gpt2_create_from_dir": (C.c_int, [C.c_char_p, C.POINTER(pg_hip_options), C.POINTER(_vp)]),
     "pg_synth_normal_f32": (None, [_f32p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double]),
     "pg_synth_token_ids": (None, [_u32p, C.c_uint64, C.c_uint64, C.c_uint64]),
     "pg_device_query": (C.c_int, [C.c_int32, C.POINTER(pg_device_info)]),

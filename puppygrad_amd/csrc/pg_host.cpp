@@ -19,6 +19,7 @@
 #include <thread>
 #include <vector>
 
+#include "pg_internal.h"
 #include "pg_kernels.h"
 
 namespace {
@@ -691,6 +692,11 @@ pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg
 
 
 }  // namespace
+
+namespace pgh {
+pg_status fail(pg_status s, const std::string& msg) { return ::fail(s, msg); }
+pg_status validate_config(const pg_gpt2_config& c) { return ::validate_config(c); }
+}  // namespace pgh
 
 extern "C" {
 

@@ -70,6 +70,18 @@ class Gpt2Config:
         return _lib.pg_gpt2_config(self.vocab_size, self.n_positions, self.n_embd, self.n_layer,
                                    self.n_head, self.n_inner, self.layer_norm_epsilon)
 
+    @classmethod
+    def from_c(cls, c: _lib.pg_gpt2_config) -> "Gpt2Config":
+        return cls(c.vocab_size, c.n_positions, c.n_embd, c.n_layer, c.n_head, c.n_inner,
+                   c.layer_norm_epsilon)
+
+    @classmethod
+    def from_json_file(cls, path) -> "Gpt2Config":
+        """load_config (src/models/gpt2/rust.rs:696-711): a Hugging Face config.json."""
+        c = _lib.pg_gpt2_config()
+        _check(_lib.load().pg_gpt2_load_config(str(path).encode(), C.byref(c)))
+        return cls.from_c(c)
+
 
 @dataclass
 class Gpt2BlockWeights:
@@ -115,6 +127,94 @@ def weights_view(weights: Gpt2Weights, keep: list) -> _lib.pg_gpt2_weights_view:
                                      _tensor(weights.ln_f_g, keep), _tensor(weights.ln_f_b, keep),
                                      C.cast(blocks, C.POINTER(_lib.pg_gpt2_block_view)),
                                      len(weights.blocks))
+
+
+class TensorStore:
+    """TensorStore (src/models/safetensors.rs:93-138) over a mapped .safetensors file.
+    Arrays returned are read-only views into the mapping and keep the store alive."""
+
+    def __init__(self, path):
+        h = C.c_void_p()
+        _check(_lib.load().pg_tensor_store_open(str(path).encode(), C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            _lib.load().pg_tensor_store_close(h)
+            self._h = None
+
+    def __len__(self) -> int:
+        return int(_lib.load().pg_tensor_store_len(self._h))
+
+    def _view(self, t: _lib.pg_tensor, shape) -> np.ndarray:
+        n = int(t.len)
+        if n == 0:
+            arr = np.zeros(0, np.float32)
+        else:
+            addr = C.cast(t.data, C.c_void_p).value
+            arr = np.frombuffer((C.c_float * n).from_address(addr), np.float32)
+        arr = arr.reshape(tuple(shape))
+        arr.flags.writeable = False  # the mapping is read-only
+        return _StoreArray.wrap(arr, self)
+
+    def required_f32(self, name: str, expected_shape: Sequence[int]) -> np.ndarray:
+        shape = (C.c_uint64 * max(len(expected_shape), 1))(*expected_shape)
+        t = _lib.pg_tensor()
+        _check(_lib.load().pg_tensor_store_required_f32(self._h, name.encode(), shape,
+                                                        len(expected_shape), C.byref(t)))
+        return self._view(t, expected_shape)
+
+    def optional_f32(self, name: str, expected_shape: Sequence[int]) -> Optional[np.ndarray]:
+        shape = (C.c_uint64 * max(len(expected_shape), 1))(*expected_shape)
+        t = _lib.pg_tensor()
+        found = C.c_int32(0)
+        _check(_lib.load().pg_tensor_store_optional_f32(self._h, name.encode(), shape,
+                                                        len(expected_shape), C.byref(found),
+                                                        C.byref(t)))
+        return self._view(t, expected_shape) if found.value else None
+
+
+class _StoreArray(np.ndarray):
+    """An ndarray that holds a reference to the TensorStore whose mapping it views."""
+
+    @classmethod
+    def wrap(cls, arr: np.ndarray, store: TensorStore) -> "np.ndarray":
+        out = arr.view(cls)
+        out._store = store
+        return out
+
+    def __array_finalize__(self, obj):
+        self._store = getattr(obj, "_store", None)
+
+
+def load_weights(path, cfg: Gpt2Config) -> Gpt2Weights:
+    """load_weights (src/models/gpt2/rust.rs:713-771) into host arrays: Hugging Face tensor
+    names, each tried bare and then with the `transformer.` prefix.  (Gpt2Model.from_dir
+    does the same inside the library without host copies.)"""
+    store = TensorStore(path)
+
+    def tensor(name: str, shape) -> np.ndarray:
+        found = store.optional_f32(name, shape)
+        return found if found is not None else store.required_f32("transformer." + name, shape)
+
+    c, i = cfg.n_embd, cfg.n_inner
+    blocks = []
+    for layer in range(cfg.n_layer):
+        p = f"h.{layer}"
+        blocks.append(Gpt2BlockWeights(
+            ln_1_g=tensor(f"{p}.ln_1.weight", [c]), ln_1_b=tensor(f"{p}.ln_1.bias", [c]),
+            c_attn_w=tensor(f"{p}.attn.c_attn.weight", [c, 3 * c]),
+            c_attn_b=tensor(f"{p}.attn.c_attn.bias", [3 * c]),
+            c_proj_w=tensor(f"{p}.attn.c_proj.weight", [c, c]),
+            c_proj_b=tensor(f"{p}.attn.c_proj.bias", [c]),
+            ln_2_g=tensor(f"{p}.ln_2.weight", [c]), ln_2_b=tensor(f"{p}.ln_2.bias", [c]),
+            c_fc_w=tensor(f"{p}.mlp.c_fc.weight", [c, i]), c_fc_b=tensor(f"{p}.mlp.c_fc.bias", [i]),
+            c_proj_mlp_w=tensor(f"{p}.mlp.c_proj.weight", [i, c]),
+            c_proj_mlp_b=tensor(f"{p}.mlp.c_proj.bias", [c])))
+    return Gpt2Weights(wte=tensor("wte.weight", [cfg.vocab_size, c]),
+                       wpe=tensor("wpe.weight", [cfg.n_positions, c]), blocks=blocks,
+                       ln_f_g=tensor("ln_f.weight", [c]), ln_f_b=tensor("ln_f.bias", [c]))
 
 
 @dataclass
@@ -290,6 +390,18 @@ class Gpt2Model:
         h = C.c_void_p()
         _check(_lib.load().pg_gpt2_create(C.byref(cfg), C.byref(view), C.byref(opts), C.byref(h)))
         return cls(h, config)
+
+    @classmethod
+    def from_dir(cls, model_dir, hip_config: Optional[Gpt2HipConfig] = None) -> "Gpt2Model":
+        """Gpt2Runtime::from_dir_with_backend without the tokenizer
+        (src/models/gpt2/rust.rs:382-393): `config.json` + `model.safetensors`."""
+        opts = (hip_config or Gpt2HipConfig()).to_c()
+        h = C.c_void_p()
+        lib = _lib.load()
+        _check(lib.pg_gpt2_create_from_dir(str(model_dir).encode(), C.byref(opts), C.byref(h)))
+        cfg = _lib.pg_gpt2_config()
+        _check(lib.pg_gpt2_get_config(h, C.byref(cfg)))
+        return cls(h, Gpt2Config.from_c(cfg))
 
     def __del__(self):
         h = getattr(self, "_h", None)
