@@ -90,6 +90,7 @@ struct pg_kv_cache {
   float *x = nullptr, *q = nullptr, *hbuf = nullptr, *part_acc = nullptr, *part_m = nullptr,
         *part_l = nullptr, *logits_buf = nullptr;
   float *qkv_b = nullptr, *xn_b = nullptr, *att_b = nullptr;  // batched step: [B][3C], [B][C], [B][C]
+  bool pack32 = false;  // batched step: xn_b, att_b and hbuf are packed (pgk::packed32_index)
   uint32_t* d_tok = nullptr;      // [B] token the next step embeds
   uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
   uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
@@ -545,19 +546,23 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   bs.out = g.C;
   // (ln_g / ln_b: the LayerNorm that reads this projection's result, written to xn_b by the
   // same call: fused into the projection's reduce where it has one)
+  // c->pack32: the inputs of the projections (xn_b, att_b, hbuf) are held in the packed form
+  // that the 32-row kernel reads with contiguous loads; their producers write them that way.
+  const int pk = c->pack32 ? 1 : 0;
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
                   int ldc, int N, int K, int epi, const float* ln_g = nullptr,
-                  const float* ln_b = nullptr) -> hipError_t {
+                  const float* ln_b = nullptr, int c_packed = 0) -> hipError_t {
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
     a.ws = c->gemm_ws; a.ws_floats = c->gemm_ws_floats;
-    if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
+    a.a_packed = pk; a.c_packed = c_packed;
+    if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; a.ln_packed = pk; }
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
   PG_HIP(pgk::launch_layer_norm_rows(c->x, c->xn_b, B, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b,
-                                     g.eps, s));
+                                     g.eps, s, pk));
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
     // the LayerNorm after this layer: the next layer's ln_1, or ln_f
@@ -573,9 +578,9 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
                                    hd, nsplit, c->part_acc, c->part_m, c->part_l, s, B, bs,
                                    fused_append ? C : 0));
     PG_HIP(pgk::launch_attn_finish(c->part_acc, c->part_m, c->part_l, H, hd, nsplit, c->att_b, s,
-                                   B, bs));
+                                   B, bs, pk));
     PG_HIP(gemm(c->att_b, C, w.c_proj_w, w.c_proj_b, c->x, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));
-    PG_HIP(gemm(c->xn_b, C, w.c_fc_w, w.c_fc_b, c->hbuf, I, I, C, pgk::GEMM_GELU));
+    PG_HIP(gemm(c->xn_b, C, w.c_fc_w, w.c_fc_b, c->hbuf, I, I, C, pgk::GEMM_GELU, nullptr, nullptr, pk));
     PG_HIP(gemm(c->hbuf, I, w.c_proj_mlp_w, w.c_proj_mlp_b, c->x, C, C, I, pgk::GEMM_RESID, next_g, next_b));
   }
   PG_HIP(gemm(c->xn_b, C, m->wte, nullptr, c->logits_buf, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
@@ -920,7 +925,13 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->kv, kv_floats * sizeof(float)));
   PG_HIP(hipMalloc(&raw->x, B * g.C * sizeof(float)));
   PG_HIP(hipMalloc(&raw->q, B * g.C * sizeof(float)));
-  PG_HIP(hipMalloc(&raw->hbuf, B * g.I * sizeof(float)));
+  // Batches whose projections all run on the 32-row kernel keep that kernel's inputs packed
+  // (32 row slots whatever B is).
+  raw->pack32 = B > 1 && B <= 32 && g.C % 16 == 0 && g.I % 16 == 0 &&
+                pgk::gemm_takes_rows32((int)B, (int)g.C, (int)g.C, m->w_bf16) &&
+                pgk::gemm_takes_rows32((int)B, (int)g.I, (int)g.I, m->w_bf16);
+  const size_t act_rows = raw->pack32 ? 32 : B;
+  PG_HIP(hipMalloc(&raw->hbuf, act_rows * g.I * sizeof(float)));
   if (B > 1) {
     raw->gemm_ws_floats = 8 * B * std::max<size_t>(3 * g.C, g.I);
     PG_HIP(hipMalloc(&raw->gemm_ws, raw->gemm_ws_floats * sizeof(float)));
@@ -930,8 +941,8 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->part_l, parts * sizeof(float)));
   PG_HIP(hipMalloc(&raw->logits_buf, B * g.V * sizeof(float)));
   PG_HIP(hipMalloc(&raw->qkv_b, B * 3 * g.C * sizeof(float)));
-  PG_HIP(hipMalloc(&raw->xn_b, B * g.C * sizeof(float)));
-  PG_HIP(hipMalloc(&raw->att_b, B * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->xn_b, act_rows * g.C * sizeof(float)));
+  PG_HIP(hipMalloc(&raw->att_b, act_rows * g.C * sizeof(float)));
   PG_HIP(hipMalloc(&raw->d_tok, B * sizeof(uint32_t)));
   PG_HIP(hipMalloc(&raw->d_out_ids, g.P * B * sizeof(uint32_t)));
   PG_HIP(hipHostMalloc(&raw->h_ids, g.P * B * sizeof(uint32_t), hipHostMallocDefault));

@@ -94,7 +94,7 @@ hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, h
 // Attention output from a single split's (acc, m, l): out = acc / l per head.
 hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
                               int H, int head_dim, int nsplit, float* out, hipStream_t s,
-                              int batch = 1, BatchStrides bs = BatchStrides{});
+                              int batch = 1, BatchStrides bs = BatchStrides{}, int out_packed = 0);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
 // dst[i] = bf16(src[i]), round to nearest even
 hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s);
@@ -122,7 +122,20 @@ struct GemmArgs {
   const float* ln_g = nullptr;
   const float* ln_b = nullptr;
   float ln_eps = 0.0f;
+  // Packed form of an activation matrix of at most 32 rows (see packed32_index): which of
+  // A, C and ln_out are held that way.  Only the 32-row decode kernel reads a packed A, so
+  // launch_gemm refuses the flags for any other form (gemm_takes_rows32 tells beforehand).
+  int a_packed = 0, c_packed = 0, ln_packed = 0;
 };
+// Element (row b < 32, column k) of a packed activation matrix: the float4 of columns
+// 4j..4j+3 of all 32 rows lie next to each other, so that 32 lanes which each read four
+// columns of "their" row read one contiguous 512 bytes.  A packed matrix of K columns takes
+// 32 K floats whatever its row count.
+__host__ __device__ inline size_t packed32_index(size_t b, size_t k) {
+  return (((k >> 2) * 32 + b) << 2) + (k & 3);
+}
+// Whether launch_gemm multiplies an M x K input with the 32-row decode kernel.
+bool gemm_takes_rows32(int M, int K, int lda, int w_bf16);
 bool gemm_supported(const GemmArgs& a);
 int gemm_split_parts(const GemmArgs& a, int num_cus);
 bool gemm_tail_plan(GemmArgs& a, int num_cus);
@@ -134,8 +147,9 @@ hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_d
                                hipStream_t s);
 hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
                              int T, int C, hipStream_t s, int w_bf16 = 0);
+// (dst_packed: dst is a packed activation matrix, rows <= 32)
 hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
-                                  const float* b, float eps, hipStream_t s);
+                                  const float* b, float eps, hipStream_t s, int dst_packed = 0);
 
 // ---- persistent batch-1 decode (pg_decode.hip) --------------------------------
 struct DecodeParams {

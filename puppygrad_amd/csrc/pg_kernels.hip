@@ -224,9 +224,15 @@ __global__ void k_embed(float* x, const float* wte, const float* wpe, const uint
 }
 
 // cached_self_attention_into (rust.rs:1721-1740) for head_dim 64, keys split
-// over blockIdx.x.  A block scores its keys with 16 lanes per key (float4 each),
-// takes the max-subtracted exponentials (softmax_in_place, cpu.rs:152-165) and
-// accumulates p.V; the per-split (acc, m, l) are merged by the consumer.
+// over blockIdx.x.  Sixteen lanes score one key (a float4 each); a wavefront takes
+// 4 keys per step and IT steps per chunk, and requests the K and the V rows of a whole
+// chunk (16 IT keys per block) before it uses the first: the kernel is a stream of
+// short rows, and only many loads in flight per lane hide its latency.  Each wavefront
+// keeps a running (max, sum, acc) over its keys (the max-subtracted exponentials of
+// softmax_in_place, cpu.rs:152-165, rescaled when the max moves); the four are merged
+// through LDS at the end, and the per-split (acc, m, l) by the consumer.
+// The launcher picks IT so that one chunk covers the split where the split count allows.
+template <int IT>
 __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restrict__ q,
                                                           const float* kcache, const float* vcache,
                                                           int pos, int P, int nsplit,
@@ -237,8 +243,7 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
   // parts of this step's interleaved qkv row (q + append_C, q + 2 append_C); the block whose
   // split holds pos uses them from there and writes them to the cache panels
   // (rust.rs:1677-1683), which saves the launch that would only copy them.
-  extern __shared__ float sc[];  // scores of this split
-  __shared__ float red[kWaves];
+  __shared__ float wm[kWaves], wl[kWaves];
   __shared__ float accs[kWaves][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int split = blockIdx.x, h = blockIdx.y;
@@ -282,36 +287,53 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
     __syncthreads();
   }
 
-  float mx = -INFINITY;
-  for (int k = k0 + wave * 4 + sub; k < k1; k += kWaves * 4) {
-    float4 kv = K4[(size_t)k * 16 + d4];
-    float s = qv.x * kv.x + qv.y * kv.y + qv.z * kv.z + qv.w * kv.w;
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
-    s += __shfl_xor(s, 4, 64);
-    s += __shfl_xor(s, 8, 64);
-    s *= scale;
-    if (d4 == 0) sc[k - k0] = s;
-    mx = fmaxf(mx, s);
-  }
-  mx = block_max(mx, red);  // includes the barrier that publishes sc[]
-
-  float lsum = 0.0f;
-  for (int i = tid; i < k1 - k0; i += kBlock) {
-    float p = expf(sc[i] - mx);
-    sc[i] = p;
-    lsum += p;
-  }
-  lsum = block_sum(lsum, red);
-
+  constexpr int kGroups = kWaves * 4;  // keys per step of the block
+  float m_run = -INFINITY, l_run = 0.0f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int k = k0 + wave * 4 + sub; k < k1; k += kWaves * 4) {
-    float p = sc[k - k0];
-    float4 vv = V4[(size_t)k * 16 + d4];
-    acc.x += p * vv.x;
-    acc.y += p * vv.y;
-    acc.z += p * vv.z;
-    acc.w += p * vv.w;
+  for (int c0 = k0; c0 < k1; c0 += IT * kGroups) {
+    float4 kr[IT], vr[IT];
+    const int kfirst = c0 + wave * 4 + sub;
+    // a key past the split re-reads the split's last row and is masked below
+#pragma unroll
+    for (int i = 0; i < IT; ++i) kr[i] = K4[(size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4];
+#pragma unroll
+    for (int i = 0; i < IT; ++i) vr[i] = V4[(size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4];
+    float sc[IT];
+    float cm = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+      float t = qv.x * kr[i].x + qv.y * kr[i].y + qv.z * kr[i].z + qv.w * kr[i].w;
+      t += __shfl_xor(t, 1, 64);
+      t += __shfl_xor(t, 2, 64);
+      t += __shfl_xor(t, 4, 64);
+      t += __shfl_xor(t, 8, 64);
+      sc[i] = kfirst + kGroups * i < k1 ? t * scale : -INFINITY;
+      cm = fmaxf(cm, sc[i]);
+    }
+    cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+    cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+    const float m_new = fmaxf(m_run, cm);
+    if (m_new == -INFINITY) continue;  // (wavefront-uniform) no key of this wavefront so far
+    const float corr = expf(m_run - m_new);
+    l_run *= corr;
+    acc.x *= corr;
+    acc.y *= corr;
+    acc.z *= corr;
+    acc.w *= corr;
+    float ls = 0.0f;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+      const float pk = expf(sc[i] - m_new);  // 0 for a masked key
+      ls += pk;
+      acc.x += pk * vr[i].x;
+      acc.y += pk * vr[i].y;
+      acc.z += pk * vr[i].z;
+      acc.w += pk * vr[i].w;
+    }
+    ls += __shfl_xor(ls, 16, 64);  // (the sixteen lanes of a key hold the same value)
+    ls += __shfl_xor(ls, 32, 64);
+    l_run += ls;
+    m_run = m_new;
   }
 #pragma unroll
   for (int off = 16; off <= 32; off <<= 1) {
@@ -321,16 +343,27 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
     acc.w += __shfl_xor(acc.w, off, 64);
   }
   if (sub == 0) reinterpret_cast<float4*>(accs[wave])[d4] = acc;
+  if (lane == 0) {
+    wm[wave] = m_run;
+    wl[wave] = l_run;
+  }
   __syncthreads();
   if (tid < 64) {
-    float t = 0.0f;
+    float M = wm[0];
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) t += accs[w][tid];
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, wm[w]);
+    float t = 0.0f, l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float f = wm[w] == -INFINITY ? 0.0f : expf(wm[w] - M);
+      t += f * accs[w][tid];
+      l += f * wl[w];
+    }
     part_acc[pidx * 64 + tid] = t;
-  }
-  if (tid == 0) {
-    part_m[pidx] = mx;
-    part_l[pidx] = lsum;
+    if (tid == 0) {
+      part_m[pidx] = M;
+      part_l[pidx] = l;
+    }
   }
 }
 
@@ -383,16 +416,16 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode_any(const float* q, cons
 }
 
 __global__ void k_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
-                              int C, int hd, int nsplit, float* out, BatchStrides bs) {
-  {
-    const size_t b = blockIdx.y;
-    part_acc += b * bs.part * hd;
-    part_m += b * bs.part;
-    part_l += b * bs.part;
-    out += b * bs.out;
-  }
+                              int C, int hd, int nsplit, float* out, BatchStrides bs,
+                              int out_packed) {
+  const size_t b = blockIdx.y;
+  part_acc += b * bs.part * hd;
+  part_m += b * bs.part;
+  part_l += b * bs.part;
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < C) out[i] = attn_combine_elem(part_acc, part_m, part_l, nsplit, hd, i);
+  if (i < C)
+    out[out_packed ? packed32_index(b, (size_t)i) : b * bs.out + i] =
+        attn_combine_elem(part_acc, part_m, part_l, nsplit, hd, i);
 }
 
 // argmax_logits (generation.rs:269-279): strict '>' from -inf, first maximum
@@ -588,10 +621,14 @@ hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint
 }
 
 int choose_nsplit(int n_keys, int H, int num_cus) {
-  // Enough (head, split) blocks to cover the CUs about twice, at least 16 keys each.
-  int want = (2 * num_cus + H - 1) / H;
+  // Enough (head, split) blocks for about four per CU, at least 16 keys each; and at most
+  // 128 keys each where the split limit allows (one chunk of the kernel: every K and V
+  // row of the block is then requested before the first is used).
+  int want = (4 * num_cus + H - 1) / H;
   int by_len = (n_keys + 15) / 16;
   int ns = want < by_len ? want : by_len;
+  int by_chunk = (n_keys + 127) / 128;
+  if (ns < by_chunk) ns = by_chunk;
   if (ns < 1) ns = 1;
   if (ns > kMaxSplits) ns = kMaxSplits;
   return ns;
@@ -602,9 +639,18 @@ hipError_t launch_attn_decode(const float* q, const float* kcache, const float* 
                               float* part_m, float* part_l, hipStream_t s, int batch,
                               BatchStrides bs, int append_C) {
   if (head_dim == kHeadDim) {
-    int per = (pos + 1 + nsplit - 1) / nsplit;
-    hipLaunchKernelGGL(k_attn_decode64, dim3(nsplit, H, batch), dim3(kBlock), per * sizeof(float),
-                       s, q, kcache, vcache, pos, P, nsplit, part_acc, part_m, part_l, bs, append_C);
+    const int per = (pos + 1 + nsplit - 1) / nsplit;
+    const dim3 grid(nsplit, H, batch);
+    // steps of 16 keys a block needs for its split: the chunk is sized to it
+    if (per <= 32)
+      hipLaunchKernelGGL(k_attn_decode64<2>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
+                         nsplit, part_acc, part_m, part_l, bs, append_C);
+    else if (per <= 64)
+      hipLaunchKernelGGL(k_attn_decode64<4>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
+                         nsplit, part_acc, part_m, part_l, bs, append_C);
+    else
+      hipLaunchKernelGGL(k_attn_decode64<8>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
+                         nsplit, part_acc, part_m, part_l, bs, append_C);
   } else {
     hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H, batch), dim3(kBlock),
                        (pos + 1) * sizeof(float), s, q, kcache, vcache, pos, P, head_dim, part_acc,
@@ -615,10 +661,11 @@ hipError_t launch_attn_decode(const float* q, const float* kcache, const float* 
 
 hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const float* part_l,
                               int H, int head_dim, int nsplit, float* out, hipStream_t s,
-                              int batch, BatchStrides bs) {
+                              int batch, BatchStrides bs, int out_packed) {
   int C = H * head_dim;
+  if (out_packed && batch > 32) return hipErrorInvalidValue;
   hipLaunchKernelGGL(k_attn_finish, dim3((C + 255) / 256, batch), dim3(256), 0, s, part_acc,
-                     part_m, part_l, C, head_dim, nsplit, out, bs);
+                     part_m, part_l, C, head_dim, nsplit, out, bs, out_packed);
   return hipGetLastError();
 }
 

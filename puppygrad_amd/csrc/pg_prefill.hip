@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
     if (p < parts) s += v[p];
   f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
   float c[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
-  float* dst = a.C + m * a.ldc + n;
+  float* dst = a.c_packed ? a.C + packed32_index(m, n) : a.C + m * a.ldc + n;  // (n % 4 == 0)
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     if (EPI == GEMM_GELU) c[k] = gelu_tanh(c[k]);
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts)
       o.y = (c[q].y - mean) * inv * g.y + b.y;
       o.z = (c[q].z - mean) * inv * g.z + b.z;
       o.w = (c[q].w - mean) * inv * g.w + b.w;
-      *reinterpret_cast<f4*>(a.ln_out + m * a.N + n) = o;
+      *reinterpret_cast<f4*>(a.ln_out + (a.ln_packed ? packed32_index(m, n) : m * a.N + n)) = o;
     }
   }
 }
@@ -432,7 +432,14 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   const int u0 = (int)(((long)piece * units) / pieces), u1 = (int)(((long)(piece + 1) * units) / pieces);
 
   const size_t wrow = (size_t)min(n0 + l32, a.N - 1) * a.K + (U / 2) * half;
-  const float* xrow = a.A + (size_t)min(l32, a.M - 1) * a.lda + (U / 2) * half;
+  // this lane's input columns of unit u: xrow + u * xstep (and xrow + u * xstep + xnext for
+  // the second float4 of a 16-column unit).  Packed: the 32 lanes of a half read 512
+  // contiguous bytes; row-major: 32 rows lda floats apart.
+  const size_t xr = (size_t)min(l32, a.M - 1);
+  const float* xrow = a.a_packed ? a.A + packed32_index(xr, (size_t)(U / 2) * half)
+                                 : a.A + xr * a.lda + (U / 2) * half;
+  const size_t xstep = a.a_packed ? (size_t)U * 32 : (size_t)U;
+  const size_t xnext = a.a_packed ? 128 : 4;
 
   f16v acc;
 #pragma unroll
@@ -442,15 +449,15 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     f4 wv[D], xa[D], xb[D];
 #pragma unroll
     for (int i = 0; i < D; ++i) {
-      const size_t k = (size_t)min(u + i, u1 - 1) * U;
+      const size_t unit = (size_t)min(u + i, u1 - 1), k = unit * U;
       if (WBF) {
         // 8 bf16 columns: widened below; the matching 8 input columns are two float4
         wv[i] = *reinterpret_cast<const f4*>(reinterpret_cast<const unsigned short*>(a.W) + wrow + k);
-        xa[i] = *reinterpret_cast<const f4*>(xrow + k);
-        xb[i] = *reinterpret_cast<const f4*>(xrow + k + 4);
+        xa[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep);
+        xb[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep + xnext);
       } else {
         wv[i] = *reinterpret_cast<const f4*>(a.W + wrow + k);
-        xa[i] = *reinterpret_cast<const f4*>(xrow + k);
+        xa[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep);
       }
     }
 #pragma unroll
@@ -500,7 +507,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     float c = (a.bias ? a.bias[n] : 0.0f) + sum;
     if (EPI == GEMM_GELU) c = gelu_tanh(c);
     if (EPI == GEMM_RESID) c = a.resid[(size_t)b * a.ldc + n] + c;
-    a.C[(size_t)b * a.ldc + n] = c;
+    a.C[a.c_packed ? packed32_index((size_t)b, (size_t)n) : (size_t)b * a.ldc + n] = c;
   }
 }
 
@@ -764,12 +771,15 @@ __global__ void k_embed_rows(float* x, const float* wte, const float* wpe, const
 }
 
 // dst[r] = LayerNorm(src[r])  (layer_norm_in_place, cpu.rs:119-143), one block per row
+// (dst_packed: dst is a packed activation matrix, see packed32_index)
 __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float* dst, int cols,
                                                          const float* g, const float* b,
-                                                         float eps) {
+                                                         float eps, int dst_packed) {
   __shared__ float red[4];
   const float* row = src + (size_t)blockIdx.x * cols;
-  float* orow = dst + (size_t)blockIdx.x * cols;
+  auto out_at = [&](int i) -> float& {
+    return dst[dst_packed ? packed32_index(blockIdx.x, (size_t)i) : (size_t)blockIdx.x * cols + i];
+  };
   auto bsum = [&](float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -801,7 +811,7 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = (int)threadIdx.x + 256 * j;
-      if (i < cols) orow[i] = (x[j] - mean) * inv * g[i] + b[i];
+      if (i < cols) out_at(i) = (x[j] - mean) * inv * g[i] + b[i];
     }
     return;
   }
@@ -815,7 +825,7 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
   }
   const float var = bsum(v) / (float)cols;
   const float inv = 1.0f / sqrtf(var + eps);
-  for (int i = threadIdx.x; i < cols; i += 256) orow[i] = (row[i] - mean) * inv * g[i] + b[i];
+  for (int i = threadIdx.x; i < cols; i += 256) out_at(i) = (row[i] - mean) * inv * g[i] + b[i];
 }
 
 template <int BM, int BN, bool WBF>
@@ -904,6 +914,9 @@ hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t
 // K parts for k_gemm_rows32 (0 = not applicable): up to one block per CU (cutting K further
 // was measured slower: the reduce and the shorter pieces cost more than the idle CUs), at
 // least sixteen units per block and part, bounded by the workspace.
+bool gemm_prefers_gemv_rows(const GemmArgs& a) {
+  return a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024;
+}
 int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 16 : 8;
   if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
@@ -995,8 +1008,14 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   bool ln_done = false;
   hipError_t e = launch_gemm_form(a, epi, num_cus, s, &ln_done);
   if (e == hipSuccess && a.ln_out && !ln_done)
-    e = launch_layer_norm_rows(a.C, a.ln_out, a.M, a.N, a.ln_g, a.ln_b, a.ln_eps, s);
+    e = launch_layer_norm_rows(a.C, a.ln_out, a.M, a.N, a.ln_g, a.ln_b, a.ln_eps, s, a.ln_packed);
   return e;
+}
+
+bool gemm_takes_rows32(int M, int K, int lda, int w_bf16) {
+  GemmArgs a{};
+  a.M = M; a.K = K; a.lda = lda; a.w_bf16 = w_bf16; a.N = 32;
+  return !gemm_prefers_gemv_rows(a) && gemm_rows32_parts(a, 1) != 0;
 }
 
 namespace {
@@ -1005,12 +1024,16 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   // A small decode batch over a short K: whole rows of W per wavefront, no MFMA tiles.
   // (Every block stages all input vectors; beyond 16 x 1024 values that costs more than it
   // saves.)
-  if (a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024)
+  const bool packed = a.a_packed || a.c_packed || a.ln_packed;
+  if (gemm_prefers_gemv_rows(a)) {
+    if (packed) return hipErrorInvalidValue;
     return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);
+  }
   // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
   if (const int rp = gemm_rows32_parts(a, num_cus))
     return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done)
                     : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
+  if (packed) return hipErrorInvalidValue;  // only the 32-row kernel knows the packed form
   const int parts = gemm_split_parts(a, num_cus);
   if (parts > 1)
     return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s, ln_done)
@@ -1055,8 +1078,10 @@ hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const
 }
 
 hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
-                                  const float* b, float eps, hipStream_t s) {
-  hipLaunchKernelGGL(k_layer_norm_rows, dim3(rows), dim3(256), 0, s, src, dst, cols, g, b, eps);
+                                  const float* b, float eps, hipStream_t s, int dst_packed) {
+  if (dst_packed && rows > 32) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(k_layer_norm_rows, dim3(rows), dim3(256), 0, s, src, dst, cols, g, b, eps,
+                     dst_packed);
   return hipGetLastError();
 }
 

@@ -17,7 +17,7 @@ def batch_case(seed, B, n, cfg):
 
 
 @pytest.mark.parametrize("prefill_path", [0, 1], ids=["gemm_prefill", "token_prefill"])
-@pytest.mark.parametrize("B,n", [(3, 21), (16, 17), (2, 5)])
+@pytest.mark.parametrize("B,n", [(3, 21), (16, 17), (2, 5), (17, 6), (20, 9), (32, 7)])
 def test_batched_steps_match_oracle(B, n, prefill_path):
     cfg = Gpt2Config(vocab_size=257, n_positions=48, n_embd=128, n_layer=2, n_head=2)
     w, ids = batch_case(B * 100 + n, B, n, cfg)
@@ -39,6 +39,33 @@ def test_batched_steps_match_oracle(B, n, prefill_path):
     for b in (0, B - 1):  # per-sequence K/V panels
         np.testing.assert_allclose(cache.read_layer(1, 0, b)[:, :cache.seq_len],
                                    rcaches[b].read_layer(1, 0)[:, :cache.seq_len], atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("storage", [0, 1], ids=["f32", "bf16"])
+def test_small_batch_of_a_wide_model_matches_oracle(storage):
+    """n_embd above 1024: even a batch of 4 runs its projections on the 32-row MFMA kernel,
+    with the activations between them in that kernel's packed layout."""
+    cfg = Gpt2Config(vocab_size=211, n_positions=40, n_embd=1088, n_layer=2, n_head=17)
+    B, n = 4, 11
+    w, ids = batch_case(31, B, n, cfg)
+    if storage:
+        for blk in w.blocks:
+            for f in ("c_attn_w", "c_proj_w", "c_fc_w", "c_proj_mlp_w"):
+                setattr(blk, f, synth.round_bf16(getattr(blk, f)))
+        w.wte = synth.round_bf16(w.wte)
+    model = Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=storage))
+    ref = oracle.Model(cfg, w, oracle.rust_config(8))
+    cache = model.new_kv_cache(B)
+    got = model.prefill_batch(ids, cache).to_host()
+    rcaches = [ref.new_kv_cache() for _ in range(B)]
+    want = np.stack([ref.prefill(ids[b], rcaches[b]) for b in range(B)])
+    assert_logits_close(got, want)
+    nxt = np.argmax(want, axis=1).astype(np.uint32)
+    for step in range(3):
+        got = model.forward_one_batch(nxt, cache).to_host()
+        want = np.stack([ref.forward_one(int(nxt[b]), rcaches[b]) for b in range(B)])
+        assert_logits_close(got, want, what=f"step {step}")
+        nxt = np.argmax(want, axis=1).astype(np.uint32)
 
 
 def test_batched_greedy_decode_matches_oracle_tokens():
