@@ -422,7 +422,7 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 template <int EPI, bool WBF>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   constexpr int U = WBF ? 16 : 8;  // columns per unit: 16 bytes of W per lane, two lane halves
-  constexpr int D = 6;             // units requested together
+  constexpr int D = 7;             // units requested together
   __shared__ float red[8][32][33];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
@@ -449,7 +449,8 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     f4 wv[D], xa[D], xb[D];
 #pragma unroll
     for (int i = 0; i < D; ++i) {
-      const size_t unit = (size_t)min(u + i, u1 - 1), k = unit * U;
+      if (u + i >= u1) break;  // (wavefront-uniform)
+      const size_t unit = (size_t)(u + i), k = unit * U;
       if (WBF) {
         // 8 bf16 columns: widened below; the matching 8 input columns are two float4
         wv[i] = *reinterpret_cast<const f4*>(reinterpret_cast<const unsigned short*>(a.W) + wrow + k);
