@@ -75,7 +75,13 @@ typedef struct pg_gpt2_weights_view {
 
 /* Stands where Gpt2RustConfig does in Gpt2BackendConfig::Rust(..)
  * (src/models/gpt2/options.rs:15-18, 54-96): the per-backend knobs. */
-typedef enum pg_weight_storage { PG_STORE_F32 = 0, PG_STORE_BF16 = 1 } pg_weight_storage;
+/* PG_STORE_INT8 is the reference's `quantized_weights` option (src/models/gpt2/options.rs:62,
+ * QuantizedRows, src/models/cpu.rs:26-56): the four matrices of every block and the lm_head
+ * copy of wte are held as int8 rows with one f32 scale per row (scale = max|row| / 127), each
+ * weight used as (float)q * scale (quantized_dot, cpu.rs:173-184); the embedding lookup keeps
+ * the f32 wte, biases and LayerNorm parameters stay f32, as in the reference
+ * (src/models/gpt2/rust.rs:1354-1376, 1438-1453).  PG_STORE_BF16 has no reference counterpart. */
+typedef enum pg_weight_storage { PG_STORE_F32 = 0, PG_STORE_BF16 = 1, PG_STORE_INT8 = 2 } pg_weight_storage;
 typedef enum pg_decode_path {
   PG_DECODE_AUTO = 0,       /* persistent kernel when the device can co-schedule it */
   PG_DECODE_KERNELS = 1,    /* one launch per fused op */

@@ -58,14 +58,15 @@ class orc_rust_config(C.Structure):
                 ("qkv_chunk_size", C.c_uint64), ("attention_projection_chunk_size", C.c_uint64),
                 ("mlp_fc_chunk_size", C.c_uint64), ("mlp_projection_chunk_size", C.c_uint64),
                 ("logits_chunk_size", C.c_uint64),
-                ("attention_head_parallel_threshold", C.c_uint64)]
+                ("attention_head_parallel_threshold", C.c_uint64),
+                ("quantized_weights", C.c_uint64)]
 
 
 def rust_config(threads: int = 1, **kw) -> orc_rust_config:
     d = dict(threads=threads, dense_parallel_threshold=262_144, qkv_chunk_size=48,
              attention_projection_chunk_size=64, mlp_fc_chunk_size=128,
              mlp_projection_chunk_size=64, logits_chunk_size=256,
-             attention_head_parallel_threshold=4_096)
+             attention_head_parallel_threshold=4_096, quantized_weights=0)
     d.update(kw)
     return orc_rust_config(**d)
 
@@ -195,6 +196,28 @@ def transpose_in_out(w, in_f, out_f) -> np.ndarray:
     out = np.empty(in_f * out_f, np.float32)
     lib().orc_transpose_in_out(_p(w), C.c_uint64(in_f), C.c_uint64(out_f), _p(out))
     return out
+
+
+def quantize_rows(values, rows: int, cols: int):
+    """QuantizedRows::from_f32 (cpu.rs:38-55) -> (int8 [rows, cols], f32 scales [rows])."""
+    v = _f(values)
+    assert v.size == rows * cols
+    q = np.empty((rows, cols), np.int8)
+    scales = np.empty(rows, np.float32)
+    lib().orc_quantize_rows(_p(v), C.c_uint64(rows), C.c_uint64(cols),
+                            q.ctypes.data_as(C.c_void_p), _p(scales))
+    return q, scales
+
+
+def quantized_dot(a, q, scales, row_index: int) -> float:
+    """quantized_dot (cpu.rs:173-184)."""
+    a = _f(a)
+    q = np.ascontiguousarray(q, np.int8)
+    scales = _f(scales)
+    f = lib().orc_quantized_dot
+    f.restype = C.c_float
+    return float(f(_p(a), q.ctypes.data_as(C.c_void_p), _p(scales), C.c_uint64(q.shape[0]),
+                   C.c_uint64(q.shape[1]), C.c_uint64(row_index)))
 
 
 def argmax_logits(v) -> int:

@@ -121,6 +121,56 @@ void dense_in_out(const float* x, size_t rows, size_t in_f, size_t out_f, const 
   }
 }
 
+// cpu.rs:26-56  QuantizedRows::from_f32: row-wise symmetric int8.  scale = max|v| / 127
+// (1 for an all-zero row); q = round(v / scale) (f32::round: halves away from zero),
+// clamped to [-127, 127].
+struct QuantizedRows {
+  std::vector<int8_t> values;
+  std::vector<float> scales;
+  size_t rows = 0, cols = 0;
+
+  static QuantizedRows from_f32(const float* values, size_t rows, size_t cols) {
+    QuantizedRows q;
+    q.rows = rows;
+    q.cols = cols;
+    q.values.reserve(rows * cols);
+    q.scales.reserve(rows);
+    for (size_t r = 0; r < rows; ++r) {
+      const float* src = values + r * cols;
+      float max_abs = 0.0f;
+      for (size_t i = 0; i < cols; ++i) max_abs = fmaxf(max_abs, fabsf(src[i]));  // f32::max
+      const float scale = max_abs == 0.0f ? 1.0f : max_abs / 127.0f;
+      q.scales.push_back(scale);
+      for (size_t i = 0; i < cols; ++i) {
+        float v = roundf(src[i] / scale);
+        v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);  // f32::clamp (NaN stays NaN)
+        q.values.push_back(v != v ? (int8_t)0 : (int8_t)v);     // `as i8`: NaN -> 0
+      }
+    }
+    return q;
+  }
+};
+
+// cpu.rs:173-184  quantized_dot: scalar, sequential, each weight dequantised as
+// (q as f32 * scale) before it meets x.
+float quantized_dot(const float* a, const QuantizedRows& rows, size_t row_index) {
+  const int8_t* values = rows.values.data() + row_index * rows.cols;
+  const float scale = rows.scales[row_index];
+  float sum = 0.0f;
+  for (size_t i = 0; i < rows.cols; ++i) sum += a[i] * ((float)values[i] * scale);
+  return sum;
+}
+
+// cpu.rs:99-117  quantized_transposed_dense_projection_into.
+void quantized_transposed_dense(const float* x, size_t rows, size_t in_f, size_t out_f,
+                                const QuantizedRows& w, const float* bias, float* out) {
+  for (size_t r = 0; r < rows; ++r) {
+    const float* src = x + r * in_f;
+    float* dst = out + r * out_f;
+    for (size_t o = 0; o < out_f; ++o) dst[o] = bias[o] + quantized_dot(src, w, o);
+  }
+}
+
 // cpu.rs:119-143  layer_norm_in_place: two-pass, biased variance, eps inside sqrt.
 void layer_norm(float* x, size_t rows, size_t cols, const float* gamma, const float* beta,
                 float eps) {
@@ -289,6 +339,7 @@ struct RustConfig {
   size_t mlp_projection_chunk_size = 64;
   size_t logits_chunk_size = 256;
   size_t attention_head_parallel_threshold = 4096;
+  bool quantized_weights = false;  // options.rs:62
 };
 
 // rust.rs:30-100  Gpt2Config.
@@ -371,11 +422,70 @@ inline double since(Clock::time_point t0) {
   return std::chrono::duration<double>(Clock::now() - t0).count();
 }
 
+// rust.rs:127-139  Gpt2QuantizedWeights / Gpt2QuantizedBlockWeights.
+struct QuantizedBlock {
+  QuantizedRows c_attn_w, c_proj_w, c_fc_w, c_proj_mlp_w;
+};
+struct QuantizedWeights {
+  QuantizedRows wte;
+  std::vector<QuantizedBlock> blocks;
+};
+
 struct Model {
   Config cfg;
   Weights w;  // dense matrices already transposed to [out,in]
   RustConfig rc;
   std::unique_ptr<ThreadPool> pool;
+  std::unique_ptr<QuantizedWeights> qw;  // rust.rs:812-816: built when rc.quantized_weights
+
+  // rust.rs:1354-1376  quantize_weights: from the transposed [out,in] matrices and wte.
+  void quantize_weights() {
+    qw = std::make_unique<QuantizedWeights>();
+    size_t C = cfg.n_embd, I = cfg.n_inner;
+    qw->wte = QuantizedRows::from_f32(w.wte.data(), cfg.vocab_size, C);
+    for (const Block& b : w.blocks) {
+      QuantizedBlock q;
+      q.c_attn_w = QuantizedRows::from_f32(b.c_attn_w.data(), 3 * C, C);
+      q.c_proj_w = QuantizedRows::from_f32(b.c_proj_w.data(), C, C);
+      q.c_fc_w = QuantizedRows::from_f32(b.c_fc_w.data(), I, C);
+      q.c_proj_mlp_w = QuantizedRows::from_f32(b.c_proj_mlp_w.data(), C, I);
+      qw->blocks.push_back(std::move(q));
+    }
+  }
+  // rust.rs:1438-1453  quantized_block_linear_slices: int8 rows, f32 bias.
+  const QuantizedRows& quantized_slice(size_t layer, BlockLinear which) const {
+    const QuantizedBlock& b = qw->blocks[layer];
+    switch (which) {
+      case C_ATTN: return b.c_attn_w;
+      case ATTN_PROJ: return b.c_proj_w;
+      case MLP_FC: return b.c_fc_w;
+      default: return b.c_proj_mlp_w;
+    }
+  }
+  // rust.rs:1535-1578  quantized_linear_into.
+  void quantized_linear_into(const float* x, size_t rows, size_t in_f, size_t out_f,
+                             const QuantizedRows& weight, const float* bias, BlockLinear which,
+                             std::vector<float>& out) const {
+    if (pool->threads() == 1 || rows * in_f * out_f < rc.dense_parallel_threshold) {
+      out.clear();
+      out.resize(rows * out_f, 0.0f);
+      quantized_transposed_dense(x, rows, in_f, out_f, weight, bias, out.data());
+      return;
+    }
+    auto chunks = pool->scoped_parallel_chunks(
+        rows * out_f, chunk_size(which), [&](size_t start, size_t end) {
+          std::vector<float> values;
+          values.reserve(end - start);
+          for (size_t index = start; index < end; ++index) {
+            size_t r = index / out_f, o = index % out_f;
+            values.push_back(bias[o] + quantized_dot(x + r * in_f, weight, o));
+          }
+          return values;
+        });
+    out.clear();
+    out.reserve(rows * out_f);
+    for (auto& c : chunks) out.insert(out.end(), c.begin(), c.end());
+  }
 
   // rust.rs:1436-1451  block_linear_slices.
   void slices(size_t layer, BlockLinear which, const float** wt, const float** bias) const {
@@ -402,6 +512,10 @@ struct Model {
                          BlockLinear which, std::vector<float>& out) const {
     const float *wt, *bias;
     slices(layer, which, &wt, &bias);
+    if (qw) {  // rust.rs:1492-1497
+      quantized_linear_into(x, rows, in_f, out_f, quantized_slice(layer, which), bias, which, out);
+      return;
+    }
     if (pool->threads() == 1 || rows * in_f * out_f < rc.dense_parallel_threshold) {
       out.clear();
       out.resize(rows * out_f, 0.0f);
@@ -512,6 +626,26 @@ struct Model {
   // rust.rs:1767-1813  logits_from_hidden_into (f32 branch): tied wte, no bias.
   void logits_from_hidden_into(const float* hidden, std::vector<float>& logits) const {
     size_t V = cfg.vocab_size, C = cfg.n_embd;
+    if (qw) {  // rust.rs:1815-1849  quantized_logits_from_hidden_into
+      if (pool->threads() == 1) {
+        logits.clear();
+        logits.resize(V, 0.0f);
+        for (size_t token = 0; token < V; ++token) logits[token] = quantized_dot(hidden, qw->wte, token);
+        return;
+      }
+      auto chunks =
+          pool->scoped_parallel_chunks(V, rc.logits_chunk_size, [&](size_t start, size_t end) {
+            std::vector<float> values;
+            values.reserve(end - start);
+            for (size_t token = start; token < end; ++token)
+              values.push_back(quantized_dot(hidden, qw->wte, token));
+            return values;
+          });
+      logits.clear();
+      logits.reserve(V);
+      for (auto& c : chunks) logits.insert(logits.end(), c.begin(), c.end());
+      return;
+    }
     if (pool->threads() == 1) {
       logits.clear();
       logits.resize(V, 0.0f);
@@ -873,7 +1007,7 @@ struct orc_weights_view {
 struct orc_rust_config {
   uint64_t threads, dense_parallel_threshold, qkv_chunk_size, attention_projection_chunk_size,
       mlp_fc_chunk_size, mlp_projection_chunk_size, logits_chunk_size,
-      attention_head_parallel_threshold;
+      attention_head_parallel_threshold, quantized_weights;
 };
 struct orc_sampling {
   float temperature;
@@ -986,6 +1120,7 @@ int orc_gpt2_create(const orc_config* c, const orc_weights_view* wv, const orc_r
     rc.mlp_projection_chunk_size = rcv->mlp_projection_chunk_size;
     rc.logits_chunk_size = rcv->logits_chunk_size;
     rc.attention_head_parallel_threshold = rcv->attention_head_parallel_threshold;
+    rc.quantized_weights = rcv->quantized_weights != 0;
   }
   if (int s = validate_rust_config(rc)) return s;
   size_t C = cfg.n_embd, I = cfg.n_inner;
@@ -1040,10 +1175,28 @@ int orc_gpt2_create(const orc_config* c, const orc_weights_view* wv, const orc_r
     d.c_proj_mlp_w = transpose_in_out(b.c_proj_mlp_w.data, I, C);
   }
   m->pool = std::make_unique<ThreadPool>(rc.threads);
+  if (rc.quantized_weights) m->quantize_weights();
   *out = m.release();
   return ORC_OK;
 }
 void orc_gpt2_destroy(void* m) { delete (Model*)m; }
+
+// QuantizedRows::from_f32 and quantized_dot for the op-level tests.
+void orc_quantize_rows(const float* values, uint64_t rows, uint64_t cols, int8_t* q_out,
+                       float* scales_out) {
+  QuantizedRows q = QuantizedRows::from_f32(values, rows, cols);
+  std::memcpy(q_out, q.values.data(), q.values.size());
+  std::memcpy(scales_out, q.scales.data(), q.scales.size() * sizeof(float));
+}
+float orc_quantized_dot(const float* a, const int8_t* q, const float* scales, uint64_t rows,
+                        uint64_t cols, uint64_t row_index) {
+  QuantizedRows r;
+  r.rows = rows;
+  r.cols = cols;
+  r.values.assign(q, q + rows * cols);
+  r.scales.assign(scales, scales + rows);
+  return quantized_dot(a, r, row_index);
+}
 
 // rust.rs:186-200, 258-266  Gpt2KvCache::new.
 int orc_cache_create(void* mp, void** out) {

@@ -12,7 +12,7 @@ from pathlib import Path
 from . import build as _build
 
 PG_OK, PG_ASSET, PG_INVALID_CONFIG, PG_INVALID_INPUT, PG_INVALID_WEIGHTS, PG_BACKEND = range(6)
-PG_STORE_F32, PG_STORE_BF16 = 0, 1
+PG_STORE_F32, PG_STORE_BF16, PG_STORE_INT8 = 0, 1, 2
 PG_DECODE_AUTO, PG_DECODE_KERNELS, PG_DECODE_PERSISTENT = 0, 1, 2
 
 

@@ -66,6 +66,13 @@ struct pg_gpt2_model {
   int persistent_grid = 0;          // workgroups of that launch (one per CU)
   int attn_splits = 1;              // key splits per head in the persistent kernel
   int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
+  // int8 storage (QuantizedRows, src/models/cpu.rs:26-56): the block matrices hold int8 rows
+  // with the scales in LayerW; wte stays f32 for the embedding (rust.rs:966-974 reads the f32
+  // table) and lm_w / lm_s are its quantised copy for the lm_head (rust.rs:1815-1849).
+  // Otherwise lm_w == wte and lm_s == nullptr.
+  int w_i8 = 0;
+  float* lm_w = nullptr;
+  float* lm_s = nullptr;
 };
 
 struct pg_logits {
@@ -183,6 +190,15 @@ pg_status validate_weights(const Cfg& c, const pg_gpt2_weights_view& w) {
 
 size_t round_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
 
+// Arena layout of an int8 matrix: rows * cols bytes, padded to a 256-byte boundary, then
+// the rows' f32 scales.  (Defined once here: model creation places tensors by it and the
+// GEMM drivers find a matrix's scales by it.)
+constexpr size_t kArenaAlign = 64;  // floats
+size_t i8_matrix_floats(size_t rows, size_t cols) { return round_up((rows * cols + 3) / 4, kArenaAlign); }
+const float* i8_scales_of(const float* W, size_t rows, size_t cols) {
+  return W + i8_matrix_floats(rows, cols);
+}
+
 struct DevBuf {
   float* p = nullptr;
   ~DevBuf() {
@@ -265,7 +281,7 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     const pgk::LayerW& w = m->layers[l];
     pgk::GemvArgs a{};
     // LN1 + c_attn + K/V append
-    a.w_bf16 = m->w_bf16; a.W = w.c_attn_w; a.bias = w.c_attn_b; a.x = x; a.y = q; a.K = C; a.nout = 3 * C;
+    a.w_bf16 = m->w_bf16; a.W = w.c_attn_w; a.w_scale = w.c_attn_s; a.bias = w.c_attn_b; a.x = x; a.y = q; a.K = C; a.nout = 3 * C;
     a.ln_g = w.ln_1_g; a.ln_b = w.ln_1_b; a.eps = g.eps;
     a.kcache = c->k_panel(l, b); a.vcache = c->v_panel(l, b);
     a.pos = (int)pos; a.P = P; a.C = C; a.head_dim = hd;
@@ -275,23 +291,23 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
                                    nsplit, pa, pm, pl, s));
     // merge splits + c_proj + residual
     a = pgk::GemvArgs{};
-    a.w_bf16 = m->w_bf16; a.W = w.c_proj_w; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
+    a.w_bf16 = m->w_bf16; a.W = w.c_proj_w; a.w_scale = w.c_proj_s; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
     a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
     // LN2 + c_fc + GELU
     a = pgk::GemvArgs{};
-    a.w_bf16 = m->w_bf16; a.W = w.c_fc_w; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
+    a.w_bf16 = m->w_bf16; a.W = w.c_fc_w; a.w_scale = w.c_fc_s; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
     a.ln_g = w.ln_2_g; a.ln_b = w.ln_2_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_GELU, s));
     // mlp c_proj + residual
     a = pgk::GemvArgs{};
-    a.w_bf16 = m->w_bf16; a.W = w.c_proj_mlp_w; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
+    a.w_bf16 = m->w_bf16; a.W = w.c_proj_mlp_w; a.w_scale = w.c_proj_mlp_s; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
     a.nout = C;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
   }
   if (want_logits) {
     pgk::GemvArgs a{};
-    a.w_bf16 = m->w_bf16; a.W = m->wte; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
+    a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
     a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   }
@@ -494,6 +510,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = T; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    if (m->w_i8) a.w_scale = i8_scales_of(W, (size_t)N, (size_t)K);
     a.ws = WS.p; a.ws_floats = ws_floats;
     if (ln_g) { a.ln_out = XN.p; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
     return pgk::launch_gemm(a, epi, m->num_cus, s);
@@ -513,13 +530,13 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   }
   if (all_logits_dst) {
     PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->ln_f_g, m->ln_f_b, g.eps, s));
-    PG_HIP(gemm(XN.p, C, m->wte, nullptr, LOG.p, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
+    PG_HIP(gemm(XN.p, C, m->lm_w, nullptr, LOG.p, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
     PG_HIP(hipMemcpyAsync(all_logits_dst, LOG.p, n * g.V * sizeof(float), hipMemcpyDeviceToHost,
                           s));
   }
   // last position -> the cache's logits row (LN_f + lm_head, rust.rs:982-1002)
   pgk::GemvArgs a{};
-  a.w_bf16 = m->w_bf16; a.W = m->wte; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
+  a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
   a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
   PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
   PG_HIP(hipStreamSynchronize(s));
@@ -555,6 +572,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     pgk::GemmArgs a{};
     a.A = A; a.w_bf16 = m->w_bf16; a.W = W; a.bias = bias; a.resid = Cout; a.C = Cout;
     a.M = B; a.N = N; a.K = K; a.lda = lda; a.ldc = ldc;
+    if (m->w_i8) a.w_scale = i8_scales_of(W, (size_t)N, (size_t)K);
     a.ws = c->gemm_ws; a.ws_floats = c->gemm_ws_floats;
     a.a_packed = pk; a.c_packed = c_packed;
     if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; a.ln_packed = pk; }
@@ -583,7 +601,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     PG_HIP(gemm(c->xn_b, C, w.c_fc_w, w.c_fc_b, c->hbuf, I, I, C, pgk::GEMM_GELU, nullptr, nullptr, pk));
     PG_HIP(gemm(c->hbuf, I, w.c_proj_mlp_w, w.c_proj_mlp_b, c->x, C, C, I, pgk::GEMM_RESID, next_g, next_b));
   }
-  PG_HIP(gemm(c->xn_b, C, m->wte, nullptr, c->logits_buf, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
+  PG_HIP(gemm(c->xn_b, C, m->lm_w, nullptr, c->logits_buf, (int)g.V, (int)g.V, C, pgk::GEMM_BIAS));
   return PG_OK;
 }
 
@@ -718,10 +736,12 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   if ((s = validate_weights(g, *weights))) return s;
   pg_hip_options opts{};
   if (options) opts = *options;
-  if (opts.weight_storage != PG_STORE_F32 && opts.weight_storage != PG_STORE_BF16)
-    return fail(PG_INVALID_CONFIG, "hip backend weight_storage must be f32 or bf16");
+  if (opts.weight_storage != PG_STORE_F32 && opts.weight_storage != PG_STORE_BF16 &&
+      opts.weight_storage != PG_STORE_INT8)
+    return fail(PG_INVALID_CONFIG, "hip backend weight_storage must be f32, bf16 or int8");
   const bool bf = opts.weight_storage == PG_STORE_BF16;
-  if (bf && opts.decode_path == PG_DECODE_PERSISTENT)
+  const bool i8 = opts.weight_storage == PG_STORE_INT8;
+  if ((bf || i8) && opts.decode_path == PG_DECODE_PERSISTENT)
     return fail(PG_INVALID_CONFIG,
                 "hip backend decode_path=persistent reads f32 weights; use weight_storage=f32");
   if (opts.decode_path > PG_DECODE_PERSISTENT)
@@ -733,6 +753,7 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   m->device = opts.device;
   m->opts = opts;
   m->w_bf16 = bf ? 1 : 0;
+  m->w_i8 = i8 ? 1 : 0;
   hipDeviceProp_t prop;
   PG_HIP(hipGetDeviceProperties(&prop, opts.device));
   m->num_cus = prop.multiProcessorCount;
@@ -741,12 +762,17 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   // With bf16 storage the token embedding and the four matrices of every block hold
   // 2-byte values (wel() floats of arena for n elements); LayerNorm parameters,
   // biases and the position embedding stay f32.
-  const size_t A = 64;
-  auto wel = [&](size_t n) { return bf ? (n + 1) / 2 : n; };
+  const size_t A = kArenaAlign;
+  // (int8: 1-byte values, plus one f32 scale per row placed right after the matrix, plus
+  // the f32 wte kept beside its quantised copy)
+  auto wel = [&](size_t n) { return bf ? (n + 1) / 2 : i8 ? (n + 3) / 4 : n; };
+  auto sel = [&](size_t rows) { return i8 ? round_up(rows, A) : 0; };
   size_t total = round_up(wel(g.V * g.C), A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A);
+  if (i8) total += round_up(g.V * g.C, A) + sel(g.V);
   const size_t per_layer = 6 * round_up(g.C, A) + round_up(wel(3 * g.C * g.C), A) +
                            round_up(3 * g.C, A) + round_up(wel(g.C * g.C), A) +
-                           2 * round_up(wel(g.C * g.I), A) + round_up(g.I, A);
+                           2 * round_up(wel(g.C * g.I), A) + round_up(g.I, A) +
+                           sel(3 * g.C) + 2 * sel(g.C) + sel(g.I);
   total += g.L * per_layer;
   PG_HIP(hipMalloc(&m->arena, total * sizeof(float)));
   m->arena_floats = total;
@@ -771,14 +797,17 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   DevBuf staging, staging_t;
   const size_t mat_max = std::max(3 * g.C * g.C, g.C * g.I);
   if ((s = staging.alloc(bf ? std::max(mat_max, g.V * g.C) : mat_max))) return s;
-  if (bf && (s = staging_t.alloc(mat_max))) return s;
+  if ((bf || i8) && (s = staging_t.alloc(mat_max))) return s;
   // transpose_dense_weights (src/models/gpt2/rust.rs:1345-1352): [in,out] -> [out,in],
-  // then rounded to bf16 (nearest even) when that is the storage type.
-  auto upload_t = [&](float* dst, const pg_tensor& t, size_t in_f, size_t out_f) -> pg_status {
+  // then rounded to bf16 (nearest even) or quantised row by row (quantize_weights,
+  // rust.rs:1354-1376: from the transposed matrix) when that is the storage type.
+  auto upload_t = [&](float* dst, const pg_tensor& t, size_t in_f, size_t out_f,
+                      float* scales) -> pg_status {
     PG_HIP(hipMemcpy(staging.p, t.data, t.len * sizeof(float), hipMemcpyHostToDevice));
-    PG_HIP(pgk::launch_transpose(staging.p, bf ? staging_t.p : dst, (int)in_f, (int)out_f,
+    PG_HIP(pgk::launch_transpose(staging.p, (bf || i8) ? staging_t.p : dst, (int)in_f, (int)out_f,
                                  nullptr));
     if (bf) PG_HIP(pgk::launch_f32_to_bf16(staging_t.p, dst, t.len, nullptr));
+    if (i8) PG_HIP(pgk::launch_quantize_rows(staging_t.p, dst, scales, out_f, (int)in_f, nullptr));
     PG_HIP(hipStreamSynchronize(nullptr));
     return PG_OK;
   };
@@ -790,11 +819,20 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     return PG_OK;
   };
 
-  m->wte = place(wel(g.V * g.C));
+  m->wte = place(i8 ? g.V * g.C : wel(g.V * g.C));
+  m->lm_w = m->wte;
+  if (i8) {
+    m->lm_w = place(wel(g.V * g.C));
+    m->lm_s = place(g.V);
+  }
   m->wpe = place(g.P * g.C);
   m->ln_f_g = place(g.C);
   m->ln_f_b = place(g.C);
   if ((s = upload_w(m->wte, weights->wte))) return s;
+  if (i8) {
+    PG_HIP(pgk::launch_quantize_rows(m->wte, m->lm_w, m->lm_s, g.V, (int)g.C, nullptr));
+    PG_HIP(hipStreamSynchronize(nullptr));
+  }
   if ((s = upload(m->wpe, weights->wpe))) return s;
   if ((s = upload(m->ln_f_g, weights->ln_f_g))) return s;
   if ((s = upload(m->ln_f_b, weights->ln_f_b))) return s;
@@ -804,29 +842,34 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     float* ln_1_g = place(g.C);
     float* ln_1_b = place(g.C);
     float* c_attn_w = place(wel(3 * g.C * g.C));
+    float* c_attn_s = i8 ? place(3 * g.C) : nullptr;  // (== i8_scales_of(c_attn_w, 3C, C))
     float* c_attn_b = place(3 * g.C);
     float* c_proj_w = place(wel(g.C * g.C));
+    float* c_proj_s = i8 ? place(g.C) : nullptr;
     float* c_proj_b = place(g.C);
     float* ln_2_g = place(g.C);
     float* ln_2_b = place(g.C);
     float* c_fc_w = place(wel(g.C * g.I));
+    float* c_fc_s = i8 ? place(g.I) : nullptr;
     float* c_fc_b = place(g.I);
     float* c_proj_mlp_w = place(wel(g.I * g.C));
+    float* c_proj_mlp_s = i8 ? place(g.C) : nullptr;
     float* c_proj_mlp_b = place(g.C);
     if ((s = upload(ln_1_g, b.ln_1_g))) return s;
     if ((s = upload(ln_1_b, b.ln_1_b))) return s;
-    if ((s = upload_t(c_attn_w, b.c_attn_w, g.C, 3 * g.C))) return s;
+    if ((s = upload_t(c_attn_w, b.c_attn_w, g.C, 3 * g.C, c_attn_s))) return s;
     if ((s = upload(c_attn_b, b.c_attn_b))) return s;
-    if ((s = upload_t(c_proj_w, b.c_proj_w, g.C, g.C))) return s;
+    if ((s = upload_t(c_proj_w, b.c_proj_w, g.C, g.C, c_proj_s))) return s;
     if ((s = upload(c_proj_b, b.c_proj_b))) return s;
     if ((s = upload(ln_2_g, b.ln_2_g))) return s;
     if ((s = upload(ln_2_b, b.ln_2_b))) return s;
-    if ((s = upload_t(c_fc_w, b.c_fc_w, g.C, g.I))) return s;
+    if ((s = upload_t(c_fc_w, b.c_fc_w, g.C, g.I, c_fc_s))) return s;
     if ((s = upload(c_fc_b, b.c_fc_b))) return s;
-    if ((s = upload_t(c_proj_mlp_w, b.c_proj_mlp_w, g.I, g.C))) return s;
+    if ((s = upload_t(c_proj_mlp_w, b.c_proj_mlp_w, g.I, g.C, c_proj_mlp_s))) return s;
     if ((s = upload(c_proj_mlp_b, b.c_proj_mlp_b))) return s;
     m->layers[l] = pgk::LayerW{ln_1_g, ln_1_b, c_attn_w, c_attn_b, c_proj_w,     c_proj_b,
-                               ln_2_g, ln_2_b, c_fc_w,   c_fc_b,   c_proj_mlp_w, c_proj_mlp_b};
+                               ln_2_g, ln_2_b, c_fc_w,   c_fc_b,   c_proj_mlp_w, c_proj_mlp_b,
+                               c_attn_s, c_proj_s, c_fc_s, c_proj_mlp_s};
   }
   PG_HIP(hipMalloc(&m->d_layers, g.L * sizeof(pgk::LayerW)));
   struct Guard2 {
@@ -845,7 +888,7 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   {
     const int grid = pgk::persistent_grid();
     int blocks_per_cu = 0;
-    bool shape_ok = !bf && g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
+    bool shape_ok = !bf && !i8 && g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
                     g.P <= 4096 && g.V >= (size_t)grid;
     if (shape_ok) {
       PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu));
@@ -891,7 +934,7 @@ pg_status pg_gpt2_get_config(const pg_gpt2_model* m, pg_gpt2_config* out) {
 pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
   if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
   std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=%s, decode=%s)", m->device,
-                m->num_cus, m->w_bf16 ? "bf16" : "f32", m->persistent ? "persistent" : "kernels");
+                m->num_cus, m->w_bf16 ? "bf16" : m->w_i8 ? "int8" : "f32", m->persistent ? "persistent" : "kernels");
   return PG_OK;
 }
 
@@ -927,7 +970,7 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->q, B * g.C * sizeof(float)));
   // Batches whose projections all run on the 32-row kernel keep that kernel's inputs packed
   // (32 row slots whatever B is).
-  raw->pack32 = B > 1 && B <= 32 && g.C % 16 == 0 && g.I % 16 == 0 &&
+  raw->pack32 = B > 1 && B <= 32 && g.C % 16 == 0 && g.I % 16 == 0 && !m->w_i8 &&
                 pgk::gemm_takes_rows32((int)B, (int)g.C, (int)g.C, m->w_bf16) &&
                 pgk::gemm_takes_rows32((int)B, (int)g.I, (int)g.I, m->w_bf16);
   const size_t act_rows = raw->pack32 ? 32 : B;

@@ -17,6 +17,8 @@ struct LayerW {
   const float *ln_2_g, *ln_2_b;
   const float *c_fc_w, *c_fc_b;       // [I][C], [I]
   const float *c_proj_mlp_w, *c_proj_mlp_b;  // [C][I], [C]
+  // int8 storage only (nullptr otherwise): one f32 scale per row of the matrix
+  const float *c_attn_s, *c_proj_s, *c_fc_s, *c_proj_mlp_s;
 };
 
 enum Prologue : int { PRO_NONE = 0, PRO_LN = 1, PRO_ATTN_COMBINE = 2 };
@@ -25,6 +27,9 @@ enum Epilogue : int { EPI_BIAS = 0, EPI_GELU = 1, EPI_RESID = 2, EPI_QKV = 3 };
 // y = epilogue(bias + W . prologue(x)) for one input vector.
 struct GemvArgs {
   int w_bf16 = 0;      // W holds bf16 values (2 bytes each) instead of f32
+  // != nullptr: W holds int8 values and w_scale[row] is the row's scale; a weight is
+  // (float)q * scale (QuantizedRows / quantized_dot, src/models/cpu.rs:26-56, 173-184)
+  const float* w_scale = nullptr;
   const float* W;      // [nout][K]
   const float* bias;   // [nout] or nullptr (treated as 0)
   const float* x;      // [K] input (PRO_NONE / PRO_LN)
@@ -98,6 +103,10 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
 // dst[i] = bf16(src[i]), round to nearest even
 hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s);
+// QuantizedRows::from_f32 (src/models/cpu.rs:38-55) for src[rows][cols]: scales[r] =
+// max|row r| / 127 (1 for an all-zero row), q = round(v / scale) clamped to [-127, 127].
+hipError_t launch_quantize_rows(const float* src, void* q, float* scales, size_t rows, int cols,
+                                hipStream_t s);
 
 // ---- full-sequence kernels (pg_prefill.hip) ----------------------------------------
 enum GemmEpilogue : int { GEMM_BIAS = 0, GEMM_GELU = 1, GEMM_RESID = 2 };
@@ -105,6 +114,7 @@ enum GemmEpilogue : int { GEMM_BIAS = 0, GEMM_GELU = 1, GEMM_RESID = 2 };
 // rows ldc apart, W dense [N][K]; bias may be nullptr.
 struct GemmArgs {
   int w_bf16 = 0;  // W holds bf16 values
+  const float* w_scale = nullptr;  // != nullptr: W holds int8 values, w_scale[n] scales row n
   const float* A;
   const float* W;
   const float* bias;

@@ -97,8 +97,12 @@ __device__ __forceinline__ float attn_combine_elem(const float* part_acc, const 
 // producer of x (LayerNorm or the attention merge) and the consumer of y
 // (GELU, residual add, K/V cache append) folded in.  One wavefront owns RPW
 // weight rows; lanes stride over the row in float4 and reduce at the end.
-// Weight access modes of k_gemv: f32 scalar / f32 float4 / bf16 x8 / bf16 scalar.
-enum : int { WM_F32 = 0, WM_F32X4 = 1, WM_BF16X8 = 2, WM_BF16 = 3 };
+// Weight access modes of k_gemv: f32 scalar / f32 float4 / bf16 x8 / bf16 scalar /
+// int8 x16 / int8 scalar.
+enum : int { WM_F32 = 0, WM_F32X4 = 1, WM_BF16X8 = 2, WM_BF16 = 3, WM_I8X16 = 4, WM_I8 = 5 };
+
+// Byte b of a 32-bit word as a signed 8-bit value, widened to f32.
+__device__ __forceinline__ float i8_at(int w, int b) { return (float)((w << (24 - 8 * b)) >> 24); }
 
 __device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned u) { return __uint_as_float(u & 0xffff0000u); }
@@ -143,6 +147,45 @@ __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
                     bf16_hi(w.y) * x0.w + bf16_lo(w.z) * x1.x + bf16_hi(w.z) * x1.y +
                     bf16_lo(w.w) * x1.z + bf16_hi(w.w) * x1.w;
         }
+      }
+    }
+  } else if (WM == WM_I8X16) {
+    // int8 weights with one scale per row: 16 per 16-byte load, each dequantised as
+    // (float)q * scale before it meets x (quantized_dot, cpu.rs:173-184)
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    const int K16 = K >> 4;
+    const float4* sx4 = reinterpret_cast<const float4*>(sx);
+    const i4* W16 = reinterpret_cast<const i4*>(a.W);
+    float sc[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) sc[r] = a.w_scale[min(row0 + r, a.nout - 1)];
+    for (int j = lane; j < K16; j += 64) {
+      const float4 x0 = sx4[4 * j], x1 = sx4[4 * j + 1], x2 = sx4[4 * j + 2], x3 = sx4[4 * j + 3];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) {
+          const i4 w = __builtin_nontemporal_load(&W16[(size_t)row * K16 + j]);
+          const float s = sc[r];
+          acc[r] += (i8_at(w.x, 0) * s) * x0.x + (i8_at(w.x, 1) * s) * x0.y +
+                    (i8_at(w.x, 2) * s) * x0.z + (i8_at(w.x, 3) * s) * x0.w +
+                    (i8_at(w.y, 0) * s) * x1.x + (i8_at(w.y, 1) * s) * x1.y +
+                    (i8_at(w.y, 2) * s) * x1.z + (i8_at(w.y, 3) * s) * x1.w +
+                    (i8_at(w.z, 0) * s) * x2.x + (i8_at(w.z, 1) * s) * x2.y +
+                    (i8_at(w.z, 2) * s) * x2.z + (i8_at(w.z, 3) * s) * x2.w +
+                    (i8_at(w.w, 0) * s) * x3.x + (i8_at(w.w, 1) * s) * x3.y +
+                    (i8_at(w.w, 2) * s) * x3.z + (i8_at(w.w, 3) * s) * x3.w;
+        }
+      }
+    }
+  } else if (WM == WM_I8) {
+    const signed char* Wq = reinterpret_cast<const signed char*>(a.W);
+    for (int j = lane; j < K; j += 64) {
+      float xv = sx[j];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        int row = row0 + r;
+        if (row < a.nout) acc[r] += ((float)Wq[(size_t)row * K + j] * a.w_scale[row]) * xv;
       }
     }
   } else if (WM == WM_BF16) {
@@ -530,6 +573,24 @@ __global__ void k_add(float* dst, const float* src, size_t n) {
   if (i < n) dst[i] += src[i];
 }
 
+// QuantizedRows::from_f32 (cpu.rs:38-55), one block per row.
+__global__ __launch_bounds__(kBlock) void k_quantize_rows(const float* src, signed char* q,
+                                                          float* scales, int cols) {
+  __shared__ float red[kWaves];
+  const float* row = src + (size_t)blockIdx.x * cols;
+  signed char* out = q + (size_t)blockIdx.x * cols;
+  float mx = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += kBlock) mx = fmaxf(mx, fabsf(row[i]));  // NaN ignored, as f32::max
+  mx = block_max(mx, red);
+  const float scale = mx == 0.0f ? 1.0f : mx / 127.0f;
+  if (threadIdx.x == 0) scales[blockIdx.x] = scale;
+  for (int i = threadIdx.x; i < cols; i += kBlock) {
+    float v = roundf(row[i] / scale);  // halves away from zero, as f32::round
+    v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+    out[i] = v != v ? (signed char)0 : (signed char)(int)v;  // `as i8` of NaN is 0
+  }
+}
+
 // f32 -> bf16, round to nearest even (NaN keeps a quiet-NaN payload).
 __global__ void k_f32_to_bf16(const float* src, unsigned short* dst, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -577,7 +638,16 @@ hipError_t launch_gemv_pe(const GemvArgs& a, hipStream_t s) {
   const int rpw = two ? 2 : 1;
   const int blocks = (a.nout + kWaves * rpw - 1) / (kWaves * rpw);
   const int blocks1 = (a.nout + kWaves - 1) / kWaves;
-  if (a.w_bf16) {
+  if (a.w_scale) {
+    if (aligned && a.K % 16 == 0) {
+      if (two)
+        hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, WM_I8X16>), dim3(blocks), dim3(kBlock), lds, s, a);
+      else
+        hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_I8X16>), dim3(blocks), dim3(kBlock), lds, s, a);
+    } else {
+      hipLaunchKernelGGL((k_gemv<PRO, EPI, 1, WM_I8>), dim3(blocks1), dim3(kBlock), lds, s, a);
+    }
+  } else if (a.w_bf16) {
     if (aligned && a.K % 8 == 0) {
       if (two)
         hipLaunchKernelGGL((k_gemv<PRO, EPI, 2, WM_BF16X8>), dim3(blocks), dim3(kBlock), lds, s, a);
@@ -711,6 +781,14 @@ hipError_t launch_transpose(const float* src, float* dst, int in_f, int out_f, h
                      dst, in_f, out_f);
   return hipGetLastError();
 }
+hipError_t launch_quantize_rows(const float* src, void* q, float* scales, size_t rows, int cols,
+                                hipStream_t s) {
+  if (rows == 0 || rows > 0x7fffffffu) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(k_quantize_rows, dim3((unsigned)rows), dim3(kBlock), 0, s, src,
+                     static_cast<signed char*>(q), scales, cols);
+  return hipGetLastError();
+}
+
 hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s) {
   size_t blocks = (n + 255) / 256;
   if (blocks > 65536) blocks = 65536;

@@ -40,9 +40,19 @@ constexpr int BK = 16;
 
 // W tile load: 4 consecutive k of one row as f32 (16 bytes) or bf16 (8 bytes, widened
 // to f32 exactly by a 16-bit shift).
-template <bool WBF>
+// (WT = 2: int8, 4 bytes; the caller multiplies by the row's scale.)
+template <int WT>
 __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
-  if (WBF) {
+  if (WT == 2) {
+    const int w = *reinterpret_cast<const int*>(reinterpret_cast<const signed char*>(W) + idx);
+    f4 r;
+    r.x = (float)((w << 24) >> 24);
+    r.y = (float)((w << 16) >> 24);
+    r.z = (float)((w << 8) >> 24);
+    r.w = (float)(w >> 24);
+    return r;
+  }
+  if (WT == 1) {
     typedef unsigned u2 __attribute__((ext_vector_type(2)));
     const u2 w = *reinterpret_cast<const u2*>(reinterpret_cast<const unsigned short*>(W) + idx);
     f4 r;
@@ -64,7 +74,9 @@ __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
 // keep a few CUs busy and the others idle) is cut into a.tail_parts parts along K, so that
 // the tail is one short item for every CU.  Their raw partial tiles go to
 // a.ws[(tile - tail_first) * parts + part][BM][BN] and k_tail_reduce finishes them.
-template <int BM, int BN, int EPI, bool WBF, int SPLIT = 0>
+// WT: how W is stored: 0 f32, 1 bf16, 2 int8 with a.w_scale[n] per row (a weight is
+// (float)q * scale, formed when the tile is loaded: QuantizedRows, cpu.rs:26-56).
+template <int BM, int BN, int EPI, int WT, int SPLIT = 0>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
@@ -104,9 +116,13 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
   for (int i = 0; i < ALD; ++i)
     Ag[i] = a.A + (size_t)min(m0 + lr + 64 * i, a.M - 1) * a.lda + lk;
+  float wsc[BLD];  // int8: the scale of each row this thread loads
 #pragma unroll
-  for (int i = 0; i < BLD; ++i)
-    Wg[i] = (size_t)min(n0 + lr + 64 * i, a.N - 1) * a.K + lk;
+  for (int i = 0; i < BLD; ++i) {
+    const int n = min(n0 + lr + 64 * i, a.N - 1);
+    Wg[i] = (size_t)n * a.K + lk;
+    wsc[i] = WT == 2 ? a.w_scale[n] : 1.0f;
+  }
 
   f16v acc[MB][NB];
 #pragma unroll
@@ -127,7 +143,10 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
   for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + kfirst);
 #pragma unroll
-  for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i] + kfirst);
+  for (int i = 0; i < BLD; ++i) {
+    rb[i] = load_w4<WT>(a.W, Wg[i] + kfirst);
+    if (WT == 2) rb[i] *= wsc[i];
+  }
 
   const int half = lane >> 5, l32 = lane & 31;
   for (int kt = kt0; kt < kt1; ++kt) {
@@ -152,7 +171,10 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + (size_t)(kt + 1) * BK);
 #pragma unroll
-      for (int i = 0; i < BLD; ++i) rb[i] = load_w4<WBF>(a.W, Wg[i] + (size_t)(kt + 1) * BK);
+      for (int i = 0; i < BLD; ++i) {
+        rb[i] = load_w4<WT>(a.W, Wg[i] + (size_t)(kt + 1) * BK);
+        if (WT == 2) rb[i] *= wsc[i];
+      }
     }
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
@@ -829,7 +851,7 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
   for (int i = threadIdx.x; i < cols; i += 256) out_at(i) = (row[i] - mean) * inv * g[i] + b[i];
 }
 
-template <int BM, int BN, bool WBF>
+template <int BM, int BN, int WBF>
 hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = (tiles + 7) / 8 * 8;  // whole rounds over the 8 XCDs
@@ -1026,6 +1048,10 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   // (Every block stages all input vectors; beyond 16 x 1024 values that costs more than it
   // saves.)
   const bool packed = a.a_packed || a.c_packed || a.ln_packed;
+  if (a.w_scale) {  // int8 rows: the 64x64 tile form dequantises them as it loads
+    if (packed || a.w_bf16) return hipErrorInvalidValue;
+    return launch_gemm_tile<64, 64, 2>(a, epi, s);
+  }
   if (gemm_prefers_gemv_rows(a)) {
     if (packed) return hipErrorInvalidValue;
     return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);

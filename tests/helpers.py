@@ -21,10 +21,11 @@ def assert_logits_close(got, want, abs_tol=ABS_TOL, rel_tol=REL_TOL, what="logit
                            f"rel; max err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}")
 
 
-def numpy_gpt2_forward(cfg: Gpt2Config, w, ids) -> np.ndarray:
+def numpy_gpt2_forward(cfg: Gpt2Config, w, ids, lm_head=None) -> np.ndarray:
     """GPT-2 in float64 with whole-matrix numpy ops on the HF [in,out] weights.
     Written from the architecture, not from the oracle's loops: a transposed
-    weight, a wrong head slice or a dropped residual fails against it."""
+    weight, a wrong head slice or a dropped residual fails against it.
+    lm_head ([vocab, n_embd]) replaces the tied wte in the final projection only."""
     f = lambda a, *s: np.asarray(a, np.float64).reshape(*s)
     C, H, I, V = cfg.n_embd, cfg.n_head, cfg.n_inner, cfg.vocab_size
     hd = C // H
@@ -50,7 +51,8 @@ def numpy_gpt2_forward(cfg: Gpt2Config, w, ids) -> np.ndarray:
         h = ln(x, b.ln_2_g, b.ln_2_b) @ f(b.c_fc_w, C, I) + f(b.c_fc_b, I)
         h = 0.5 * h * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (h + 0.044715 * h ** 3)))
         x = x + h @ f(b.c_proj_mlp_w, I, C) + f(b.c_proj_mlp_b, C)
-    return ln(x, w.ln_f_g, w.ln_f_b) @ wte.T
+    head = wte if lm_head is None else f(lm_head, V, C)
+    return ln(x, w.ln_f_g, w.ln_f_b) @ head.T
 
 
 def load_golden(name: str):

@@ -72,7 +72,7 @@ def test_bf16_rejects_persistent_path():
     with pytest.raises(Gpt2Error, match="reads f32 weights"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_BF16,
                                             decode_path=PG_DECODE_PERSISTENT))
-    with pytest.raises(Gpt2Error, match="weight_storage must be f32 or bf16"):
+    with pytest.raises(Gpt2Error, match="weight_storage must be f32, bf16 or int8"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=7))
 
 
