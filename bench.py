@@ -29,10 +29,16 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def weight_bytes(cfg) -> int:
+def weight_bytes(cfg, int8: bool = False) -> int:
     """Bytes of parameters one decode step reads: every block tensor, ln_f, wte
-    (as lm_head) and the two embedding rows."""
+    (as lm_head) and the two embedding rows.  With int8 storage the four block matrices
+    and the lm_head are one byte per element plus one f32 scale per row."""
     C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    if int8:
+        mats = 3 * C_ * C_ + C_ * C_ + 2 * C_ * I              # bytes
+        scales = 3 * C_ + C_ + I + C_                          # f32 each
+        small = 3 * C_ + C_ + I + C_ + 4 * C_                  # biases and LayerNorm, f32
+        return L * (mats + 4 * (scales + small)) + V * C_ + 4 * V + 4 * (2 * C_ + 2 * C_)
     per_layer = 3 * C_ * C_ + 3 * C_ + C_ * C_ + C_ + 2 * C_ * I + I + C_ + 4 * C_
     return 4 * (L * per_layer + 2 * C_ + V * C_ + 2 * C_)
 
@@ -56,6 +62,9 @@ def main() -> int:
                          "batch-decode: a step is one greedy step of --batch sequences")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--bf16", action="store_true", help="store the weights as bf16 (fp32 arithmetic)")
+    ap.add_argument("--int8", action="store_true",
+                    help="store the weights as int8 rows with f32 scales (the reference's "
+                         "quantized_weights; fp32 arithmetic); --workload decode")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this path runs on ONE GPU (a batch-1 decode step has one all-reduce of "
@@ -78,9 +87,12 @@ def main() -> int:
     t0 = time.time()
     path = {"auto": _lib.PG_DECODE_AUTO, "kernels": _lib.PG_DECODE_KERNELS,
             "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
-    storage = _lib.PG_STORE_BF16 if args.bf16 else _lib.PG_STORE_F32
+    storage = _lib.PG_STORE_BF16 if args.bf16 else _lib.PG_STORE_INT8 if args.int8 else _lib.PG_STORE_F32
     if args.bf16 and args.workload != "batch-decode":
         log("bench.py: --bf16 is for --workload batch-decode")
+        return 2
+    if args.int8 and (args.workload != "decode" or args.bf16):
+        log("bench.py: --int8 is for --workload decode, without --bf16")
         return 2
     model = Gpt2Model.new(cfg, weights, Gpt2HipConfig(device=0, weight_storage=storage, decode_path=path))
     log(f"[bench] upload: {time.time() - t0:.1f}s; backend: {model.describe()}")
@@ -137,7 +149,7 @@ def main() -> int:
     # lm_head, argmax); its duration is the HIP-event time the library takes on the
     # launch stream (gpu_decode_time).  Algorithmic bytes: the parameters once per
     # forward plus the K/V rows of positions [0, pos] that forward attends over.
-    algo_bytes = weight_bytes(cfg) + kv_total / K            # per forward
+    algo_bytes = weight_bytes(cfg, args.int8) + kv_total / K  # per forward
     bytes_per_launch = algo_bytes * K / launches
     launch_s = gpu / launches
     achieved = bytes_per_launch / launch_s / 1e9
@@ -149,8 +161,9 @@ def main() -> int:
     _lib.load().pg_device_query(0, C.byref(info))
 
     result = {
-        "metric": "decode tokens/sec, GPT-2 XL 1.5B fp32 bs=1" if args.model == "xl"
-                  else f"decode tokens/sec, GPT-2 {args.model} fp32 bs=1",
+        "metric": (f"decode tokens/sec, GPT-2 {args.model} int8-stored weights bs=1" if args.int8
+                   else "decode tokens/sec, GPT-2 XL 1.5B fp32 bs=1" if args.model == "xl"
+                   else f"decode tokens/sec, GPT-2 {args.model} fp32 bs=1"),
         "value": round(tok_s, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -162,7 +175,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"GPT-2 {args.model} fp32 B=1 greedy decode, KV cache prefilled to "
+        "config": {"workload": f"GPT-2 {args.model} {'int8-stored weights, fp32 arithmetic,' if args.int8 else 'fp32'} "
+                               f"B=1 greedy decode, KV cache prefilled to "
                                f"{n_prefill} tokens, positions {n_prefill}..{n_prefill + min(K, room - 1) - 1}",
                    "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
                    "device": info.name.decode() or info.arch.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
@@ -181,7 +195,7 @@ def main() -> int:
     }
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, weights, ids, n_prefill)
+        result["cpu_baseline"] = cpu_baseline(cfg, weights, ids, n_prefill, args.int8)
 
     print(json.dumps(result), flush=True)
     return 0
@@ -295,7 +309,7 @@ def measured_traffic(args, n_prefill, persistent, launches):
     return None
 
 
-def cpu_baseline(cfg, weights, ids, n_prefill):
+def cpu_baseline(cfg, weights, ids, n_prefill, int8=False):
     """The oracle (a C++ restatement of the reference's CPU path, AVX dot and
     round-robin chunked thread pool) timed on this host: a bounded sample of
     forward_one steps at the benchmark's context length."""
@@ -303,7 +317,8 @@ def cpu_baseline(cfg, weights, ids, n_prefill):
     cores = len(os.sched_getaffinity(0))
     threads = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
     t0 = time.time()
-    ref = oracle.Model(cfg, weights, oracle.rust_config(threads))
+    q = 1 if int8 else 0  # quantized_weights (src/models/gpt2/options.rs:62)
+    ref = oracle.Model(cfg, weights, oracle.rust_config(threads, quantized_weights=q))
     log(f"[bench] cpu oracle build: {time.time() - t0:.1f}s, threads={threads}")
     rcache = ref.new_kv_cache()
     step_ids = [int(ids[i % len(ids)]) for i in range(64)]
@@ -315,7 +330,7 @@ def cpu_baseline(cfg, weights, ids, n_prefill):
         s, _ = ref.timed_forward_steps(rcache, n_prefill, step_ids[:max(1, n // 3)])
         runs.append(max(1, n // 3) / s)
     runs.sort()
-    one = oracle.Model(cfg, weights, oracle.rust_config(1))
+    one = oracle.Model(cfg, weights, oracle.rust_config(1, quantized_weights=q))
     c1 = one.new_kv_cache()
     one.timed_forward_steps(c1, n_prefill, step_ids[:1])
     s1, _ = one.timed_forward_steps(c1, n_prefill, step_ids[:3])

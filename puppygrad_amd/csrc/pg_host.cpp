@@ -289,11 +289,19 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     // attention over keys [0, pos]
     PG_HIP(pgk::launch_attn_decode(q, c->k_panel(l, b), c->v_panel(l, b), (int)pos, P, H, hd,
                                    nsplit, pa, pm, pl, s));
-    // merge splits + c_proj + residual
+    // merge splits + c_proj + residual.  Every block of the projection repeats the merge in
+    // its prologue, which is cheap for a few splits; beyond that the merge gets a launch of
+    // its own (into q, which the attention has finished reading).
     a = pgk::GemvArgs{};
     a.w_bf16 = m->w_bf16; a.W = w.c_proj_w; a.w_scale = w.c_proj_s; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
-    a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
-    PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
+    if (nsplit > 2 && hd == pgk::kHeadDim) {
+      PG_HIP(pgk::launch_attn_finish(pa, pm, pl, H, hd, nsplit, q, s));
+      a.x = q;
+      PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
+    } else {
+      a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
+      PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
+    }
     // LN2 + c_fc + GELU
     a = pgk::GemvArgs{};
     a.w_bf16 = m->w_bf16; a.W = w.c_fc_w; a.w_scale = w.c_fc_s; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
