@@ -82,13 +82,25 @@ __device__ __forceinline__ float attn_combine_elem(const float* part_acc, const 
   int h = i / hd, d = i - h * hd;
   const float* m = part_m + h * nsplit;
   const float* l = part_l + h * nsplit;
-  float M = m[0];
-  for (int s = 1; s < nsplit; ++s) M = fmaxf(M, m[s]);
+  // every value is requested before the first is used (a loop over the splits would wait for
+  // one memory round trip per split); splits past nsplit re-read the last one and weigh 0
+  float mv[kMaxSplits], lv[kMaxSplits], av[kMaxSplits];
+#pragma unroll
+  for (int s = 0; s < kMaxSplits; ++s) {
+    const int t = min(s, nsplit - 1);
+    mv[s] = m[t];
+    lv[s] = l[t];
+    av[s] = part_acc[(size_t)(h * nsplit + t) * hd + d];
+  }
+  float M = mv[0];
+#pragma unroll
+  for (int s = 1; s < kMaxSplits; ++s) M = fmaxf(M, mv[s]);
   float num = 0.0f, den = 0.0f;
-  for (int s = 0; s < nsplit; ++s) {
-    float w = expf(m[s] - M);
-    den += w * l[s];
-    num += w * part_acc[(size_t)(h * nsplit + s) * hd + d];
+#pragma unroll
+  for (int s = 0; s < kMaxSplits; ++s) {
+    const float w = s < nsplit ? expf(mv[s] - M) : 0.0f;
+    den += w * lv[s];
+    num += w * av[s];
   }
   return num / den;
 }
