@@ -265,7 +265,7 @@ pg_status pg_op_argmax(int32_t device, const float* values, uint64_t n, uint32_t
  * .safetensors file; read_safetensors_file + TensorStore::from_bytes
  * (safetensors.rs:79-101).  Failures are PG_ASSET with the reference's wording
  * ("failed to read safetensors file {path}: ...", "failed to parse safetensors
- * file {path}: ...", safetensors.rs:40-70). */
+ * file {path}: ...", safetensors.rs:40-70).  A store handle is single-threaded. */
 typedef struct pg_tensor_store pg_tensor_store;
 pg_status pg_tensor_store_open(const char* path, pg_tensor_store** out);
 void pg_tensor_store_close(pg_tensor_store* store);

@@ -119,12 +119,61 @@ __device__ __forceinline__ float i8_at(int w, int b) { return (float)((w << (24 
 __device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(unsigned u) { return __uint_as_float(u & 0xffff0000u); }
 
+typedef unsigned gv_u4 __attribute__((ext_vector_type(4)));
+
+// One 16-byte chunk of a weight row (chunk j of the row) against the input vector in LDS:
+// 4 f32, 8 bf16 or 16 int8 weights meet 1, 2 or 4 float4 of x.  An int8 weight is
+// dequantised as (float)q * scale before it meets x (quantized_dot, cpu.rs:173-184).
+template <int WM>
+__device__ __forceinline__ float chunk_dot(gv_u4 w, const float4* sx4, int j, float scale) {
+  if (WM == WM_F32X4) {
+    const float4 xv = sx4[j];
+    return __uint_as_float(w.x) * xv.x + __uint_as_float(w.y) * xv.y + __uint_as_float(w.z) * xv.z +
+           __uint_as_float(w.w) * xv.w;
+  }
+  if (WM == WM_BF16X8) {
+    const float4 x0 = sx4[2 * j], x1 = sx4[2 * j + 1];
+    return bf16_lo(w.x) * x0.x + bf16_hi(w.x) * x0.y + bf16_lo(w.y) * x0.z + bf16_hi(w.y) * x0.w +
+           bf16_lo(w.z) * x1.x + bf16_hi(w.z) * x1.y + bf16_lo(w.w) * x1.z + bf16_hi(w.w) * x1.w;
+  }
+  const float4 x0 = sx4[4 * j], x1 = sx4[4 * j + 1], x2 = sx4[4 * j + 2], x3 = sx4[4 * j + 3];
+  const float s = scale;
+  const int wx = (int)w.x, wy = (int)w.y, wz = (int)w.z, ww = (int)w.w;
+  return (i8_at(wx, 0) * s) * x0.x + (i8_at(wx, 1) * s) * x0.y + (i8_at(wx, 2) * s) * x0.z +
+         (i8_at(wx, 3) * s) * x0.w + (i8_at(wy, 0) * s) * x1.x + (i8_at(wy, 1) * s) * x1.y +
+         (i8_at(wy, 2) * s) * x1.z + (i8_at(wy, 3) * s) * x1.w + (i8_at(wz, 0) * s) * x2.x +
+         (i8_at(wz, 1) * s) * x2.y + (i8_at(wz, 2) * s) * x2.z + (i8_at(wz, 3) * s) * x2.w +
+         (i8_at(ww, 0) * s) * x3.x + (i8_at(ww, 1) * s) * x3.y + (i8_at(ww, 2) * s) * x3.z +
+         (i8_at(ww, 3) * s) * x3.w;
+}
+
 template <int PRO, int EPI, int RPW, int WM>
 __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
   extern __shared__ float sx[];  // K floats
   __shared__ float red[kWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int K = a.K;
+  const int row0 = (blockIdx.x * kWaves + wave) * RPW;
+
+  // Vector modes: the first chunks of this wavefront's rows are requested before the input
+  // vector is staged and normalised, so that the two latencies overlap (a short row is
+  // in registers in full by the time the prologue ends).
+  constexpr bool kVec = WM == WM_F32X4 || WM == WM_BF16X8 || WM == WM_I8X16;
+  constexpr int kPre = 4;
+  const int KV = WM == WM_F32X4 ? K >> 2 : WM == WM_BF16X8 ? K >> 3 : K >> 4;  // chunks per row
+  const gv_u4* Wv = reinterpret_cast<const gv_u4*>(a.W);
+  gv_u4 pre[RPW][kPre];
+  if (kVec) {
+#pragma unroll
+    for (int r = 0; r < RPW; ++r)
+#pragma unroll
+      for (int i = 0; i < kPre; ++i) {
+        const int j = lane + 64 * i;
+        pre[r][i] = gv_u4{0u, 0u, 0u, 0u};
+        if (row0 + r < a.nout && j < KV)
+          pre[r][i] = __builtin_nontemporal_load(&Wv[(size_t)(row0 + r) * KV + j]);
+      }
+  }
 
   if (PRO == PRO_ATTN_COMBINE) {
     for (int i = tid; i < K; i += kBlock)
@@ -135,58 +184,34 @@ __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
   __syncthreads();
   if (PRO == PRO_LN) ln_in_lds(sx, K, a.ln_g, a.ln_b, a.eps, red);
 
-  const int row0 = (blockIdx.x * kWaves + wave) * RPW;
   if (row0 >= a.nout) return;
   float acc[RPW];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) acc[r] = 0.0f;
 
-  if (WM == WM_BF16X8) {
-    // weights stored as bf16 (exactly representable in f32): 8 per 16-byte load
-    typedef unsigned u4 __attribute__((ext_vector_type(4)));
-    const int K8 = K >> 3;
+  if (kVec) {
     const float4* sx4 = reinterpret_cast<const float4*>(sx);
-    const u4* W8 = reinterpret_cast<const u4*>(a.W);
-#pragma unroll 2
-    for (int j = lane; j < K8; j += 64) {
-      float4 x0 = sx4[2 * j], x1 = sx4[2 * j + 1];
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) {
-        int row = row0 + r;
-        if (row < a.nout) {
-          u4 w = __builtin_nontemporal_load(&W8[(size_t)row * K8 + j]);
-          acc[r] += bf16_lo(w.x) * x0.x + bf16_hi(w.x) * x0.y + bf16_lo(w.y) * x0.z +
-                    bf16_hi(w.y) * x0.w + bf16_lo(w.z) * x1.x + bf16_hi(w.z) * x1.y +
-                    bf16_lo(w.w) * x1.z + bf16_hi(w.w) * x1.w;
-        }
-      }
-    }
-  } else if (WM == WM_I8X16) {
-    // int8 weights with one scale per row: 16 per 16-byte load, each dequantised as
-    // (float)q * scale before it meets x (quantized_dot, cpu.rs:173-184)
-    typedef int i4 __attribute__((ext_vector_type(4)));
-    const int K16 = K >> 4;
-    const float4* sx4 = reinterpret_cast<const float4*>(sx);
-    const i4* W16 = reinterpret_cast<const i4*>(a.W);
     float sc[RPW];
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) sc[r] = a.w_scale[min(row0 + r, a.nout - 1)];
-    for (int j = lane; j < K16; j += 64) {
-      const float4 x0 = sx4[4 * j], x1 = sx4[4 * j + 1], x2 = sx4[4 * j + 2], x3 = sx4[4 * j + 3];
+    for (int r = 0; r < RPW; ++r)
+      sc[r] = WM == WM_I8X16 ? a.w_scale[min(row0 + r, a.nout - 1)] : 1.0f;
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+      const int j = lane + 64 * i;
+      if (j < KV) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r)
+          if (row0 + r < a.nout) acc[r] += chunk_dot<WM>(pre[r][i], sx4, j, sc[r]);
+      }
+    }
+#pragma unroll 2
+    for (int j = lane + 64 * kPre; j < KV; j += 64) {
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
-        int row = row0 + r;
+        const int row = row0 + r;
         if (row < a.nout) {
-          const i4 w = __builtin_nontemporal_load(&W16[(size_t)row * K16 + j]);
-          const float s = sc[r];
-          acc[r] += (i8_at(w.x, 0) * s) * x0.x + (i8_at(w.x, 1) * s) * x0.y +
-                    (i8_at(w.x, 2) * s) * x0.z + (i8_at(w.x, 3) * s) * x0.w +
-                    (i8_at(w.y, 0) * s) * x1.x + (i8_at(w.y, 1) * s) * x1.y +
-                    (i8_at(w.y, 2) * s) * x1.z + (i8_at(w.y, 3) * s) * x1.w +
-                    (i8_at(w.z, 0) * s) * x2.x + (i8_at(w.z, 1) * s) * x2.y +
-                    (i8_at(w.z, 2) * s) * x2.z + (i8_at(w.z, 3) * s) * x2.w +
-                    (i8_at(w.w, 0) * s) * x3.x + (i8_at(w.w, 1) * s) * x3.y +
-                    (i8_at(w.w, 2) * s) * x3.z + (i8_at(w.w, 3) * s) * x3.w;
+          const gv_u4 w = __builtin_nontemporal_load(&Wv[(size_t)row * KV + j]);
+          acc[r] += chunk_dot<WM>(w, sx4, j, sc[r]);
         }
       }
     }
@@ -208,22 +233,6 @@ __global__ __launch_bounds__(kBlock) void k_gemv(GemvArgs a) {
       for (int r = 0; r < RPW; ++r) {
         int row = row0 + r;
         if (row < a.nout) acc[r] += bf16_lo(Wh[(size_t)row * K + j]) * xv;
-      }
-    }
-  } else if (WM == WM_F32X4) {
-    const int K4 = K >> 2;
-    const float4* sx4 = reinterpret_cast<const float4*>(sx);
-    const f4* W4 = reinterpret_cast<const f4*>(a.W);
-#pragma unroll 2
-    for (int j = lane; j < K4; j += 64) {
-      float4 xv = sx4[j];
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) {
-        int row = row0 + r;
-        if (row < a.nout) {
-          f4 w = __builtin_nontemporal_load(&W4[(size_t)row * K4 + j]);
-          acc[r] += w.x * xv.x + w.y * xv.y + w.z * xv.z + w.w * xv.w;
-        }
       }
     }
   } else {
