@@ -303,6 +303,48 @@ __device__ __forceinline__ void dot_tiles(const Tile<J> (&W)[T], lfp xs, int K4s
   for (int i = 0; i < T; ++i) out[i] = wsum((acc[i].x + acc[i].y) + (acc[i].z + acc[i].w));
 }
 
+// ---- int8 rows (QuantizedRows, src/models/cpu.rs:26-56): a 16-byte chunk is 16 weights ----
+// Sixteen int8 weights against sixteen inputs (four float4), each weight dequantised as
+// (float)q * scale before it meets x (quantized_dot, cpu.rs:173-184).  The chunk travels
+// in a float4 register like the f32 rows do; only its bits are used.
+__device__ __forceinline__ float i8_chunk(const f4& w, const f4& x0, const f4& x1, const f4& x2,
+                                          const f4& x3, float s) {
+  const int a = __float_as_int(w.x), b = __float_as_int(w.y), c = __float_as_int(w.z),
+            d = __float_as_int(w.w);
+#define PG_Q(v, k) ((float)(((v) << (24 - 8 * (k))) >> 24) * s)
+  const float r0 = PG_Q(a, 0) * x0.x + PG_Q(a, 1) * x0.y + PG_Q(a, 2) * x0.z + PG_Q(a, 3) * x0.w;
+  const float r1 = PG_Q(b, 0) * x1.x + PG_Q(b, 1) * x1.y + PG_Q(b, 2) * x1.z + PG_Q(b, 3) * x1.w;
+  const float r2 = PG_Q(c, 0) * x2.x + PG_Q(c, 1) * x2.y + PG_Q(c, 2) * x2.z + PG_Q(c, 3) * x2.w;
+  const float r3 = PG_Q(d, 0) * x3.x + PG_Q(d, 1) * x3.y + PG_Q(d, 2) * x3.z + PG_Q(d, 3) * x3.w;
+#undef PG_Q
+  return (r0 + r1) + (r2 + r3);
+}
+// The inputs of chunk c (columns 16 c .. 16 c + 15) out of LDS; zeros past the row.
+__device__ __forceinline__ void load_x16(f4* x, lfp xs, int chunks, int c, bool whole) {
+  lf4p x4 = (lf4p)xs + 4 * min(c, chunks - 1);
+  const bool valid = whole || c < chunks;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) x[b] = valid ? x4[b] : f4{0.f, 0.f, 0.f, 0.f};
+}
+// dot_tiles for int8 rows: chunks = 16-byte chunks per row, sc[i] = the rows' scales.
+template <int T, int J>
+__device__ __forceinline__ void dot_tiles_i8(const Tile<J> (&W)[T], lfp xs, int chunks, int lane,
+                                             const float (&sc)[T], float (&out)[T]) {
+  float acc[T];
+#pragma unroll
+  for (int i = 0; i < T; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    asm volatile("" ::: "memory");  // one chunk's inputs live at a time
+    f4 x[4];
+    load_x16(x, xs, chunks, lane + 64 * j, 64 * (j + 1) <= chunks);
+#pragma unroll
+    for (int i = 0; i < T; ++i) acc[i] += i8_chunk(W[i].w[j], x[0], x[1], x[2], x[3], sc[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < T; ++i) out[i] = wsum(acc[i]);
+}
+
 struct Best {
   float v;
   unsigned i;
@@ -1074,13 +1116,16 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 // products, and on the two "credits" it raises during the attention phases).  Each
 // slice drains while the dependency chain makes its next hop; each is requested at
 // least one phase before its rows are used.
-template <int C_>
+// WB = bytes per weight: 4 (f32 rows) or 1 (int8 rows with one f32 scale per row).  Rows
+// are streamed in 16-byte chunks either way: KC chunks per C-wide row, KF per 4C-wide row.
+template <int C_, int WB = 4>
 struct StreamPlan {
   static constexpr int C = C_, I = 4 * C_, K4 = C_ / 4, G = kGrid;
+  static constexpr int KC = C_ * WB / 16, KF = 4 * C_ * WB / 16;
   static constexpr int RA = cdiv(3 * C, G), RD = cdiv(C, G), RE = cdiv(I, G);  // max rows per band
   static constexpr int TA = cdiv(RA, kSW), TE = cdiv(RE, kSW);
-  static constexpr int J = cdiv(K4, 64);
-  static constexpr int JF = C_ / 64;  // float4 per lane of one 4C-wide row
+  static constexpr int J = cdiv(KC, 64);
+  static constexpr int JF = cdiv(KF, 64);  // 16-byte chunks per lane of one 4C-wide row
   // loads per layer and wavefront, in stream order
   static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
   // Loads into registers, in stream order:
@@ -1117,12 +1162,16 @@ struct StreamPlan {
   static_assert(in_regs(cut(4)) >= ND + NE, "c_fc rows are requested before they are used");
   static_assert(ND + NE + NF <= cut(5), "mlp projection row is requested before it is used");
   static_assert(RD <= kSW, "one mlp projection row per streamer");
-  static_assert(C_ % 64 == 0, "4C-wide rows are whole runs of 64 float4");
+  static_assert(WB == 4 || WB == 1, "f32 or int8 rows");
+  static_assert(WB == 1 || C_ % 64 == 0, "4C-wide f32 rows are whole runs of 64 float4");
+  static_assert((C_ * WB) % 16 == 0, "rows are whole 16-byte chunks");
+  static_assert(WB == 4 || !kTight, "only f32 rows are staged");
 };
 
-template <int C_>
+template <int C_, int WB>
 __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
-  typedef StreamPlan<C_> SP;
+  typedef StreamPlan<C_, WB> SP;
+  constexpr bool kI8 = WB == 1;
   constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
   constexpr int G = kGrid;
   constexpr int TA = SP::TA, TE = SP::TE, J = SP::J, JF = SP::JF;
@@ -1153,9 +1202,15 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
   // float4 and meet a zero in x).  Unconditional, like every load here: a load under a
   // branch would make the compiler lose count of the loads in flight.
   auto ld_c = [&](const float* W, int row, int j, int ln) -> f4 {
-    const unsigned c = (64 * (j + 1) <= K4) ? (unsigned)ln + 64u * j
-                                            : (unsigned)min(ln + 64 * j, K4 - 1);
-    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * K4, c * 16u);
+    const unsigned c = (64 * (j + 1) <= SP::KC) ? (unsigned)ln + 64u * j
+                                                : (unsigned)min(ln + 64 * j, SP::KC - 1);
+    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * SP::KC, c * 16u);
+  };
+  // One chunk of the 4C-wide mlp projection row (f32 rows are whole runs of 64 chunks).
+  auto ld_f = [&](const float* W, int row, int j, int ln) -> f4 {
+    const unsigned c = (64 * (j + 1) <= SP::KF) ? (unsigned)ln + 64u * j
+                                                : (unsigned)min(ln + 64 * j, SP::KF - 1);
+    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * SP::KF, c * 16u);
   };
   // Requests loads [N0, N1) of the layer stream: `w` is the layer whose c_proj, c_fc and
   // mlp projection rows are meant, `wn` the one whose c_attn rows follow.
@@ -1175,7 +1230,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       const int m = n < SP::PS ? n : n - SP::FS;  // index among the loads into registers
       if (n >= SP::PS && n < SP::PS + SP::FS) {
         const int j = n - SP::PS;
-        ld_row_lds(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
+        ld_row_lds(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * SP::KF,
                    ((unsigned)ln + 64u * j) * 16u, lds.stage + (wave_id() * SP::FS + j) * 256);
       } else if (m < SP::ND) {
         WD[0].w[m] = ld_c(w.c_proj_w, row_of(d0, d1, 0), m, ln);
@@ -1184,8 +1239,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
       } else if (m < SP::ND + SP::NE + SP::NF - SP::FS) {
         const int j = m - SP::ND - SP::NE + SP::FS;  // FS <= j < NF
-        WF.w[j] = ld_row(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * C,
-                         ((unsigned)ln + 64u * j) * 16u);
+        WF.w[j] = ld_f(w.c_proj_mlp_w, row_of(d0, d1, 0), j, ln);
       } else {
         const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
         WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
@@ -1225,6 +1279,9 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       float biasA[TA];
 #pragma unroll
       for (int i = 0; i < TA; ++i) biasA[i] = cld(w.c_attn_b + row_of(a0, a1, i));
+      float scA[TA];  // int8 rows: their scales
+#pragma unroll
+      for (int i = 0; i < TA; ++i) scA[i] = kI8 ? cld(w.c_attn_s + row_of(a0, a1, i)) : 1.0f;
       if (!wait_flag(ctl, 0, epoch_of(p, t, l, 0), abort_word)) {
         ok = false;
         break;
@@ -1234,7 +1291,10 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       PG_SLICE(0, w, wn);
       {
         float v[TA];
-        dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
+        if constexpr (kI8)
+          dot_tiles_i8<TA, J>(WA, lds.xsA, SP::KC, lane, scA, v);
+        else
+          dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 0);
 #pragma unroll
         for (int i = 0; i < TA; ++i) {
@@ -1276,13 +1336,17 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
 
       // ================= D: c_proj row + residual =================
       const float biasD = cld(w.c_proj_b + row_of(d0, d1, 0));
+      const float scD[1] = {kI8 ? cld(w.c_proj_s + row_of(d0, d1, 0)) : 1.0f};
       if (!wait_flag(ctl, 1, epoch_of(p, t, l, 2), abort_word)) {
         ok = false;
         break;
       }
       {
         float v[1];
-        dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
+        if constexpr (kI8)
+          dot_tiles_i8<1, J>(WD, lds.xsD, SP::KC, lane, scD, v);
+        else
+          dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
         const int r = d0 + wave;
         if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v[0])));
       }
@@ -1292,13 +1356,19 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       float biasE[TE];
 #pragma unroll
       for (int i = 0; i < TE; ++i) biasE[i] = cld(w.c_fc_b + row_of(e0, e1, i));
+      float scE[TE];
+#pragma unroll
+      for (int i = 0; i < TE; ++i) scE[i] = kI8 ? cld(w.c_fc_s + row_of(e0, e1, i)) : 1.0f;
       if (!wait_flag(ctl, 2, epoch_of(p, t, l, 3), abort_word)) {
         ok = false;
         break;
       }
       {
         float v[TE];
-        dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
+        if constexpr (kI8)
+          dot_tiles_i8<TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
+        else
+          dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 4);
         // lane i finishes row i: one GELU and one store for all of the wavefront's rows
         float mine = 0.0f;
@@ -1316,6 +1386,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
 
       // ================= F: mlp projection row + residual =================
       const float biasF = cld(w.c_proj_mlp_b + row_of(d0, d1, 0));
+      const float scF = kI8 ? cld(w.c_proj_mlp_s + row_of(d0, d1, 0)) : 1.0f;
       // rounds of reading this wavefront's share of h, until the service wavefront has
       // seen a complete one
       for (;;) {
@@ -1333,7 +1404,22 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         vm_drain();
         SSTAMP(12);
       }
-      {
+      if constexpr (kI8) {
+        // int8 row: KF chunks of 16 weights against the 4C inputs in LDS
+        const int ln = opaque(lane);
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < JF; ++j) {
+          asm volatile("" ::: "memory");
+          f4 x[4];
+          load_x16(x, lds.xsF, SP::KF, ln + 64 * j, 64 * (j + 1) <= SP::KF);
+          acc += i8_chunk(WF.w[j], x[0], x[1], x[2], x[3], scF);
+          if (j == 0) SSTAMP(8);
+        }
+        const float v = wsum(acc);
+        const int r = d0 + wave;
+        if (lane == 0 && r < d1) PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), lds.xraw2[r] + (biasF + v)));
+      } else {
         // the staged part of the row: complete once only the c_attn rows requested after
         // the row's last registers are still in flight
         if (SP::FS) stage_wait<SP::cut(5) - (SP::ND + SP::NE + SP::NF)>();
@@ -1375,26 +1461,52 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
     // ================= lm_head rows (rust.rs:982-1002) + band argmax =================
     if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
       const int wave = wave_id();
-      const f4* wte4 = reinterpret_cast<const f4*>(p.wte);
+      // (int8: the quantised copy of wte and its row scales; f32: wte itself)
+      const f4* wte4 = reinterpret_cast<const f4*>(p.lm_w);
       float* const logits = p.logits;
       Tile<J> T[kLmTiles];
+      float ts[kLmTiles];  // int8: the scale of the row in T[k]
 #pragma unroll
-      for (int k = 0; k < kLmTiles; ++k)
-        load_tile<J>(T[k], wte4 + (size_t)min(v0 + wave + kSW * k, v1 - 1) * K4, K4, lane);
+      for (int k = 0; k < kLmTiles; ++k) {
+        const int row = min(v0 + wave + kSW * k, v1 - 1);
+        load_tile<J>(T[k], wte4 + (size_t)row * SP::KC, SP::KC, lane);
+        ts[k] = kI8 ? cld(p.lm_s + row) : 1.0f;
+      }
       const unsigned epl = epoch_of(p, t, p.L, 5);
       if (!wait_flag(ctl, 4, epl, abort_word)) {
         ok = false;
         break;
       }
-      f4 xr[J];
-      load_x<J>(xr, lds.xsD, K4, lane);
+      // the input vector in registers for the whole phase: one float4 per f32 chunk, four
+      // per int8 chunk
+      constexpr int XPC = kI8 ? 4 : 1;
+      f4 xr[J * XPC];
+      if constexpr (kI8) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) load_x16(xr + 4 * j, lds.xsD, SP::KC, lane + 64 * j, 64 * (j + 1) <= SP::KC);
+      } else {
+        load_x<J>(xr, lds.xsD, K4, lane);
+      }
       Best best{-INFINITY, 0xffffffffu};
       for (int r = v0 + wave; r < v1; r += kSW * kLmTiles) {
 #pragma unroll
         for (int k = 0; k < kLmTiles; ++k) {
           const int rk = r + kSW * k;
-          const float v = dot_tile<J>(T[k], xr);
-          load_tile<J>(T[k], wte4 + (size_t)min(rk + kSW * kLmTiles, v1 - 1) * K4, K4, lane);
+          float v;
+          if constexpr (kI8) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < J; ++j)
+              acc += i8_chunk(T[k].w[j], xr[4 * j], xr[4 * j + 1], xr[4 * j + 2], xr[4 * j + 3], ts[k]);
+            v = wsum(acc);
+          } else {
+            v = dot_tile<J>(T[k], xr);
+          }
+          {
+            const int row = min(rk + kSW * kLmTiles, v1 - 1);
+            load_tile<J>(T[k], wte4 + (size_t)row * SP::KC, SP::KC, lane);
+            if (kI8) ts[k] = cld(p.lm_s + row);
+          }
           if (rk < v1) {
             if (lane == 0) gst(logits + rk, v);
             if (v > best.v) best = Best{v, (unsigned)rk};
@@ -1415,7 +1527,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
 }
 
 // C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
-template <int C_>
+template <int C_, int WB>
 __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
   constexpr int C = C_, I = 4 * C_;
   // 16-byte LDS accesses run at full speed only on 16-byte boundaries: the dynamic block
@@ -1447,54 +1559,79 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
   if ((threadIdx.x >> 6) == kSW)
     service_wave<C_>(p, ctl, lds);
   else
-    streamer_wave<C_>(p, ctl, lds);
+    streamer_wave<C_, WB>(p, ctl, lds);
 }
 
 }  // namespace
 
-size_t persistent_lds_bytes(int C) {
-  const int fs = C == 1600 ? StreamPlan<1600>::FS : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
+size_t persistent_lds_bytes(int C, int w_i8) {
+  const int fs = w_i8 ? 0
+                      : C == 1600 ? StreamPlan<1600>::FS : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
   return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8 + (size_t)kSW * fs * 1024;
 }
-// n_embd values the kernel is instantiated for (GPT-2 small, medium, XL).
+// n_embd values the kernel is instantiated for (GPT-2 small, medium, XL), each for f32 and
+// for int8 rows.
 bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }
 int persistent_grid() { return kGrid; }
 int persistent_max_item_keys() { return kMaxItemKeys; }
 
 namespace {
-template <int C_>
+template <int C_, int WB>
 hipError_t launch_one(const DecodeParams& p, hipStream_t s) {
-  const size_t lds = persistent_lds_bytes(C_);
+  const size_t lds = persistent_lds_bytes(C_, WB == 1);
   // more than the 64 KiB default of dynamic LDS: opt in once per device
   static thread_local int armed_device = -1;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (armed_device != dev) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_persistent<C_>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_persistent<C_, WB>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     armed_device = dev;
   }
-  hipLaunchKernelGGL(k_decode_persistent<C_>, dim3(kGrid), dim3(kThreads), lds, s, p);
+  hipLaunchKernelGGL((k_decode_persistent<C_, WB>), dim3(kGrid), dim3(kThreads), lds, s, p);
   return hipGetLastError();
+}
+template <int WB>
+hipError_t launch_width(const DecodeParams& p, hipStream_t s) {
+  if (p.C == 768) return launch_one<768, WB>(p, s);
+  if (p.C == 1024) return launch_one<1024, WB>(p, s);
+  if (p.C == 1600) return launch_one<1600, WB>(p, s);
+  return hipErrorInvalidValue;
+}
+// Whether one workgroup of the kernel fits on a CU (then the grid of one workgroup per CU is
+// resident at once on an otherwise idle device): the block size the code object allows and
+// the LDS it may be given.  Taken from the function's attributes, not from the occupancy
+// query: a process that has loaded another copy of the HIP runtime first (PyTorch bundles
+// one) was seen to get 0 blocks from that query for the 161..167-register instances, which
+// launch and run correctly (8 wavefronts of up to 256 registers are one block per CU here).
+template <int C_, int WB>
+hipError_t fits_one(int* out) {
+  hipFuncAttributes at{};
+  hipError_t e = hipFuncGetAttributes(&at, reinterpret_cast<const void*>(&k_decode_persistent<C_, WB>));
+  if (e != hipSuccess) return e;
+  const size_t lds = persistent_lds_bytes(C_, WB == 1);
+  *out = (at.maxThreadsPerBlock >= kThreads && lds <= (size_t)at.maxDynamicSharedSizeBytes) ? 1 : 0;
+  return hipSuccess;
+}
+template <int WB>
+hipError_t max_blocks(int C, int* out) {
+  if (C == 768) return fits_one<768, WB>(out);
+  if (C == 1024) return fits_one<1024, WB>(out);
+  if (C == 1600) return fits_one<1600, WB>(out);
+  *out = 0;
+  return hipSuccess;
 }
 }  // namespace
 
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
-  if (p.C == 768) return launch_one<768>(p, s);
-  if (p.C == 1024) return launch_one<1024>(p, s);
-  if (p.C == 1600) return launch_one<1600>(p, s);
-  return hipErrorInvalidValue;
+  if (p.w_i8 && (!p.lm_s || !p.lm_w)) return hipErrorInvalidValue;
+  return p.w_i8 ? launch_width<1>(p, s) : launch_width<4>(p, s);
 }
 
-hipError_t persistent_max_blocks_per_cu(int C, int* out) {
-  const size_t lds = persistent_lds_bytes(C);
-  if (C == 768) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<768>, kThreads, lds);
-  if (C == 1024) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1024>, kThreads, lds);
-  if (C == 1600) return hipOccupancyMaxActiveBlocksPerMultiprocessor(out, k_decode_persistent<1600>, kThreads, lds);
-  *out = 0;
-  return hipSuccess;
+hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_i8) {
+  return w_i8 ? max_blocks<1>(C, out) : max_blocks<4>(C, out);
 }
 
 }  // namespace pgk

@@ -69,7 +69,7 @@ def test_bf16_batched_steps():
 def test_bf16_rejects_persistent_path():
     cfg = Gpt2Config(vocab_size=257, n_positions=48, n_embd=128, n_layer=1, n_head=2)
     w = synth.random_weights(cfg, 3)
-    with pytest.raises(Gpt2Error, match="reads f32 weights"):
+    with pytest.raises(Gpt2Error, match="reads f32 or int8 weights, not bf16"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_BF16,
                                             decode_path=PG_DECODE_PERSISTENT))
     with pytest.raises(Gpt2Error, match="weight_storage must be f32, bf16 or int8"):

@@ -8,7 +8,7 @@ import pytest
 import oracle
 from helpers import ABS_TOL, REL_TOL, assert_logits_close, small_cases
 from puppygrad_amd import Gpt2Config, Gpt2Error, Gpt2HipConfig, Gpt2Model, synth
-from puppygrad_amd._lib import PG_DECODE_PERSISTENT, PG_STORE_INT8
+from puppygrad_amd._lib import PG_STORE_INT8
 
 pytestmark = pytest.mark.gpu
 
@@ -114,11 +114,42 @@ def test_int8_gpt2_small_decode_steps():
         assert_logits_close(got, want, what=f"step {step}")
 
 
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1600, 25, 40)])
+def test_int8_persistent_decode_matches_oracle(n_embd, n_head, n_prompt):
+    """The persistent decode kernel on int8 rows (16 weights per 16-byte chunk; the XL rows
+    are not whole runs of 64 chunks): single forwards and a multi-token launch against the
+    quantised oracle, and against the per-op path on the same device weights."""
+    cfg = Gpt2Config(vocab_size=300, n_positions=256, n_embd=n_embd, n_layer=2, n_head=n_head)
+    w = synth.random_weights(cfg, 0x5EED0610 + n_head, perturb=True)
+    ids = list(synth.token_ids(n_prompt, 0x70C00610, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w, INT8), qref(cfg, w, threads=8)
+    assert "weights=int8" in model.describe() and "decode=persistent" in model.describe()
+    per_op = Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_INT8, decode_path=1))
+    assert "decode=kernels" in per_op.describe()
+    cache, pcache, rcache = model.new_kv_cache(), per_op.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    per_op.prefill(ids, pcache)
+    rlog = None
+    for tok in (7, 123, 42):
+        rlog = ref.forward_one(tok, rcache)
+        got = model.forward_one(tok, cache).to_host()
+        assert_logits_close(got, rlog)
+        assert_logits_close(got, per_op.forward_one(tok, pcache).to_host(), abs_tol=2e-5, rel_tol=1e-4)
+    got, _ = model.decode_greedy(cache, 6)  # five forwards in one launch
+    want, clear = [], True
+    for i in range(6):
+        top = np.sort(rlog)[-2:]
+        clear = clear and (top[1] - top[0]) > 2 * (ABS_TOL + REL_TOL * abs(float(top[1])))
+        want.append(oracle.argmax_logits(rlog))
+        if i < 5:
+            rlog = ref.forward_one(want[-1], rcache)
+    assert len(got) == 6
+    if clear:
+        assert got == want
+
+
 def test_int8_options_are_validated():
     cfg = synth.tiny_config()
     w = synth.tiny_weights(cfg)
-    with pytest.raises(Gpt2Error, match="decode_path=persistent reads f32 weights"):
-        Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_INT8,
-                                            decode_path=PG_DECODE_PERSISTENT))
     with pytest.raises(Gpt2Error, match="weight_storage must be f32, bf16 or int8"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=3))
