@@ -154,7 +154,7 @@ def main() -> int:
     launch_s = gpu / launches
     achieved = bytes_per_launch / launch_s / 1e9
     persistent = "decode=persistent" in model.describe()
-    kernel = (f"k_decode_persistent<{cfg.n_embd}>" if persistent
+    kernel = (f"k_decode_persistent<{cfg.n_embd}{', int8 rows' if args.int8 else ''}>" if persistent
               else "all launches of one decode step (k_gemv dominant)")
 
     info = _lib.pg_device_info()
@@ -304,7 +304,7 @@ TRAFFIC_XL_DEFAULT = 891.8e9
 
 def measured_traffic(args, n_prefill, persistent, launches):
     if (args.model == "xl" and n_prefill == 896 and args.steps == 127 and persistent
-            and launches == 1):
+            and launches == 1 and not args.int8):
         return TRAFFIC_XL_DEFAULT
     return None
 
