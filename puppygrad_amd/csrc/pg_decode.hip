@@ -35,6 +35,12 @@
 //             F  mlp c_proj rows + residual   -> xm_t    (tagged)
 // then LN_f + lm_head rows -> logits (plain) and per-workgroup argmax -> best_t.
 //
+// The weight rows are f32, or int8 with one f32 scale per row (QuantizedRows,
+// src/models/cpu.rs:26-56; template parameter WB): either way a row is a stream of 16-byte
+// chunks, and an int8 chunk's 16 weights are dequantised as (float)q * scale before they
+// meet the input (quantized_dot, cpu.rs:173-184).  Embedding, biases, LayerNorm, K/V and
+// every exchanged activation are f32 in both.
+//
 // Every wait is bounded: a poll that does not complete within its spin limit sets
 // the abort word (global) and the halt word (LDS); every other wait observes one of
 // them and all wavefronts leave the kernel.
