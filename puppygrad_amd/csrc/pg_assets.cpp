@@ -382,7 +382,7 @@ pg_status open_store(const char* path, std::unique_ptr<pg_tensor_store>& out) {
   st->data = bytes + 8 + n;
   st->data_len = st->map_len - 8 - (size_t)n;
 
-  std::vector<std::pair<uint64_t, std::string>> order;
+  std::vector<std::pair<std::pair<uint64_t, uint64_t>, std::string>> order;  // (begin, end), name
   for (const auto& kv : header.obj) {
     if (kv.first == "__metadata__") continue;
     const Json& t = kv.second;
@@ -416,7 +416,7 @@ pg_status open_store(const char* path, std::unique_ptr<pg_tensor_store>& out) {
     if ((unsigned __int128)(info.end - info.begin) != count * esz)
       return parse_error(st->path, "invalid tensor info for tensor `" + kv.first +
                                        "`: byte range does not match dtype and shape");
-    order.emplace_back(info.begin, kv.first);
+    order.emplace_back(std::make_pair(info.begin, info.end), kv.first);
     st->tensors[kv.first] = std::move(info);
   }
   // The data section is the tensors back to back, without holes or overlap, to its end.
