@@ -29,16 +29,19 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def weight_bytes(cfg, int8: bool = False) -> int:
+def weight_bytes(cfg, int8: bool = False, bf16: bool = False) -> int:
     """Bytes of parameters one decode step reads: every block tensor, ln_f, wte
     (as lm_head) and the two embedding rows.  With int8 storage the four block matrices
-    and the lm_head are one byte per element plus one f32 scale per row."""
+    and the lm_head are one byte per element plus one f32 scale per row; with bf16 storage
+    they (and the wte embedding row) are two bytes per element."""
     C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
-    if int8:
-        mats = 3 * C_ * C_ + C_ * C_ + 2 * C_ * I              # bytes
-        scales = 3 * C_ + C_ + I + C_                          # f32 each
+    if int8 or bf16:
+        eb = 1 if int8 else 2
+        mats = eb * (3 * C_ * C_ + C_ * C_ + 2 * C_ * I)       # bytes
+        scales = (3 * C_ + C_ + I + C_) if int8 else 0         # f32 each
         small = 3 * C_ + C_ + I + C_ + 4 * C_                  # biases and LayerNorm, f32
-        return L * (mats + 4 * (scales + small)) + V * C_ + 4 * V + 4 * (2 * C_ + 2 * C_)
+        embed = 4 * C_ + (4 if int8 else 2) * C_               # wpe row + wte row
+        return L * (mats + 4 * (scales + small)) + eb * V * C_ + (4 * V if int8 else 0) + 4 * 2 * C_ + embed
     per_layer = 3 * C_ * C_ + 3 * C_ + C_ * C_ + C_ + 2 * C_ * I + I + C_ + 4 * C_
     return 4 * (L * per_layer + 2 * C_ + V * C_ + 2 * C_)
 
@@ -88,8 +91,8 @@ def main() -> int:
     path = {"auto": _lib.PG_DECODE_AUTO, "kernels": _lib.PG_DECODE_KERNELS,
             "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
     storage = _lib.PG_STORE_BF16 if args.bf16 else _lib.PG_STORE_INT8 if args.int8 else _lib.PG_STORE_F32
-    if args.bf16 and args.workload != "batch-decode":
-        log("bench.py: --bf16 is for --workload batch-decode")
+    if args.bf16 and args.workload == "prefill":
+        log("bench.py: --bf16 is for --workload decode or batch-decode")
         return 2
     if args.int8 and (args.workload != "decode" or args.bf16):
         log("bench.py: --int8 is for --workload decode, without --bf16")
@@ -149,12 +152,12 @@ def main() -> int:
     # lm_head, argmax); its duration is the HIP-event time the library takes on the
     # launch stream (gpu_decode_time).  Algorithmic bytes: the parameters once per
     # forward plus the K/V rows of positions [0, pos] that forward attends over.
-    algo_bytes = weight_bytes(cfg, args.int8) + kv_total / K  # per forward
+    algo_bytes = weight_bytes(cfg, args.int8, args.bf16) + kv_total / K  # per forward
     bytes_per_launch = algo_bytes * K / launches
     launch_s = gpu / launches
     achieved = bytes_per_launch / launch_s / 1e9
     persistent = "decode=persistent" in model.describe()
-    kernel = (f"k_decode_persistent<{cfg.n_embd}{', int8 rows' if args.int8 else ''}>" if persistent
+    kernel = (f"k_decode_persistent<{cfg.n_embd}{', int8 rows' if args.int8 else ', bf16 rows' if args.bf16 else ''}>" if persistent
               else "all launches of one decode step (k_gemv dominant)")
 
     info = _lib.pg_device_info()
@@ -162,6 +165,7 @@ def main() -> int:
 
     result = {
         "metric": (f"decode tokens/sec, GPT-2 {args.model} int8-stored weights bs=1" if args.int8
+                   else f"decode tokens/sec, GPT-2 {args.model} bf16-stored weights bs=1" if args.bf16
                    else "decode tokens/sec, GPT-2 XL 1.5B fp32 bs=1" if args.model == "xl"
                    else f"decode tokens/sec, GPT-2 {args.model} fp32 bs=1"),
         "value": round(tok_s, 2),
@@ -175,7 +179,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"GPT-2 {args.model} {'int8-stored weights, fp32 arithmetic,' if args.int8 else 'fp32'} "
+        "config": {"workload": f"GPT-2 {args.model} {'int8-stored weights, fp32 arithmetic,' if args.int8 else 'bf16-stored weights, fp32 arithmetic,' if args.bf16 else 'fp32'} "
                                f"B=1 greedy decode, KV cache prefilled to "
                                f"{n_prefill} tokens, positions {n_prefill}..{n_prefill + min(K, room - 1) - 1}",
                    "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
@@ -195,7 +199,8 @@ def main() -> int:
     }
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, weights, ids, n_prefill, args.int8)
+        result["cpu_baseline"] = cpu_baseline(cfg, synth.bf16_rounded(weights) if args.bf16 else weights,
+                                              ids, n_prefill, args.int8)
 
     print(json.dumps(result), flush=True)
     return 0
@@ -304,7 +309,7 @@ TRAFFIC_XL_DEFAULT = 891.8e9
 
 def measured_traffic(args, n_prefill, persistent, launches):
     if (args.model == "xl" and n_prefill == 896 and args.steps == 127 and persistent
-            and launches == 1 and not args.int8):
+            and launches == 1 and not args.int8 and not args.bf16):
         return TRAFFIC_XL_DEFAULT
     return None
 

@@ -325,27 +325,50 @@ __device__ __forceinline__ float i8_chunk(const f4& w, const f4& x0, const f4& x
 #undef PG_Q
   return (r0 + r1) + (r2 + r3);
 }
-// The inputs of chunk c (columns 16 c .. 16 c + 15) out of LDS; zeros past the row.
-__device__ __forceinline__ void load_x16(f4* x, lfp xs, int chunks, int c, bool whole) {
-  lf4p x4 = (lf4p)xs + 4 * min(c, chunks - 1);
+// Eight bf16 weights (exactly representable in f32) against eight inputs (two float4).
+__device__ __forceinline__ float bf16_chunk(const f4& w, const f4& x0, const f4& x1) {
+  const unsigned a = __float_as_uint(w.x), b = __float_as_uint(w.y), c = __float_as_uint(w.z),
+                 d = __float_as_uint(w.w);
+#define PG_LO(v) __uint_as_float((v) << 16)
+#define PG_HI(v) __uint_as_float((v) & 0xffff0000u)
+  const float r0 = PG_LO(a) * x0.x + PG_HI(a) * x0.y + PG_LO(b) * x0.z + PG_HI(b) * x0.w;
+  const float r1 = PG_LO(c) * x1.x + PG_HI(c) * x1.y + PG_LO(d) * x1.z + PG_HI(d) * x1.w;
+#undef PG_LO
+#undef PG_HI
+  return r0 + r1;
+}
+// One 16-byte chunk of WB-byte weights against its XPC = 4 / WB float4 of inputs.
+template <int WB>
+__device__ __forceinline__ float packed_chunk(const f4& w, const f4* x, float s) {
+  if constexpr (WB == 1)
+    return i8_chunk(w, x[0], x[1], x[2], x[3], s);
+  else
+    return bf16_chunk(w, x[0], x[1]);
+}
+// The inputs of chunk c (XPC float4 = the chunk's columns) out of LDS; zeros past the row.
+template <int XPC>
+__device__ __forceinline__ void load_xc(f4* x, lfp xs, int chunks, int c, bool whole) {
+  lf4p x4 = (lf4p)xs + XPC * min(c, chunks - 1);
   const bool valid = whole || c < chunks;
 #pragma unroll
-  for (int b = 0; b < 4; ++b) x[b] = valid ? x4[b] : f4{0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < XPC; ++b) x[b] = valid ? x4[b] : f4{0.f, 0.f, 0.f, 0.f};
 }
-// dot_tiles for int8 rows: chunks = 16-byte chunks per row, sc[i] = the rows' scales.
-template <int T, int J>
-__device__ __forceinline__ void dot_tiles_i8(const Tile<J> (&W)[T], lfp xs, int chunks, int lane,
-                                             const float (&sc)[T], float (&out)[T]) {
+// dot_tiles for packed rows (int8 or bf16): chunks = 16-byte chunks per row, sc[i] = the
+// rows' scales (int8).
+template <int WB, int T, int J>
+__device__ __forceinline__ void dot_tiles_packed(const Tile<J> (&W)[T], lfp xs, int chunks, int lane,
+                                                 const float (&sc)[T], float (&out)[T]) {
+  constexpr int XPC = 4 / WB;
   float acc[T];
 #pragma unroll
   for (int i = 0; i < T; ++i) acc[i] = 0.0f;
 #pragma unroll
   for (int j = 0; j < J; ++j) {
     asm volatile("" ::: "memory");  // one chunk's inputs live at a time
-    f4 x[4];
-    load_x16(x, xs, chunks, lane + 64 * j, 64 * (j + 1) <= chunks);
+    f4 x[XPC];
+    load_xc<XPC>(x, xs, chunks, lane + 64 * j, 64 * (j + 1) <= chunks);
 #pragma unroll
-    for (int i = 0; i < T; ++i) acc[i] += i8_chunk(W[i].w[j], x[0], x[1], x[2], x[3], sc[i]);
+    for (int i = 0; i < T; ++i) acc[i] += packed_chunk<WB>(W[i].w[j], x, sc[i]);
   }
 #pragma unroll
   for (int i = 0; i < T; ++i) out[i] = wsum(acc[i]);
@@ -753,9 +776,15 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         if (l == 0) {
           // embedding (rust.rs:966-974)
 #pragma unroll
-          for (int j = 0; j < NW; ++j)
-            lds.xraw1[lane + 64 * j] = gld_at(p.wte + (size_t)tok * C, (unsigned)ln + 64u * j) +
-                                       gld_at(p.wpe + (size_t)pos * C, (unsigned)ln + 64u * j);
+          for (int j = 0; j < NW; ++j) {
+            const unsigned col = (unsigned)ln + 64u * j;
+            // (wte is bf16 when the rows are; wpe is always f32)
+            typedef const unsigned short __attribute__((address_space(1)))* ghp;
+            const float e = p.w_bytes == 2
+                                ? __uint_as_float((unsigned)((ghp)p.wte)[(size_t)tok * C + col] << 16)
+                                : gld_at(p.wte + (size_t)tok * C, col);
+            lds.xraw1[lane + 64 * j] = e + gld_at(p.wpe + (size_t)pos * C, col);
+          }
         } else {
           if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, l - 1, 5), lds.xraw1, abort_word, wg))
             PG_SERVICE_FAIL();
@@ -1122,7 +1151,8 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 // products, and on the two "credits" it raises during the attention phases).  Each
 // slice drains while the dependency chain makes its next hop; each is requested at
 // least one phase before its rows are used.
-// WB = bytes per weight: 4 (f32 rows) or 1 (int8 rows with one f32 scale per row).  Rows
+// WB = bytes per weight: 4 (f32 rows), 2 (bf16 rows) or 1 (int8 rows with one f32 scale per
+// row).  Rows
 // are streamed in 16-byte chunks either way: KC chunks per C-wide row, KF per 4C-wide row.
 template <int C_, int WB = 4>
 struct StreamPlan {
@@ -1168,8 +1198,8 @@ struct StreamPlan {
   static_assert(in_regs(cut(4)) >= ND + NE, "c_fc rows are requested before they are used");
   static_assert(ND + NE + NF <= cut(5), "mlp projection row is requested before it is used");
   static_assert(RD <= kSW, "one mlp projection row per streamer");
-  static_assert(WB == 4 || WB == 1, "f32 or int8 rows");
-  static_assert(WB == 1 || C_ % 64 == 0, "4C-wide f32 rows are whole runs of 64 float4");
+  static_assert(WB == 4 || WB == 2 || WB == 1, "f32, bf16 or int8 rows");
+  static_assert(WB != 4 || C_ % 64 == 0, "4C-wide f32 rows are whole runs of 64 float4");
   static_assert((C_ * WB) % 16 == 0, "rows are whole 16-byte chunks");
   static_assert(WB == 4 || !kTight, "only f32 rows are staged");
 };
@@ -1177,7 +1207,8 @@ struct StreamPlan {
 template <int C_, int WB>
 __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
   typedef StreamPlan<C_, WB> SP;
-  constexpr bool kI8 = WB == 1;
+  constexpr bool kI8 = WB == 1, kPacked = WB != 4;  // packed: several weights per 32-bit word
+  constexpr int XPC = kPacked ? 4 / WB : 1;          // float4 of inputs per 16-byte chunk
   constexpr int C = C_, I = 4 * C_, K4 = C_ / 4;
   constexpr int G = kGrid;
   constexpr int TA = SP::TA, TE = SP::TE, J = SP::J, JF = SP::JF;
@@ -1297,8 +1328,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       PG_SLICE(0, w, wn);
       {
         float v[TA];
-        if constexpr (kI8)
-          dot_tiles_i8<TA, J>(WA, lds.xsA, SP::KC, lane, scA, v);
+        if constexpr (kPacked)
+          dot_tiles_packed<WB, TA, J>(WA, lds.xsA, SP::KC, lane, scA, v);
         else
           dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 0);
@@ -1349,8 +1380,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       }
       {
         float v[1];
-        if constexpr (kI8)
-          dot_tiles_i8<1, J>(WD, lds.xsD, SP::KC, lane, scD, v);
+        if constexpr (kPacked)
+          dot_tiles_packed<WB, 1, J>(WD, lds.xsD, SP::KC, lane, scD, v);
         else
           dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
         const int r = d0 + wave;
@@ -1371,8 +1402,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       }
       {
         float v[TE];
-        if constexpr (kI8)
-          dot_tiles_i8<TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
+        if constexpr (kPacked)
+          dot_tiles_packed<WB, TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
         else
           dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
         const unsigned ep = epoch_of(p, t, l, 4);
@@ -1410,16 +1441,16 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         vm_drain();
         SSTAMP(12);
       }
-      if constexpr (kI8) {
-        // int8 row: KF chunks of 16 weights against the 4C inputs in LDS
+      if constexpr (kPacked) {
+        // packed row: KF chunks of 16 or 8 weights against the 4C inputs in LDS
         const int ln = opaque(lane);
         float acc = 0.0f;
 #pragma unroll
         for (int j = 0; j < JF; ++j) {
           asm volatile("" ::: "memory");
-          f4 x[4];
-          load_x16(x, lds.xsF, SP::KF, ln + 64 * j, 64 * (j + 1) <= SP::KF);
-          acc += i8_chunk(WF.w[j], x[0], x[1], x[2], x[3], scF);
+          f4 x[XPC];
+          load_xc<XPC>(x, lds.xsF, SP::KF, ln + 64 * j, 64 * (j + 1) <= SP::KF);
+          acc += packed_chunk<WB>(WF.w[j], x, scF);
           if (j == 0) SSTAMP(8);
         }
         const float v = wsum(acc);
@@ -1483,13 +1514,13 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         ok = false;
         break;
       }
-      // the input vector in registers for the whole phase: one float4 per f32 chunk, four
-      // per int8 chunk
-      constexpr int XPC = kI8 ? 4 : 1;
+      // the input vector in registers for the whole phase: one float4 per f32 chunk, two
+      // per bf16 chunk, four per int8 chunk
       f4 xr[J * XPC];
-      if constexpr (kI8) {
+      if constexpr (kPacked) {
 #pragma unroll
-        for (int j = 0; j < J; ++j) load_x16(xr + 4 * j, lds.xsD, SP::KC, lane + 64 * j, 64 * (j + 1) <= SP::KC);
+        for (int j = 0; j < J; ++j)
+          load_xc<XPC>(xr + XPC * j, lds.xsD, SP::KC, lane + 64 * j, 64 * (j + 1) <= SP::KC);
       } else {
         load_x<J>(xr, lds.xsD, K4, lane);
       }
@@ -1499,11 +1530,10 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         for (int k = 0; k < kLmTiles; ++k) {
           const int rk = r + kSW * k;
           float v;
-          if constexpr (kI8) {
+          if constexpr (kPacked) {
             float acc = 0.0f;
 #pragma unroll
-            for (int j = 0; j < J; ++j)
-              acc += i8_chunk(T[k].w[j], xr[4 * j], xr[4 * j + 1], xr[4 * j + 2], xr[4 * j + 3], ts[k]);
+            for (int j = 0; j < J; ++j) acc += packed_chunk<WB>(T[k].w[j], xr + XPC * j, ts[k]);
             v = wsum(acc);
           } else {
             v = dot_tile<J>(T[k], xr);
@@ -1570,8 +1600,8 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 
 }  // namespace
 
-size_t persistent_lds_bytes(int C, int w_i8) {
-  const int fs = w_i8 ? 0
+size_t persistent_lds_bytes(int C, int w_packed) {
+  const int fs = w_packed ? 0
                       : C == 1600 ? StreamPlan<1600>::FS : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
   return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8 + (size_t)kSW * fs * 1024;
 }
@@ -1584,7 +1614,7 @@ int persistent_max_item_keys() { return kMaxItemKeys; }
 namespace {
 template <int C_, int WB>
 hipError_t launch_one(const DecodeParams& p, hipStream_t s) {
-  const size_t lds = persistent_lds_bytes(C_, WB == 1);
+  const size_t lds = persistent_lds_bytes(C_, WB != 4);
   // more than the 64 KiB default of dynamic LDS: opt in once per device
   static thread_local int armed_device = -1;
   int dev = 0;
@@ -1617,7 +1647,7 @@ hipError_t fits_one(int* out) {
   hipFuncAttributes at{};
   hipError_t e = hipFuncGetAttributes(&at, reinterpret_cast<const void*>(&k_decode_persistent<C_, WB>));
   if (e != hipSuccess) return e;
-  const size_t lds = persistent_lds_bytes(C_, WB == 1);
+  const size_t lds = persistent_lds_bytes(C_, WB != 4);
   *out = (at.maxThreadsPerBlock >= kThreads && lds <= (size_t)at.maxDynamicSharedSizeBytes) ? 1 : 0;
   return hipSuccess;
 }
@@ -1632,12 +1662,17 @@ hipError_t max_blocks(int C, int* out) {
 }  // namespace
 
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
-  if (p.w_i8 && (!p.lm_s || !p.lm_w)) return hipErrorInvalidValue;
-  return p.w_i8 ? launch_width<1>(p, s) : launch_width<4>(p, s);
+  if (!p.lm_w || (p.w_bytes == 1 && !p.lm_s)) return hipErrorInvalidValue;
+  if (p.w_bytes == 1) return launch_width<1>(p, s);
+  if (p.w_bytes == 2) return launch_width<2>(p, s);
+  if (p.w_bytes == 4) return launch_width<4>(p, s);
+  return hipErrorInvalidValue;
 }
 
-hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_i8) {
-  return w_i8 ? max_blocks<1>(C, out) : max_blocks<4>(C, out);
+hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes) {
+  if (w_bytes == 1) return max_blocks<1>(C, out);
+  if (w_bytes == 2) return max_blocks<2>(C, out);
+  return max_blocks<4>(C, out);
 }
 
 }  // namespace pgk

@@ -400,7 +400,7 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   pgk::DecodeParams p{};
   p.layers = m->d_layers;
   p.wte = m->wte; p.wpe = m->wpe; p.ln_f_g = m->ln_f_g; p.ln_f_b = m->ln_f_b;
-  p.lm_w = m->lm_w; p.lm_s = m->lm_s; p.w_i8 = m->w_i8;
+  p.lm_w = m->lm_w; p.lm_s = m->lm_s; p.w_bytes = m->w_i8 ? 1 : m->w_bf16 ? 2 : 4;
   p.C = (int)g.C; p.I = (int)g.I; p.H = (int)g.H; p.L = (int)g.L; p.V = (int)g.V; p.P = (int)g.P;
   p.eps = g.eps;
   p.kv = c->kv;
@@ -750,9 +750,6 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     return fail(PG_INVALID_CONFIG, "hip backend weight_storage must be f32, bf16 or int8");
   const bool bf = opts.weight_storage == PG_STORE_BF16;
   const bool i8 = opts.weight_storage == PG_STORE_INT8;
-  if (bf && opts.decode_path == PG_DECODE_PERSISTENT)
-    return fail(PG_INVALID_CONFIG,
-                "hip backend decode_path=persistent reads f32 or int8 weights, not bf16");
   if (opts.decode_path > PG_DECODE_PERSISTENT)
     return fail(PG_INVALID_CONFIG, "hip backend decode_path out of range");
   if ((s = select_device(opts.device))) return s;
@@ -897,10 +894,10 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   {
     const int grid = pgk::persistent_grid();
     int blocks_per_cu = 0;
-    bool shape_ok = !bf && g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
+    bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
                     g.P <= 4096 && g.V >= (size_t)grid;
     if (shape_ok) {
-      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu, m->w_i8));
+      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu, i8 ? 1 : bf ? 2 : 4));
       shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
     }
     if (shape_ok) {

@@ -165,10 +165,12 @@ hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int co
 struct DecodeParams {
   const LayerW* layers;
   const float *wte, *wpe, *ln_f_g, *ln_f_b;
-  // lm_head rows: wte itself, or with int8 rows (w_i8) its quantised copy and row scales;
-  // the block matrices are then int8 as well, with the scales in LayerW.
+  // w_bytes: bytes per weight of the block matrices and the lm_head rows: 4 (f32), 2 (bf16)
+  // or 1 (int8, with the row scales in LayerW).  lm_head rows: wte itself, or with int8 rows
+  // its quantised copy lm_w and row scales lm_s (wte stays f32 for the embedding; with bf16
+  // rows wte is bf16 as well).
   const float *lm_w, *lm_s;
-  int w_i8;
+  int w_bytes;
   int C, I, H, L, V, P;
   float eps;
   float* kv;               // [L][2][H][P][64] of this sequence
@@ -196,9 +198,9 @@ struct DecodeParams {
 // dynamic LDS need, and how many of its workgroups fit on one CU.
 bool persistent_supports(int C);
 int persistent_grid();
-size_t persistent_lds_bytes(int C, int w_i8 = 0);
+size_t persistent_lds_bytes(int C, int w_packed = 0);
 int persistent_max_item_keys();
-hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_i8 = 0);
+hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes = 4);
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
 
 }  // namespace pgk

@@ -66,14 +66,48 @@ def test_bf16_batched_steps():
         nxt = np.argmax(want, axis=1).astype(np.uint32)
 
 
-def test_bf16_rejects_persistent_path():
+def test_bf16_options_are_validated():
     cfg = Gpt2Config(vocab_size=257, n_positions=48, n_embd=128, n_layer=1, n_head=2)
     w = synth.random_weights(cfg, 3)
-    with pytest.raises(Gpt2Error, match="reads f32 or int8 weights, not bf16"):
+    with pytest.raises(Gpt2Error, match="decode_path=persistent needs head_dim 64"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_BF16,
                                             decode_path=PG_DECODE_PERSISTENT))
     with pytest.raises(Gpt2Error, match="weight_storage must be f32, bf16 or int8"):
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=7))
+
+
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1600, 25, 40)])
+def test_bf16_persistent_decode_matches_oracle(n_embd, n_head, n_prompt):
+    """The persistent decode kernel on bf16 rows (8 weights per 16-byte chunk, bf16 embedding
+    table): single forwards and a multi-token launch against the oracle on the rounded
+    weights, and against the per-op path."""
+    cfg = Gpt2Config(vocab_size=300, n_positions=256, n_embd=n_embd, n_layer=2, n_head=n_head)
+    w = synth.random_weights(cfg, 0x5EED0510 + n_head, perturb=True)
+    ids = list(synth.token_ids(n_prompt, 0x70C00510, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w, BF16), oracle.Model(cfg, synth.bf16_rounded(w), oracle.rust_config(8))
+    assert "weights=bf16" in model.describe() and "decode=persistent" in model.describe()
+    per_op = Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=PG_STORE_BF16, decode_path=1))
+    assert "decode=kernels" in per_op.describe()
+    cache, pcache, rcache = model.new_kv_cache(), per_op.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    per_op.prefill(ids, pcache)
+    rlog = None
+    for tok in (7, 123, 42):
+        rlog = ref.forward_one(tok, rcache)
+        got = model.forward_one(tok, cache).to_host()
+        assert_logits_close(got, rlog)
+        assert_logits_close(got, per_op.forward_one(tok, pcache).to_host(), abs_tol=2e-5, rel_tol=1e-4)
+    got, _ = model.decode_greedy(cache, 6)  # five forwards in one launch
+    want, clear = [], True
+    for i in range(6):
+        top = np.sort(rlog)[-2:]
+        clear = clear and (top[1] - top[0]) > 2 * (1e-4 + 1e-3 * abs(float(top[1])))
+        want.append(oracle.argmax_logits(rlog))
+        if i < 5:
+            rlog = ref.forward_one(want[-1], rcache)
+    assert len(got) == 6
+    if clear:
+        assert got == want
 
 
 def test_config5_gpt2_xl_bf16_batch32_subsample():
