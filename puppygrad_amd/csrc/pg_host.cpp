@@ -680,10 +680,21 @@ pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg
   if (cand.empty())
     return fail(PG_INVALID_INPUT,
                 "token sampling failed: cannot sample from empty or non-finite logits");
-  std::stable_sort(cand.begin(), cand.end(), [](const auto& l, const auto& r) {
-    return total_order_key(r.second) < total_order_key(l.second);
-  });
-  if (cfg.has_top_k) cand.resize((size_t)std::min<uint64_t>(cfg.top_k, cand.size()));
+  // Stable sort, descending by total_cmp (generation.rs:311-312): among equal keys the lower
+  // id comes first, because the candidates were collected in id order.  With top_k only the
+  // first k of that order are kept (generation.rs:313-315), so only they are sorted; the
+  // explicit id tie-break makes the partial sort pick exactly the stable sort's prefix.
+  const auto before = [](const std::pair<uint32_t, float>& l, const std::pair<uint32_t, float>& r) {
+    const int32_t kl = total_order_key(l.second), kr = total_order_key(r.second);
+    return kl != kr ? kl > kr : l.first < r.first;
+  };
+  if (cfg.has_top_k && cfg.top_k < cand.size()) {
+    const size_t k = (size_t)cfg.top_k;
+    std::partial_sort(cand.begin(), cand.begin() + k, cand.end(), before);
+    cand.resize(k);
+  } else {
+    std::sort(cand.begin(), cand.end(), before);
+  }
   const double T = (double)cfg.temperature;
   const double max_logit = (double)cand[0].second / T;
   std::vector<std::pair<uint32_t, double>> w;

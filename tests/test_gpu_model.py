@@ -238,6 +238,31 @@ def test_sampler_on_device_logits_matches_oracle():
             assert got == want, (kw, seed)
 
 
+def test_sampler_with_tied_logits_keeps_the_stable_order():
+    """Tokens with identical wte rows have bit-identical logits.  The reference sorts the
+    candidates stably (generation.rs:311-312), so among ties the lower id ranks first and
+    top_k may cut through a group of ties: the library's sampler, fed its own device
+    logits, must pick what the oracle's sampler picks on those same values."""
+    _, cfg, w, ids = small_cases()[1]
+    wte = np.asarray(w.wte, np.float32).reshape(cfg.vocab_size, cfg.n_embd).copy()
+    for i in range(cfg.vocab_size):
+        wte[i] = wte[i % 7]  # seven distinct rows: 18-19 exact ties each
+    w.wte = wte.reshape(-1)
+    model = Gpt2Model.new(cfg, w)
+    cache = model.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    host = logits.to_host()
+    assert len(np.unique(host)) <= 7
+    for kw in [dict(temperature=0.9, top_k=3), dict(temperature=1.3, top_k=20), dict(temperature=0.7, top_k=25, top_p=0.9),
+               dict(temperature=1.0, top_k=130), dict(temperature=1.0, top_k=131), dict(temperature=1.1, top_k=500),
+               dict(temperature=0.8, top_p=0.6), dict(temperature=1.0), dict(temperature=1.0, top_k=40, repeat_penalty=1.5)]:
+        for seed in (1, 2, 3, 299792458):
+            g = TextGenerationConfig(1, seed=seed, **kw)
+            got = LogitsSampler(seed).select_next_token(logits, ids, g)
+            want = oracle.LogitsSampler(seed).select_next_token(host, ids, oracle.sampling(seed=seed, **kw))
+            assert got == want, (kw, seed)
+
+
 def test_sampled_stream_matches_oracle():
     _, cfg, w, ids = small_cases()[1]
     model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
