@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Headline benchmark: GPT-2 XL 1.5B fp32, batch-1 greedy decode with a KV cache
-prefilled to 896 tokens (BASELINE.json configs[3]), on one MI355X.
+prefilled to 896 tokens (the configuration the headline metric is quoted on), on one MI355X.
 
 A step is one cached decoder forward (one token).  The timed region holds
 weights, KV cache and the first logits resident in HBM; token selection
@@ -210,7 +210,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 
 
 def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
-    """Secondary workload (BASELINE.json configs[1]-style prompt processing): a step is one
+    """Secondary workload (prompt processing, e.g. GPT-2 124M with 1024 tokens): a step is one
     prefill of n_prefill tokens into an empty cache through the GEMM path.  Algorithmic
     flops: the four projections of every layer over all tokens, causal attention
     (QK^T and PV over the lower triangle), and the lm_head row of the last token."""
@@ -254,7 +254,7 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
 
 
 def bench_batch_decode(args, cfg, model, n_prefill) -> int:
-    """Secondary workload (BASELINE.json configs[2] / configs[4] style): --batch sequences
+    """Secondary workload (batched decode, e.g. 355M batch 16 or XL bf16 batch 32): --batch sequences
     prefilled to n_prefill tokens each, then --steps greedy steps for all of them.  A step
     reads every weight once plus the K/V rows of every sequence: HBM-bound."""
     from puppygrad_amd import synth

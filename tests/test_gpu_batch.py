@@ -1,4 +1,4 @@
-"""Batched decode (BASELINE configs 3 and 5 shapes): every sequence of a batch must
+"""Batched decode (the batched benchmark configurations: 355M batch 16, XL bf16 batch 32): every sequence of a batch must
 match the oracle run on that sequence alone."""
 import numpy as np
 import pytest
@@ -102,7 +102,7 @@ def test_batch_argument_errors():
 
 
 def test_config3_gpt2_medium_batch16_subsample():
-    """BASELINE config 3 (355M, batch 16, 128-token prompts): all 16 sequences run on the
+    """Benchmark configuration 3 (355M, batch 16, 128-token prompts): all 16 sequences run on the
     GPU; sequences 0, 7 and 15 are checked against the oracle for the prompt and the
     first 6 greedy steps (teacher-forced with the oracle's tokens)."""
     cfg = Gpt2Config(**synth.GPT2_MEDIUM)

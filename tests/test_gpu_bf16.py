@@ -1,4 +1,4 @@
-"""bf16 weight storage (BASELINE config 5): the token embedding and the block matrices
+"""bf16 weight storage (benchmark configuration 5): the token embedding and the block matrices
 are kept as bf16 in HBM, accumulation / LayerNorm / softmax / KV cache stay f32.  The
 oracle runs on the same bf16-rounded weights widened to f32, so both sides multiply
 identical values and the f32 tolerance applies; the 2e-2 relative bound the config
@@ -111,7 +111,7 @@ def test_bf16_persistent_decode_matches_oracle(n_embd, n_head, n_prompt):
 
 
 def test_config5_gpt2_xl_bf16_batch32_subsample():
-    """BASELINE config 5 shape (XL, bf16 weights, batch 32, 512-token prompts): all 32
+    """Benchmark configuration 5 shape (XL, bf16 weights, batch 32, 512-token prompts): all 32
     sequences run on the GPU; sequence 0 and 31 are checked against the oracle (on the
     rounded weights) for the prompt and 3 teacher-forced steps."""
     cfg = Gpt2Config(**synth.GPT2_XL)

@@ -297,7 +297,7 @@ def greedy_with_teacher_forcing(model, ref, ids, max_new, check_every=1):
 
 
 def test_config1_gpt2_small_greedy_decode_parity():
-    """BASELINE config 1: 124M, 32 prompt ids, 128 greedy tokens with KV cache."""
+    """Benchmark configuration 1: 124M, 32 prompt ids, 128 greedy tokens with KV cache."""
     cfg = synth.Gpt2Config(**synth.GPT2_SMALL)
     w = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 1)
     ids = list(synth.token_ids(32, synth.TOKEN_SEED_BASE + 1, cfg.vocab_size))
