@@ -921,10 +921,13 @@ hipError_t launch_gemv_rows_r(const GemmArgs& a, int epi, hipStream_t s) {
     return hipErrorInvalidValue;
   return hipGetLastError();
 }
-// Rows per wavefront: as many as leave about two blocks per CU (and one sum per lane).
+// Rows per wavefront: as many as leave about one and a half blocks per CU (and one sum per
+// lane): every block stages all input vectors, so fewer, longer blocks win until the CUs
+// run short of blocks (355M, 16 rows: 2 rows per wavefront for the 3072- and 4096-row
+// matrices; measured against 1 and 4).
 template <bool WBF>
 hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
-  const long want = 2L * num_cus;
+  const long want = 3L * num_cus / 2;
   if (a.M <= 16) {
     if ((a.N + 15) / 16 >= want) return launch_gemv_rows_r<16, 4, WBF>(a, epi, s);
     if ((a.N + 7) / 8 >= want) return launch_gemv_rows_r<16, 2, WBF>(a, epi, s);
