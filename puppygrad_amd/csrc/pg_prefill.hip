@@ -937,9 +937,11 @@ hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t
   return launch_gemv_rows_r<32, 1, WBF>(a, epi, s);
 }
 
-// K parts for k_gemm_rows32 (0 = not applicable): up to one block per CU (cutting K further
-// was measured slower: the reduce and the shorter pieces cost more than the idle CUs), at
-// least sixteen units per block and part, bounded by the workspace.
+// K parts for k_gemm_rows32 (0 = not applicable): as many as keep the blocks within one per
+// CU, rounded down (150 row blocks stay uncut, 50 are cut five times: rounding to nearest or
+// up, or cutting less, were all measured slower: the reduce launch and the shorter pieces
+// cost more than the idle CUs), at least sixteen units per block and part, bounded by the
+// workspace.
 bool gemm_prefers_gemv_rows(const GemmArgs& a) {
   return a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024;
 }
@@ -947,7 +949,7 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 16 : 8;
   if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
   const long tiles = (a.N + 31) / 32;
-  long parts = std::max<long>(1, (num_cus + tiles / 2) / tiles);
+  long parts = std::max<long>(1, num_cus / tiles);
   parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 16));
   parts = std::min<long>(parts, 8);
   if (parts > 1) {
