@@ -1002,7 +1002,7 @@ hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
 int gemm_split_parts(const GemmArgs& a, int num_cus) {
   const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
   if (!a.ws || a.N % 4 != 0 || tiles * 2 >= 3L * num_cus) return 1;
-  const int depth = a.M < 64 ? 128 : 512;
+  const int depth = a.M < 64 ? 128 : (tiles * 10 < 9L * num_cus ? 192 : 512);
   int parts = (int)((3L * num_cus) / tiles);
   parts = std::min(parts, a.K / depth);
   parts = std::min(parts, 8);
