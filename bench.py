@@ -56,7 +56,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=127)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--model", default="xl", choices=["xl", "medium", "small"])
+    ap.add_argument("--model", default="xl", choices=["xl", "large", "medium", "small"])
     ap.add_argument("--prefill", type=int, default=None, help="tokens in the cache before decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
@@ -77,10 +77,11 @@ def main() -> int:
 
     from puppygrad_amd import Gpt2Config, Gpt2HipConfig, Gpt2Model, _lib, synth
 
-    model_kw = {"xl": synth.GPT2_XL, "medium": synth.GPT2_MEDIUM, "small": synth.GPT2_SMALL}[args.model]
-    cfg_no = {"xl": 4, "medium": 3, "small": 1}[args.model]
+    model_kw = {"xl": synth.GPT2_XL, "large": synth.GPT2_LARGE, "medium": synth.GPT2_MEDIUM,
+                "small": synth.GPT2_SMALL}[args.model]
+    cfg_no = {"xl": 4, "large": 6, "medium": 3, "small": 1}[args.model]
     cfg = Gpt2Config(**model_kw)
-    n_prefill = args.prefill if args.prefill is not None else {"xl": 896, "medium": 128, "small": 32}[args.model]
+    n_prefill = args.prefill if args.prefill is not None else {"xl": 896, "large": 512, "medium": 128, "small": 32}[args.model]
     room = cfg.n_positions - n_prefill  # tokens one pass can generate
 
     t0 = time.time()

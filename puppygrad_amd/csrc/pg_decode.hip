@@ -1602,12 +1602,14 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
 
 size_t persistent_lds_bytes(int C, int w_packed) {
   const int fs = w_packed ? 0
-                      : C == 1600 ? StreamPlan<1600>::FS : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
+                      : C == 1600 ? StreamPlan<1600>::FS
+                      : C == 1280 ? StreamPlan<1280>::FS
+                      : C == 1024 ? StreamPlan<1024>::FS : StreamPlan<768>::FS;
   return (size_t)(9 * C) * sizeof(float) + (size_t)kTsLayers * 16 * 8 + (size_t)kSW * fs * 1024;
 }
-// n_embd values the kernel is instantiated for (GPT-2 small, medium, XL), each for f32 and
-// for int8 rows.
-bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1600; }
+// n_embd values the kernel is instantiated for (GPT-2 small, medium, large, XL), each for
+// f32, bf16 and int8 rows.
+bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1280 || C == 1600; }
 int persistent_grid() { return kGrid; }
 int persistent_max_item_keys() { return kMaxItemKeys; }
 
@@ -1633,6 +1635,7 @@ template <int WB>
 hipError_t launch_width(const DecodeParams& p, hipStream_t s) {
   if (p.C == 768) return launch_one<768, WB>(p, s);
   if (p.C == 1024) return launch_one<1024, WB>(p, s);
+  if (p.C == 1280) return launch_one<1280, WB>(p, s);
   if (p.C == 1600) return launch_one<1600, WB>(p, s);
   return hipErrorInvalidValue;
 }
@@ -1655,6 +1658,7 @@ template <int WB>
 hipError_t max_blocks(int C, int* out) {
   if (C == 768) return fits_one<768, WB>(out);
   if (C == 1024) return fits_one<1024, WB>(out);
+  if (C == 1280) return fits_one<1280, WB>(out);
   if (C == 1600) return fits_one<1600, WB>(out);
   *out = 0;
   return hipSuccess;

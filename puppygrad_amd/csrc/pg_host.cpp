@@ -923,7 +923,7 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     if (opts.decode_path == PG_DECODE_PERSISTENT && !shape_ok)
       return fail(PG_INVALID_CONFIG,
                   "hip backend decode_path=persistent needs head_dim 64, n_inner = 4*n_embd, "
-                  "n_embd in {768, 1024, 1600} and a device that holds 256 workgroups at once");
+                  "n_embd in {768, 1024, 1280, 1600} and a device that holds 256 workgroups at once");
     m->persistent = shape_ok && opts.decode_path != PG_DECODE_KERNELS;
     m->persistent_grid = grid;
   }

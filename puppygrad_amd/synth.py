@@ -17,6 +17,7 @@ from .gpt2 import Gpt2BlockWeights, Gpt2Config, Gpt2Weights
 
 GPT2_SMALL = dict(vocab_size=50257, n_positions=1024, n_embd=768, n_layer=12, n_head=12)
 GPT2_MEDIUM = dict(vocab_size=50257, n_positions=1024, n_embd=1024, n_layer=24, n_head=16)
+GPT2_LARGE = dict(vocab_size=50257, n_positions=1024, n_embd=1280, n_layer=36, n_head=20)
 GPT2_XL = dict(vocab_size=50257, n_positions=1024, n_embd=1600, n_layer=48, n_head=25)
 
 WEIGHT_SEED_BASE = 0x5EED_0000

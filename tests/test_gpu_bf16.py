@@ -76,7 +76,7 @@ def test_bf16_options_are_validated():
         Gpt2Model.new(cfg, w, Gpt2HipConfig(weight_storage=7))
 
 
-@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1600, 25, 40)])
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1280, 20, 70), (1600, 25, 40)])
 def test_bf16_persistent_decode_matches_oracle(n_embd, n_head, n_prompt):
     """The persistent decode kernel on bf16 rows (8 weights per 16-byte chunk, bf16 embedding
     table): single forwards and a multi-token launch against the oracle on the rounded

@@ -114,7 +114,7 @@ def test_int8_gpt2_small_decode_steps():
         assert_logits_close(got, want, what=f"step {step}")
 
 
-@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1600, 25, 40)])
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 20), (1024, 16, 150), (1280, 20, 70), (1600, 25, 40)])
 def test_int8_persistent_decode_matches_oracle(n_embd, n_head, n_prompt):
     """The persistent decode kernel on int8 rows (16 weights per 16-byte chunk; the XL rows
     are not whole runs of 64 chunks): single forwards and a multi-token launch against the

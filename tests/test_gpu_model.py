@@ -191,6 +191,34 @@ def test_gemm_prefill_and_forward_match_oracle(case):
     assert_logits_close(tok_model.prefill(ids, c2).to_host(), want_all[-1])
 
 
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(768, 12, 30), (1024, 16, 140), (1280, 20, 60), (1600, 25, 200)])
+def test_persistent_decode_every_width_matches_oracle(n_embd, n_head, n_prompt):
+    """The four GPT-2 widths the persistent decode kernel is built for (small, medium, large,
+    XL), f32 rows: single forwards and a multi-token launch against the oracle."""
+    cfg = synth.Gpt2Config(vocab_size=300, n_positions=256, n_embd=n_embd, n_layer=2, n_head=n_head)
+    w = synth.random_weights(cfg, 0x5EED0220 + n_head, perturb=True)
+    ids = list(synth.token_ids(n_prompt, 0x70C00220, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(8))
+    assert "decode=persistent" in model.describe()
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    assert_logits_close(model.prefill(ids, cache).to_host(), ref.prefill(ids, rcache))
+    rlog = None
+    for tok in (7, 123, 42):
+        rlog = ref.forward_one(tok, rcache)
+        assert_logits_close(model.forward_one(tok, cache).to_host(), rlog)
+    got, _ = model.decode_greedy(cache, 6)
+    want, clear = [], True
+    for i in range(6):
+        top = np.sort(rlog)[-2:]
+        clear = clear and (top[1] - top[0]) > 2 * (ABS_TOL + REL_TOL * abs(float(top[1])))
+        want.append(oracle.argmax_logits(rlog))
+        if i < 5:
+            rlog = ref.forward_one(want[-1], rcache)
+    assert len(got) == 6
+    if clear:
+        assert got == want
+
+
 @pytest.mark.parametrize("n_prompt", [100, 1500, 2750])
 def test_persistent_decode_split_counts_match_oracle(n_prompt):
     """The persistent decode kernel picks the number of key splits per head from the position:
