@@ -683,15 +683,17 @@ pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg
   // Stable sort, descending by total_cmp (generation.rs:311-312): among equal keys the lower
   // id comes first, because the candidates were collected in id order.  With top_k only the
   // first k of that order are kept (generation.rs:313-315), so only they are sorted; the
-  // explicit id tie-break makes the partial sort pick exactly the stable sort's prefix.
+  // explicit id tie-break makes the selection pick exactly the stable sort's prefix.
   const auto before = [](const std::pair<uint32_t, float>& l, const std::pair<uint32_t, float>& r) {
     const int32_t kl = total_order_key(l.second), kr = total_order_key(r.second);
     return kl != kr ? kl > kr : l.first < r.first;
   };
   if (cfg.has_top_k && cfg.top_k < cand.size()) {
     const size_t k = (size_t)cfg.top_k;
-    std::partial_sort(cand.begin(), cand.begin() + k, cand.end(), before);
+    // (`before` is a strict total order, so the k first are a unique set: select, then sort)
+    std::nth_element(cand.begin(), cand.begin() + k, cand.end(), before);
     cand.resize(k);
+    std::sort(cand.begin(), cand.end(), before);
   } else {
     std::sort(cand.begin(), cand.end(), before);
   }
