@@ -190,7 +190,10 @@ double pg_rng_next_unit_f64(pg_rng_state* rng);
 /* LogitsSampler::select_next_token (src/models/generation.rs:221-241) on row
  * `row` of the logits: repeat penalty over the last repeat_last_n history ids,
  * argmax when temperature <= 0, otherwise top-k / top-p / inverse-CDF sampling
- * (generation.rs:281-362). */
+ * (generation.rs:281-362).  Greedy selection is an argmax on the device; with top_k the
+ * penalty, the finite filter and the choice of the k candidates run on the device and only
+ * those k pairs reach the host, which draws from them in f64 as the reference does; without
+ * top_k the row is copied to the host. */
 pg_status pg_logits_sample(pg_logits* logits, uint32_t row, const uint32_t* history, size_t n_hist,
                            const pg_sampling* sampling, pg_rng_state* rng, uint32_t* out);
 

@@ -98,6 +98,13 @@ struct pg_kv_cache {
         *part_l = nullptr, *logits_buf = nullptr;
   float *qkv_b = nullptr, *xn_b = nullptr, *att_b = nullptr;  // batched step: [B][3C], [B][C], [B][C]
   bool pack32 = false;  // batched step: xn_b, att_b and hbuf are packed (pgk::packed32_index)
+  // device-side candidate selection for sampling, allocated at first use: kept candidates
+  // (ids, then values, then [count]) and the recent ids of the repeat penalty, with pinned
+  // host mirrors
+  uint32_t* d_cand = nullptr;
+  uint32_t* h_cand = nullptr;
+  uint32_t* d_recent = nullptr;
+  uint32_t* h_recent = nullptr;
   uint32_t* d_tok = nullptr;      // [B] token the next step embeds
   uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
   uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
@@ -672,9 +679,46 @@ inline int32_t total_order_key(float f) {
   return b;
 }
 
+using Candidate = std::pair<uint32_t, float>;  // (token id, logit)
+
+// The stable descending order of sample_logits (generation.rs:311-312): by total_cmp, and
+// among equal values by id (the candidates are collected in id order and the sort is stable).
+bool candidate_before(const Candidate& l, const Candidate& r) {
+  const int32_t kl = total_order_key(l.second), kr = total_order_key(r.second);
+  return kl != kr ? kl > kr : l.first < r.first;
+}
+
+pg_status sample_sorted(std::vector<Candidate>& cand, const pg_sampling& cfg, pg_rng_state* rng,
+                        uint32_t* out, bool in_id_order = false);
+
+// The same order for a long list that is in id order: a stable radix sort on the 32-bit
+// order-preserving image of the values, descending (two passes of 16 bits; stability keeps
+// equal values in id order).  A comparison sort of 50k candidates costs about 3 ms per token.
+void radix_sort_descending(std::vector<Candidate>& cand) {
+  const size_t n = cand.size();
+  std::vector<Candidate> tmp(n);
+  std::vector<uint32_t> count(65536);
+  auto inv_key = [](const Candidate& c) {  // ascending inv_key == descending total_cmp
+    return ~((uint32_t)total_order_key(c.second) ^ 0x80000000u);
+  };
+  for (int pass = 0; pass < 2; ++pass) {
+    const int shift = 16 * pass;
+    std::fill(count.begin(), count.end(), 0u);
+    for (size_t i = 0; i < n; ++i) ++count[(inv_key(cand[i]) >> shift) & 0xffffu];
+    uint32_t at = 0;
+    for (auto& c : count) {
+      const uint32_t here = c;
+      c = at;
+      at += here;
+    }
+    for (size_t i = 0; i < n; ++i) tmp[count[(inv_key(cand[i]) >> shift) & 0xffffu]++] = cand[i];
+    cand.swap(tmp);
+  }
+}
+
 pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg,
                         pg_rng_state* rng, uint32_t* out) {
-  std::vector<std::pair<uint32_t, float>> cand;
+  std::vector<Candidate> cand;
   for (size_t i = 0; i < logits.size(); ++i)
     if (std::isfinite(logits[i])) cand.emplace_back((uint32_t)i, logits[i]);
   if (cand.empty())
@@ -684,19 +728,27 @@ pg_status sample_logits(const std::vector<float>& logits, const pg_sampling& cfg
   // id comes first, because the candidates were collected in id order.  With top_k only the
   // first k of that order are kept (generation.rs:313-315), so only they are sorted; the
   // explicit id tie-break makes the selection pick exactly the stable sort's prefix.
-  const auto before = [](const std::pair<uint32_t, float>& l, const std::pair<uint32_t, float>& r) {
-    const int32_t kl = total_order_key(l.second), kr = total_order_key(r.second);
-    return kl != kr ? kl > kr : l.first < r.first;
-  };
   if (cfg.has_top_k && cfg.top_k < cand.size()) {
     const size_t k = (size_t)cfg.top_k;
-    // (`before` is a strict total order, so the k first are a unique set: select, then sort)
-    std::nth_element(cand.begin(), cand.begin() + k, cand.end(), before);
+    // (a strict total order, so the k first are a unique set: select, then sort)
+    std::nth_element(cand.begin(), cand.begin() + k, cand.end(), candidate_before);
     cand.resize(k);
-    std::sort(cand.begin(), cand.end(), before);
-  } else {
-    std::sort(cand.begin(), cand.end(), before);
+    return sample_sorted(cand, cfg, rng, out);
   }
+  return sample_sorted(cand, cfg, rng, out, /*in_id_order=*/true);
+}
+
+// The rest of sample_logits (generation.rs:311-362) on the kept candidates, in any order:
+// sort, f64 weights exp(l/T - max), top_p prefix, inverse-CDF walk.
+pg_status sample_sorted(std::vector<Candidate>& cand, const pg_sampling& cfg, pg_rng_state* rng,
+                        uint32_t* out, bool in_id_order) {
+  if (cand.empty())
+    return fail(PG_INVALID_INPUT,
+                "token sampling failed: cannot sample from empty or non-finite logits");
+  if (in_id_order && cand.size() > 4096)
+    radix_sort_descending(cand);
+  else
+    std::sort(cand.begin(), cand.end(), candidate_before);
   const double T = (double)cfg.temperature;
   const double max_logit = (double)cand[0].second / T;
   std::vector<std::pair<uint32_t, double>> w;
@@ -1049,6 +1101,10 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->logits_buf);
     (void)hipFree(c->qkv_b);
     (void)hipFree(c->xn_b);
+    if (c->d_cand) (void)hipFree(c->d_cand);
+    if (c->h_cand) (void)hipHostFree(c->h_cand);
+    if (c->d_recent) (void)hipFree(c->d_recent);
+    if (c->h_recent) (void)hipHostFree(c->h_recent);
     (void)hipFree(c->att_b);
     (void)hipFree(c->d_tok);
     (void)hipFree(c->d_out_ids);
@@ -1278,6 +1334,44 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
     PG_HIP(hipStreamSynchronize(c->stream));
     *out = c->h_ids[0];
     return PG_OK;
+  }
+  // Sampling with top_k: the candidates are chosen on the device (penalty, finite filter, the
+  // k first of the stable order) and only they cross to the host, which does the f64
+  // arithmetic of the draw exactly as the reference does.
+  constexpr uint64_t kMaxCand = 4096, kMaxRecent = 8192;
+  const uint64_t recent = penalised ? std::min<uint64_t>(sampling->repeat_last_n, n_hist) : 0;
+  if (sampling->temperature > 0.0f && sampling->has_top_k && sampling->top_k <= kMaxCand &&
+      l->vocab <= (uint64_t)pgk::kTopkMaxVocab && recent <= kMaxRecent && (recent == 0 || history)) {
+    if (!c->d_cand) {
+      PG_HIP(hipMalloc(&c->d_cand, (2 * kMaxCand + 4) * sizeof(uint32_t)));
+      PG_HIP(hipHostMalloc(&c->h_cand, (2 * kMaxCand + 4) * sizeof(uint32_t), hipHostMallocDefault));
+      PG_HIP(hipMalloc(&c->d_recent, kMaxRecent * sizeof(uint32_t)));
+      PG_HIP(hipHostMalloc(&c->h_recent, kMaxRecent * sizeof(uint32_t), hipHostMallocDefault));
+    }
+    const int k = (int)sampling->top_k;
+    if (recent) {
+      std::memcpy(c->h_recent, history + (n_hist - recent), recent * sizeof(uint32_t));
+      PG_HIP(hipMemcpyAsync(c->d_recent, c->h_recent, recent * sizeof(uint32_t),
+                            hipMemcpyHostToDevice, c->stream));
+    }
+    uint32_t* d_ids = c->d_cand;
+    float* d_vals = reinterpret_cast<float*>(c->d_cand + kMaxCand);
+    uint32_t* d_count = c->d_cand + 2 * kMaxCand;
+    PG_HIP(pgk::launch_topk_select(l->data + (size_t)row * l->vocab, (int)l->vocab, c->d_recent,
+                                   (int)recent, sampling->repeat_penalty, k, d_ids, d_vals, d_count,
+                                   c->stream));
+    // ids and values of the k slots that can be filled, and the count
+    PG_HIP(hipMemcpyAsync(c->h_cand, d_ids, (size_t)k * sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_cand + kMaxCand, d_vals, (size_t)k * sizeof(float), hipMemcpyDeviceToHost,
+                          c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_cand + 2 * kMaxCand, d_count, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));
+    const uint32_t count = std::min<uint32_t>(c->h_cand[2 * kMaxCand], (uint32_t)k);
+    std::vector<Candidate> cand(count);
+    const float* vals = reinterpret_cast<const float*>(c->h_cand + kMaxCand);
+    for (uint32_t i = 0; i < count; ++i) cand[i] = Candidate(c->h_cand[i], vals[i]);
+    return sample_sorted(cand, *sampling, rng, out);
   }
   std::vector<float> adjusted(l->vocab);
   PG_HIP(hipStreamSynchronize(c->stream));

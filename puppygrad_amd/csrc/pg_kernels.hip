@@ -533,6 +533,137 @@ __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t
   }
 }
 
+// ---- candidate selection for sampling (generation.rs:281-315) on the device -------------
+// sample_logits sorts the finite logits descending (total_cmp; the sort is stable, so equal
+// values keep id order) and keeps the first top_k.  Which k those are is decided here, so
+// that only k (id, logit) pairs cross to the host instead of the whole row: the repeat
+// penalty is applied first (apply_repeat_penalty, generation.rs:281-298: once per distinct
+// recent id, negative logits multiplied, others divided), then a radix select over the
+// order-preserving integer image of the values finds the k-th largest key, and an ordered
+// compaction writes every candidate above it plus, among those equal to it, the lowest ids.
+// One block per call; out_count[0] = number of candidates (fewer than k when fewer are finite).
+__device__ __forceinline__ unsigned order_key(float f) {  // total_cmp order, as unsigned
+  int b = __float_as_int(f);
+  b ^= (int)(((unsigned)(b >> 31)) >> 1);
+  return (unsigned)b ^ 0x80000000u;
+}
+__global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V,
+                                                      const uint32_t* pen_ids, int n_pen,
+                                                      float penalty, int k, uint32_t* out_ids,
+                                                      float* out_vals, uint32_t* out_count) {
+  extern __shared__ unsigned pen_bits[];  // one bit per id: among the recent ids
+  __shared__ unsigned hist[256];
+  __shared__ unsigned sh_prefix, sh_remaining, sh_total;
+  __shared__ unsigned wave_gt[16], wave_eq[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int words = (V + 31) / 32;
+  for (int i = tid; i < words; i += 1024) pen_bits[i] = 0u;
+  if (tid == 0) sh_total = 0u;
+  __syncthreads();
+  for (int i = tid; i < n_pen; i += 1024) {
+    const uint32_t id = pen_ids[i];
+    if (id < (uint32_t)V) atomicOr(&pen_bits[id >> 5], 1u << (id & 31));
+  }
+  __syncthreads();
+  auto value = [&](int i) {
+    const float l = logits[i];
+    if (n_pen && ((pen_bits[i >> 5] >> (i & 31)) & 1u)) return l < 0.0f ? l * penalty : l / penalty;
+    return l;
+  };
+  auto finite = [](float v) { return fabsf(v) <= 3.402823466e+38f; };  // false for NaN and inf
+  // finite candidates in all
+  {
+    unsigned c = 0;
+    for (int i = tid; i < V; i += 1024) c += finite(value(i)) ? 1u : 0u;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+    if (lane == 0) atomicAdd(&sh_total, c);
+  }
+  __syncthreads();
+  const unsigned total = sh_total;
+  const unsigned kk = total < (unsigned)k ? total : (unsigned)k;
+  if (tid == 0) out_count[0] = kk;
+  if (kk == 0) return;
+  // radix select, most significant byte first: key of the kk-th largest candidate
+  unsigned prefix = 0u, mask = 0u;
+  if (tid == 0) sh_remaining = kk;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (tid < 256) hist[tid] = 0u;
+    __syncthreads();
+    for (int i = tid; i < V; i += 1024) {
+      const float v = value(i);
+      if (!finite(v)) continue;
+      const unsigned key = order_key(v);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      unsigned remaining = sh_remaining, cum = 0u;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (cum + hist[b] >= remaining) break;
+        cum += hist[b];
+      }
+      sh_remaining = remaining - cum;  // how many to take inside bin b
+      sh_prefix = prefix | ((unsigned)b << shift);
+    }
+    __syncthreads();
+    prefix = sh_prefix;
+    mask |= 255u << shift;
+    __syncthreads();
+  }
+  const unsigned T = prefix;            // key of the kk-th largest
+  const unsigned need = sh_remaining;   // candidates equal to T that are kept: the lowest ids
+  const unsigned n_gt = kk - need;
+  // ordered compaction: thread t owns ids [t * per, (t + 1) * per)
+  const int per = (V + 1023) / 1024;
+  const int i0 = tid * per, i1 = min(V, i0 + per);
+  unsigned c_gt = 0u, c_eq = 0u;
+  for (int i = i0; i < i1; ++i) {
+    const float v = value(i);
+    if (!finite(v)) continue;
+    const unsigned key = order_key(v);
+    c_gt += key > T ? 1u : 0u;
+    c_eq += key == T ? 1u : 0u;
+  }
+  // exclusive prefix sums over the block, in thread (= id) order
+  unsigned s_gt = c_gt, s_eq = c_eq;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned a = __shfl_up(s_gt, off, 64), b = __shfl_up(s_eq, off, 64);
+    if (lane >= off) {
+      s_gt += a;
+      s_eq += b;
+    }
+  }
+  if (lane == 63) {
+    wave_gt[wave] = s_gt;
+    wave_eq[wave] = s_eq;
+  }
+  __syncthreads();
+  unsigned base_gt = s_gt - c_gt, base_eq = s_eq - c_eq;
+  for (int w = 0; w < wave; ++w) {
+    base_gt += wave_gt[w];
+    base_eq += wave_eq[w];
+  }
+  for (int i = i0; i < i1; ++i) {
+    const float v = value(i);
+    if (!finite(v)) continue;
+    const unsigned key = order_key(v);
+    if (key > T) {
+      out_ids[base_gt] = (uint32_t)i;
+      out_vals[base_gt] = v;
+      ++base_gt;
+    } else if (key == T) {
+      if (base_eq < need) {
+        out_ids[n_gt + base_eq] = (uint32_t)i;
+        out_vals[n_gt + base_eq] = v;
+      }
+      ++base_eq;
+    }
+  }
+}
+
 // Embedding of one token per sequence at a common position (rust.rs:966-974).
 __global__ void k_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
                               int pos, int C, int w_bf16) {
@@ -771,6 +902,16 @@ hipError_t launch_kv_append(const float* qkv, int batch, int C, int head_dim, in
                             float* kcache, float* vcache, size_t kv_stride, hipStream_t s) {
   hipLaunchKernelGGL(k_kv_append, dim3((C + 255) / 256, batch), dim3(256), 0, s, qkv, C, head_dim,
                      P, pos, kcache, vcache, kv_stride);
+  return hipGetLastError();
+}
+
+hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
+                              float penalty, int k, uint32_t* out_ids, float* out_vals,
+                              uint32_t* out_count, hipStream_t s) {
+  const size_t lds = (size_t)((V + 31) / 32) * sizeof(unsigned);
+  if (V < 1 || k < 1 || lds > 60000 || n_pen < 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(k_topk_select, dim3(1), dim3(1024), lds, s, logits, V, pen_ids, n_pen,
+                     penalty, k, out_ids, out_vals, out_count);
   return hipGetLastError();
 }
 

@@ -281,14 +281,74 @@ def test_sampler_with_tied_logits_keeps_the_stable_order():
     logits = model.prefill(ids, cache)
     host = logits.to_host()
     assert len(np.unique(host)) <= 7
-    for kw in [dict(temperature=0.9, top_k=3), dict(temperature=1.3, top_k=20), dict(temperature=0.7, top_k=25, top_p=0.9),
-               dict(temperature=1.0, top_k=130), dict(temperature=1.0, top_k=131), dict(temperature=1.1, top_k=500),
-               dict(temperature=0.8, top_p=0.6), dict(temperature=1.0), dict(temperature=1.0, top_k=40, repeat_penalty=1.5)]:
+    cases = [dict(temperature=0.9, top_k=3), dict(temperature=1.3, top_k=20), dict(temperature=0.7, top_k=25, top_p=0.9),
+             dict(temperature=1.0, top_k=1), dict(temperature=1.0, top_k=19), dict(temperature=1.0, top_k=130),
+             dict(temperature=1.0, top_k=131), dict(temperature=1.1, top_k=500), dict(temperature=0.8, top_p=0.6),
+             dict(temperature=1.0), dict(temperature=1.0, top_k=40, repeat_penalty=1.5),
+             dict(temperature=0.6, top_k=7, repeat_penalty=3.0, repeat_last_n=5),
+             dict(temperature=2.0, top_k=60, repeat_penalty=0.5, repeat_last_n=1000)]
+    for kw in cases:
         for seed in (1, 2, 3, 299792458):
             g = TextGenerationConfig(1, seed=seed, **kw)
             got = LogitsSampler(seed).select_next_token(logits, ids, g)
             want = oracle.LogitsSampler(seed).select_next_token(host, ids, oracle.sampling(seed=seed, **kw))
             assert got == want, (kw, seed)
+
+
+def test_sampler_over_a_large_vocabulary_with_ties():
+    """More than 4096 candidates: without top_k the host orders the whole row (a stable radix
+    sort on the values' integer image); with top_k the device picks the candidates.  Rows of
+    wte are repeated so that the order among exact ties matters."""
+    cfg = synth.Gpt2Config(vocab_size=6011, n_positions=32, n_embd=128, n_layer=1, n_head=2)
+    w = synth.random_weights(cfg, 0x5EED0230, perturb=True)
+    wte = np.asarray(w.wte, np.float32).reshape(cfg.vocab_size, cfg.n_embd).copy()
+    for i in range(cfg.vocab_size):
+        wte[i] = wte[i % 997]  # six or seven exact ties per value
+    wte[11] = np.inf           # and a few non-finite logits
+    wte[4999] = -np.inf
+    w.wte = wte.reshape(-1)
+    ids = [int(t) for t in synth.token_ids(9, 0x70C00230, 997) if t not in (11,)]
+    model = Gpt2Model.new(cfg, w)
+    cache = model.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    host = logits.to_host()
+    assert len(np.unique(host[np.isfinite(host)])) <= 997
+    for kw in [dict(temperature=1.0), dict(temperature=0.7, top_p=0.9), dict(temperature=1.5, top_p=0.999),
+               dict(temperature=1.0, repeat_penalty=1.3), dict(temperature=1.0, top_k=5000),
+               dict(temperature=1.0, top_k=4096), dict(temperature=0.9, top_k=300, top_p=0.95),
+               dict(temperature=1.0, top_k=6, repeat_penalty=2.0, repeat_last_n=4)]:
+        for seed in (1, 2, 3, 4, 5):
+            g = TextGenerationConfig(1, seed=seed, **kw)
+            got = LogitsSampler(seed).select_next_token(logits, ids, g)
+            want = oracle.LogitsSampler(seed).select_next_token(host, ids, oracle.sampling(seed=seed, **kw))
+            assert got == want, (kw, seed)
+
+
+def test_sampler_skips_non_finite_logits():
+    """Rows of wte made of infinities give +inf, -inf and NaN logits: sample_logits keeps the
+    finite ones only (generation.rs:300-310), on the device path (top_k) as on the host path."""
+    _, cfg, w, ids = small_cases()[1]
+    ids = [t for t in ids if t not in (3, 4, 5)] or [1]
+    wte = np.asarray(w.wte, np.float32).reshape(cfg.vocab_size, cfg.n_embd).copy()
+    wte[3] = np.inf                                                   # mixed-sign hidden state: NaN
+    wte[4] = 0.0
+    wte[4, 0] = np.inf                                                # +inf or -inf
+    wte[5] = 0.0
+    wte[5, 0] = -np.inf
+    w.wte = wte.reshape(-1)
+    model = Gpt2Model.new(cfg, w)
+    cache = model.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    host = logits.to_host()
+    assert not np.isfinite(host[[3, 4, 5]]).any() and np.isfinite(np.delete(host, [3, 4, 5])).all()
+    for kw in [dict(temperature=1.0, top_k=5), dict(temperature=1.0, top_k=cfg.vocab_size - 3),
+               dict(temperature=1.0, top_k=cfg.vocab_size - 1), dict(temperature=0.9, top_k=64, repeat_penalty=1.4),
+               dict(temperature=1.0), dict(temperature=1.2, top_p=0.7)]:
+        for seed in (5, 6, 7):
+            g = TextGenerationConfig(1, seed=seed, **kw)
+            got = LogitsSampler(seed).select_next_token(logits, ids, g)
+            want = oracle.LogitsSampler(seed).select_next_token(host, ids, oracle.sampling(seed=seed, **kw))
+            assert got == want and got not in (3, 4, 5), (kw, seed)
 
 
 def test_sampled_stream_matches_oracle():
