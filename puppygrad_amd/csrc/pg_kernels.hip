@@ -508,12 +508,22 @@ __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t
   __shared__ float sv[16];
   __shared__ uint32_t si[16];
   Best b{-INFINITY, 0xffffffffu};
-  for (int i = threadIdx.x; i < n; i += 1024) {
-    float x = v[i];
-    if (x > b.v) {
-      b.v = x;
-      b.i = (uint32_t)i;
+  // eight loads in flight per thread (one per iteration would wait a memory round trip each
+  // time); a thread still visits its ids in ascending order, so the first maximum wins
+  constexpr int U = 8;
+  for (int i0 = threadIdx.x; i0 < n; i0 += 1024 * U) {
+    float x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + 1024 * u;
+      x[u] = i < n ? v[i] : -INFINITY;
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (x[u] > b.v) {
+        b.v = x[u];
+        b.i = (uint32_t)(i0 + 1024 * u);
+      }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
