@@ -1354,23 +1354,19 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
       PG_HIP(hipMemcpyAsync(c->d_recent, c->h_recent, recent * sizeof(uint32_t),
                             hipMemcpyHostToDevice, c->stream));
     }
-    uint32_t* d_ids = c->d_cand;
-    float* d_vals = reinterpret_cast<float*>(c->d_cand + kMaxCand);
-    uint32_t* d_count = c->d_cand + 2 * kMaxCand;
     PG_HIP(pgk::launch_topk_select(l->data + (size_t)row * l->vocab, (int)l->vocab, c->d_recent,
-                                   (int)recent, sampling->repeat_penalty, k, d_ids, d_vals, d_count,
-                                   c->stream));
-    // ids and values of the k slots that can be filled, and the count
-    PG_HIP(hipMemcpyAsync(c->h_cand, d_ids, (size_t)k * sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
-    PG_HIP(hipMemcpyAsync(c->h_cand + kMaxCand, d_vals, (size_t)k * sizeof(float), hipMemcpyDeviceToHost,
-                          c->stream));
-    PG_HIP(hipMemcpyAsync(c->h_cand + 2 * kMaxCand, d_count, sizeof(uint32_t), hipMemcpyDeviceToHost,
-                          c->stream));
+                                   (int)recent, sampling->repeat_penalty, k, c->d_cand, c->stream));
+    // the count and the k (id, logit) slots that can be filled, in one copy
+    PG_HIP(hipMemcpyAsync(c->h_cand, c->d_cand, (size_t)(1 + 2 * k) * sizeof(uint32_t),
+                          hipMemcpyDeviceToHost, c->stream));
     PG_HIP(hipStreamSynchronize(c->stream));
-    const uint32_t count = std::min<uint32_t>(c->h_cand[2 * kMaxCand], (uint32_t)k);
+    const uint32_t count = std::min<uint32_t>(c->h_cand[0], (uint32_t)k);
     std::vector<Candidate> cand(count);
-    const float* vals = reinterpret_cast<const float*>(c->h_cand + kMaxCand);
-    for (uint32_t i = 0; i < count; ++i) cand[i] = Candidate(c->h_cand[i], vals[i]);
+    for (uint32_t i = 0; i < count; ++i) {
+      float v;
+      std::memcpy(&v, &c->h_cand[2 + 2 * i], sizeof v);
+      cand[i] = Candidate(c->h_cand[1 + 2 * i], v);
+    }
     return sample_sorted(cand, *sampling, rng, out);
   }
   std::vector<float> adjusted(l->vocab);

@@ -83,11 +83,11 @@ int choose_nsplit(int n_keys, int H, int num_cus);
 hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, int rows = 1);
 // Candidates of sample_logits (src/models/generation.rs:281-315) for one row of V logits: the
 // repeat penalty over the n_pen recent ids, then the k first of the stable descending order
-// (unsorted: out_ids / out_vals hold them, out_count[0] their number).  V <= 480000.
-constexpr int kTopkMaxVocab = 480000;
+// (unsorted: out[0] = their number, then (id, logit bits) pairs; out holds 1 + 2 k words).
+// V <= 131072.
+constexpr int kTopkMaxVocab = 131072;
 hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
-                              float penalty, int k, uint32_t* out_ids, float* out_vals,
-                              uint32_t* out_count, hipStream_t s);
+                              float penalty, int k, uint32_t* out, hipStream_t s);
 // x[b] = wte[ids[b]] + wpe[pos]
 hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
                               int batch, int pos, int C, hipStream_t s, int w_bf16 = 0);

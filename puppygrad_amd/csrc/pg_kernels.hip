@@ -551,20 +551,26 @@ __global__ __launch_bounds__(1024) void k_argmax(const float* v, int n, uint32_t
 // recent id, negative logits multiplied, others divided), then a radix select over the
 // order-preserving integer image of the values finds the k-th largest key, and an ordered
 // compaction writes every candidate above it plus, among those equal to it, the lowest ids.
-// One block per call; out_count[0] = number of candidates (fewer than k when fewer are finite).
+// One block per call; out[0] = number of candidates (fewer than k when fewer are finite),
+// followed by that many (id, logit) pairs in no particular order.
 __device__ __forceinline__ unsigned order_key(float f) {  // total_cmp order, as unsigned
   int b = __float_as_int(f);
   b ^= (int)(((unsigned)(b >> 31)) >> 1);
   return (unsigned)b ^ 0x80000000u;
 }
+constexpr int kTopkRows = (kTopkMaxVocab + 1023) / 1024;  // ids are visited in rows of 1024
 __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V,
                                                       const uint32_t* pen_ids, int n_pen,
-                                                      float penalty, int k, uint32_t* out_ids,
-                                                      float* out_vals, uint32_t* out_count) {
+                                                      float penalty, int k, uint32_t* out) {
+  // out[0] = number of candidates, then (id, logit bits) pairs: one block to copy back
+  uint32_t* const out_count = out;
+  auto put = [&](unsigned at, int i, float v) {
+    out[1 + 2 * at] = (uint32_t)i;
+    out[2 + 2 * at] = __float_as_uint(v);
+  };
   extern __shared__ unsigned pen_bits[];  // one bit per id: among the recent ids
   __shared__ unsigned hist[256];
   __shared__ unsigned sh_prefix, sh_remaining, sh_total;
-  __shared__ unsigned wave_gt[16], wave_eq[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int words = (V + 31) / 32;
   for (int i = tid; i < words; i += 1024) pen_bits[i] = 0u;
@@ -575,16 +581,35 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
     if (id < (uint32_t)V) atomicOr(&pen_bits[id >> 5], 1u << (id & 31));
   }
   __syncthreads();
-  auto value = [&](int i) {
-    const float l = logits[i];
+  auto adjust = [&](int i, float l) {
     if (n_pen && ((pen_bits[i >> 5] >> (i & 31)) & 1u)) return l < 0.0f ? l * penalty : l / penalty;
     return l;
   };
   auto finite = [](float v) { return fabsf(v) <= 3.402823466e+38f; };  // false for NaN and inf
+  // One pass over the row: thread t visits ids t, t + 1024, ...; eight loads are in flight
+  // before the first is used.  f(i, key) sees the finite candidates only.
+  constexpr int U = 8;
+  auto for_each = [&](auto f) {
+    for (int i0 = tid; i0 < V; i0 += 1024 * U) {
+      float x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + 1024 * u;
+        x[u] = i < V ? logits[i] : INFINITY;  // (infinity: skipped below)
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + 1024 * u;
+        if (i >= V) break;
+        const float v = adjust(i, x[u]);
+        if (finite(v)) f(i, v);
+      }
+    }
+  };
   // finite candidates in all
   {
     unsigned c = 0;
-    for (int i = tid; i < V; i += 1024) c += finite(value(i)) ? 1u : 0u;
+    for_each([&](int, float) { ++c; });
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
     if (lane == 0) atomicAdd(&sh_total, c);
@@ -600,12 +625,10 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
   for (int shift = 24; shift >= 0; shift -= 8) {
     if (tid < 256) hist[tid] = 0u;
     __syncthreads();
-    for (int i = tid; i < V; i += 1024) {
-      const float v = value(i);
-      if (!finite(v)) continue;
+    for_each([&](int, float v) {
       const unsigned key = order_key(v);
       if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-    }
+    });
     __syncthreads();
     if (tid == 0) {
       unsigned remaining = sh_remaining, cum = 0u;
@@ -625,51 +648,83 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
   const unsigned T = prefix;            // key of the kk-th largest
   const unsigned need = sh_remaining;   // candidates equal to T that are kept: the lowest ids
   const unsigned n_gt = kk - need;
-  // ordered compaction: thread t owns ids [t * per, (t + 1) * per)
-  const int per = (V + 1023) / 1024;
-  const int i0 = tid * per, i1 = min(V, i0 + per);
-  unsigned c_gt = 0u, c_eq = 0u;
-  for (int i = i0; i < i1; ++i) {
-    const float v = value(i);
-    if (!finite(v)) continue;
-    const unsigned key = order_key(v);
-    c_gt += key > T ? 1u : 0u;
-    c_eq += key == T ? 1u : 0u;
-  }
-  // exclusive prefix sums over the block, in thread (= id) order
-  unsigned s_gt = c_gt, s_eq = c_eq;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const unsigned a = __shfl_up(s_gt, off, 64), b = __shfl_up(s_eq, off, 64);
-    if (lane >= off) {
-      s_gt += a;
-      s_eq += b;
+  // Ordered compaction.  Id order is (row, wavefront, lane) order; the rank of a candidate
+  // among those above T (or among those equal to T) is the sum of the counts of the
+  // (row, wavefront) cells before its own plus its rank inside its wavefront.
+  __shared__ unsigned short cell_gt[kTopkRows * 16], cell_eq[kTopkRows * 16];
+  __shared__ unsigned base_gt[kTopkRows * 16], base_eq[kTopkRows * 16];
+  const int rows = (V + 1023) / 1024;
+  for (int r = 0; r < rows; ++r) {
+    const int i = r * 1024 + tid;
+    bool gt = false, eq = false;
+    if (i < V) {
+      const float v = adjust(i, logits[i]);
+      if (finite(v)) {
+        const unsigned key = order_key(v);
+        gt = key > T;
+        eq = key == T;
+      }
+    }
+    const unsigned long long mg = __ballot(gt), me = __ballot(eq);
+    if (lane == 0) {
+      cell_gt[r * 16 + wave] = (unsigned short)__popcll(mg);
+      cell_eq[r * 16 + wave] = (unsigned short)__popcll(me);
     }
   }
-  if (lane == 63) {
-    wave_gt[wave] = s_gt;
-    wave_eq[wave] = s_eq;
+  __syncthreads();
+  {  // exclusive scans over the rows * 16 <= 2048 cells: two cells per thread
+    __shared__ unsigned wtot_gt[16], wtot_eq[16];
+    const int cells = rows * 16, c0 = 2 * tid, c1 = 2 * tid + 1;
+    const unsigned g0 = c0 < cells ? cell_gt[c0] : 0u, g1 = c1 < cells ? cell_gt[c1] : 0u;
+    const unsigned e0 = c0 < cells ? cell_eq[c0] : 0u, e1 = c1 < cells ? cell_eq[c1] : 0u;
+    unsigned sg = g0 + g1, se = e0 + e1;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned a = __shfl_up(sg, off, 64), b = __shfl_up(se, off, 64);
+      if (lane >= off) {
+        sg += a;
+        se += b;
+      }
+    }
+    if (lane == 63) {
+      wtot_gt[wave] = sg;
+      wtot_eq[wave] = se;
+    }
+    __syncthreads();
+    unsigned bg = sg - (g0 + g1), be = se - (e0 + e1);
+    for (int w = 0; w < wave; ++w) {
+      bg += wtot_gt[w];
+      be += wtot_eq[w];
+    }
+    if (c0 < cells) {
+      base_gt[c0] = bg;
+      base_eq[c0] = be;
+    }
+    if (c1 < cells) {
+      base_gt[c1] = bg + g0;
+      base_eq[c1] = be + e0;
+    }
   }
   __syncthreads();
-  unsigned base_gt = s_gt - c_gt, base_eq = s_eq - c_eq;
-  for (int w = 0; w < wave; ++w) {
-    base_gt += wave_gt[w];
-    base_eq += wave_eq[w];
-  }
-  for (int i = i0; i < i1; ++i) {
-    const float v = value(i);
-    if (!finite(v)) continue;
-    const unsigned key = order_key(v);
-    if (key > T) {
-      out_ids[base_gt] = (uint32_t)i;
-      out_vals[base_gt] = v;
-      ++base_gt;
-    } else if (key == T) {
-      if (base_eq < need) {
-        out_ids[n_gt + base_eq] = (uint32_t)i;
-        out_vals[n_gt + base_eq] = v;
+  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int r = 0; r < rows; ++r) {
+    const int i = r * 1024 + tid;
+    bool gt = false, eq = false;
+    float v = 0.0f;
+    if (i < V) {
+      v = adjust(i, logits[i]);
+      if (finite(v)) {
+        const unsigned key = order_key(v);
+        gt = key > T;
+        eq = key == T;
       }
-      ++base_eq;
+    }
+    const unsigned long long mg = __ballot(gt), me = __ballot(eq);
+    if (gt) {
+      put(base_gt[r * 16 + wave] + (unsigned)__popcll(mg & below), i, v);
+    } else if (eq) {
+      const unsigned rank = base_eq[r * 16 + wave] + (unsigned)__popcll(me & below);
+      if (rank < need) put(n_gt + rank, i, v);
     }
   }
 }
@@ -916,12 +971,11 @@ hipError_t launch_kv_append(const float* qkv, int batch, int C, int head_dim, in
 }
 
 hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
-                              float penalty, int k, uint32_t* out_ids, float* out_vals,
-                              uint32_t* out_count, hipStream_t s) {
+                              float penalty, int k, uint32_t* out, hipStream_t s) {
   const size_t lds = (size_t)((V + 31) / 32) * sizeof(unsigned);
-  if (V < 1 || k < 1 || lds > 60000 || n_pen < 0) return hipErrorInvalidValue;
+  if (V < 1 || V > kTopkMaxVocab || k < 1 || n_pen < 0) return hipErrorInvalidValue;
   hipLaunchKernelGGL(k_topk_select, dim3(1), dim3(1024), lds, s, logits, V, pen_ids, n_pen,
-                     penalty, k, out_ids, out_vals, out_count);
+                     penalty, k, out);
   return hipGetLastError();
 }
 
