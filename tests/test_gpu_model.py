@@ -408,3 +408,52 @@ def test_config1_gpt2_small_greedy_decode_parity():
         model.prefill(ids, cache)
         again, _ = model.decode_greedy(cache, 128)
         assert again == got
+
+
+def test_config2_gpt2_small_full_context_prefill_parity():
+    """Benchmark configuration 2: 124M, one prompt of 1024 ids (the whole context) through the
+    MFMA GEMM path and the full causal attention; final-position logits and the cache it
+    leaves against the oracle's token-by-token prefill (rust.rs:906-927)."""
+    cfg = synth.Gpt2Config(**synth.GPT2_SMALL)
+    w = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 2)
+    ids = list(synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(16))
+    cache, rcache = model.new_kv_cache(), ref.new_kv_cache()
+    want = ref.prefill(ids, rcache)
+    got = model.prefill(ids, cache)
+    assert_logits_close(got.to_host(), want)
+    assert model.select_next_token(got) == oracle.argmax_logits(want) or \
+        np.diff(np.sort(want)[-2:])[0] <= 2 * (ABS_TOL + REL_TOL * abs(float(want.max())))
+    assert cache.seq_len == 1024 == cache.max_seq_len
+    for layer in (0, cfg.n_layer - 1):
+        for which in (0, 1):
+            np.testing.assert_allclose(cache.read_layer(layer, which), rcache.read_layer(layer, which),
+                                       atol=2e-5, rtol=1e-4)
+    # the context is used up (rust.rs:957-961)
+    with pytest.raises(Gpt2Error, match="cache is full at seq_len 1024"):
+        model.forward_one(1, cache)
+    # prefill clears the cache first (rust.rs:913): a second prompt starts from position 0
+    short = ids[:40]
+    assert_logits_close(model.prefill(short, cache).to_host(), ref.prefill(short, rcache))
+    assert cache.seq_len == 40
+
+
+def test_config4_gpt2_xl_long_context_greedy_decode_parity():
+    """Benchmark configuration 4, the headline workload: XL, cache prefilled with 896 ids, 128
+    greedy tokens at positions 896..1022 (the context ends exactly there).  Logits of every
+    step against the oracle with its tokens teacher-forced, then the fused on-device loop."""
+    cfg = synth.Gpt2Config(**synth.GPT2_XL)
+    w = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 4)
+    ids = list(synth.token_ids(896, synth.TOKEN_SEED_BASE + 4, cfg.vocab_size))
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(16))
+    assert "decode=persistent" in model.describe()
+    steps, explained, unexplained, want = greedy_with_teacher_forcing(model, ref, ids, 128)
+    assert steps == 128 and unexplained == 0
+    assert len(want) == 1024  # stopped by the context limit, not short of it
+    cache = model.new_kv_cache()
+    model.prefill(ids, cache)
+    got, stats = model.decode_greedy(cache, 128)
+    assert stats.generated_tokens == 128 and len(got) == 128
+    if explained == 0:
+        assert got == want[896:]
+    assert cache.seq_len == 896 + 127  # the forward after the last token is skipped
