@@ -238,6 +238,37 @@ pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* model, const 
                                               pg_on_token on_token, void* user, uint32_t* out_ids,
                                               size_t* out_n, pg_generation_stats* stats);
 
+/* Gpt2OperationProfile (src/models/gpt2/rust.rs:336-347) in seconds, accumulated over the
+ * prefill and the decode steps of one generation as forward_one_profiled and
+ * prefill_profiled do (rust.rs:906-1006, 1136-1250).  The spans are measured with HIP
+ * events between the launches of the per-operation decode path.  On this backend a
+ * LayerNorm runs inside the launch of the projection that consumes it, so its time is
+ * part of that projection's bucket and layer_norm_s stays 0; tokenization_s and
+ * decoding_s are tokenizer work (rust.rs:473-478, 651), 0 for streams of token ids. */
+typedef struct pg_gpt2_operation_profile {
+  double tokenization_s;
+  double layer_norm_s;
+  double qkv_projection_s;
+  double attention_s;
+  double attention_projection_s;
+  double mlp_fc_projection_s;
+  double mlp_projection_s;
+  double final_logits_s;
+  double decoding_s;
+} pg_gpt2_operation_profile;
+
+/* pg_gpt2_stream_token_ids_with_stats with every forward (the prompt's included, token by
+ * token as prefill_profiled does) run as separate launches per operation and timed into
+ * `profile` (must not be NULL).  Tokens are the same as the unprofiled stream's; the
+ * wall-clock fields of `stats` include the per-step synchronisation the timing needs, so
+ * throughput is quoted from the unprofiled call. */
+pg_status pg_gpt2_stream_token_ids_profiled(const pg_gpt2_model* model, const uint32_t* ids,
+                                            size_t n, uint32_t max_new, int64_t eos,
+                                            const pg_sampling* sampling, uint64_t seed,
+                                            pg_on_token on_token, void* user, uint32_t* out_ids,
+                                            size_t* out_n, pg_generation_stats* stats,
+                                            pg_gpt2_operation_profile* profile);
+
 /* Op-level entry points with the semantics of src/models/cpu.rs; operands are
  * host pointers, the work runs on `device`.  They exist for kernel parity tests
  * and as the seam for other models that share these kernels. */

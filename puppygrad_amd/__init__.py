@@ -5,10 +5,10 @@ package is its Python host-side mirror, used by the tests and the benchmark.
 """
 from .gpt2 import (GPT2_EOS_TOKEN_ID, DeviceLogits, GenerationStats, Gpt2BlockWeights, Gpt2Config,
                    Gpt2Error, Gpt2GenerationConfig, Gpt2HipConfig, Gpt2KvCache, Gpt2Model,
-                   Gpt2Output, Gpt2Weights, LogitsSampler, TensorStore, TextGenerationConfig,
+                   Gpt2OperationProfile, Gpt2Output, Gpt2Weights, LogitsSampler, TensorStore, TextGenerationConfig,
                    argmax_logits, generate, load_weights)
 
 __all__ = ["GPT2_EOS_TOKEN_ID", "DeviceLogits", "GenerationStats", "Gpt2BlockWeights",
            "Gpt2Config", "Gpt2Error", "Gpt2GenerationConfig", "Gpt2HipConfig", "Gpt2KvCache",
-           "Gpt2Model", "Gpt2Output", "Gpt2Weights", "LogitsSampler", "TensorStore",
+           "Gpt2Model", "Gpt2OperationProfile", "Gpt2Output", "Gpt2Weights", "LogitsSampler", "TensorStore",
            "TextGenerationConfig", "argmax_logits", "generate", "load_weights"]

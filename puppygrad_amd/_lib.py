@@ -61,6 +61,13 @@ class pg_generation_stats(C.Structure):
                 ("first_token_s", C.c_double), ("gpu_decode_s", C.c_double)]
 
 
+class pg_gpt2_operation_profile(C.Structure):
+    _fields_ = [(name, C.c_double) for name in (
+        "tokenization_s", "layer_norm_s", "qkv_projection_s", "attention_s",
+        "attention_projection_s", "mlp_fc_projection_s", "mlp_projection_s", "final_logits_s",
+        "decoding_s")]
+
+
 class pg_device_info(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_uint32),
                 ("total_mem_bytes", C.c_uint64), ("lds_bytes_per_block", C.c_uint32)]
@@ -113,6 +120,12 @@ SIGNATURES = {
                                                       C.c_uint64, ON_TOKEN, _vp, _u32p,
                                                       C.POINTER(C.c_size_t),
                                                       C.POINTER(pg_generation_stats)]),
+    "pg_gpt2_stream_token_ids_profiled": (C.c_int, [_vp, _u32p, C.c_size_t, C.c_uint32,
+                                                    C.c_int64, C.POINTER(pg_sampling),
+                                                    C.c_uint64, ON_TOKEN, _vp, _u32p,
+                                                    C.POINTER(C.c_size_t),
+                                                    C.POINTER(pg_generation_stats),
+                                                    C.POINTER(pg_gpt2_operation_profile)]),
     "pg_op_dense": (C.c_int, [C.c_int32, _f32p, C.c_uint64, C.c_uint64, C.c_uint64, _f32p, _f32p,
                               _f32p]),
     "pg_op_layer_norm": (C.c_int, [C.c_int32, _f32p, C.c_uint64, C.c_uint64, _f32p, _f32p,

@@ -268,9 +268,57 @@ pg_status check_compatible(const pg_gpt2_model* m, const pg_kv_cache* c) {
 // launches on the cache's stream.  The token comes from tok_ptr (device) when
 // it is non-null.  With want_logits false the final LayerNorm and lm_head are
 // skipped (prefill discards those logits, rust.rs:922-926).
+// Time stamps between the launches of one step, for the buckets of Gpt2OperationProfile
+// (src/models/gpt2/rust.rs:336-347): an event is recorded on the step's stream after each
+// operation; the span since the previous event belongs to that operation's bucket.
+struct ProfileMarks {
+  enum Bucket { kNone, kQkv, kAttention, kAttnProj, kMlpFc, kMlpProj, kLogits };
+  std::vector<hipEvent_t> events;
+  std::vector<Bucket> bucket;
+  size_t used = 0;
+  hipError_t mark(hipStream_t s, Bucket b) {
+    if (used == events.size()) {
+      hipEvent_t e = nullptr;
+      hipError_t r = hipEventCreate(&e);
+      if (r != hipSuccess) return r;
+      events.push_back(e);
+      bucket.push_back(kNone);
+    }
+    bucket[used] = b;
+    return hipEventRecord(events[used++], s);
+  }
+  // Adds the spans of the step just synchronised to `p` and rewinds.
+  hipError_t collect(pg_gpt2_operation_profile* p) {
+    for (size_t i = 1; i < used; ++i) {
+      float ms = 0.0f;
+      hipError_t r = hipEventElapsedTime(&ms, events[i - 1], events[i]);
+      if (r != hipSuccess) return r;
+      const double sec = (double)ms * 1e-3;
+      switch (bucket[i]) {
+        case kQkv: p->qkv_projection_s += sec; break;
+        case kAttention: p->attention_s += sec; break;
+        case kAttnProj: p->attention_projection_s += sec; break;
+        case kMlpFc: p->mlp_fc_projection_s += sec; break;
+        case kMlpProj: p->mlp_projection_s += sec; break;
+        case kLogits: p->final_logits_s += sec; break;
+        case kNone: break;
+      }
+    }
+    used = 0;
+    return hipSuccess;
+  }
+  ~ProfileMarks() {
+    for (hipEvent_t e : events) (void)hipEventDestroy(e);
+  }
+};
+#define PG_MARK(b) \
+  do {             \
+    if (marks) PG_HIP(marks->mark(s, ProfileMarks::b)); \
+  } while (0)
+
 pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
                               const uint32_t* tok_ptr, uint32_t tok, size_t pos,
-                              bool want_logits) {
+                              bool want_logits, ProfileMarks* marks = nullptr) {
   const Cfg& g = m->cfg;
   const int C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
   hipStream_t s = c->stream;
@@ -284,6 +332,7 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
   const int nsplit = hd == pgk::kHeadDim ? pgk::choose_nsplit((int)pos + 1, H, m->num_cus) : 1;
 
   PG_HIP(pgk::launch_embed(x, m->wte, m->wpe, tok_ptr, tok, (int)pos, C, s, m->w_bf16));
+  PG_MARK(kNone);  // the embedding is in no bucket (rust.rs:966-974)
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
     pgk::GemvArgs a{};
@@ -293,9 +342,11 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     a.kcache = c->k_panel(l, b); a.vcache = c->v_panel(l, b);
     a.pos = (int)pos; a.P = P; a.C = C; a.head_dim = hd;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_QKV, s));
+    PG_MARK(kQkv);
     // attention over keys [0, pos]
     PG_HIP(pgk::launch_attn_decode(q, c->k_panel(l, b), c->v_panel(l, b), (int)pos, P, H, hd,
                                    nsplit, pa, pm, pl, s));
+    if (!(nsplit > 2 && hd == pgk::kHeadDim)) PG_MARK(kAttention);
     // merge splits + c_proj + residual.  Every block of the projection repeats the merge in
     // its prologue, which is cheap for a few splits; beyond that the merge gets a launch of
     // its own (into q, which the attention has finished reading).
@@ -303,31 +354,37 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
     a.w_bf16 = m->w_bf16; a.W = w.c_proj_w; a.w_scale = w.c_proj_s; a.bias = w.c_proj_b; a.y = x; a.resid = x; a.K = C; a.nout = C;
     if (nsplit > 2 && hd == pgk::kHeadDim) {
       PG_HIP(pgk::launch_attn_finish(pa, pm, pl, H, hd, nsplit, q, s));
+      PG_MARK(kAttention);
       a.x = q;
       PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
     } else {
       a.part_acc = pa; a.part_m = pm; a.part_l = pl; a.nsplit = nsplit; a.head_dim = hd;
       PG_HIP(pgk::launch_gemv(a, pgk::PRO_ATTN_COMBINE, pgk::EPI_RESID, s));
     }
+    PG_MARK(kAttnProj);
     // LN2 + c_fc + GELU
     a = pgk::GemvArgs{};
     a.w_bf16 = m->w_bf16; a.W = w.c_fc_w; a.w_scale = w.c_fc_s; a.bias = w.c_fc_b; a.x = x; a.y = hb; a.K = C; a.nout = I;
     a.ln_g = w.ln_2_g; a.ln_b = w.ln_2_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_GELU, s));
+    PG_MARK(kMlpFc);
     // mlp c_proj + residual
     a = pgk::GemvArgs{};
     a.w_bf16 = m->w_bf16; a.W = w.c_proj_mlp_w; a.w_scale = w.c_proj_mlp_s; a.bias = w.c_proj_mlp_b; a.x = hb; a.y = x; a.resid = x; a.K = I;
     a.nout = C;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_RESID, s));
+    PG_MARK(kMlpProj);
   }
   if (want_logits) {
     pgk::GemvArgs a{};
     a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = x; a.y = c->logits_buf + b * g.V; a.K = C;
     a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
     PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+    PG_MARK(kLogits);
   }
   return PG_OK;
 }
+#undef PG_MARK
 
 // The tagged activation words live in uncached device memory: a word written by one
 // workgroup is read by workgroups on other dies, and without a cache level that has to be
@@ -1499,13 +1556,34 @@ pg_status pg_gpt2_decode_greedy(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t
   return PG_OK;
 }
 
-pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint32_t* ids,
-                                              size_t n, uint32_t max_new, int64_t eos,
-                                              const pg_sampling* sampling, uint64_t seed,
-                                              pg_on_token on_token, void* user, uint32_t* out_ids,
-                                              size_t* out_n, pg_generation_stats* stats) {
+// One forward of the per-operation path with its spans added to `profile`
+// (forward_one_profiled_with_scratch, src/models/gpt2/rust.rs:943-1006).
+static pg_status forward_one_profiled(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t id,
+                                      bool want_logits, ProfileMarks* marks,
+                                      pg_gpt2_operation_profile* profile, pg_logits** out) {
+  pg_status s;
+  if ((s = check_compatible(m, c))) return s;
+  if (id >= m->cfg.V)  // rust.rs:951-956
+    return fail(PG_INVALID_INPUT, "token id " + std::to_string(id) + " exceeds vocab_size " +
+                                      std::to_string(m->cfg.V));
+  if ((s = check_step(m, c))) return s;
+  if ((s = select_device(m->device))) return s;
+  if ((s = enqueue_forward_one(m, c, 0, nullptr, id, c->seq_len, want_logits, marks))) return s;
+  PG_HIP(hipStreamSynchronize(c->stream));
+  PG_HIP(marks->collect(profile));
+  c->seq_len += 1;  // rust.rs:1004
+  return want_logits ? finish_logits(c, out) : PG_OK;
+}
+
+static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t n,
+                             uint32_t max_new, int64_t eos, const pg_sampling* sampling,
+                             uint64_t seed, pg_on_token on_token, void* user, uint32_t* out_ids,
+                             size_t* out_n, pg_generation_stats* stats,
+                             pg_gpt2_operation_profile* profile) {
   if (!m || !sampling || !out_ids || !out_n) return fail(PG_INVALID_INPUT, "null argument");
   pg_status s;
+  ProfileMarks marks;
+  if (profile) *profile = pg_gpt2_operation_profile{};
   if ((s = pg_sampling_validate(sampling))) return s;
   if (eos >= 0 && (uint64_t)eos >= m->cfg.V)  // rust.rs:558-566
     return fail(PG_INVALID_CONFIG, "generation eos_token_id " + std::to_string(eos) +
@@ -1516,7 +1594,16 @@ pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint
   auto first_start = Clock::now();
   auto prefill_start = Clock::now();
   pg_logits* logits = nullptr;
-  if ((s = pg_gpt2_prefill(m, c, ids, n, &logits))) return s;
+  if (profile) {
+    // prefill_profiled (rust.rs:906-927): the checks of prefill, then the prompt token by
+    // token, logits from the last one
+    if ((s = validate_input(m->cfg, ids, n))) return s;
+    if ((s = pg_kv_cache_clear(c))) return s;
+    for (size_t i = 0; i < n; ++i)
+      if ((s = forward_one_profiled(m, c, ids[i], i + 1 == n, &marks, profile, &logits))) return s;
+  } else if ((s = pg_gpt2_prefill(m, c, ids, n, &logits))) {
+    return s;
+  }
   double prefill_s = since(prefill_start);
   std::vector<uint32_t> output(ids, ids + n);
   auto decode_start = Clock::now();
@@ -1536,8 +1623,13 @@ pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint
     generated += 1;
     if (first_token_s < 0) first_token_s = since(first_start);
     bool needs_next = generated < max_new && output.size() < m->cfg.P;
-    if (needs_next)
-      if ((s = pg_gpt2_forward_one(m, c, tok, &logits))) return s;
+    if (needs_next) {
+      if (profile)
+        s = forward_one_profiled(m, c, tok, true, &marks, profile, &logits);
+      else
+        s = pg_gpt2_forward_one(m, c, tok, &logits);
+      if (s) return s;
+    }
   }
   double decode_s = since(decode_start);
   std::memcpy(out_ids, output.data(), output.size() * sizeof(uint32_t));
@@ -1551,6 +1643,26 @@ pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint
     stats->gpu_decode_s = 0.0;
   }
   return PG_OK;
+}
+
+pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* m, const uint32_t* ids,
+                                              size_t n, uint32_t max_new, int64_t eos,
+                                              const pg_sampling* sampling, uint64_t seed,
+                                              pg_on_token on_token, void* user, uint32_t* out_ids,
+                                              size_t* out_n, pg_generation_stats* stats) {
+  return stream_core(m, ids, n, max_new, eos, sampling, seed, on_token, user, out_ids, out_n,
+                     stats, nullptr);
+}
+
+pg_status pg_gpt2_stream_token_ids_profiled(const pg_gpt2_model* m, const uint32_t* ids,
+                                            size_t n, uint32_t max_new, int64_t eos,
+                                            const pg_sampling* sampling, uint64_t seed,
+                                            pg_on_token on_token, void* user, uint32_t* out_ids,
+                                            size_t* out_n, pg_generation_stats* stats,
+                                            pg_gpt2_operation_profile* profile) {
+  if (!profile) return fail(PG_INVALID_INPUT, "null argument");
+  return stream_core(m, ids, n, max_new, eos, sampling, seed, on_token, user, out_ids, out_n,
+                     stats, profile);
 }
 
 // ---- op-level entry points ---------------------------------------------------

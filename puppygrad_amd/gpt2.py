@@ -261,6 +261,21 @@ def Gpt2GenerationConfig(max_new_tokens: int) -> TextGenerationConfig:
 
 
 @dataclass
+class Gpt2OperationProfile:
+    """Gpt2OperationProfile (src/models/gpt2/rust.rs:336-347), seconds per bucket.  LayerNorm
+    runs inside the projection that consumes it on this backend: its bucket stays 0."""
+    tokenization: float = 0.0
+    layer_norm: float = 0.0
+    qkv_projection: float = 0.0
+    attention: float = 0.0
+    attention_projection: float = 0.0
+    mlp_fc_projection: float = 0.0
+    mlp_projection: float = 0.0
+    final_logits: float = 0.0
+    decoding: float = 0.0
+
+
+@dataclass
 class GenerationStats:
     """GenerationStats (src/models/generation.rs:129-180)."""
     prompt_tokens: int = 0
@@ -508,9 +523,11 @@ class Gpt2Model:
 
     def stream_token_ids_with_stats(self, input_ids: Sequence[int],
                                     generation: TextGenerationConfig,
-                                    on_token: Optional[Callable[[int], None]] = None):
+                                    on_token: Optional[Callable[[int], None]] = None,
+                                    profiled: bool = False):
         """Gpt2Runtime::stream_token_ids_with_stats with ids in place of a prompt
-        string (rust.rs:548-634)."""
+        string (rust.rs:548-634).  With profiled=True every forward runs as one launch per
+        operation, timed into a Gpt2OperationProfile, and a third value is returned."""
         ids = _u32(input_ids)
         out = np.empty(ids.size + generation.max_new_tokens + 1, dtype=np.uint32)
         n = C.c_size_t()
@@ -528,14 +545,22 @@ class Gpt2Model:
                 return 1
 
         cb = _lib.ON_TOKEN(_cb)
-        status = _lib.load().pg_gpt2_stream_token_ids_with_stats(
-            self._h, _lib.u32p(ids), ids.size, generation.max_new_tokens,
-            -1 if generation.eos_token_id is None else generation.eos_token_id, C.byref(samp),
-            generation.seed, cb, None, _lib.u32p(out), C.byref(n), C.byref(st))
+        args = (self._h, _lib.u32p(ids), ids.size, generation.max_new_tokens,
+                -1 if generation.eos_token_id is None else generation.eos_token_id, C.byref(samp),
+                generation.seed, cb, None, _lib.u32p(out), C.byref(n), C.byref(st))
+        prof = _lib.pg_gpt2_operation_profile()
+        if profiled:
+            status = _lib.load().pg_gpt2_stream_token_ids_profiled(*args, C.byref(prof))
+        else:
+            status = _lib.load().pg_gpt2_stream_token_ids_with_stats(*args)
         if err:
             raise err[0]
         _check(status)
-        return [int(t) for t in out[:n.value]], _stats(st)
+        tokens = [int(t) for t in out[:n.value]]
+        if profiled:
+            return tokens, _stats(st), Gpt2OperationProfile(
+                **{f[0][:-2]: getattr(prof, f[0]) for f in prof._fields_})
+        return tokens, _stats(st)
 
 
 def _stats(st: _lib.pg_generation_stats) -> GenerationStats:
