@@ -5,6 +5,9 @@ prefilled to 896 tokens (the configuration the headline metric is quoted on), on
 A step is one cached decoder forward (one token).  The timed region holds
 weights, KV cache and the first logits resident in HBM; token selection
 (argmax) runs on the device and only the ids return to the host afterwards.
+The same invocation then measures the other configurations the metric names (124M batch-1
+decode, 124M full-context prefill, 355M batch-16 and XL bf16 batch-32 decode steps) and reports
+them under "secondary", each with the roofline of its own bound.
 Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this path runs on one GPU.
 """
 from __future__ import annotations
@@ -59,6 +62,8 @@ def main() -> int:
     ap.add_argument("--model", default="xl", choices=["xl", "large", "medium", "small"])
     ap.add_argument("--prefill", type=int, default=None, help="tokens in the cache before decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the other configurations (they run only beside the default workload)")
     ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "batch-decode"],
                     help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound); "
@@ -106,60 +111,11 @@ def main() -> int:
     if args.workload == "batch-decode":
         return bench_batch_decode(args, cfg, model, n_prefill)
 
-    cache = model.new_kv_cache()
-    t0 = time.time()
-    model.prefill(ids, cache)
-    prefill_s = time.time() - t0
-    log(f"[bench] prefill {n_prefill} tokens: {prefill_s:.2f}s")
-
-    def rewind():
-        """Back to the prefilled state with valid logits (one untimed forward)."""
-        cache.seq_len = n_prefill - 1
-        model.forward_one(int(ids[-1]), cache)
-
-    # warmup
-    done = 0
-    while done < args.warmup:
-        n = min(args.warmup - done, room - 1)
-        model.decode_greedy(cache, n + 1)
-        done += n
-        rewind()
-
-    # timed: K forwards in passes of at most room-1 forwards (room tokens)
-    steps_left = args.steps
-    wall = gpu = 0.0
-    tokens = 0
-    kv_total = 0
-    launches = 0
-    while steps_left > 0:
-        n = min(steps_left, room - 1)
-        start = cache.seq_len
-        toks, st = model.decode_greedy(cache, n + 1)  # n+1 tokens selected, n forwards
-        assert len(toks) == n + 1 and cache.seq_len == start + n
-        wall += st.decode_time
-        gpu += st.gpu_decode_time
-        tokens += n + 1
-        kv_total += sum(kv_bytes(cfg, p) for p in range(start, start + n))
-        steps_left -= n
-        launches += 1
-        if steps_left > 0:
-            rewind()
-    K = args.steps
-    ms_per_step = wall / K * 1e3
-    gpu_ms_per_step = gpu / K * 1e3
-    tok_s = K / wall  # forwards per second; the reference's tokens/sec adds the free last token
-    # Roofline of the dominant kernel.  On the persistent path one launch of
-    # k_decode_persistent<n_embd> runs every forward of a pass (embedding, all blocks,
-    # lm_head, argmax); its duration is the HIP-event time the library takes on the
-    # launch stream (gpu_decode_time).  Algorithmic bytes: the parameters once per
-    # forward plus the K/V rows of positions [0, pos] that forward attends over.
-    algo_bytes = weight_bytes(cfg, args.int8, args.bf16) + kv_total / K  # per forward
-    bytes_per_launch = algo_bytes * K / launches
-    launch_s = gpu / launches
-    achieved = bytes_per_launch / launch_s / 1e9
-    persistent = "decode=persistent" in model.describe()
-    kernel = (f"k_decode_persistent<{cfg.n_embd}{', int8 rows' if args.int8 else ', bf16 rows' if args.bf16 else ''}>" if persistent
-              else "all launches of one decode step (k_gemv dominant)")
+    d = measure_decode(model, cfg, ids, n_prefill, args.steps, args.warmup, args.int8, args.bf16)
+    K, room, launches = args.steps, d["room"], d["launches"]
+    ms_per_step, gpu_ms_per_step, tok_s, prefill_s = d["ms_per_step"], d["gpu_ms_per_step"], d["tok_s"], d["prefill_s"]
+    tokens, wall, achieved, launch_s = d["tokens"], d["wall"], d["achieved"], d["launch_s"]
+    bytes_per_launch, algo_bytes, persistent, kernel = d["bytes_per_launch"], d["algo_bytes"], d["persistent"], d["kernel"]
 
     info = _lib.pg_device_info()
     _lib.load().pg_device_query(0, C.byref(info))
@@ -184,6 +140,7 @@ def main() -> int:
                                f"B=1 greedy decode, KV cache prefilled to "
                                f"{n_prefill} tokens, positions {n_prefill}..{n_prefill + min(K, room - 1) - 1}",
                    "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
+                   "weight_storage": "int8" if args.int8 else "bf16" if args.bf16 else "f32",
                    "device": info.name.decode() or info.arch.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "backend": model.describe()},
         "reference_metric_tokens_per_s": round(tokens / wall, 2),
@@ -191,13 +148,20 @@ def main() -> int:
         "prefill_s": round(prefill_s, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic(args, n_prefill, persistent, launches),
+                     "traffic": measured_traffic(args, n_prefill, persistent, bytes_per_launch),
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel": kernel, "launches": launches,
                      "forwards_per_launch": K // launches,
                      "launch_ms": round(launch_s * 1e3, 3),
                      "algorithmic_bytes_per_launch": int(bytes_per_launch),
                      "algorithmic_bytes_per_forward": int(algo_bytes)},
     }
+
+    default_workload = (args.model == "xl" and args.prefill is None and args.decode_path == "auto"
+                        and not args.int8 and not args.bf16)
+    if default_workload and not args.no_secondary:
+        del model
+        result["secondary"] = secondary_workloads(cfg, weights)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, synth.bf16_rounded(weights) if args.bf16 else weights,
@@ -208,6 +172,165 @@ def main() -> int:
 
 
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+
+
+def measure_decode(model, cfg, ids, n_prefill, steps, warmup, int8=False, bf16=False):
+    """Batch-1 greedy decode from a cache prefilled with `ids`: `steps` forwards in passes that
+    end at the context limit.  Returns the timings and the HBM roofline figures of the pass."""
+    room = cfg.n_positions - n_prefill  # tokens one pass can generate
+    cache = model.new_kv_cache()
+    t0 = time.time()
+    model.prefill(ids, cache)
+    prefill_s = time.time() - t0
+    log(f"[bench] prefill {n_prefill} tokens: {prefill_s:.2f}s")
+
+    def rewind():
+        """Back to the prefilled state with valid logits (one untimed forward)."""
+        cache.seq_len = n_prefill - 1
+        model.forward_one(int(ids[-1]), cache)
+
+    done = 0
+    while done < warmup:
+        n = min(warmup - done, room - 1)
+        model.decode_greedy(cache, n + 1)
+        done += n
+        rewind()
+
+    # timed: K forwards in passes of at most room-1 forwards (room tokens)
+    steps_left = steps
+    wall = gpu = 0.0
+    tokens = 0
+    kv_total = 0
+    launches = 0
+    while steps_left > 0:
+        n = min(steps_left, room - 1)
+        start = cache.seq_len
+        toks, st = model.decode_greedy(cache, n + 1)  # n+1 tokens selected, n forwards
+        assert len(toks) == n + 1 and cache.seq_len == start + n
+        wall += st.decode_time
+        gpu += st.gpu_decode_time
+        tokens += n + 1
+        kv_total += sum(kv_bytes(cfg, p) for p in range(start, start + n))
+        steps_left -= n
+        launches += 1
+        if steps_left > 0:
+            rewind()
+    K = steps
+    # Roofline of the dominant kernel.  On the persistent path one launch of
+    # k_decode_persistent<n_embd> runs every forward of a pass (embedding, all blocks,
+    # lm_head, argmax); its duration is the HIP-event time the library takes on the
+    # launch stream (gpu_decode_time).  Algorithmic bytes: the parameters once per
+    # forward plus the K/V rows of positions [0, pos] that forward attends over.
+    algo_bytes = weight_bytes(cfg, int8, bf16) + kv_total / K  # per forward
+    bytes_per_launch = algo_bytes * K / launches
+    launch_s = gpu / launches
+    persistent = "decode=persistent" in model.describe()
+    kernel = (f"k_decode_persistent<{cfg.n_embd}{', int8 rows' if int8 else ', bf16 rows' if bf16 else ''}>" if persistent
+              else "all launches of one decode step (k_gemv dominant)")
+    return {"room": room, "launches": launches, "ms_per_step": wall / K * 1e3, "gpu_ms_per_step": gpu / K * 1e3,
+            "tok_s": K / wall,  # forwards per second; the reference's tokens/sec adds the free last token
+            "prefill_s": prefill_s, "tokens": tokens, "wall": wall,
+            "achieved": bytes_per_launch / launch_s / 1e9, "launch_s": launch_s,
+            "bytes_per_launch": bytes_per_launch, "algo_bytes": algo_bytes, "persistent": persistent, "kernel": kernel}
+
+
+def hbm_roofline(achieved_gbs, kernel, **extra):
+    return {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel, **extra}
+
+
+def secondary_workloads(xl_cfg, xl_weights):
+    """The other configurations of the metric, measured in this same process: small fixed
+    step counts, inputs resident, each with the roofline of its own bound."""
+    from puppygrad_amd import Gpt2Config, Gpt2HipConfig, Gpt2Model, _lib, synth
+    out = {}
+    # GPT-2 124M: batch-1 decode of 96 tokens from a 32-token prompt, and the 1024-token prefill
+    cfg = Gpt2Config(**synth.GPT2_SMALL)
+    w = synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 1)
+    model = Gpt2Model.new(cfg, w)
+    ids = synth.token_ids(32, synth.TOKEN_SEED_BASE + 1, cfg.vocab_size)
+    d = measure_decode(model, cfg, ids, 32, 96, 8)
+    out["gpt2_124m_decode_b1"] = {
+        "workload": "GPT-2 small 124M fp32 B=1 greedy decode, KV cache prefilled to 32 tokens, positions 32..127",
+        "value": round(d["tok_s"], 1), "unit": "tokens/s", "steps": 96, "ms_per_step": round(d["ms_per_step"], 4),
+        "gpu_ms_per_step": round(d["gpu_ms_per_step"], 4),
+        "reference_metric_tokens_per_s": round(d["tokens"] / d["wall"], 1),
+        "roofline": hbm_roofline(d["achieved"], d["kernel"], launches=d["launches"],
+                                 launch_ms=round(d["launch_s"] * 1e3, 3),
+                                 algorithmic_bytes_per_forward=int(d["algo_bytes"]))}
+    ids = synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size)
+    out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 10, 2)
+    del model, w
+    # GPT-2 355M: batch-16 decode steps from 128-token prompts
+    cfg = Gpt2Config(**synth.GPT2_MEDIUM)
+    model = Gpt2Model.new(cfg, synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 3))
+    out["gpt2_355m_decode_b16"] = measure_batch_decode(model, cfg, 16, 128, 64, False)
+    del model
+    # GPT-2 XL with bf16-stored weights: batch-32 decode steps from 512-token prompts
+    model = Gpt2Model.new(xl_cfg, xl_weights, Gpt2HipConfig(weight_storage=_lib.PG_STORE_BF16))
+    out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 512, 24, True)
+    del model
+    return out
+
+
+def measure_prefill(model, cfg, ids, T, steps, warmup):
+    """One prefill of T tokens into an empty cache through the full-sequence path, MFMA-bound:
+    wall time over `steps` runs for the whole prefill, and one profiled run (HIP events between
+    the launches) for the share of the four projections."""
+    C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    gemm_flops = 2.0 * T * L * (3 * C_ * C_ + C_ * C_ + 2 * C_ * I)
+    attn_flops = 4.0 * C_ * (T * (T + 1) / 2) * L
+    flops = gemm_flops + attn_flops + 2.0 * V * C_
+    cache = model.new_kv_cache()
+    for _ in range(max(1, warmup)):
+        model.prefill(ids, cache).argmax()
+    t0 = time.time()
+    for _ in range(steps):
+        lg = model.prefill(ids, cache)
+    lg.argmax()
+    sec = (time.time() - t0) / steps
+    _, prof = model.prefill_profiled(ids, cache)
+    gemm_s = prof.qkv_projection + prof.attention_projection + prof.mlp_fc_projection + prof.mlp_projection
+    whole = flops / sec / 1e12
+    gemm = gemm_flops / gemm_s / 1e12 if gemm_s > 0 else 0.0
+    attn = attn_flops / prof.attention / 1e12 if prof.attention > 0 else 0.0
+    return {"workload": f"GPT-2 124M fp32 B=1 prefill of {T} tokens into an empty KV cache, final-position logits",
+            "value": round(T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 4),
+            "roofline": {"bound": "mfma", "achieved": round(whole, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(whole / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                         "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
+                         "algorithmic_flops_per_step": int(flops)},
+            "gemm_part": {"ms": round(gemm_s * 1e3, 4), "achieved": round(gemm, 2), "unit": "TFLOP/s",
+                          "frac": round(gemm / FP32_MFMA_PEAK_TFLOPS, 4), "flops": int(gemm_flops),
+                          "how": "HIP events between the launches of one profiled prefill: the four "
+                                 "projections of every layer with their split-K reduces and fused LayerNorms"},
+            "attention_part": {"ms": round(prof.attention * 1e3, 4), "achieved": round(attn, 2), "unit": "TFLOP/s",
+                               "frac": round(attn / FP32_MFMA_PEAK_TFLOPS, 4), "flops": int(attn_flops)}}
+
+
+def measure_batch_decode(model, cfg, B, n_prefill, steps, bf16):
+    """B sequences prefilled to n_prefill tokens each, then `steps` greedy steps for all of them.
+    A step reads every weight once plus the K/V rows of every sequence: HBM-bound."""
+    from puppygrad_amd import synth
+    steps = min(steps, cfg.n_positions - n_prefill - 1)
+    ids = np.stack([synth.token_ids(n_prefill, synth.TOKEN_SEED_BASE + 100 + b, cfg.vocab_size) for b in range(B)])
+    cache = model.new_kv_cache(B)
+    model.prefill_batch(ids, cache).argmax()
+    toks, st = model.decode_greedy_batch(cache, 4)  # warm-up steps
+    model.forward_one_batch(toks[-1], cache)        # the forward of the last selected tokens
+    start = cache.seq_len
+    toks, st = model.decode_greedy_batch(cache, steps + 1)  # steps + 1 tokens per sequence, steps forwards
+    n = st.generated_tokens - 1
+    sec = st.gpu_decode_time / n
+    C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    wbytes = (2 if bf16 else 4) * (L * (4 * C_ * C_ + 2 * C_ * I) + V * C_)
+    kvb = sum(kv_bytes(cfg, p) for p in range(start, start + n)) / n * B
+    achieved = (wbytes + kvb) / sec / 1e9
+    return {"workload": f"GPT-2 n_embd={C_} B={B} greedy decode steps, every KV cache at {start}..{start + n - 1} "
+                        f"tokens, weights stored as {'bf16' if bf16 else 'f32'}, fp32 arithmetic",
+            "value": round(B / sec, 1), "unit": "tokens/s", "steps": n, "ms_per_step": round(sec * 1e3, 4),
+            "roofline": hbm_roofline(achieved, "all launches of one batched step",
+                                     algorithmic_bytes_per_step=int(wbytes + kvb))}
 
 
 def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
@@ -301,17 +424,20 @@ def _devinfo():
     return info
 
 
-# HBM bytes one launch of k_decode_persistent<1600> moves on the default workload
-# (127 forwards from cache length 896), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this file (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the
-# counters and the copy-kernel scale factors).  None for any other workload.
-TRAFFIC_XL_DEFAULT = 891.8e9
+# HBM bytes per algorithmic byte of k_decode_persistent<1600> on the headline workload, from
+# rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by what the same
+# counter reads for a plain copy kernel of known size
+# (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the counters and the factors).
+TRAFFIC_RATIO_XL = 1.031
+TRAFFIC_SOURCE = "profiles/k_decode_persistent_1600_xl_decode_traffic.txt"
 
 
-def measured_traffic(args, n_prefill, persistent, launches):
-    if (args.model == "xl" and n_prefill == 896 and args.steps == 127 and persistent
-            and launches == 1 and not args.int8 and not args.bf16):
-        return TRAFFIC_XL_DEFAULT
+def measured_traffic(args, n_prefill, persistent, bytes_per_launch):
+    """The kernel's HBM traffic per launch: the measured ratio applied to this launch's
+    algorithmic bytes (the ratio was taken at 127 forwards per launch; it does not depend on
+    their number, every forward streams the same weights)."""
+    if args.model == "xl" and n_prefill == 896 and persistent and not args.int8 and not args.bf16:
+        return round(TRAFFIC_RATIO_XL * bytes_per_launch)
     return None
 
 

@@ -293,6 +293,15 @@ pg_status pg_op_attention_decode(int32_t device, const float* qkv, uint64_t pos,
 /* argmax_logits (src/models/generation.rs:269-279) on a host vector. */
 pg_status pg_op_argmax(int32_t device, const float* values, uint64_t n, uint32_t* out);
 
+/* Gpt2Model::prefill_profiled (src/models/gpt2/rust.rs:906-927 with a profile): pg_gpt2_prefill
+ * with the time of every launch added to its bucket of `profile` (HIP events on the cache's
+ * stream).  A prompt that takes the full-sequence path is timed as that path runs it, one
+ * launch per projection over all positions; LayerNorms that run inside a projection's reduce
+ * count with that projection, the stand-alone first one goes to layer_norm_s. */
+pg_status pg_gpt2_prefill_profiled(const pg_gpt2_model* model, pg_kv_cache* cache,
+                                   const uint32_t* ids, size_t n, pg_logits** out,
+                                   pg_gpt2_operation_profile* profile);
+
 /* ---- model assets: safetensors store, config.json, model directory ---- */
 
 /* TensorStore (src/models/safetensors.rs:93-138) over a read-only mapping of one
@@ -344,6 +353,15 @@ pg_status pg_gpt2_create_from_dir(const char* model_dir, const pg_hip_options* o
 void pg_synth_normal_f32(float* dst, uint64_t n, uint64_t seed, uint64_t first, double std);
 /* ids[i] = next_u64() % vocab from SmallRng::new(seed). */
 void pg_synth_token_ids(uint32_t* dst, uint64_t n, uint64_t seed, uint64_t vocab);
+
+/* Test hooks for the batch-1 decode kernel's exchange words (no reference counterpart).  Every
+ * activation the kernel hands from one workgroup to another carries a 32-bit epoch that counts
+ * up over the cache's life; when it nears its limit the next launch clears the words and starts
+ * from 1 again.  debug_epoch reads the next unused epoch (0 for a cache without that kernel);
+ * debug_set_epoch moves it forward (never back) so that a test can reach the restart without
+ * generating 2^31 tokens first. */
+uint32_t pg_kv_cache_debug_epoch(const pg_kv_cache* cache);
+pg_status pg_kv_cache_debug_set_epoch(pg_kv_cache* cache, uint32_t epoch);
 
 /* Device facts for the benchmark harness. */
 typedef struct pg_device_info {

@@ -126,6 +126,8 @@ SIGNATURES = {
                                                     C.POINTER(C.c_size_t),
                                                     C.POINTER(pg_generation_stats),
                                                     C.POINTER(pg_gpt2_operation_profile)]),
+    "pg_gpt2_prefill_profiled": (C.c_int, [_vp, _vp, _u32p, C.c_size_t, C.POINTER(_vp),
+                                           C.POINTER(pg_gpt2_operation_profile)]),
     "pg_op_dense": (C.c_int, [C.c_int32, _f32p, C.c_uint64, C.c_uint64, C.c_uint64, _f32p, _f32p,
                               _f32p]),
     "pg_op_layer_norm": (C.c_int, [C.c_int32, _f32p, C.c_uint64, C.c_uint64, _f32p, _f32p,
@@ -136,6 +138,8 @@ SIGNATURES = {
     "pg_op_attention_decode": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _f32p, _f32p, C.c_uint64,
                                          C.c_uint64, C.c_uint64, _f32p]),
     "pg_op_argmax": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _u32p]),
+    "pg_kv_cache_debug_epoch": (C.c_uint32, [_vp]),
+    "pg_kv_cache_debug_set_epoch": (C.c_int, [_vp, C.c_uint32]),
     "pg_tensor_store_open": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
     "pg_tensor_store_close": (None, [_vp]),
     "pg_tensor_store_len": (C.c_uint64, [_vp]),

@@ -186,6 +186,12 @@ __device__ __forceinline__ void gst(float* p, float v) {
 __device__ __forceinline__ void gst_u(unsigned* p, unsigned v) {
   *(unsigned __attribute__((address_space(1)))*)p = v;
 }
+// An id for the host: out_ids may be pinned host memory that the host reads while the kernel
+// runs, so the store goes all the way out (system scope).
+__device__ __forceinline__ void gst_id(unsigned* p, unsigned v) {
+  __hip_atomic_store((__attribute__((address_space(1))) unsigned*)p, v, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_SYSTEM);
+}
 __device__ __forceinline__ void gst_u64(u64* p, u64 v) {
   *(u64 __attribute__((address_space(1)))*)p = v;
 }
@@ -752,7 +758,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           PG_SERVICE_FAIL();
         }
     }
-    if (wg == 0 && lane == 0 && p.out_ids) gst_u(p.out_ids + t, tok);
+    if (wg == 0 && lane == 0 && p.out_ids) gst_id(p.out_ids + t, tok);
     if (p.eos >= 0 && tok == (unsigned)p.eos) {
       stopped = 1;
       break;
@@ -1122,7 +1128,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       PG_SERVICE_FAIL();
     }
     if (wg == 0 && lane == 0) {
-      if (p.out_ids) gst_u(p.out_ids + p.n_fwd, tk);
+      if (p.out_ids) gst_id(p.out_ids + p.n_fwd, tk);
       gst_u(p.d_tok, tk);
     }
   }

@@ -108,6 +108,10 @@ struct pg_kv_cache {
   uint32_t* d_tok = nullptr;      // [B] token the next step embeds
   uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
   uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
+  // streamed greedy generation: ids the persistent kernel writes straight into pinned host
+  // memory as it selects them ([P + 1], batch 1), and the device's address of that block
+  uint32_t* h_stream = nullptr;
+  uint32_t* h_stream_dev = nullptr;
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   pg_logits logits{};
@@ -272,7 +276,7 @@ pg_status check_compatible(const pg_gpt2_model* m, const pg_kv_cache* c) {
 // (src/models/gpt2/rust.rs:336-347): an event is recorded on the step's stream after each
 // operation; the span since the previous event belongs to that operation's bucket.
 struct ProfileMarks {
-  enum Bucket { kNone, kQkv, kAttention, kAttnProj, kMlpFc, kMlpProj, kLogits };
+  enum Bucket { kNone, kLayerNorm, kQkv, kAttention, kAttnProj, kMlpFc, kMlpProj, kLogits };
   std::vector<hipEvent_t> events;
   std::vector<Bucket> bucket;
   size_t used = 0;
@@ -295,6 +299,7 @@ struct ProfileMarks {
       if (r != hipSuccess) return r;
       const double sec = (double)ms * 1e-3;
       switch (bucket[i]) {
+        case kLayerNorm: p->layer_norm_s += sec; break;
         case kQkv: p->qkv_projection_s += sec; break;
         case kAttention: p->attention_s += sec; break;
         case kAttnProj: p->attention_projection_s += sec; break;
@@ -436,6 +441,10 @@ void exchange_release(int device, size_t bytes, void* p) {
   g_exchange_free.push_back(ExchangeBlock{device, bytes, p});
 }
 
+// Epochs of the tagged words count up over a cache's life; past this value the next launch
+// clears every tag and starts again from 1.
+constexpr unsigned kEpochWrap = 0xE0000000u;
+
 // Persistent launches are serialised process-wide: two of them resident at once
 // could each hold part of the CUs while waiting for workgroups that cannot start.
 std::mutex g_persistent_mu;
@@ -444,18 +453,46 @@ bool use_persistent(const pg_gpt2_model* m, const pg_kv_cache* c) {
   return m->persistent && c->B == 1 && c->qkv_t != nullptr;
 }
 
-// Runs n_fwd cached decoder steps of sequence 0 in ONE launch of the persistent
-// kernel and waits for it.  Token t is force_ids[t] when force_ids is set (prefill),
-// otherwise the first token comes from d_tok / tok and later ones from the argmax
-// of the previous step.  On return *done is the number of forwards executed and
-// *stopped says whether an EOS token ended the run early.
-pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
-                         bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
-                         size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
-                         size_t* done, bool* stopped, bool timed) {
+// Set while this thread has a persistent launch in flight: a callback that re-enters the
+// library from inside a streamed generation must not start a second one (it would wait for
+// workgroups that cannot become resident).
+thread_local bool t_persistent_in_flight = false;
+
+// One launch of the persistent kernel, in two halves so that the host can read the ids the
+// kernel writes to pinned memory while it runs.  persistent_begin enqueues the launch and
+// returns with the process-wide lock held; persistent_end waits for the kernel, releases the
+// lock and reports how many forwards ran and whether an EOS token ended the run early.
+struct PersistentRun {
+  std::unique_lock<std::mutex> lock;
+  bool begun = false;
+  hipStream_t stream = nullptr;
+  // (a caller that leaves early still waits for the kernel before the lock is released)
+  ~PersistentRun() {
+    if (begun) {
+      (void)hipStreamSynchronize(stream);
+      t_persistent_in_flight = false;
+    }
+  }
+#ifdef PG_DECODE_PROF_BUILD
+  float* prof = nullptr;
+  size_t prof_words = 0;
+  const char* prof_path = nullptr;
+#endif
+};
+
+// n_fwd cached decoder steps of sequence 0.  Token t is force_ids[t] when force_ids is set
+// (prefill), otherwise the first token comes from d_tok / tok and later ones from the argmax
+// of the previous step.
+pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
+                           bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
+                           size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
+                           bool timed, PersistentRun* run) {
   const Cfg& g = m->cfg;
+  if (t_persistent_in_flight)
+    return fail(PG_INVALID_INPUT,
+                "a token callback must not call the model while its generation is running");
   const unsigned span = (unsigned)(n_fwd * (g.L + 1) * 8 + 8);
-  if (c->epoch > 0xE0000000u - span) {
+  if (c->epoch > kEpochWrap - span) {
     // epochs would wrap: clear every tag and start over
     PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->qkv_t), c->tagged_words * 2,
                                  c->stream));
@@ -486,41 +523,79 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   p.epoch0 = c->epoch;
   p.ns = m->attn_splits;
   p.status = c->status;
-  // Development aid: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
+#ifdef PG_DECODE_PROF_BUILD
+  // Development builds only: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
   // of the last token of each persistent launch (raw u64, [grid][L+1][16]).
-  const char* prof_path = std::getenv("PG_DECODE_PROF");
-  DevBuf prof;
-  const size_t prof_words = (size_t)m->persistent_grid * (g.L + 1) * 16;
-  if (prof_path && g.L + 1 > 64) prof_path = nullptr;  // the kernel keeps 64 rows of stamps
-  if (prof_path) {
-    pg_status ps = prof.alloc(prof_words * 2);
-    if (ps) return ps;
-    PG_HIP(pgk::launch_fill_zero(prof.p, prof_words * 2, c->stream));
-    p.prof = reinterpret_cast<unsigned long long*>(prof.p);
+  run->prof_path = std::getenv("PG_DECODE_PROF");
+  run->prof_words = (size_t)m->persistent_grid * (g.L + 1) * 16;
+  if (run->prof_path && g.L + 1 > 64) run->prof_path = nullptr;  // the kernel keeps 64 rows of stamps
+  if (run->prof_path) {
+    PG_HIP(hipMalloc(&run->prof, run->prof_words * 8));
+    PG_HIP(pgk::launch_fill_zero(run->prof, run->prof_words * 2, c->stream));
+    p.prof = reinterpret_cast<unsigned long long*>(run->prof);
   }
+#endif
   c->epoch += span;
-  std::lock_guard<std::mutex> lk(g_persistent_mu);
-  PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
-  if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
-  PG_HIP(pgk::launch_decode_persistent(p, c->stream));
-  if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
-  PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
-                        c->stream));
-  PG_HIP(hipStreamSynchronize(c->stream));
-  if (prof_path) {
-    std::vector<unsigned long long> host(prof_words);
-    PG_HIP(hipMemcpy(host.data(), prof.p, prof_words * 8, hipMemcpyDeviceToHost));
-    if (FILE* f = std::fopen(prof_path, "wb")) {
-      std::fwrite(host.data(), 8, prof_words, f);
+  run->lock = std::unique_lock<std::mutex>(g_persistent_mu);
+  auto enqueue = [&]() -> pg_status {
+    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
+    if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
+    PG_HIP(pgk::launch_decode_persistent(p, c->stream));
+    if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
+                          c->stream));
+    return PG_OK;
+  };
+  pg_status s = enqueue();
+  if (s) {
+    (void)hipStreamSynchronize(c->stream);
+    run->lock.unlock();
+    return s;
+  }
+  run->begun = true;
+  run->stream = c->stream;
+  t_persistent_in_flight = true;
+  return PG_OK;
+}
+
+pg_status persistent_end(pg_kv_cache* c, PersistentRun* run, size_t* done, bool* stopped) {
+  if (!run->begun) return PG_OK;
+  run->begun = false;
+  const hipError_t e = hipStreamSynchronize(c->stream);
+  t_persistent_in_flight = false;
+  run->lock.unlock();
+  PG_HIP(e);
+#ifdef PG_DECODE_PROF_BUILD
+  if (run->prof_path) {
+    std::vector<unsigned long long> host(run->prof_words);
+    PG_HIP(hipMemcpy(host.data(), run->prof, run->prof_words * 8, hipMemcpyDeviceToHost));
+    if (FILE* f = std::fopen(run->prof_path, "wb")) {
+      std::fwrite(host.data(), 8, run->prof_words, f);
       std::fclose(f);
     }
   }
+  if (run->prof) (void)hipFree(run->prof);
+  run->prof = nullptr;
+#endif
   if (c->h_status[0] != 0)
     return fail(PG_BACKEND, "persistent decode kernel gave up waiting for a dependency "
                             "(another kernel may be occupying the device)");
   if (done) *done = c->h_status[1];
   if (stopped) *stopped = c->h_status[2] != 0;
   return PG_OK;
+}
+
+// The whole launch: begin, wait, end.  On return *done is the number of forwards executed and
+// *stopped says whether an EOS token ended the run early.
+pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
+                         bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
+                         size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
+                         size_t* done, bool* stopped, bool timed) {
+  PersistentRun run;
+  pg_status s = persistent_begin(m, c, force_ids, lm_last_only, tok_from_ptr, tok, pos0, n_fwd,
+                                 select_last, eos, out_ids_dev, timed, &run);
+  if (s) return s;
+  return persistent_end(c, &run, done, stopped);
 }
 
 // Sequences at least this long take the GEMM path in prefill / forward.
@@ -538,7 +613,7 @@ bool gemm_path_ok(const pg_gpt2_model* m, size_t n) {
 // position's logits go to the cache's logits row b; with all_logits set, the logits
 // of every position are also copied to dst ([n][V], host).
 pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, const uint32_t* ids,
-                            size_t n, float* all_logits_dst) {
+                            size_t n, float* all_logits_dst, ProfileMarks* marks = nullptr) {
   const Cfg& g = m->cfg;
   const int T = (int)n, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
   hipStream_t s = c->stream;
@@ -574,7 +649,12 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
   PG_HIP(hipMemcpyAsync(d_ids, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
   PG_HIP(hipStreamSynchronize(s));  // ids is the caller's pageable memory
+#define PG_MARK(bk) \
+  do {              \
+    if (marks) PG_HIP(marks->mark(s, ProfileMarks::bk)); \
+  } while (0)
   PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s, m->w_bf16));
+  PG_MARK(kNone);
   // (ln_g / ln_b: the LayerNorm that reads this projection's result, written to XN by the
   // same call: fused into the projection's reduce where it has one)
   auto gemm = [&](const float* A, int lda, const float* W, const float* bias, float* Cout,
@@ -589,17 +669,23 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b, g.eps, s));
+  PG_MARK(kLayerNorm);
   for (size_t l = 0; l < g.L; ++l) {
     const pgk::LayerW& w = m->layers[l];
     // the LayerNorm after this layer: the next layer's ln_1; ln_f is applied where it is needed
     const float* next_g = l + 1 < g.L ? m->layers[l + 1].ln_1_g : nullptr;
     const float* next_b = l + 1 < g.L ? m->layers[l + 1].ln_1_b : nullptr;
     PG_HIP(gemm(XN.p, C, w.c_attn_w, w.c_attn_b, QKV.p, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
+    PG_MARK(kQkv);
     PG_HIP(pgk::launch_attn_prefill(QKV.p, T, C, H, hd, P, c->k_panel(l, b), c->v_panel(l, b),
                                     ATT.p, SCR.p, s));
+    PG_MARK(kAttention);
     PG_HIP(gemm(ATT.p, C, w.c_proj_w, w.c_proj_b, X.p, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));
+    PG_MARK(kAttnProj);
     PG_HIP(gemm(XN.p, C, w.c_fc_w, w.c_fc_b, HB.p, I, I, C, pgk::GEMM_GELU));
+    PG_MARK(kMlpFc);
     PG_HIP(gemm(HB.p, I, w.c_proj_mlp_w, w.c_proj_mlp_b, X.p, C, C, I, pgk::GEMM_RESID, next_g, next_b));
+    PG_MARK(kMlpProj);
   }
   if (all_logits_dst) {
     PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->ln_f_g, m->ln_f_b, g.eps, s));
@@ -612,6 +698,8 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
   a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
   PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+  PG_MARK(kLogits);
+#undef PG_MARK
   PG_HIP(hipStreamSynchronize(s));
   return PG_OK;
 }
@@ -1132,6 +1220,9 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
     PG_HIP(hipMalloc(&raw->status, 4 * sizeof(unsigned)));
     PG_HIP(hipHostMalloc(&raw->h_status, 4 * sizeof(unsigned), hipHostMallocDefault));
     PG_HIP(hipMalloc(&raw->d_force, g.P * sizeof(uint32_t)));
+    PG_HIP(hipHostMalloc(&raw->h_stream, (g.P + 1) * sizeof(uint32_t),
+                         hipHostMallocMapped | hipHostMallocCoherent));
+    PG_HIP(hipHostGetDevicePointer(reinterpret_cast<void**>(&raw->h_stream_dev), raw->h_stream, 0));
     PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(raw->qkv_t), words * 2, raw->stream));
   }
   // Gpt2LayerKvCache::new zero-fills (src/models/gpt2/rust.rs:258-266).
@@ -1170,6 +1261,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->status);
     (void)hipFree(c->d_force);
     if (c->h_status) (void)hipHostFree(c->h_status);
+    if (c->h_stream) (void)hipHostFree(c->h_stream);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -1193,6 +1285,18 @@ pg_status pg_kv_cache_set_seq_len(pg_kv_cache* c, uint64_t n) {
                                       std::to_string(c->cfg.P));
   c->seq_len = n;
   c->logits_valid = false;
+  return PG_OK;
+}
+
+uint32_t pg_kv_cache_debug_epoch(const pg_kv_cache* c) { return c && c->qkv_t ? c->epoch : 0; }
+pg_status pg_kv_cache_debug_set_epoch(pg_kv_cache* c, uint32_t epoch) {
+  if (!c) return fail(PG_INVALID_INPUT, "null argument");
+  if (!c->qkv_t) return fail(PG_INVALID_INPUT, "this cache does not use the persistent decode kernel");
+  // words in memory carry epochs below c->epoch: a lower value could meet one of them again
+  if (epoch < c->epoch)
+    return fail(PG_INVALID_INPUT, "epoch " + std::to_string(epoch) + " is behind the cache's " +
+                                      std::to_string(c->epoch));
+  c->epoch = epoch;
   return PG_OK;
 }
 
@@ -1249,6 +1353,32 @@ pg_status pg_gpt2_prefill(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t
   if (!m || !c) return fail(PG_INVALID_INPUT, "null argument");
   if (c->B != 1) return fail(PG_INVALID_INPUT, "prefill needs a cache of batch 1");
   return pg_gpt2_prefill_batch(m, c, ids, n, out);
+}
+
+pg_status pg_gpt2_prefill_profiled(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* ids,
+                                   size_t n, pg_logits** out, pg_gpt2_operation_profile* profile) {
+  if (!m || !c || !profile) return fail(PG_INVALID_INPUT, "null argument");
+  if (c->B != 1) return fail(PG_INVALID_INPUT, "prefill needs a cache of batch 1");
+  *profile = pg_gpt2_operation_profile{};
+  pg_status s;
+  if ((s = validate_input(m->cfg, ids, n))) return s;
+  if ((s = check_compatible(m, c))) return s;
+  if ((s = select_device(m->device))) return s;
+  c->seq_len = 0;  // cache.clear() (rust.rs:918)
+  c->logits_valid = false;
+  ProfileMarks marks;
+  if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) {
+    if ((s = run_sequence_gemm(m, c, 0, ids, n, nullptr, &marks))) return s;
+    PG_HIP(marks.collect(profile));
+  } else {
+    for (size_t i = 0; i < n; ++i) {
+      if ((s = enqueue_forward_one(m, c, 0, nullptr, ids[i], i, i + 1 == n, &marks))) return s;
+      PG_HIP(hipStreamSynchronize(c->stream));
+      PG_HIP(marks.collect(profile));
+    }
+  }
+  c->seq_len = n;
+  return finish_logits(c, out);
 }
 
 pg_status pg_gpt2_forward_one_batch(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* ids,
@@ -1380,6 +1510,7 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
   pg_kv_cache* c = l->owner;
   if (!c->logits_valid) return fail(PG_INVALID_INPUT, "logits handle is stale");
   pg_status s;
+  if ((s = pg_sampling_validate(sampling))) return s;
   if ((s = select_device(c->device))) return s;
   const bool penalised = !(sampling->repeat_penalty == 1.0f || sampling->repeat_last_n == 0);
   if (sampling->temperature <= 0.0f && !penalised) {
@@ -1608,9 +1739,82 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
   std::vector<uint32_t> output(ids, ids + n);
   auto decode_start = Clock::now();
   double first_token_s = -1.0;
+  double gpu_decode_s = 0.0;
   uint64_t generated = 0;
   pg_rng_state rng;
   pg_rng_seed(&rng, seed);
+  const bool penalised = !(sampling->repeat_penalty == 1.0f || sampling->repeat_last_n == 0);
+  if (!profile && use_persistent(m, c) && sampling->temperature <= 0.0f && !penalised) {
+    // Greedy selection without a penalty (the reference's defaults, generation.rs:72-84): the
+    // same loop (rust.rs:495-531: select, EOS test before the push, on_token, forward_one
+    // unless it was the last token) with whole runs of steps inside one launch of the
+    // persistent kernel.  The kernel writes every id it selects into pinned host memory; this
+    // thread reads them from there while the kernel runs and hands them to on_token as they
+    // appear.  A launch holds at most kStreamChunk forwards, which bounds the work that is
+    // thrown away when on_token asks to stop.
+    constexpr size_t kStreamChunk = 64;
+    constexpr uint32_t kUnset = 0xffffffffu;  // not a token id (vocab_size < 2^31)
+    const size_t N = std::min<size_t>(max_new, m->cfg.P - output.size());  // tokens to select
+    volatile uint32_t* slot = c->h_stream;
+    size_t delivered = 0;  // tokens read from slot[0 .. delivered)
+    bool ended = N == 0;   // EOS seen or every token delivered
+    bool callback_stop = false;
+    // takes slot[delivered] once it is set; false while it is not
+    auto take = [&]() -> bool {
+      const uint32_t tok = slot[delivered];
+      if (tok == kUnset) return false;
+      ++delivered;
+      if (eos >= 0 && (uint32_t)eos == tok) {
+        ended = true;
+        return true;
+      }
+      output.push_back(tok);
+      if (on_token && on_token(tok, user) != 0) {
+        callback_stop = ended = true;
+        return true;
+      }
+      generated += 1;
+      if (first_token_s < 0) first_token_s = since(first_start);
+      if (delivered == N) ended = true;
+      return true;
+    };
+    if (N > 0) {
+      PG_HIP(pgk::launch_argmax(c->logits_buf, (int)m->cfg.V, c->d_tok, c->stream));
+      slot[0] = kUnset;
+      PG_HIP(hipMemcpyAsync(c->h_stream, c->d_tok, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                            c->stream));
+      PG_HIP(hipStreamSynchronize(c->stream));
+      take();
+    }
+    size_t base = 0;  // slot index of the token the next launch starts from (it is in d_tok)
+    while (!ended) {
+      const size_t nf = std::min(N - 1 - base, kStreamChunk);  // forwards of this launch
+      for (size_t i = 1; i <= nf; ++i) slot[base + i] = kUnset;
+      PersistentRun run;
+      if ((s = persistent_begin(m, c, nullptr, false, true, 0, c->seq_len, nf, true, eos,
+                                c->h_stream_dev + base, true, &run)))
+        return s;
+      bool running = true;
+      while (!ended && delivered <= base + nf) {
+        if (take()) continue;
+        if (!running) break;  // the kernel has ended without writing this id: it gave up
+        if (hipStreamQuery(c->stream) != hipErrorNotReady) running = false;  // one more look
+      }
+      size_t done = 0;
+      bool stopped = false;
+      if ((s = persistent_end(c, &run, &done, &stopped))) return s;
+      float ms = 0.0f;
+      PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
+      gpu_decode_s += ms * 1e-3;
+      if (callback_stop) return fail(PG_INVALID_INPUT, "on_token callback stopped generation");
+      if (!ended && delivered <= base + nf)
+        return fail(PG_BACKEND, "persistent decode kernel ended without the expected token");
+      // the forwards the reference would have run: one per token pushed, except the last
+      c->seq_len += stopped ? done : nf;
+      base += nf;
+    }
+    c->logits_valid = false;
+  } else {
   for (uint32_t it = 0; it < max_new; ++it) {
     if (output.size() >= m->cfg.P) break;
     uint32_t tok = 0;
@@ -1631,6 +1835,7 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
       if (s) return s;
     }
   }
+  }
   double decode_s = since(decode_start);
   std::memcpy(out_ids, output.data(), output.size() * sizeof(uint32_t));
   *out_n = output.size();
@@ -1640,7 +1845,7 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
     stats->prefill_s = prefill_s;
     stats->decode_s = decode_s;
     stats->first_token_s = first_token_s;
-    stats->gpu_decode_s = 0.0;
+    stats->gpu_decode_s = gpu_decode_s;
   }
   return PG_OK;
 }

@@ -445,6 +445,16 @@ class Gpt2Model:
                                            C.byref(out)))
         return DeviceLogits(out, cache)
 
+    def prefill_profiled(self, input_ids: Sequence[int], cache: Gpt2KvCache):
+        """prefill_profiled (rust.rs:906-927): the logits and the per-operation times."""
+        ids = _u32(input_ids)
+        out = C.c_void_p()
+        prof = _lib.pg_gpt2_operation_profile()
+        _check(_lib.load().pg_gpt2_prefill_profiled(self._h, cache._h, _lib.u32p(ids), ids.size,
+                                                    C.byref(out), C.byref(prof)))
+        return DeviceLogits(out, cache), Gpt2OperationProfile(
+            **{f[0][:-2]: getattr(prof, f[0]) for f in prof._fields_})
+
     def forward_one(self, token_id: int, cache: Gpt2KvCache) -> DeviceLogits:
         if token_id < 0 or token_id > 0xFFFFFFFF:
             raise Gpt2Error("InvalidInput", f"token id {token_id} exceeds vocab_size "
