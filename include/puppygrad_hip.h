@@ -302,6 +302,31 @@ pg_status pg_gpt2_prefill_profiled(const pg_gpt2_model* model, pg_kv_cache* cach
                                    const uint32_t* ids, size_t n, pg_logits** out,
                                    pg_gpt2_operation_profile* profile);
 
+/* ---- device operands for the op-level seam ---- */
+
+/* Plain device buffers for callers that keep operands in HBM between calls (no reference
+ * counterpart: the reference's operands are host slices).  upload / download are
+ * synchronous; download first waits for all work queued on the device. */
+pg_status pg_device_alloc(int32_t device, size_t bytes, void** out);
+pg_status pg_device_free(int32_t device, void* ptr);
+pg_status pg_device_upload(int32_t device, void* dst_device, const void* src_host, size_t bytes);
+pg_status pg_device_download(int32_t device, void* dst_host, const void* src_device, size_t bytes);
+
+/* pg_op_attention_decode for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  qkv ([3 * n_head * head_dim]), keys and values ([head][max_seq_len][head_dim],
+ * updated in place at `pos`) and out ([n_head * head_dim]) are DEVICE pointers; the three
+ * launches are queued on `stream` (a hipStream_t, NULL for the default stream) and the call
+ * returns without waiting for them.  The partial results of the key splits live in a fixed
+ * array inside the library (576 KiB per GPU, held until the process ends) instead of an
+ * allocation, which limits the call to n_head <= 256 and n_head * head_dim <= 4096; larger
+ * shapes are refused with PG_INVALID_INPUT.  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU (different streams or threads) race. */
+pg_status pg_op_attention_decode_noalloc(int32_t device, void* stream, const float* qkv,
+                                         uint64_t pos, float* keys, float* values,
+                                         uint64_t max_seq_len, uint64_t n_head, uint64_t head_dim,
+                                         float* out);
+
 /* ---- model assets: safetensors store, config.json, model directory ---- */
 
 /* TensorStore (src/models/safetensors.rs:93-138) over a read-only mapping of one

@@ -138,6 +138,12 @@ SIGNATURES = {
     "pg_op_attention_decode": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _f32p, _f32p, C.c_uint64,
                                          C.c_uint64, C.c_uint64, _f32p]),
     "pg_op_argmax": (C.c_int, [C.c_int32, _f32p, C.c_uint64, _u32p]),
+    "pg_device_alloc": (C.c_int, [C.c_int32, C.c_size_t, C.POINTER(_vp)]),
+    "pg_device_free": (C.c_int, [C.c_int32, _vp]),
+    "pg_device_upload": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
+    "pg_device_download": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
+    "pg_op_attention_decode_noalloc": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, _vp, _vp,
+                                                 C.c_uint64, C.c_uint64, C.c_uint64, _vp]),
     "pg_kv_cache_debug_epoch": (C.c_uint32, [_vp]),
     "pg_kv_cache_debug_set_epoch": (C.c_int, [_vp, C.c_uint32]),
     "pg_tensor_store_open": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
