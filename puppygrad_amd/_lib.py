@@ -164,7 +164,11 @@ _lib = None
 
 
 def lib_path() -> Path:
-    return _build.LIB_PATH
+    """The built library; PUPPYGRAD_HIP_LIB names another build of it (e.g. one with the
+    decode kernel's development timestamps compiled in)."""
+    import os
+    override = os.environ.get("PUPPYGRAD_HIP_LIB")
+    return Path(override) if override else _build.LIB_PATH
 
 
 def load() -> C.CDLL:

@@ -1393,6 +1393,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         const int r = d0 + wave;
         if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v[0])));
       }
+      SSTAMP(11);
       PG_SLICE(3, w, wn);
 
       // ================= E: c_fc rows + GELU =================
