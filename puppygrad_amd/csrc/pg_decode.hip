@@ -67,6 +67,10 @@ constexpr unsigned kSpinLimit = 1u << 21;
 constexpr int kMaxItemKeys = 128;  // keys per (head, split) attention item
 constexpr int kPace = 4;           // loads per pacing group of a slice
 constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
+// Widths whose instances leave registers free request the K and V rows of a workgroup's first
+// attention item at the top of the layer, before they wait for the layer's input: the rows do
+// not depend on the current token, and on these widths nothing else hides their latency.
+constexpr bool early_kv(int C) { return C <= 1024; }
 
 // Tagged words and the abort word live in global memory; saying so in the pointer type
 // gets global_ instead of flat_ instructions (a flat access also counts as an LDS one).
@@ -770,6 +774,22 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       float* kc = p.kv + (size_t)l * p.kv_layer_stride;
       float* vc = kc + p.kv_v_offset;
 
+      // the first attention item of this workgroup, known before the layer starts
+      const int items = H * ns, n = pos + 1;
+      const int per = (n + ns - 1) / ns;
+      KvRegs kv;
+      bool kv_early = false;
+      if constexpr (early_kv(C_)) {
+        if (wg < items) {
+          const int h0 = wg / ns, s0 = wg - h0 * ns;
+          const int k0 = s0 * per, k1 = min(n, k0 + per);
+          if (k0 < k1) {
+            attn_load_kv(kv, kc, vc, h0, P, k0, pos, kSW * 4 + (lane >> 4), lane & 15);
+            kv_early = true;
+          }
+        }
+      }
+
       // ================= A: block input -> LN1 -> xsA =================
       {
         const int ln = opaque(lane);  // per-lane addresses are built here, not hoisted
@@ -806,8 +826,6 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // All eight wavefronts work on an item: each loads the K/V rows of its slots as
       // soon as the item is known; this wavefront waits for q, stages it in LDS, counts
       // the item in flag[5], and merges the eight partial results.
-      const int items = H * ns, n = pos + 1;
-      const int per = (n + ns - 1) / ns;
       const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
 #pragma unroll 1
       for (int item = wg; item < items; item += G) {
@@ -822,8 +840,8 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           continue;
         }
         const bool owns_new = (k1 == n);
-        KvRegs kv;
-        attn_load_kv(kv, kc, vc, h, P, k0, pos, kSW * 4 + (lane >> 4), lane & 15);
+        if (!(kv_early && item == wg))
+          attn_load_kv(kv, kc, vc, h, P, k0, pos, kSW * 4 + (lane >> 4), lane & 15);
         // q of this head, and this token's own K/V rows if the split holds pos
         float qn[3];
         {
@@ -1316,6 +1334,25 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       const LayerW wn = layer_of(p.layers, (l + 1 < p.L) ? l + 1 : 0);
       const int wave = wave_id();
 
+      // the first attention item of this workgroup: its K/V rows are requested here on the
+      // widths that have the registers for it (see early_kv)
+      const int H = p.H, P = p.P, pos = p.pos0 + t, ns = splits_at(p, pos);
+      const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
+      const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
+      const float* vc = kc + p.kv_v_offset;
+      KvRegs kv;
+      bool kv_early = false;
+      if constexpr (early_kv(C_)) {
+        if (wg < items) {
+          const int h0 = wg / ns, s0 = wg - h0 * ns;
+          const int k0 = s0 * per, k1 = min(n, k0 + per);
+          if (k0 < k1) {
+            attn_load_kv(kv, kc, vc, h0, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
+            kv_early = true;
+          }
+        }
+      }
+
       // ================= A: c_attn rows =================
       // (biases are scalar loads: requested before each wait, they neither use vector
       // registers while the rows are in flight nor queue behind them)
@@ -1348,18 +1385,14 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       SSTAMP(5);
       // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
       {
-        const int H = p.H, P = p.P, pos = p.pos0 + t, ns = splits_at(p, pos);
-        const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
-        const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
-        const float* vc = kc + p.kv_v_offset;
 #pragma unroll 1
         for (int item = wg; item < items; item += G) {
           const int h = item / ns, sp = item - h * ns;
           const int k0 = sp * per, k1 = min(n, k0 + per);
           ++bseq;
           if (k0 >= k1) continue;
-          KvRegs kv;
-          attn_load_kv(kv, kc, vc, h, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
+          if (!(kv_early && item == wg))
+            attn_load_kv(kv, kc, vc, h, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
           if (!wait_flag(ctl, 5, bseq, abort_word)) {
             ok = false;
             break;
