@@ -92,6 +92,16 @@ typedef struct pg_hip_options {
   uint32_t weight_storage; /* pg_weight_storage: how the dense matrices and wte are kept in HBM */
   uint32_t decode_path;    /* pg_decode_path */
   uint32_t prefill_path;   /* 0: GEMM prefill for prompts of 16+ tokens; 1: always token by token */
+  /* Tunables, the counterpart of the thresholds and chunk sizes of Gpt2RustConfig
+   * (src/models/gpt2/options.rs:54-96) that the reference's `autotune gpt2` scans
+   * (src/main.rs:2732-2870).  0 selects the built-in default. */
+  uint32_t attn_item_keys;          /* fused batch-1 decode kernel: keys per (head, key split)
+                                       attention item, 128 (default) or 256 */
+  uint32_t attn_blocks_per_cu;      /* per-operation and batched decode attention: (head, split)
+                                       blocks per CU the split count aims for (default 4) */
+  uint32_t gemm_split_items_per_cu; /* tile GEMM: a product that leaves CUs idle is cut along K
+                                       into about this many work items per CU (default 3) */
+  uint32_t reserved;                /* must be 0 */
 } pg_hip_options;
 
 typedef struct pg_gpt2_model pg_gpt2_model;
@@ -361,12 +371,20 @@ pg_status pg_tensor_store_optional_f32(const pg_tensor_store* store, const char*
  * "failed to parse config {path}: ...", src/models/config.rs:19-29). */
 pg_status pg_gpt2_load_config(const char* path, pg_gpt2_config* out);
 
+/* load_gpt2_tuning (src/main.rs:2564-2586): reads the `hip` object of a puppygrad-tune.json
+ * written by the autotune scan (SavedGpt2Tuning, src/main.rs:2611-2623, with `hip` in the place
+ * of `rust`) and copies its tunables into the fields of *options that are still 0.  A file
+ * that does not exist is not an error (*found = 0); an unreadable or malformed one is
+ * PG_ASSET ("failed to read tuning file ...", "failed to parse tuning file ..."). */
+pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t* found);
+
 /* Gpt2Runtime::from_dir_with_backend without the tokenizer
  * (src/models/gpt2/rust.rs:382-393): {model_dir}/config.json and
  * {model_dir}/model.safetensors (src/models/gpt2/assets.rs:20-30), tensor names and
  * shapes as load_weights with the `transformer.` prefix fallback
  * (rust.rs:713-771), then pg_gpt2_create.  Tensors are uploaded straight from the
- * file mapping; no host copy of the weights is made. */
+ * file mapping; no host copy of the weights is made.  {model_dir}/puppygrad-tune.json, when
+ * present, supplies the tunables that `options` leaves at 0 (src/main.rs:2564-2586). */
 pg_status pg_gpt2_create_from_dir(const char* model_dir, const pg_hip_options* options,
                                   pg_gpt2_model** out);
 

@@ -42,7 +42,9 @@ class pg_gpt2_weights_view(C.Structure):
 
 class pg_hip_options(C.Structure):
     _fields_ = [("device", C.c_int32), ("weight_storage", C.c_uint32),
-                ("decode_path", C.c_uint32), ("prefill_path", C.c_uint32)]
+                ("decode_path", C.c_uint32), ("prefill_path", C.c_uint32),
+                ("attn_item_keys", C.c_uint32), ("attn_blocks_per_cu", C.c_uint32),
+                ("gemm_split_items_per_cu", C.c_uint32), ("reserved", C.c_uint32)]
 
 
 class pg_sampling(C.Structure):
@@ -154,6 +156,7 @@ SIGNATURES = {
     "pg_tensor_store_optional_f32": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.c_size_t,
                                                C.POINTER(C.c_int32), C.POINTER(pg_tensor)]),
     "pg_gpt2_load_config": (C.c_int, [C.c_char_p, C.POINTER(pg_gpt2_config)]),
+    "pg_hip_load_tuning": (C.c_int, [C.c_char_p, C.POINTER(pg_hip_options), C.POINTER(C.c_int32)]),
     "pg_gpt2_create_from_dir": (C.c_int, [C.c_char_p, C.POINTER(pg_hip_options), C.POINTER(_vp)]),
     "pg_synth_normal_f32": (None, [_f32p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double]),
     "pg_synth_token_ids": (None, [_u32p, C.c_uint64, C.c_uint64, C.c_uint64]),

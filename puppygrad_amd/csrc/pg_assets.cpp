@@ -596,10 +596,58 @@ pg_status pg_gpt2_load_config(const char* path, pg_gpt2_config* out) {
   return PG_OK;
 }
 
+pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t* found) {
+  if (!path || !options) return fail(PG_INVALID_INPUT, "null argument");
+  if (found) *found = 0;
+  std::ifstream in(path, std::ios::binary);
+  if (!in) {
+    if (errno == ENOENT) return PG_OK;  // load_gpt2_tuning: a missing default file is no error
+    return fail(PG_ASSET, std::string("failed to read tuning file ") + path + ": " +
+                              std::strerror(errno));
+  }
+  std::stringstream buf;
+  buf << in.rdbuf();
+  const std::string text = buf.str();
+  Json root;
+  std::string err;
+  if (!JsonParser(text.data(), text.data() + text.size()).parse(root, err))
+    return fail(PG_ASSET, std::string("failed to parse tuning file ") + path + ": " + err);
+  const Json* hip = root.kind == Json::Obj ? root.find("hip") : nullptr;
+  if (!hip || hip->kind != Json::Obj)
+    return fail(PG_ASSET, std::string("failed to parse tuning file ") + path +
+                              ": missing field `hip`");
+  struct Field {
+    const char* key;
+    uint32_t* dst;
+  } fields[] = {{"attn_item_keys", &options->attn_item_keys},
+                {"attn_blocks_per_cu", &options->attn_blocks_per_cu},
+                {"gemm_split_items_per_cu", &options->gemm_split_items_per_cu}};
+  for (const Field& f : fields) {
+    const Json* v = hip->find(f.key);
+    if (!v || v->kind == Json::Null) continue;
+    if (v->kind != Json::Num || v->num < 0 || v->num > 4294967295.0 || v->num != std::floor(v->num))
+      return fail(PG_ASSET, std::string("failed to parse tuning file ") + path +
+                                ": invalid type for field `" + f.key + "`, expected u32");
+    if (*f.dst == 0) *f.dst = (uint32_t)v->num;  // a value the caller set explicitly wins
+  }
+  if (found) *found = 1;
+  return PG_OK;
+}
+
 pg_status pg_gpt2_create_from_dir(const char* model_dir, const pg_hip_options* options,
                                   pg_gpt2_model** out) {
   if (!model_dir || !out) return fail(PG_INVALID_INPUT, "null argument");
   *out = nullptr;
+  // load_gpt2_tuning (src/main.rs:2564-2586): {model_dir}/puppygrad-tune.json, when it exists,
+  // supplies the tunables the caller left at their defaults
+  pg_hip_options tuned{};
+  if (options) tuned = *options;
+  {
+    const std::string tune_path = join(model_dir, "puppygrad-tune.json");
+    pg_status ts = pg_hip_load_tuning(tune_path.c_str(), &tuned, nullptr);
+    if (ts) return ts;
+    options = &tuned;
+  }
   // Gpt2AssetPaths::new (src/models/gpt2/assets.rs:20-30)
   const std::string config_path = join(model_dir, "config.json");
   const std::string weights_path = join(model_dir, "model.safetensors");

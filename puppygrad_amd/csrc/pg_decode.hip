@@ -64,7 +64,11 @@ constexpr int kThreads = 512;
 constexpr int kSW = 7;      // streamer wavefronts (0..6); wavefront 7 is the service wavefront
 constexpr int kGrid = 256;  // workgroups; row bands are computed for exactly this many
 constexpr unsigned kSpinLimit = 1u << 21;
-constexpr int kMaxItemKeys = 128;  // keys per (head, split) attention item
+// Keys per (head, split) attention item: 128 (four steps of 32 key slots) or 256 (eight steps,
+// half as many splits to merge but twice the K/V rows per item).  Which one is faster depends on
+// the width and the context length, so it is a launch parameter with one kernel instance each
+// (template parameter KS = steps per slot).
+constexpr int kItemKeysDefault = 128;
 constexpr int kPace = 4;           // loads per pacing group of a slice
 constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
 // Widths whose instances leave registers free request the K and V rows of a workgroup's first
@@ -462,11 +466,11 @@ __device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, 
 }
 
 // Key splits per head at position pos: as few as hold the pos + 1 keys in items of at
-// most kMaxItemKeys (never more than the launch's count, which covers the longest context).
+// most p.item_keys (never more than the launch's count, which covers the longest context).
 // With one split there is no merge hop: the item's result is the head's attention output.
 // Every wavefront of the grid derives the same value.
 __device__ __forceinline__ int splits_at(const DecodeParams& p, int pos) {
-  return min((pos + kMaxItemKeys) / kMaxItemKeys, p.ns);
+  return min((pos + p.item_keys) / p.item_keys, p.ns);
 }
 
 // ---- service side: poll tagged words ---------------------------------------------------
@@ -615,19 +619,19 @@ constexpr int kTsLayers = 64;  // room for L + 1 <= 64 rows of 16 stamps
 // ---- attention item: shared by all eight wavefronts ----------------------------------
 // An item is the keys [k0, k1) of one head (at most 128).  Key k0 + slot + 32 i belongs
 // to slot = 4 wave + (lane >> 4), step i < 4; the 16 lanes of a slot hold 4 dims each.
-constexpr int kAttnSteps = kMaxItemKeys / 32;
-static_assert(kMaxItemKeys % 32 == 0, "an item is whole steps of 32 key slots");
+template <int KS>
 struct KvRegs {
-  f4 k[kAttnSteps], v[kAttnSteps];
+  f4 k[KS], v[KS];
 };
 // Requests this wavefront's K and V rows.  Unconditional: keys past the split, and the
 // key `pos` that is not in the cache yet, re-read an older row and are masked / replaced.
-__device__ __forceinline__ void attn_load_kv(KvRegs& r, const float* kc, const float* vc, int h, int P,
+template <int KS>
+__device__ __forceinline__ void attn_load_kv(KvRegs<KS>& r, const float* kc, const float* vc, int h, int P,
                                              int k0, int pos, int slot, int d4) {
   gf4p Kh = as_global(reinterpret_cast<const f4*>(kc + (size_t)h * P * 64));
   gf4p Vh = as_global(reinterpret_cast<const f4*>(vc + (size_t)h * P * 64));
 #pragma unroll
-  for (int i = 0; i < kAttnSteps; ++i) {
+  for (int i = 0; i < KS; ++i) {
     const int key = min(k0 + slot + 32 * i, max(pos - 1, 0));
     r.k[i] = __builtin_nontemporal_load(Kh + (size_t)key * 16 + d4);
     r.v[i] = __builtin_nontemporal_load(Vh + (size_t)key * 16 + d4);
@@ -636,8 +640,10 @@ __device__ __forceinline__ void attn_load_kv(KvRegs& r, const float* kc, const f
 // This wavefront's part of cached_self_attention_into (src/models/gpt2/rust.rs:1662-1741)
 // once q (and the new K/V rows) are in LDS: max, sum of exp and weighted V rows over its
 // keys, written to the control block.  A wavefront without keys writes the neutral element.
-__device__ __forceinline__ void attn_wave_partial(KvRegs& r, ctlp ctl, int k0, int k1, int pos,
+template <int KS>
+__device__ __forceinline__ void attn_wave_partial(KvRegs<KS>& r, ctlp ctl, int k0, int k1, int pos,
                                                   int wave, int lane) {
+  constexpr int kAttnSteps = KS;
   const int sub = lane >> 4, d4 = lane & 15, slot = wave * 4 + sub;
   const f4 qv = ((lf4p)&ctl->qs[0])[d4];
   float sc[kAttnSteps];
@@ -707,7 +713,7 @@ __device__ __forceinline__ unsigned h_share(const u64* src, unsigned epoch, lfp 
 // ===================================================================================
 // Service wavefront
 // ===================================================================================
-template <int C_>
+template <int C_, int KS>
 __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
   constexpr int C = C_, I = 4 * C_, NW = C_ / 64, NWI = I / 64;
   constexpr int G = kGrid;
@@ -777,7 +783,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // the first attention item of this workgroup, known before the layer starts
       const int items = H * ns, n = pos + 1;
       const int per = (n + ns - 1) / ns;
-      KvRegs kv;
+      KvRegs<KS> kv;
       bool kv_early = false;
       if constexpr (early_kv(C_)) {
         if (wg < items) {
@@ -1228,7 +1234,7 @@ struct StreamPlan {
   static_assert(WB == 4 || !kTight, "only f32 rows are staged");
 };
 
-template <int C_, int WB>
+template <int C_, int WB, int KS>
 __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, const Lds& lds) {
   typedef StreamPlan<C_, WB> SP;
   constexpr bool kI8 = WB == 1, kPacked = WB != 4;  // packed: several weights per 32-bit word
@@ -1340,7 +1346,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
       const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
       const float* vc = kc + p.kv_v_offset;
-      KvRegs kv;
+      KvRegs<KS> kv;
       bool kv_early = false;
       if constexpr (early_kv(C_)) {
         if (wg < items) {
@@ -1603,7 +1609,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
 }
 
 // C_ = n_embd (compile time); n_inner = 4 C_; head_dim 64; grid = kGrid.
-template <int C_, int WB>
+template <int C_, int WB, int KS>
 __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
   constexpr int C = C_, I = 4 * C_;
   // 16-byte LDS accesses run at full speed only on 16-byte boundaries: the dynamic block
@@ -1633,9 +1639,9 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
   __syncthreads();
 
   if ((threadIdx.x >> 6) == kSW)
-    service_wave<C_>(p, ctl, lds);
+    service_wave<C_, KS>(p, ctl, lds);
   else
-    streamer_wave<C_, WB>(p, ctl, lds);
+    streamer_wave<C_, WB, KS>(p, ctl, lds);
 }
 
 }  // namespace
@@ -1651,10 +1657,11 @@ size_t persistent_lds_bytes(int C, int w_packed) {
 // f32, bf16 and int8 rows.
 bool persistent_supports(int C) { return C == 768 || C == 1024 || C == 1280 || C == 1600; }
 int persistent_grid() { return kGrid; }
-int persistent_max_item_keys() { return kMaxItemKeys; }
+int persistent_default_item_keys() { return kItemKeysDefault; }
+bool persistent_item_keys_ok(int keys) { return keys == 128 || keys == 256; }
 
 namespace {
-template <int C_, int WB>
+template <int C_, int WB, int KS>
 hipError_t launch_one(const DecodeParams& p, hipStream_t s) {
   const size_t lds = persistent_lds_bytes(C_, WB != 4);
   // more than the 64 KiB default of dynamic LDS: opt in once per device
@@ -1663,20 +1670,26 @@ hipError_t launch_one(const DecodeParams& p, hipStream_t s) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (armed_device != dev) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_persistent<C_, WB>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_persistent<C_, WB, KS>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     armed_device = dev;
   }
-  hipLaunchKernelGGL((k_decode_persistent<C_, WB>), dim3(kGrid), dim3(kThreads), lds, s, p);
+  hipLaunchKernelGGL((k_decode_persistent<C_, WB, KS>), dim3(kGrid), dim3(kThreads), lds, s, p);
   return hipGetLastError();
 }
-template <int WB>
+template <int WB, int KS>
 hipError_t launch_width(const DecodeParams& p, hipStream_t s) {
-  if (p.C == 768) return launch_one<768, WB>(p, s);
-  if (p.C == 1024) return launch_one<1024, WB>(p, s);
-  if (p.C == 1280) return launch_one<1280, WB>(p, s);
-  if (p.C == 1600) return launch_one<1600, WB>(p, s);
+  if (p.C == 768) return launch_one<768, WB, KS>(p, s);
+  if (p.C == 1024) return launch_one<1024, WB, KS>(p, s);
+  if (p.C == 1280) return launch_one<1280, WB, KS>(p, s);
+  if (p.C == 1600) return launch_one<1600, WB, KS>(p, s);
+  return hipErrorInvalidValue;
+}
+template <int WB>
+hipError_t launch_keys(const DecodeParams& p, hipStream_t s) {
+  if (p.item_keys == 128) return launch_width<WB, 4>(p, s);
+  if (p.item_keys == 256) return launch_width<WB, 8>(p, s);
   return hipErrorInvalidValue;
 }
 // Whether one workgroup of the kernel fits on a CU (then the grid of one workgroup per CU is
@@ -1685,21 +1698,21 @@ hipError_t launch_width(const DecodeParams& p, hipStream_t s) {
 // query: a process that has loaded another copy of the HIP runtime first (PyTorch bundles
 // one) was seen to get 0 blocks from that query for the 161..167-register instances, which
 // launch and run correctly (8 wavefronts of up to 256 registers are one block per CU here).
-template <int C_, int WB>
+template <int C_, int WB, int KS>
 hipError_t fits_one(int* out) {
   hipFuncAttributes at{};
-  hipError_t e = hipFuncGetAttributes(&at, reinterpret_cast<const void*>(&k_decode_persistent<C_, WB>));
+  hipError_t e = hipFuncGetAttributes(&at, reinterpret_cast<const void*>(&k_decode_persistent<C_, WB, KS>));
   if (e != hipSuccess) return e;
   const size_t lds = persistent_lds_bytes(C_, WB != 4);
   *out = (at.maxThreadsPerBlock >= kThreads && lds <= (size_t)at.maxDynamicSharedSizeBytes) ? 1 : 0;
   return hipSuccess;
 }
-template <int WB>
+template <int WB, int KS>
 hipError_t max_blocks(int C, int* out) {
-  if (C == 768) return fits_one<768, WB>(out);
-  if (C == 1024) return fits_one<1024, WB>(out);
-  if (C == 1280) return fits_one<1280, WB>(out);
-  if (C == 1600) return fits_one<1600, WB>(out);
+  if (C == 768) return fits_one<768, WB, KS>(out);
+  if (C == 1024) return fits_one<1024, WB, KS>(out);
+  if (C == 1280) return fits_one<1280, WB, KS>(out);
+  if (C == 1600) return fits_one<1600, WB, KS>(out);
   *out = 0;
   return hipSuccess;
 }
@@ -1707,16 +1720,21 @@ hipError_t max_blocks(int C, int* out) {
 
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
   if (!p.lm_w || (p.w_bytes == 1 && !p.lm_s)) return hipErrorInvalidValue;
-  if (p.w_bytes == 1) return launch_width<1>(p, s);
-  if (p.w_bytes == 2) return launch_width<2>(p, s);
-  if (p.w_bytes == 4) return launch_width<4>(p, s);
+  if (p.w_bytes == 1) return launch_keys<1>(p, s);
+  if (p.w_bytes == 2) return launch_keys<2>(p, s);
+  if (p.w_bytes == 4) return launch_keys<4>(p, s);
   return hipErrorInvalidValue;
 }
 
-hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes) {
-  if (w_bytes == 1) return max_blocks<1>(C, out);
-  if (w_bytes == 2) return max_blocks<2>(C, out);
-  return max_blocks<4>(C, out);
+hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes, int item_keys) {
+  if (item_keys == 256) {
+    if (w_bytes == 1) return max_blocks<1, 8>(C, out);
+    if (w_bytes == 2) return max_blocks<2, 8>(C, out);
+    return max_blocks<4, 8>(C, out);
+  }
+  if (w_bytes == 1) return max_blocks<1, 4>(C, out);
+  if (w_bytes == 2) return max_blocks<2, 4>(C, out);
+  return max_blocks<4, 4>(C, out);
 }
 
 }  // namespace pgk

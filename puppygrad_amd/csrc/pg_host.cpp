@@ -65,6 +65,10 @@ struct pg_gpt2_model {
   bool persistent = false;          // batch-1 decode runs as one persistent launch
   int persistent_grid = 0;          // workgroups of that launch (one per CU)
   int attn_splits = 1;              // key splits per head in the persistent kernel
+  // tunables (pg_hip_options; defaults filled in at creation)
+  int item_keys = 128;              // keys per attention item of the persistent kernel
+  int attn_blocks_per_cu = 4;       // per-operation / batched decode attention
+  int gemm_split_items = 3;         // tile GEMM split-K
   int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
   // int8 storage (QuantizedRows, src/models/cpu.rs:26-56): the block matrices hold int8 rows
   // with the scales in LayerW; wte stays f32 for the embedding (rust.rs:966-974 reads the f32
@@ -334,7 +338,7 @@ pg_status enqueue_forward_one(const pg_gpt2_model* m, pg_kv_cache* c, size_t b,
   float* pa = c->part_acc + b * part_stride * hd;
   float* pm = c->part_m + b * part_stride;
   float* pl = c->part_l + b * part_stride;
-  const int nsplit = hd == pgk::kHeadDim ? pgk::choose_nsplit((int)pos + 1, H, m->num_cus) : 1;
+  const int nsplit = hd == pgk::kHeadDim ? pgk::choose_nsplit((int)pos + 1, H, m->num_cus, m->attn_blocks_per_cu) : 1;
 
   PG_HIP(pgk::launch_embed(x, m->wte, m->wpe, tok_ptr, tok, (int)pos, C, s, m->w_bf16));
   PG_MARK(kNone);  // the embedding is in no bucket (rust.rs:966-974)
@@ -522,6 +526,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   p.eos = (int)eos;
   p.epoch0 = c->epoch;
   p.ns = m->attn_splits;
+  p.item_keys = m->item_keys;
   p.status = c->status;
 #ifdef PG_DECODE_PROF_BUILD
   // Development builds only: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
@@ -666,6 +671,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     if (m->w_i8) a.w_scale = i8_scales_of(W, (size_t)N, (size_t)K);
     a.ws = WS.p; a.ws_floats = ws_floats;
     if (ln_g) { a.ln_out = XN.p; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
+    a.split_items_per_cu = m->gemm_split_items;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b, g.eps, s));
@@ -716,7 +722,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
             P = (int)g.P;
   hipStream_t s = c->stream;
   const int nsplit = hd == pgk::kHeadDim
-                         ? pgk::choose_nsplit((int)pos + 1, H * B, m->num_cus) : 1;
+                         ? pgk::choose_nsplit((int)pos + 1, H * B, m->num_cus, m->attn_blocks_per_cu) : 1;
   pgk::BatchStrides bs;
   bs.q = 3 * g.C;
   bs.kv = g.H * g.P * g.hd();
@@ -737,6 +743,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     a.ws = c->gemm_ws; a.ws_floats = c->gemm_ws_floats;
     a.a_packed = pk; a.c_packed = c_packed;
     if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; a.ln_packed = pk; }
+    a.split_items_per_cu = m->gemm_split_items;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
@@ -962,6 +969,13 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   const bool i8 = opts.weight_storage == PG_STORE_INT8;
   if (opts.decode_path > PG_DECODE_PERSISTENT)
     return fail(PG_INVALID_CONFIG, "hip backend decode_path out of range");
+  if (opts.attn_item_keys != 0 && !pgk::persistent_item_keys_ok((int)opts.attn_item_keys))
+    return fail(PG_INVALID_CONFIG, "hip backend attn_item_keys must be 0 (default), 128 or 256");
+  if (opts.attn_blocks_per_cu > 64)
+    return fail(PG_INVALID_CONFIG, "hip backend attn_blocks_per_cu must be at most 64");
+  if (opts.gemm_split_items_per_cu > 16)
+    return fail(PG_INVALID_CONFIG, "hip backend gemm_split_items_per_cu must be at most 16");
+  if (opts.reserved != 0) return fail(PG_INVALID_CONFIG, "hip backend options: reserved must be 0");
   if ((s = select_device(opts.device))) return s;
 
   auto m = std::make_unique<pg_gpt2_model>();
@@ -970,6 +984,9 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   m->opts = opts;
   m->w_bf16 = bf ? 1 : 0;
   m->w_i8 = i8 ? 1 : 0;
+  m->item_keys = opts.attn_item_keys ? (int)opts.attn_item_keys : pgk::persistent_default_item_keys();
+  m->attn_blocks_per_cu = opts.attn_blocks_per_cu ? (int)opts.attn_blocks_per_cu : 4;
+  m->gemm_split_items = opts.gemm_split_items_per_cu ? (int)opts.gemm_split_items_per_cu : 3;
   hipDeviceProp_t prop;
   PG_HIP(hipGetDeviceProperties(&prop, opts.device));
   m->num_cus = prop.multiProcessorCount;
@@ -1107,15 +1124,15 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     bool shape_ok = g.hd() == 64 && g.I == 4 * g.C && pgk::persistent_supports((int)g.C) &&
                     g.P <= 4096 && g.V >= (size_t)grid;
     if (shape_ok) {
-      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu, i8 ? 1 : bf ? 2 : 4));
+      PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu, i8 ? 1 : bf ? 2 : 4,
+                                                   m->item_keys));
       shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
     }
     if (shape_ok) {
       // key splits per head at the longest context (the kernel uses as few as the position
       // at hand needs: fewer splits are fewer partials to merge and fewer workgroups held
       // up by attention)
-      int ns = std::max<int>(1, (int)((g.P + pgk::persistent_max_item_keys() - 1) /
-                                      pgk::persistent_max_item_keys()));
+      int ns = std::max<int>(1, (int)((g.P + m->item_keys - 1) / m->item_keys));
       shape_ok = ns <= pgk::kMaxSplits && (size_t)ns * 66 <= g.I;
       m->attn_splits = ns;
     }
@@ -1149,8 +1166,12 @@ pg_status pg_gpt2_get_config(const pg_gpt2_model* m, pg_gpt2_config* out) {
 
 pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
   if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
-  std::snprintf(dst, cap, "hip (device=%d, compute_units=%d, weights=%s, decode=%s)", m->device,
-                m->num_cus, m->w_bf16 ? "bf16" : m->w_i8 ? "int8" : "f32", m->persistent ? "persistent" : "kernels");
+  std::snprintf(dst, cap,
+                "hip (device=%d, compute_units=%d, weights=%s, decode=%s, attn_item_keys=%d, "
+                "attn_blocks_per_cu=%d, gemm_split_items_per_cu=%d)",
+                m->device, m->num_cus, m->w_bf16 ? "bf16" : m->w_i8 ? "int8" : "f32",
+                m->persistent ? "persistent" : "kernels", m->item_keys, m->attn_blocks_per_cu,
+                m->gemm_split_items);
   return PG_OK;
 }
 

@@ -77,7 +77,8 @@ hipError_t launch_attn_decode(const float* q, const float* kcache, const float* 
                               int P, int H, int head_dim, int nsplit, float* part_acc,
                               float* part_m, float* part_l, hipStream_t s, int batch = 1,
                               BatchStrides bs = BatchStrides{}, int append_C = 0);
-int choose_nsplit(int n_keys, int H, int num_cus);
+// blocks_per_cu: (head, split) blocks per CU to aim for (tunable, 4 by default).
+int choose_nsplit(int n_keys, int H, int num_cus, int blocks_per_cu = 4);
 
 // out[r] = argmax of row r of v[rows][n] with the reference's tie/NaN rules.
 hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, int rows = 1);
@@ -143,6 +144,9 @@ struct GemmArgs {
   // A, C and ln_out are held that way.  Only the 32-row decode kernel reads a packed A, so
   // launch_gemm refuses the flags for any other form (gemm_takes_rows32 tells beforehand).
   int a_packed = 0, c_packed = 0, ln_packed = 0;
+  // Tunable: a GEMM whose M x N leaves CUs idle is cut along K into about this many work items
+  // per CU (gemm_split_parts).
+  int split_items_per_cu = 3;
 };
 // Element (row b < 32, column k) of a packed activation matrix: the float4 of columns
 // 4j..4j+3 of all 32 rows lie next to each other, so that 32 lanes which each read four
@@ -193,7 +197,8 @@ struct DecodeParams {
   int lm_last_only;           // with force_ids: LN_f + lm_head only after the last token
   int pos0, n_fwd, select_last, eos;
   unsigned epoch0;
-  int ns;
+  int ns;         // key splits per head at the longest context
+  int item_keys;  // keys per (head, split) attention item: 128 or 256
   unsigned* status;  // [0] abort, [1] forwards done, [2] stopped at eos
   // Optional [grid][L+1][8] timestamps (100 MHz wall clock) of the last token's phase
   // completions per workgroup; slot [L][7] holds the token's start.
@@ -206,8 +211,9 @@ struct DecodeParams {
 bool persistent_supports(int C);
 int persistent_grid();
 size_t persistent_lds_bytes(int C, int w_packed = 0);
-int persistent_max_item_keys();
-hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes = 4);
+int persistent_default_item_keys();
+bool persistent_item_keys_ok(int keys);
+hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes = 4, int item_keys = 128);
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
 
 }  // namespace pgk

@@ -907,11 +907,12 @@ hipError_t launch_embed(float* x, const float* wte, const float* wpe, const uint
   return hipGetLastError();
 }
 
-int choose_nsplit(int n_keys, int H, int num_cus) {
-  // Enough (head, split) blocks for about four per CU, at least 16 keys each; and at most
-  // 128 keys each where the split limit allows (one chunk of the kernel: every K and V
-  // row of the block is then requested before the first is used).
-  int want = (4 * num_cus + H - 1) / H;
+int choose_nsplit(int n_keys, int H, int num_cus, int blocks_per_cu) {
+  // Enough (head, split) blocks for about blocks_per_cu (four by default) per CU, at least 16
+  // keys each; and at most 128 keys each where the split limit allows (one chunk of the
+  // kernel: every K and V row of the block is then requested before the first is used).
+  if (blocks_per_cu < 1) blocks_per_cu = 4;
+  int want = (blocks_per_cu * num_cus + H - 1) / H;
   int by_len = (n_keys + 15) / 16;
   int ns = want < by_len ? want : by_len;
   int by_chunk = (n_keys + 127) / 128;

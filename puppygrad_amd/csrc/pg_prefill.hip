@@ -1003,7 +1003,7 @@ int gemm_split_parts(const GemmArgs& a, int num_cus) {
   const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
   if (!a.ws || a.N % 4 != 0 || tiles * 2 >= 3L * num_cus) return 1;
   const int depth = a.M < 64 ? 128 : (tiles * 10 < 9L * num_cus ? 192 : 512);
-  int parts = (int)((3L * num_cus) / tiles);
+  int parts = (int)(((long)std::max(a.split_items_per_cu, 1) * num_cus) / tiles);
   parts = std::min(parts, a.K / depth);
   parts = std::min(parts, 8);
   while (parts > 1 && (size_t)parts * a.M * a.N > a.ws_floats) --parts;
