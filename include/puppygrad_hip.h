@@ -322,6 +322,37 @@ pg_status pg_device_free(int32_t device, void* ptr);
 pg_status pg_device_upload(int32_t device, void* dst_device, const void* src_host, size_t bytes);
 pg_status pg_device_download(int32_t device, void* dst_host, const void* src_device, size_t bytes);
 
+/* The op-level entry points above on DEVICE operands: the launches are queued on `stream`
+ * (a hipStream_t, NULL for the default stream) and nothing is waited for, so a model that
+ * shares these kernels (src/models/whisper/runtime.rs:43-47 is where a backend would plug
+ * in) keeps its activations in HBM from one op to the next. */
+/* transposed_dense_projection_into (cpu.rs:58-75): weight is [out,in]. */
+pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                          uint64_t in_features, uint64_t out_features, const float* weight,
+                          const float* bias, float* out);
+/* dense_projection_into (cpu.rs:77-97): weight is [in,out] (in_features <= 4096). */
+pg_status pg_op_dense_in_out_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                                 uint64_t in_features, uint64_t out_features, const float* weight,
+                                 const float* bias, float* out);
+/* layer_norm_in_place (cpu.rs:119-143), gelu_in_place (145-150), softmax_in_place per row
+ * (152-165), add_in_place (167-171), argmax_logits (generation.rs:269-279; out is a device
+ * pointer to one id). */
+pg_status pg_op_layer_norm_dev(int32_t device, void* stream, float* x, uint64_t rows, uint64_t cols,
+                               const float* gamma, const float* beta, float eps);
+pg_status pg_op_gelu_dev(int32_t device, void* stream, float* values, uint64_t n);
+pg_status pg_op_softmax_dev(int32_t device, void* stream, float* values, uint64_t rows, uint64_t cols);
+pg_status pg_op_add_dev(int32_t device, void* stream, float* dst, const float* src, uint64_t n);
+pg_status pg_op_argmax_dev(int32_t device, void* stream, const float* values, uint64_t n,
+                           uint32_t* out);
+/* attention_values_into (src/models/whisper/model.rs:1262-1357), the attention of the
+ * reference's other model family: q is [query_rows][state], k and v are [key_rows][state]
+ * with the heads side by side in a row; every query attends to all keys (cross attention,
+ * encoder self attention) or, with causal != 0, to keys <= its own index; out is
+ * [query_rows][state].  head_dim = state / heads <= 256, key_rows <= 15360. */
+pg_status pg_op_attention_dev(int32_t device, void* stream, const float* q, const float* k,
+                              const float* v, uint64_t query_rows, uint64_t key_rows, uint64_t state,
+                              uint64_t heads, int32_t causal, float* out);
+
 /* pg_op_attention_decode for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
  * the reference.  qkv ([3 * n_head * head_dim]), keys and values ([head][max_seq_len][head_dim],

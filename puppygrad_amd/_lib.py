@@ -144,6 +144,16 @@ SIGNATURES = {
     "pg_device_free": (C.c_int, [C.c_int32, _vp]),
     "pg_device_upload": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
     "pg_device_download": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
+    "pg_op_dense_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64, _vp, _vp, _vp]),
+    "pg_op_dense_in_out_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64, _vp,
+                                         _vp, _vp]),
+    "pg_op_layer_norm_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, _vp, _vp, C.c_float]),
+    "pg_op_gelu_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64]),
+    "pg_op_softmax_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64]),
+    "pg_op_add_dev": (C.c_int, [C.c_int32, _vp, _vp, _vp, C.c_uint64]),
+    "pg_op_argmax_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, _vp]),
+    "pg_op_attention_dev": (C.c_int, [C.c_int32, _vp, _vp, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64,
+                                      C.c_uint64, C.c_int32, _vp]),
     "pg_op_attention_decode_noalloc": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, _vp, _vp,
                                                  C.c_uint64, C.c_uint64, C.c_uint64, _vp]),
     "pg_kv_cache_debug_epoch": (C.c_uint32, [_vp]),

@@ -1,6 +1,8 @@
 // Device-operand side of the op-level seam of libpuppygrad_hip.so: plain device buffers for
-// callers that keep their operands in HBM between calls, and the one entry point of the
-// library that allocates nothing (pg_op_attention_decode_noalloc).  The public contract is
+// callers that keep their operands in HBM between calls, the cpu.rs ops on such operands
+// (with the [in,out] dense projection and the row-major multi-query attention that the
+// reference's other model family uses), and the one entry point of the library that
+// allocates nothing (pg_op_attention_decode_noalloc).  The public contract is
 // include/puppygrad_hip.h.
 #include "../../include/puppygrad_hip.h"
 
@@ -70,6 +72,103 @@ pg_status scratch_of(int device, float** ptr, int* num_cus) {
   *ptr = g_scratch_ptr[device];
   *num_cus = g_scratch_cus[device];
   return PG_OK;
+}
+
+
+// ---- kernels of the ops that only exist with device operands ------------------------------
+constexpr int kBlk = 256;
+
+// dense_projection_into (src/models/cpu.rs:77-97): weight is [in,out].  A thread owns one
+// output column and kRowsPerBlock rows of x (staged in LDS); consecutive threads read
+// consecutive floats of a weight row, and every weight is read once per row group.  The sum
+// starts from the bias and adds in ascending i, as the reference does.
+constexpr int kRowsPerBlock = 4;
+__global__ __launch_bounds__(kBlk) void k_dense_in_out(const float* __restrict__ x, int rows, int in_f,
+                                                       int out_f, const float* __restrict__ w,
+                                                       const float* __restrict__ bias,
+                                                       float* __restrict__ out) {
+  extern __shared__ float xs[];  // [kRowsPerBlock][in_f]
+  const int r0 = blockIdx.y * kRowsPerBlock;
+  const int nr = min(kRowsPerBlock, rows - r0);
+  for (int i = threadIdx.x; i < nr * in_f; i += kBlk) xs[i] = x[(size_t)r0 * in_f + i];
+  __syncthreads();
+  const int o = blockIdx.x * kBlk + threadIdx.x;
+  if (o >= out_f) return;
+  float acc[kRowsPerBlock];
+#pragma unroll
+  for (int r = 0; r < kRowsPerBlock; ++r) acc[r] = bias[o];
+  for (int i = 0; i < in_f; ++i) {
+    const float wv = w[(size_t)i * out_f + o];
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; ++r)
+      if (r < nr) acc[r] += xs[r * in_f + i] * wv;
+  }
+  for (int r = 0; r < nr; ++r) out[(size_t)(r0 + r) * out_f + o] = acc[r];
+}
+
+__device__ __forceinline__ float blk_reduce(float v, float* red, bool is_max) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = is_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int w = 1; w < kBlk / 64; ++w) t = is_max ? fmaxf(t, red[w]) : t + red[w];
+  return t;
+}
+
+// attention_values_into (src/models/whisper/model.rs:1262-1357): q [query_rows][state], k and v
+// [key_rows][state], heads side by side in a row; scores = q . k * 1/sqrt(head_dim), softmax
+// over the keys a query may see (all of them, or keys <= query when causal), out = weights . v.
+// One block per (query, head); the scores of the row live in LDS.
+__global__ __launch_bounds__(kBlk) void k_attention_rows(const float* __restrict__ q,
+                                                         const float* __restrict__ k,
+                                                         const float* __restrict__ v, int key_rows,
+                                                         int state, int hd, int causal,
+                                                         float* __restrict__ out) {
+  extern __shared__ float sc[];  // [key_rows]
+  __shared__ float red[kBlk / 64];
+  const int query = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int max_key = causal ? min(query + 1, key_rows) : key_rows;
+  const float scale = 1.0f / sqrtf((float)hd);
+  const float* qh = q + (size_t)query * state + (size_t)head * hd;
+  float mx = -INFINITY;
+  for (int key = tid; key < max_key; key += kBlk) {
+    const float* kh = k + (size_t)key * state + (size_t)head * hd;
+    float s = 0.0f;
+    for (int i = 0; i < hd; ++i) s += qh[i] * kh[i];
+    s *= scale;
+    sc[key] = s;
+    mx = fmaxf(mx, s);
+  }
+  mx = blk_reduce(mx, red, true);
+  float sum = 0.0f;
+  for (int key = tid; key < max_key; key += kBlk) {
+    const float p = expf(sc[key] - mx);  // softmax_in_place (cpu.rs:152-165)
+    sc[key] = p;
+    sum += p;
+  }
+  sum = blk_reduce(sum, red, false);
+  const float inv = 1.0f / sum;
+  __syncthreads();
+  // groups of threads share an output dimension and split the keys between them
+  const int groups = max(1, kBlk / hd);  // threads per dimension
+  const int d = tid % hd, g = tid / hd;
+  float acc = 0.0f;
+  if (g < groups && d < hd && tid < groups * hd)
+    for (int key = g; key < max_key; key += groups)
+      acc += sc[key] * inv * v[(size_t)key * state + (size_t)head * hd + d];
+  __shared__ float part[kBlk];
+  part[tid] = (tid < groups * hd) ? acc : 0.0f;
+  __syncthreads();
+  if (tid < hd && tid < kBlk) {
+    float t = 0.0f;
+    for (int gg = 0; gg < groups; ++gg) t += part[gg * hd + tid];
+    out[(size_t)query * state + (size_t)head * hd + tid] = t;
+  }
 }
 
 }  // namespace
@@ -142,6 +241,118 @@ pg_status pg_op_attention_decode_noalloc(int32_t device, void* stream, const flo
   PG_HIP(pgk::launch_kv_append(qkv, 1, C, hd, P, (int)pos, keys, values, 0, st));
   PG_HIP(pgk::launch_attn_decode(qkv, keys, values, (int)pos, P, H, hd, nsplit, pa, pm, pl, st));
   PG_HIP(pgk::launch_attn_finish(pa, pm, pl, H, hd, nsplit, out, st));
+  return PG_OK;
+}
+
+// ---- the cpu.rs ops on device operands: queued on `stream`, nothing is waited for -----------
+
+pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                          uint64_t in_f, uint64_t out_f, const float* weight, const float* bias,
+                          float* out) {
+  if (!x || !weight || !bias || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
+    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0) return PG_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  pgk::GemmArgs ga{};
+  ga.A = x; ga.W = weight; ga.bias = bias; ga.resid = nullptr; ga.C = out;
+  ga.M = (int)rows; ga.N = (int)out_f; ga.K = (int)in_f; ga.lda = (int)in_f; ga.ldc = (int)out_f;
+  if (rows >= 16 && pgk::gemm_supported(ga)) {
+    int cus = 0;
+    PG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    PG_HIP(pgk::launch_gemm(ga, pgk::GEMM_BIAS, cus, st));  // no workspace: never cut along K
+  } else {
+    for (uint64_t r = 0; r < rows; ++r) {
+      pgk::GemvArgs a{};
+      a.W = weight; a.bias = bias; a.x = x + r * in_f; a.y = out + r * out_f;
+      a.K = (int)in_f; a.nout = (int)out_f;
+      PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_BIAS, st));
+    }
+  }
+  return PG_OK;
+}
+
+pg_status pg_op_dense_in_out_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                                 uint64_t in_f, uint64_t out_f, const float* weight,
+                                 const float* bias, float* out) {
+  if (!x || !weight || !bias || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (in_f == 0 || in_f > 4096 || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
+    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,4096] for [in,out] weights, "
+                                       "out_features >= 1");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0) return PG_OK;
+  const dim3 grid((unsigned)((out_f + kBlk - 1) / kBlk), (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock));
+  hipLaunchKernelGGL(k_dense_in_out, grid, dim3(kBlk), kRowsPerBlock * in_f * sizeof(float),
+                     static_cast<hipStream_t>(stream), x, (int)rows, (int)in_f, (int)out_f, weight,
+                     bias, out);
+  PG_HIP(hipGetLastError());
+  return PG_OK;
+}
+
+pg_status pg_op_layer_norm_dev(int32_t device, void* stream, float* x, uint64_t rows, uint64_t cols,
+                               const float* gamma, const float* beta, float eps) {
+  if (!x || !gamma || !beta) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (cols == 0 || cols > 16384 || rows > (1u << 30))
+    return pgh::fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16384]");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0) return PG_OK;
+  PG_HIP(pgk::launch_layer_norm(x, (int)rows, (int)cols, gamma, beta, eps, static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_gelu_dev(int32_t device, void* stream, float* v, uint64_t n) {
+  if (!v) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (n) PG_HIP(pgk::launch_gelu(v, n, static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_softmax_dev(int32_t device, void* stream, float* v, uint64_t rows, uint64_t cols) {
+  if (!v) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (rows > (1u << 30) || cols > (1u << 30)) return pgh::fail(PG_INVALID_INPUT, "softmax: rows/cols too large");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows && cols) PG_HIP(pgk::launch_softmax(v, (int)rows, (int)cols, static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_add_dev(int32_t device, void* stream, float* dst, const float* src, uint64_t n) {
+  if (!dst || !src) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (n) PG_HIP(pgk::launch_add(dst, src, n, static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_argmax_dev(int32_t device, void* stream, const float* v, uint64_t n, uint32_t* out) {
+  if (!v || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (n == 0 || n > (1u << 30)) return pgh::fail(PG_INVALID_INPUT, "argmax: n must be in [1, 2^30]");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  PG_HIP(pgk::launch_argmax(v, (int)n, out, static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_attention_dev(int32_t device, void* stream, const float* q, const float* k,
+                              const float* v, uint64_t query_rows, uint64_t key_rows, uint64_t state,
+                              uint64_t heads, int32_t causal, float* out) {
+  if (!q || !k || !v || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (heads == 0 || state == 0 || state % heads != 0 || state > 16384 || state / heads > kBlk ||
+      key_rows == 0 || key_rows > 15360 || query_rows > (1u << 20) || heads > 65535)
+    return pgh::fail(PG_INVALID_INPUT, "attention: state must be heads * head_dim with head_dim <= 256, "
+                                       "key_rows in [1,15360]");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (query_rows == 0) return PG_OK;
+  hipLaunchKernelGGL(k_attention_rows, dim3((unsigned)query_rows, (unsigned)heads), dim3(kBlk),
+                     key_rows * sizeof(float), static_cast<hipStream_t>(stream), q, k, v, (int)key_rows,
+                     (int)state, (int)(state / heads), causal ? 1 : 0, out);
+  PG_HIP(hipGetLastError());
   return PG_OK;
 }
 

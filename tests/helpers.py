@@ -76,3 +76,26 @@ def small_cases():
     out.append(("odd", cfg, synth.random_weights(cfg, 0x5EED0202, std=0.08, perturb=True),
                 list(synth.token_ids(23, 0x70C00202, 300))))
     return out
+
+
+class DeviceArray:
+    """A host array mirrored in a device buffer of the library (pg_device_*)."""
+
+    def __init__(self, host, dtype=np.float32):
+        import ctypes as C
+        from puppygrad_amd import _lib
+        self._C, self.lib = C, _lib.load()
+        self.host = np.ascontiguousarray(host, dtype=dtype)
+        self.ptr = C.c_void_p()
+        assert self.lib.pg_device_alloc(0, self.host.nbytes, C.byref(self.ptr)) == 0
+        assert self.lib.pg_device_upload(0, self.ptr, self.host.ctypes.data_as(C.c_void_p),
+                                         self.host.nbytes) == 0
+
+    def download(self) -> np.ndarray:
+        out = np.empty_like(self.host)
+        assert self.lib.pg_device_download(0, out.ctypes.data_as(self._C.c_void_p), self.ptr,
+                                           out.nbytes) == 0
+        return out
+
+    def free(self):
+        assert self.lib.pg_device_free(0, self.ptr) == 0

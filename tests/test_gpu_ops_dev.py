@@ -1,0 +1,129 @@
+"""The op-level seam on device operands (what a second model family would call between its own
+steps): each op against the oracle's restatement of src/models/cpu.rs, the [in,out] dense
+projection (cpu.rs:77-97) and the multi-query attention of the reference's Whisper model
+(src/models/whisper/model.rs:1262-1357), chained without leaving the device."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import DeviceArray
+from puppygrad_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def ok(status):
+    assert status == 0, _lib.load().pg_last_error_message().decode()
+
+
+def attention_values(q, k, v, heads, causal):
+    """attention_values_into restated in float64 with the oracle's softmax per row."""
+    Tq, state = q.shape
+    Tk = k.shape[0]
+    hd = state // heads
+    out = np.zeros((Tq, state), np.float64)
+    for h in range(heads):
+        sl = slice(h * hd, (h + 1) * hd)
+        for i in range(Tq):
+            n = min(i + 1, Tk) if causal else Tk
+            s = (k[:n, sl].astype(np.float64) @ q[i, sl].astype(np.float64)) / np.sqrt(np.float32(hd))
+            p = oracle.softmax(s.astype(np.float32)).astype(np.float64)
+            out[i, sl] = p @ v[:n, sl].astype(np.float64)
+    return out
+
+
+@pytest.mark.parametrize("rows,in_f,out_f", [(1, 8, 5), (3, 100, 257), (7, 384, 1536), (20, 768, 768),
+                                             (1, 4096, 33), (5, 1, 300)])
+def test_dense_with_in_out_weights_matches_oracle(rows, in_f, out_f):
+    rng = np.random.default_rng(rows * 1000 + in_f)
+    x = rng.standard_normal((rows, in_f)).astype(np.float32)
+    w = (rng.standard_normal((in_f, out_f)) / np.sqrt(in_f)).astype(np.float32)
+    b = rng.standard_normal(out_f).astype(np.float32)
+    dx, dw, db, dy = DeviceArray(x), DeviceArray(w), DeviceArray(b), DeviceArray(np.zeros((rows, out_f)))
+    ok(_lib.load().pg_op_dense_in_out_dev(0, None, dx.ptr, rows, in_f, out_f, dw.ptr, db.ptr, dy.ptr))
+    want = oracle.dense(x, rows, in_f, out_f, w, b).reshape(rows, out_f)
+    np.testing.assert_allclose(dy.download(), want, atol=2e-5, rtol=1e-4)
+    # the same product through the [out,in] entry point on the transposed weights
+    dwt = DeviceArray(np.ascontiguousarray(w.T))
+    ok(_lib.load().pg_op_dense_dev(0, None, dx.ptr, rows, in_f, out_f, dwt.ptr, db.ptr, dy.ptr))
+    np.testing.assert_allclose(dy.download(), want, atol=2e-5, rtol=1e-4)
+    for d in (dx, dw, db, dy, dwt):
+        d.free()
+
+
+@pytest.mark.parametrize("Tq,Tk,state,heads,causal", [(1, 1, 8, 2, 0), (5, 5, 24, 3, 1), (6, 1500, 384, 6, 0),
+                                                      (40, 40, 384, 6, 1), (3, 700, 1280, 20, 0),
+                                                      (9, 4, 64, 1, 1), (2, 33, 512, 2, 0)])
+def test_attention_rows_matches_the_reference_formula(Tq, Tk, state, heads, causal):
+    rng = np.random.default_rng(Tq * 100 + Tk)
+    q = rng.standard_normal((Tq, state)).astype(np.float32)
+    k = rng.standard_normal((Tk, state)).astype(np.float32)
+    v = rng.standard_normal((Tk, state)).astype(np.float32)
+    dq, dk, dv, dout = DeviceArray(q), DeviceArray(k), DeviceArray(v), DeviceArray(np.zeros((Tq, state)))
+    ok(_lib.load().pg_op_attention_dev(0, None, dq.ptr, dk.ptr, dv.ptr, Tq, Tk, state, heads, causal, dout.ptr))
+    np.testing.assert_allclose(dout.download(), attention_values(q, k, v, heads, bool(causal)),
+                               atol=2e-5, rtol=1e-4)
+    for d in (dq, dk, dv, dout):
+        d.free()
+
+
+def test_an_encoder_style_block_stays_on_the_device():
+    """LayerNorm -> q/k/v projections -> attention over all keys -> projection + residual ->
+    LayerNorm -> fc + GELU -> projection + residual -> argmax, op by op on device buffers,
+    against the same chain of oracle ops on the host."""
+    rng = np.random.default_rng(7)
+    T, S, H, I = 12, 128, 4, 512
+    lib = _lib.load()
+    x = rng.standard_normal((T, S)).astype(np.float32)
+    p = {n: (rng.standard_normal(shape) * 0.1).astype(np.float32) for n, shape in
+         [("wq", (S, S)), ("wk", (S, S)), ("wv", (S, S)), ("wo", (S, S)), ("w1", (I, S)), ("w2", (S, I)),
+          ("bq", S), ("bk", S), ("bv", S), ("bo", S), ("b1", I), ("b2", S), ("g1", S), ("be1", S),
+          ("g2", S), ("be2", S)]}
+    # host chain with the oracle's ops
+    xn = oracle.layer_norm(x, T, S, p["g1"], p["be1"], 1e-5).reshape(T, S)
+    q = oracle.transposed_dense(xn, T, S, S, p["wq"], p["bq"]).reshape(T, S)
+    k = oracle.transposed_dense(xn, T, S, S, p["wk"], p["bk"]).reshape(T, S)
+    v = oracle.transposed_dense(xn, T, S, S, p["wv"], p["bv"]).reshape(T, S)
+    att = attention_values(q, k, v, H, False).astype(np.float32)
+    x1 = oracle.add(x.reshape(-1), oracle.transposed_dense(att, T, S, S, p["wo"], p["bo"])).reshape(T, S)
+    xn2 = oracle.layer_norm(x1, T, S, p["g2"], p["be2"], 1e-5).reshape(T, S)
+    h = oracle.gelu(oracle.transposed_dense(xn2, T, S, I, p["w1"], p["b1"]))
+    want = oracle.add(x1.reshape(-1), oracle.transposed_dense(h.reshape(T, I), T, I, S, p["w2"], p["b2"]))
+    # device chain
+    d = {n: DeviceArray(a) for n, a in p.items()}
+    dx, dxn = DeviceArray(x), DeviceArray(x)
+    dq, dk, dv, datt, dtmp = (DeviceArray(np.zeros((T, S))) for _ in range(5))
+    dh = DeviceArray(np.zeros((T, I)))
+    did = DeviceArray(np.zeros(1, np.uint32), dtype=np.uint32)
+    ok(lib.pg_op_layer_norm_dev(0, None, dxn.ptr, T, S, d["g1"].ptr, d["be1"].ptr, 1e-5))
+    for w, b, dst in (("wq", "bq", dq), ("wk", "bk", dk), ("wv", "bv", dv)):
+        ok(lib.pg_op_dense_dev(0, None, dxn.ptr, T, S, S, d[w].ptr, d[b].ptr, dst.ptr))
+    ok(lib.pg_op_attention_dev(0, None, dq.ptr, dk.ptr, dv.ptr, T, T, S, H, 0, datt.ptr))
+    ok(lib.pg_op_dense_dev(0, None, datt.ptr, T, S, S, d["wo"].ptr, d["bo"].ptr, dtmp.ptr))
+    ok(lib.pg_op_add_dev(0, None, dx.ptr, dtmp.ptr, T * S))
+    ok(lib.pg_device_upload(0, dxn.ptr, dx.download().ctypes.data_as(C.c_void_p), T * S * 4))
+    ok(lib.pg_op_layer_norm_dev(0, None, dxn.ptr, T, S, d["g2"].ptr, d["be2"].ptr, 1e-5))
+    ok(lib.pg_op_dense_dev(0, None, dxn.ptr, T, S, I, d["w1"].ptr, d["b1"].ptr, dh.ptr))
+    ok(lib.pg_op_gelu_dev(0, None, dh.ptr, T * I))
+    ok(lib.pg_op_dense_dev(0, None, dh.ptr, T, I, S, d["w2"].ptr, d["b2"].ptr, dtmp.ptr))
+    ok(lib.pg_op_add_dev(0, None, dx.ptr, dtmp.ptr, T * S))
+    got = dx.download().reshape(-1)
+    np.testing.assert_allclose(got, want, atol=1e-4, rtol=1e-3)
+    ok(lib.pg_op_softmax_dev(0, None, dx.ptr, T, S))
+    np.testing.assert_allclose(dx.download(), np.stack([oracle.softmax(r) for r in got.reshape(T, S)]),
+                               atol=1e-6, rtol=1e-4)
+    ok(lib.pg_op_argmax_dev(0, None, dx.ptr, T * S, did.ptr))
+    assert int(did.download()[0]) == oracle.argmax_logits(dx.download().reshape(-1))
+
+
+def test_device_ops_refuse_bad_shapes():
+    lib = _lib.load()
+    one = DeviceArray(np.zeros(8))
+    assert lib.pg_op_dense_in_out_dev(0, None, one.ptr, 1, 5000, 4, one.ptr, one.ptr, one.ptr) == _lib.PG_INVALID_INPUT
+    assert lib.pg_op_attention_dev(0, None, one.ptr, one.ptr, one.ptr, 1, 1, 10, 3, 0, one.ptr) == _lib.PG_INVALID_INPUT
+    assert b"state must be heads * head_dim" in lib.pg_last_error_message()
+    assert lib.pg_op_attention_dev(0, None, one.ptr, one.ptr, one.ptr, 1, 0, 8, 2, 0, one.ptr) == _lib.PG_INVALID_INPUT
+    assert lib.pg_op_layer_norm_dev(0, None, None, 1, 8, one.ptr, one.ptr, 1e-5) == _lib.PG_INVALID_INPUT
+    one.free()

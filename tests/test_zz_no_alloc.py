@@ -7,27 +7,10 @@ import ctypes as C
 import numpy as np
 import pytest
 
+from helpers import DeviceArray
 from puppygrad_amd import _lib
 
 pytestmark = pytest.mark.gpu
-
-
-class DeviceArray:
-    def __init__(self, host: np.ndarray):
-        self.lib = _lib.load()
-        self.host = np.ascontiguousarray(host, dtype=np.float32)
-        self.ptr = C.c_void_p()
-        assert self.lib.pg_device_alloc(0, self.host.nbytes, C.byref(self.ptr)) == 0
-        assert self.lib.pg_device_upload(0, self.ptr, self.host.ctypes.data_as(C.c_void_p),
-                                         self.host.nbytes) == 0
-
-    def download(self) -> np.ndarray:
-        out = np.empty_like(self.host)
-        assert self.lib.pg_device_download(0, out.ctypes.data_as(C.c_void_p), self.ptr, out.nbytes) == 0
-        return out
-
-    def free(self):
-        assert self.lib.pg_device_free(0, self.ptr) == 0
 
 
 def attention_case(seed, H, hd, P, pos):
