@@ -203,7 +203,12 @@ double pg_rng_next_unit_f64(pg_rng_state* rng);
  * (generation.rs:281-362).  Greedy selection is an argmax on the device; with top_k the
  * penalty, the finite filter and the choice of the k candidates run on the device and only
  * those k pairs reach the host, which draws from them in f64 as the reference does; without
- * top_k the row is copied to the host. */
+ * top_k the whole draw (f64 weights of every finite candidate, top-p prefix, inverse-CDF walk
+ * for the generator's next uniform value) runs on the device and only the id comes back.  The
+ * device leaves a draw undecided when its target lies within a relative 1e-9 of the boundary
+ * between two candidates (its sums are f64 but not added in the reference's order); such a
+ * draw, a top_k above 4096 and a greedy selection under a repeat penalty copy the row to the
+ * host and use the reference's exact arithmetic there. */
 pg_status pg_logits_sample(pg_logits* logits, uint32_t row, const uint32_t* history, size_t n_hist,
                            const pg_sampling* sampling, pg_rng_state* rng, uint32_t* out);
 
@@ -436,6 +441,10 @@ void pg_synth_token_ids(uint32_t* dst, uint64_t n, uint64_t seed, uint64_t vocab
  * generating 2^31 tokens first. */
 uint32_t pg_kv_cache_debug_epoch(const pg_kv_cache* cache);
 pg_status pg_kv_cache_debug_set_epoch(pg_kv_cache* cache, uint32_t epoch);
+
+/* Test hook: selections that pg_logits_sample drew entirely on the device since the process
+ * started, and selections for which it copied the row of logits to the host. */
+void pg_debug_sample_counts(uint64_t* device_draws, uint64_t* host_rows);
 
 /* Device facts for the benchmark harness. */
 typedef struct pg_device_info {

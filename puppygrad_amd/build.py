@@ -9,7 +9,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libpuppygrad_hip.so"
-SOURCES = ["pg_kernels.hip", "pg_decode.hip", "pg_prefill.hip", "pg_ops_dev.hip",
+SOURCES = ["pg_kernels.hip", "pg_decode.hip", "pg_prefill.hip", "pg_ops_dev.hip", "pg_sample.hip",
            "pg_host.cpp", "pg_assets.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

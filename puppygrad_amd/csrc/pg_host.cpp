@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -25,6 +26,10 @@
 namespace {
 
 thread_local std::string g_err;
+
+// Test hook counters: selections drawn entirely on the device, and selections for which the row
+// of logits was copied to the host.
+std::atomic<uint64_t> g_device_draws{0}, g_host_draws{0};
 
 pg_status fail(pg_status s, const std::string& msg) {
   g_err = msg;
@@ -1578,6 +1583,46 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
     }
     return sample_sorted(cand, *sampling, rng, out);
   }
+  // Sampling without top_k: the whole draw runs on the device (weights of every finite candidate
+  // in f64, top-p prefix, inverse-CDF walk) and only the id comes back.  The uniform value is
+  // drawn here from a copy of the generator, which is committed only when the device used it;
+  // a draw the device leaves undecided (a target within a relative 1e-9 of the boundary between
+  // two candidates, or thousands of nearly equal logits) is repeated below on the host with the
+  // reference's exact arithmetic.
+  if (sampling->temperature > 0.0f && !sampling->has_top_k &&
+      l->vocab <= (uint64_t)pgk::kTopkMaxVocab && recent <= kMaxRecent && (recent == 0 || history)) {
+    if (!c->d_cand) {
+      PG_HIP(hipMalloc(&c->d_cand, (2 * kMaxCand + 4) * sizeof(uint32_t)));
+      PG_HIP(hipHostMalloc(&c->h_cand, (2 * kMaxCand + 4) * sizeof(uint32_t), hipHostMallocDefault));
+      PG_HIP(hipMalloc(&c->d_recent, kMaxRecent * sizeof(uint32_t)));
+      PG_HIP(hipHostMalloc(&c->h_recent, kMaxRecent * sizeof(uint32_t), hipHostMallocDefault));
+    }
+    if (recent) {
+      std::memcpy(c->h_recent, history + (n_hist - recent), recent * sizeof(uint32_t));
+      PG_HIP(hipMemcpyAsync(c->d_recent, c->h_recent, recent * sizeof(uint32_t),
+                            hipMemcpyHostToDevice, c->stream));
+    }
+    pg_rng_state ahead = *rng;
+    const double u = pg_rng_next_unit_f64(&ahead);
+    PG_HIP(pgk::launch_sample_select(l->data + (size_t)row * l->vocab, (int)l->vocab, c->d_recent,
+                                     (int)recent, sampling->repeat_penalty,
+                                     (double)sampling->temperature, sampling->has_top_p ? 1 : 0,
+                                     (double)sampling->top_p, u, c->d_cand, c->stream));
+    PG_HIP(hipMemcpyAsync(c->h_cand, c->d_cand, 2 * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                          c->stream));
+    PG_HIP(hipStreamSynchronize(c->stream));
+    if (c->h_cand[0] == 0u) {
+      *rng = ahead;
+      *out = c->h_cand[1];
+      g_device_draws.fetch_add(1, std::memory_order_relaxed);
+      return PG_OK;
+    }
+    if (c->h_cand[0] == 3u)
+      return fail(PG_INVALID_INPUT,
+                  "token sampling failed: cannot sample from empty or non-finite logits");
+    // undecided: fall through to the host
+  }
+  g_host_draws.fetch_add(1, std::memory_order_relaxed);
   std::vector<float> adjusted(l->vocab);
   PG_HIP(hipStreamSynchronize(c->stream));
   PG_HIP(hipMemcpy(adjusted.data(), l->data + (size_t)row * l->vocab, l->vocab * sizeof(float),
@@ -1589,6 +1634,11 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
     return PG_OK;
   }
   return sample_logits(adjusted, *sampling, rng, out);
+}
+
+void pg_debug_sample_counts(uint64_t* device_draws, uint64_t* host_rows) {
+  if (device_draws) *device_draws = g_device_draws.load(std::memory_order_relaxed);
+  if (host_rows) *host_rows = g_host_draws.load(std::memory_order_relaxed);
 }
 
 // Shared body of the two greedy-decode entry points.  Selects up to `steps`

@@ -89,6 +89,15 @@ hipError_t launch_argmax(const float* v, int n, uint32_t* out, hipStream_t s, in
 constexpr int kTopkMaxVocab = 131072;
 hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
                               float penalty, int k, uint32_t* out, hipStream_t s);
+// sample_logits (src/models/generation.rs:300-362) without top_k for one row of V logits: the
+// repeat penalty over the n_pen recent ids, f64 weights exp(l / T - max / T) of the finite
+// candidates in the stable descending order, the top-p prefix and the inverse-CDF walk for the
+// uniform draw u.  out[0] = 0: out[1] is the drawn id; 2: not decided on the device (a target
+// within a relative 1e-9 of a boundary, or too many nearly equal logits): the caller repeats
+// the selection on the host; 3: no finite candidate.  V <= kTopkMaxVocab.
+hipError_t launch_sample_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
+                                float penalty, double temperature, int has_top_p, double top_p,
+                                double u, uint32_t* out, hipStream_t s);
 // x[b] = wte[ids[b]] + wpe[pos]
 hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
                               int batch, int pos, int C, hipStream_t s, int w_bf16 = 0);

@@ -457,3 +457,85 @@ def test_config4_gpt2_xl_long_context_greedy_decode_parity():
     if explained == 0:
         assert got == want[896:]
     assert cache.seq_len == 896 + 127  # the forward after the last token is skipped
+
+
+def sample_counts():
+    import ctypes as C
+    from puppygrad_amd import _lib
+    dev, host = C.c_uint64(), C.c_uint64()
+    _lib.load().pg_debug_sample_counts(C.byref(dev), C.byref(host))
+    return dev.value, host.value
+
+
+@pytest.mark.parametrize("vocab,ties", [(131, 0), (6011, 0), (50257, 0), (6011, 997)])
+def test_sampling_without_top_k_is_drawn_on_the_device(vocab, ties):
+    """Temperature and top-p sampling over the whole vocabulary (sample_logits,
+    generation.rs:300-362) without the row of logits leaving the device: every draw equals the
+    oracle's sampler on the same logits, and the library's counters show that no row was copied
+    to the host.  With `ties`, wte rows repeat so that the stable order among equal logits
+    decides which id a draw lands on."""
+    cfg = synth.Gpt2Config(vocab_size=vocab, n_positions=32, n_embd=128, n_layer=1, n_head=2)
+    w = synth.random_weights(cfg, 0x5EED0700 + vocab, std=0.05, perturb=True)
+    if ties:
+        wte = np.asarray(w.wte, np.float32).reshape(vocab, cfg.n_embd).copy()
+        for i in range(vocab):
+            wte[i] = wte[i % ties]
+        wte[11] = np.inf
+        wte[vocab - 5] = -np.inf
+        w.wte = wte.reshape(-1)
+    ids = [int(t) for t in synth.token_ids(9, 0x70C00700, min(vocab, 900)) if t != 11] or [1]
+    model = Gpt2Model.new(cfg, w)
+    cache = model.new_kv_cache()
+    logits = model.prefill(ids, cache)
+    host = logits.to_host()
+    cases = [dict(temperature=1.0), dict(temperature=0.7), dict(temperature=2.5), dict(temperature=0.05),
+             dict(temperature=1.0, top_p=0.9), dict(temperature=0.8, top_p=0.5), dict(temperature=1.3, top_p=0.05),
+             dict(temperature=1.0, top_p=1.0), dict(temperature=1.0, top_p=0.999),
+             dict(temperature=1.0, repeat_penalty=1.3), dict(temperature=0.9, top_p=0.8, repeat_penalty=0.7, repeat_last_n=4)]
+    dev0, host0 = sample_counts()
+    calls = 0
+    for kw in cases:
+        for seed in range(1, 13):
+            g = TextGenerationConfig(1, seed=seed, **kw)
+            sampler, ref_sampler = LogitsSampler(seed), oracle.LogitsSampler(seed)
+            for draw in range(3):  # consecutive draws: the generator advances exactly as the oracle's
+                got = sampler.select_next_token(logits, ids, g)
+                want = ref_sampler.select_next_token(host, ids, oracle.sampling(seed=seed, **kw))
+                assert got == want, (kw, seed, draw)
+                calls += 1
+    dev1, host1 = sample_counts()
+    assert (dev1 - dev0) + (host1 - host0) == calls
+    # (a draw within 1e-9 of a boundary would be repeated on the host; none is expected here)
+    assert host1 - host0 <= 2 and dev1 - dev0 >= calls - 2
+
+
+def test_sampling_over_equal_logits_falls_back_to_the_host():
+    """A vocabulary whose logits are all equal: more candidates in one value bin than the device
+    sorts, so the draw is repeated on the host, and still equals the oracle's."""
+    cfg = synth.Gpt2Config(vocab_size=5003, n_positions=16, n_embd=64, n_layer=1, n_head=1)
+    w = synth.random_weights(cfg, 0x5EED0710, perturb=True)
+    wte = np.asarray(w.wte, np.float32).reshape(cfg.vocab_size, cfg.n_embd).copy()
+    wte[:] = wte[0]
+    w.wte = wte.reshape(-1)
+    model = Gpt2Model.new(cfg, w)
+    cache = model.new_kv_cache()
+    logits = model.prefill([3, 4], cache)
+    host = logits.to_host()
+    assert len(np.unique(host)) == 1
+    dev0, host0 = sample_counts()
+    for seed in (1, 2, 3):
+        got = LogitsSampler(seed).select_next_token(logits, [3, 4], TextGenerationConfig(1, seed=seed, temperature=1.0, top_p=0.7))
+        want = oracle.LogitsSampler(seed).select_next_token(host, [3, 4], oracle.sampling(seed=seed, temperature=1.0, top_p=0.7))
+        assert got == want
+    dev1, host1 = sample_counts()
+    assert host1 - host0 == 3 and dev1 == dev0
+
+
+def test_sampled_stream_without_top_k_matches_oracle():
+    _, cfg, w, ids = small_cases()[1]
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w)
+    for kw in (dict(temperature=1.0), dict(temperature=0.8, top_p=0.9, repeat_penalty=1.2)):
+        g = TextGenerationConfig(20, seed=11, **kw)
+        toks, stats = model.stream_token_ids_with_stats(ids, g)
+        want, st, _, _ = ref.stream_token_ids_with_stats(ids, 20, None, oracle.sampling(seed=11, **kw))
+        assert toks == want and stats.generated_tokens == st.generated_tokens
