@@ -143,6 +143,7 @@ struct GemmArgs {
   size_t ws_floats = 0;   // its size
   int tail_first = 0;     // filled by gemm_tail_plan: first tile of the tail that is cut along K,
   int tail_parts = 1;     // and the number of parts
+  int band_rows = 1;      // tile numbering of the tile forms (set by the launcher)
   // Optional: also write LayerNorm(row of C) to ln_out[M][N] (needs ldc == N).  Fused into the
   // split-K reduce where the chosen form has one, a separate launch otherwise.
   float* ln_out = nullptr;
@@ -156,6 +157,12 @@ struct GemmArgs {
   // Tunable: a GEMM whose M x N leaves CUs idle is cut along K into about this many work items
   // per CU (gemm_split_parts).
   int split_items_per_cu = 3;
+  // A forced plan for the tile forms (benchmarks and tests; 0 = the planner chooses): tile
+  // shape, form (1 whole tiles, 2 every tile cut along K into plan_parts, 3 only the last
+  // partial round of tiles cut).
+  int plan_bm = 0, plan_bn = 0, plan_form = 0, plan_parts = 0;
+  int plan_band = 0;  // band height of the tile numbering (0: chosen by the launcher)
+  int plan_bk16 = 0;  // 1: k-tiles of 16 columns also where K would allow 32
 };
 // Element (row b < 32, column k) of a packed activation matrix: the float4 of columns
 // 4j..4j+3 of all 32 rows lie next to each other, so that 32 lanes which each read four
@@ -167,8 +174,8 @@ __host__ __device__ inline size_t packed32_index(size_t b, size_t k) {
 // Whether launch_gemm multiplies an M x K input with the 32-row decode kernel.
 bool gemm_takes_rows32(int M, int K, int lda, int w_bf16);
 bool gemm_supported(const GemmArgs& a);
-int gemm_split_parts(const GemmArgs& a, int num_cus);
-bool gemm_tail_plan(GemmArgs& a, int num_cus);
+int gemm_split_parts(const GemmArgs& a, int num_cus, int bm = 64, int bn = 64);
+bool gemm_tail_plan(GemmArgs& a, int num_cus, int bm = 64, int bn = 64);
 hipError_t launch_gemm(const GemmArgs& a, int epilogue, int num_cus, hipStream_t s);
 // Causal attention over qkv[T][3C] -> out[T][C]; also appends K, V to the cache panels.
 // scratch ([T*H][T] floats) is only used when head_dim != 64.

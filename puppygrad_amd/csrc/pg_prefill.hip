@@ -11,6 +11,8 @@
 
 #include <algorithm>
 
+#include <type_traits>
+
 namespace pgk {
 
 namespace {
@@ -65,6 +67,54 @@ __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
   return *reinterpret_cast<const f4*>(W + idx);
 }
 
+// The same in two steps, so that a tile's widening happens when it is stored to LDS and
+// not where it would wait for the load: the raw 16, 8 or 4 bytes, and their four floats.
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+template <int WT>
+__device__ __forceinline__ auto load_w_raw(const float* W, size_t idx) {
+  if constexpr (WT == 2) {
+    return *reinterpret_cast<const int*>(reinterpret_cast<const signed char*>(W) + idx);
+  } else if constexpr (WT == 1) {
+    return *reinterpret_cast<const u2v*>(reinterpret_cast<const unsigned short*>(W) + idx);
+  } else {
+    return *reinterpret_cast<const f4*>(W + idx);
+  }
+}
+template <int WT, typename R>
+__device__ __forceinline__ f4 widen_w(R w) {
+  if constexpr (WT == 2) {
+    f4 r;
+    r.x = (float)((w << 24) >> 24);
+    r.y = (float)((w << 16) >> 24);
+    r.z = (float)((w << 8) >> 24);
+    r.w = (float)(w >> 24);
+    return r;
+  } else if constexpr (WT == 1) {
+    f4 r;
+    r.x = __uint_as_float(w.x << 16);
+    r.y = __uint_as_float(w.x & 0xffff0000u);
+    r.z = __uint_as_float(w.y << 16);
+    r.w = __uint_as_float(w.y & 0xffff0000u);
+    return r;
+  } else {
+    return w;
+  }
+}
+
+// Tile number -> tile coordinates.  Tiles are numbered band by band (a band is `band` tile
+// rows high), down the columns of a band, so that a run of consecutive numbers, which is
+// what one XCD computes, is a compact block of C: its tiles share few rows of A and of W,
+// which that XCD's L2 then fetches once.  (Row-major numbering makes every XCD read all of
+// W.)
+__device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int band, int* tm, int* tn) {
+  const int per_band = band * tiles_n;
+  const int b = tile / per_band, rem = tile - b * per_band;
+  const int bh = min(band, tiles_m - b * band);
+  const int col = rem / bh;
+  *tn = col;
+  *tm = b * band + (rem - col * bh);
+}
+
 // SPLIT = 1: the K range is cut into gridDim.y parts: part blockIdx.y multiplies its
 // k-tiles and writes the raw partial tile to a.ws[part][M][N]; k_splitk_reduce adds the
 // parts in order and applies bias and epilogue (a fixed order: results do not depend on
@@ -76,14 +126,20 @@ __device__ __forceinline__ f4 load_w4(const float* W, size_t idx) {
 // a.ws[(tile - tail_first) * parts + part][BM][BN] and k_tail_reduce finishes them.
 // WT: how W is stored: 0 f32, 1 bf16, 2 int8 with a.w_scale[n] per row (a weight is
 // (float)q * scale, formed when the tile is loaded: QuantizedRows, cpu.rs:26-56).
-template <int BM, int BN, int EPI, int WT, int SPLIT = 0>
+template <int BM, int BN, int EPI, int WT, int SPLIT = 0, int BKT = BK>
 __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
-  constexpr int LDA = BM + 4, LDB = BN + 4;
-  constexpr int ALD = BM / 64, BLD = BN / 64;  // float4 global loads per thread per tile
-  __shared__ float As[2][BK][LDA];
-  __shared__ float Bs[2][BK][LDB];
+  // BKT columns per k-tile: 32 when K allows (a row's 128 bytes are one cache line, asked
+  // for by one load instruction), 16 otherwise.  LPR lanes load one row's columns; the row
+  // padding keeps the transposing stores of a wavefront (LPR columns-of-four x 64 / LPR
+  // rows) on different banks.
+  constexpr int LPR = BKT / 4, RPP = 256 / LPR;  // lanes per row, rows per pass
+  constexpr int PADR = BKT == 32 ? 2 : 4;
+  constexpr int LDA = BM + PADR, LDB = BN + PADR;
+  constexpr int ALD = BM / RPP, BLD = BN / RPP;  // float4 global loads per thread per tile
+  __shared__ float As[2][BKT][LDA];
+  __shared__ float Bs[2][BKT][LDB];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -106,20 +162,21 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     tile = xcd * per_xcd + slot;
   }
   if (tile >= tiles_all) return;
-  const int tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  int tm, tn;
+  tile_coords(tile, (a.M + BM - 1) / BM, tiles_n, a.band_rows, &tm, &tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   // global load mapping: 4 lanes cover 16 consecutive k of one row
-  const int lr = tid >> 2, lk = (tid & 3) * 4;
+  const int lr = tid / LPR, lk = (tid % LPR) * 4;
   const float* Ag[ALD];
   size_t Wg[BLD];  // element offsets into W
 #pragma unroll
   for (int i = 0; i < ALD; ++i)
-    Ag[i] = a.A + (size_t)min(m0 + lr + 64 * i, a.M - 1) * a.lda + lk;
+    Ag[i] = a.A + (size_t)min(m0 + lr + RPP * i, a.M - 1) * a.lda + lk;
   float wsc[BLD];  // int8: the scale of each row this thread loads
 #pragma unroll
   for (int i = 0; i < BLD; ++i) {
-    const int n = min(n0 + lr + 64 * i, a.N - 1);
+    const int n = min(n0 + lr + RPP * i, a.N - 1);
     Wg[i] = (size_t)n * a.K + lk;
     wsc[i] = WT == 2 ? a.w_scale[n] : 1.0f;
   }
@@ -132,65 +189,116 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  f4 ra[ALD], rb[BLD];
-  const int ktiles_all = a.K / BK;
+  const int ktiles_all = a.K / BKT;
   // this block's k-tiles [kt0, kt1)
   const int kpart = SPLIT == 1 ? (int)blockIdx.y : tail_part;
   const int kparts = SPLIT == 1 ? (int)gridDim.y : (in_tail ? a.tail_parts : 1);
   const int kt0 = (int)(((long)kpart * ktiles_all) / kparts);
   const int kt1 = (int)(((long)(kpart + 1) * ktiles_all) / kparts);
-  const size_t kfirst = (size_t)kt0 * BK;
-#pragma unroll
-  for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + kfirst);
-#pragma unroll
-  for (int i = 0; i < BLD; ++i) {
-    rb[i] = load_w4<WT>(a.W, Wg[i] + kfirst);
-    if (WT == 2) rb[i] *= wsc[i];
-  }
-
+  const int T = kt1 - kt0;
   const int half = lane >> 5, l32 = lane & 31;
-  for (int kt = kt0; kt < kt1; ++kt) {
-    const int buf = (kt - kt0) & 1;
-    // registers -> LDS (transposed)
+
+  // The k loop is software-pipelined by hand.  A wavefront issues in order and an MFMA
+  // occupies the matrix core for 64 clocks, so every LDS access of a tile is placed between
+  // two MFMAs, where its issue and latency cost nothing:
+  //   tile t, first half of the MFMA steps  + LDS stores of tile t+1 (loaded a tile ago)
+  //   barrier; global loads of tile t+2
+  //   tile t, second half of the MFMA steps + LDS reads of tile t+1's operands
+  // so the operands of a tile are in registers (two sets, used in turn) before its first
+  // MFMA.  Left to itself the compiler reads two operands, waits for the LDS, multiplies,
+  // and reads again: the matrix core idles for the LDS latency at every step.
+  constexpr int STEPS = BKT / 2;      // MFMA steps (two columns each) per tile
+  constexpr int H = STEPS / 2;        // steps before the barrier
+  constexpr int NST = 4 * (ALD + BLD);  // scalar LDS stores per thread and tile
+  constexpr int NRD = STEPS * (MB + NB);  // operand reads per lane and tile
+  static_assert(NST % H == 0 && NRD % (STEPS - H) == 0, "whole LDS accesses per step");
+  typedef decltype(load_w_raw<WT>(a.W, 0)) WRaw;
+  f4 ra0[ALD];  // load registers: a tile is asked for one tile's time before it is stored
+  WRaw rb0[BLD];
+  auto load_tile = [&](int t, f4 (&ra)[ALD], WRaw (&rb)[BLD]) __attribute__((always_inline)) {  // global -> registers
+    const size_t k = (size_t)(kt0 + t) * BKT;
 #pragma unroll
-    for (int i = 0; i < ALD; ++i) {
-      As[buf][lk + 0][lr + 64 * i] = ra[i].x;
-      As[buf][lk + 1][lr + 64 * i] = ra[i].y;
-      As[buf][lk + 2][lr + 64 * i] = ra[i].z;
-      As[buf][lk + 3][lr + 64 * i] = ra[i].w;
-    }
+    for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + k);
 #pragma unroll
-    for (int i = 0; i < BLD; ++i) {
-      Bs[buf][lk + 0][lr + 64 * i] = rb[i].x;
-      Bs[buf][lk + 1][lr + 64 * i] = rb[i].y;
-      Bs[buf][lk + 2][lr + 64 * i] = rb[i].z;
-      Bs[buf][lk + 3][lr + 64 * i] = rb[i].w;
-    }
-    __syncthreads();
-    if (kt + 1 < kt1) {
+    for (int i = 0; i < BLD; ++i) rb[i] = load_w_raw<WT>(a.W, Wg[i] + k);
+  };
+  // stores [u0, u1) of a loaded tile into LDS buffer `buf` (transposed)
+  auto store_units = [&](int buf, int u0, int u1, f4 (&ra)[ALD], WRaw (&rb)[BLD]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + (size_t)(kt + 1) * BK);
-#pragma unroll
-      for (int i = 0; i < BLD; ++i) {
-        rb[i] = load_w4<WT>(a.W, Wg[i] + (size_t)(kt + 1) * BK);
-        if (WT == 2) rb[i] *= wsc[i];
+    for (int u = u0; u < u1; ++u) {
+      const int i = u >> 2, j = u & 3;
+      if (i < ALD) {
+        As[buf][lk + j][lr + RPP * i] = ra[i][j];
+      } else {
+        f4 w = widen_w<WT>(rb[i - ALD]);
+        if (WT == 2) w *= wsc[i - ALD];
+        Bs[buf][lk + j][lr + RPP * (i - ALD)] = w[j];
       }
     }
+  };
+  // operand reads [r0, r1) of LDS buffer `buf` into the register set (oa, ob)
+  auto read_units = [&](int buf, int r0, int r1, float (&oa)[STEPS][MB], float (&ob)[STEPS][NB])
+                        __attribute__((always_inline)) {
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float av[MB], bv[NB];
-#pragma unroll
-      for (int i = 0; i < MB; ++i) av[i] = As[buf][kk + half][wm * WM + 32 * i + l32];
-#pragma unroll
-      for (int j = 0; j < NB; ++j) bv[j] = Bs[buf][kk + half][wn * WN + 32 * j + l32];
-#pragma unroll
-      for (int i = 0; i < MB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+    for (int r = r0; r < r1; ++r) {
+      const int st = r / (MB + NB), x = r % (MB + NB);
+      if (x < MB) oa[st][x] = As[buf][2 * st + half][wm * WM + 32 * x + l32];
+      else ob[st][x - MB] = Bs[buf][2 * st + half][wn * WN + 32 * (x - MB) + l32];
     }
-    // the other buffer is free once every wavefront has left it: the barrier at the
-    // top of the next iteration's store is preceded by this iteration's compute
+  };
+  auto mfma_step = [&](int st, float (&oa)[STEPS][MB], float (&ob)[STEPS][NB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(oa[st][i], ob[st][j], acc[i][j], 0, 0, 0);
+  };
+  // Tile t from the set (ca, cb); when `more`, tile t+1 goes load registers (ra, rb) -> LDS ->
+  // (na, nb), and tile t+2 is asked for into (ra, rb).
+  auto tile_step = [&](auto more_c, int t, float (&ca)[STEPS][MB], float (&cb)[STEPS][NB],
+                       float (&na)[STEPS][MB], float (&nb)[STEPS][NB], f4 (&ra)[ALD],
+                       WRaw (&rb)[BLD]) __attribute__((always_inline)) {
+    constexpr bool more = decltype(more_c)::value;
+    const int nbuf = (t + 1) & 1;
+#pragma unroll
+    for (int st = 0; st < H; ++st) {
+      mfma_step(st, ca, cb);
+      if (more) store_units(nbuf, st * (NST / H), (st + 1) * (NST / H), ra, rb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (more) {
+      __syncthreads();
+      load_tile(min(t + 2, T - 1), ra, rb);  // past the end: the last tile again, never used
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int st = H; st < STEPS; ++st) {
+      mfma_step(st, ca, cb);
+      if (more) read_units(nbuf, (st - H) * (NRD / (STEPS - H)), (st - H + 1) * (NRD / (STEPS - H)), na, nb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  if (T > 0) {
+    float pa[STEPS][MB], pb[STEPS][NB], qa[STEPS][MB], qb[STEPS][NB];
+    load_tile(0, ra0, rb0);
+    store_units(0, 0, NST, ra0, rb0);
+    __syncthreads();
+    load_tile(min(1, T - 1), ra0, rb0);
+    read_units(0, 0, NRD, pa, pb);
+    const std::true_type yes;
+    const std::false_type no;
+    int t = 0;
+    for (; t + 2 < T; t += 2) {
+      tile_step(yes, t, pa, pb, qa, qb, ra0, rb0);
+      tile_step(yes, t + 1, qa, qb, pa, pb, ra0, rb0);
+    }
+    if (T - t == 2) {
+      tile_step(yes, t, pa, pb, qa, qb, ra0, rb0);
+      tile_step(no, t + 1, qa, qb, pa, pb, ra0, rb0);
+    } else {
+      tile_step(no, t, pa, pb, qa, qb, ra0, rb0);
+    }
   }
 
   // epilogue
@@ -534,20 +642,22 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   }
 }
 
-// The same for the tail tiles of the SPLIT = 2 form: block (x, y) finishes a quarter of
-// tail tile y (tile-local partials, BM = BN = 64).
-template <int EPI>
+// The same for the tail tiles of the SPLIT = 2 form: block (x, y) finishes 256 float4 of
+// tail tile y (tile-local partials of BM x BN floats).
+template <int BM, int BN, int EPI>
 __global__ __launch_bounds__(256) void k_tail_reduce(GemmArgs a) {
+  constexpr int kTile = BM * BN, kRow4 = BN / 4;
   const int tile = a.tail_first + (int)blockIdx.y;
-  const int tiles_n = (a.N + 63) / 64;
-  const int tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  const int tiles_n = (a.N + BN - 1) / BN;
+  int tm, tn;
+  tile_coords(tile, (a.M + BM - 1) / BM, tiles_n, a.band_rows, &tm, &tn);
   const int e4 = (int)blockIdx.x * 256 + (int)threadIdx.x;  // float4 index in the tile
-  const int lm = e4 >> 4, ln = (e4 & 15) * 4;
-  const int m = tm * 64 + lm, n = tn * 64 + ln;
+  const int lm = e4 / kRow4, ln = (e4 - lm * kRow4) * 4;
+  const int m = tm * BM + lm, n = tn * BN + ln;
   if (m >= a.M || n >= a.N) return;
-  const float* part = a.ws + (size_t)blockIdx.y * a.tail_parts * 4096 + lm * 64 + ln;
+  const float* part = a.ws + (size_t)blockIdx.y * a.tail_parts * kTile + lm * BN + ln;
   f4 s = *reinterpret_cast<const f4*>(part);
-  for (int p = 1; p < a.tail_parts; ++p) s += *reinterpret_cast<const f4*>(part + (size_t)p * 4096);
+  for (int p = 1; p < a.tail_parts; ++p) s += *reinterpret_cast<const f4*>(part + (size_t)p * kTile);
   f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
   float c[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
   float* dst = a.C + (size_t)m * a.ldc + n;
@@ -851,16 +961,16 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
   for (int i = threadIdx.x; i < cols; i += 256) out_at(i) = (row[i] - mean) * inv * g[i] + b[i];
 }
 
-template <int BM, int BN, int WBF>
+template <int BM, int BN, int WBF, int BKT = BK>
 hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = (tiles + 7) / 8 * 8;  // whole rounds over the 8 XCDs
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS, WBF>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS, WBF, 0, BKT>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU, WBF>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU, WBF, 0, BKT>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID, WBF>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID, WBF, 0, BKT>), dim3(grid), dim3(256), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
@@ -901,11 +1011,11 @@ hipError_t launch_splitk_reduce(const GemmArgs& a, int epi, int parts, hipStream
   return hipGetLastError();
 }
 
-template <bool WBF>
+template <int BM, int BN, bool WBF, int BKT>
 hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
-  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = (tiles + 7) / 8 * 8;
-  hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 1>), dim3(grid, parts), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS, WBF, 1, BKT>), dim3(grid, parts), dim3(256), 0, s, a);
   return launch_splitk_reduce(a, epi, parts, s, ln_done);
 }
 template <int MB, int R, bool WBF>
@@ -973,21 +1083,21 @@ hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t
   return hipGetLastError();
 }
 
-// 64x64 tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
-template <bool WBF>
+// Tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
+template <int BM, int BN, bool WBF, int BKT>
 hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
-  const int tiles = ((a.M + 63) / 64) * ((a.N + 63) / 64);
+  const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = a.tail_first + (tiles - a.tail_first) * a.tail_parts;
-  const dim3 rgrid(4, (unsigned)(tiles - a.tail_first));
+  const dim3 rgrid(BM * BN / 1024, (unsigned)(tiles - a.tail_first));
   if (epi == GEMM_BIAS) {
-    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_BIAS, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(k_tail_reduce<GEMM_BIAS>, rgrid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_BIAS, WBF, 2, BKT>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_tail_reduce<BM, BN, GEMM_BIAS>), rgrid, dim3(256), 0, s, a);
   } else if (epi == GEMM_GELU) {
-    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_GELU, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(k_tail_reduce<GEMM_GELU>, rgrid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_GELU, WBF, 2, BKT>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_tail_reduce<BM, BN, GEMM_GELU>), rgrid, dim3(256), 0, s, a);
   } else if (epi == GEMM_RESID) {
-    hipLaunchKernelGGL((k_gemm<64, 64, GEMM_RESID, WBF, 2>), dim3(grid), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(k_tail_reduce<GEMM_RESID>, rgrid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm<BM, BN, GEMM_RESID, WBF, 2, BKT>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_tail_reduce<BM, BN, GEMM_RESID>), rgrid, dim3(256), 0, s, a);
   } else {
     return hipErrorInvalidValue;
   }
@@ -995,17 +1105,30 @@ hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
 }
 }  // namespace
 
-// Parts the K range is cut into (1 = no split): when the 64x64 tiles of C are fewer than
-// about 1.5 per CU, enough parts for about three work items per CU.  A part is at least
-// 512 deep for tall operands; for a batch of a few rows (decode), where the job is to
-// stream W at the speed of HBM, 128.  Needs the workspace a.ws of parts x M x N floats.
-int gemm_split_parts(const GemmArgs& a, int num_cus) {
-  const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
-  if (!a.ws || a.N % 4 != 0 || tiles * 2 >= 3L * num_cus) return 1;
-  const int depth = a.M < 64 ? 128 : (tiles * 10 < 9L * num_cus ? 192 : 512);
-  int parts = (int)(((long)std::max(a.split_items_per_cu, 1) * num_cus) / tiles);
-  parts = std::min(parts, a.K / depth);
-  parts = std::min(parts, 8);
+// Parts the K range is cut into (1 = no split).  Needs the workspace a.ws of parts x M x N
+// floats.
+//  - A batch of a few rows (decode), where the job is to stream W at the speed of HBM: with
+//    fewer than 1.5 tiles per CU, about split_items_per_cu work items per CU, a part at least
+//    128 deep.
+//  - Tall operands whose tiles occupy at most half of the CUs: the same, a part at least 192
+//    deep.
+//  - Tall operands with up to two tiles per CU and a deep K (the MLP's second projection):
+//    up to four parts of at least 768 columns; more blocks per CU hide each other's waits
+//    and the parts even out the load.
+//  - Otherwise whole tiles: a tile that has a CU to itself runs its k loop faster than two
+//    halves and a reduction would.
+int gemm_split_parts(const GemmArgs& a, int num_cus, int bm, int bn) {
+  const long tiles = (long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
+  if (!a.ws || a.N % 4 != 0) return 1;
+  int parts = 1;
+  if (a.M < 64 ? tiles * 2 < 3L * num_cus : tiles * 2 <= num_cus) {
+    const int depth = a.M < 64 ? 128 : 192;
+    parts = (int)(((long)std::max(a.split_items_per_cu, 1) * num_cus) / tiles);
+    parts = std::min(parts, a.K / depth);
+    parts = std::min(parts, 8);
+  } else if (a.M >= 64 && tiles <= 2L * num_cus && a.K >= 2048) {
+    parts = std::min(4, a.K / 768);
+  }
   while (parts > 1 && (size_t)parts * a.M * a.N > a.ws_floats) --parts;
   return std::max(parts, 1);
 }
@@ -1013,19 +1136,97 @@ int gemm_split_parts(const GemmArgs& a, int num_cus) {
 // The tail split of the 64x64 form: with more tiles than CUs and a last round that would
 // occupy at most half of them, that round's tiles are cut into as many K parts as make it
 // one item per CU.  Fills a.tail_first / a.tail_parts; false when it does not apply.
-bool gemm_tail_plan(GemmArgs& a, int num_cus) {
-  const long tiles = (long)((a.M + 63) / 64) * ((a.N + 63) / 64);
+bool gemm_tail_plan(GemmArgs& a, int num_cus, int bm, int bn) {
+  const long tiles = (long)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
   if (!a.ws || a.N % 4 != 0 || num_cus % 8 != 0 || tiles <= num_cus) return false;
   const int r = (int)(tiles % num_cus);
   if (r == 0 || 2 * r > num_cus) return false;
   int parts = std::min(8, num_cus / r);
   parts = std::min(parts, a.K / (4 * BK));  // at least four k-tiles per part
-  while (parts > 1 && (size_t)r * parts * 4096 > a.ws_floats) --parts;
+  while (parts > 1 && (size_t)r * parts * bm * bn > a.ws_floats) --parts;
   if (parts < 2) return false;
   a.tail_first = (int)(tiles - r);
   a.tail_parts = parts;
   return true;
 }
+
+namespace {
+// form: 1 whole tiles, 2 every tile cut along K into `parts` (a.ws), 3 only the last partial
+// round of tiles cut (a.tail_first / a.tail_parts are set in a)
+template <int BM, int BN, bool WBF, int BKT>
+hipError_t launch_tiles_depth(const GemmArgs& a, int epi, int form, int parts, hipStream_t s, bool* ln_done) {
+  if (form == 2) return launch_gemm_split<BM, BN, WBF, BKT>(a, epi, parts, s, ln_done);
+  if (form == 3) return launch_gemm_tail<BM, BN, WBF, BKT>(a, epi, s);
+  return launch_gemm_tile<BM, BN, WBF, BKT>(a, epi, s);
+}
+template <int BM, int BN, bool WBF>
+hipError_t launch_tiles_shape(const GemmArgs& a, int epi, int form, int parts, hipStream_t s, bool* ln_done) {
+  // k-tiles of 32 columns where K allows
+  if (a.K % 32 == 0 && !a.plan_bk16) return launch_tiles_depth<BM, BN, WBF, 32>(a, epi, form, parts, s, ln_done);
+  return launch_tiles_depth<BM, BN, WBF, 16>(a, epi, form, parts, s, ln_done);
+}
+// Band height for tile_coords: a run of `run` consecutive tiles (one XCD's share) should
+// touch as few rows of A and W as it can: hb tile rows and run / hb tile columns.
+int choose_band(int tiles_m, int run, int bm, int bn) {
+  int best = 1;
+  long best_cost = -1;
+  for (int hb = 1; hb <= tiles_m; ++hb) {
+    const int bands = (tiles_m + hb - 1) / hb;
+    const int last = tiles_m - (bands - 1) * hb;  // a short last band makes short, wide runs
+    const long cost = (long)hb * bm + (long)((run + hb - 1) / hb) * bn + (last < hb ? (long)(hb - last) * bm / 2 : 0);
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = hb;
+    }
+  }
+  return best;
+}
+
+template <bool WBF>
+hipError_t launch_tiles(const GemmArgs& a0, int epi, int bm, int bn, int form, int parts, hipStream_t s,
+                        bool* ln_done) {
+  GemmArgs a = a0;
+  {
+    const int tiles_m = (a.M + bm - 1) / bm, tiles_n = (a.N + bn - 1) / bn;
+    const int whole = form == 3 ? a.tail_first : tiles_m * tiles_n;
+    a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band(tiles_m, std::max(1, (whole + 7) / 8), bm, bn);
+  }
+  if (bm == 128 && bn == 128) return launch_tiles_shape<128, 128, WBF>(a, epi, form, parts, s, ln_done);
+  if (bm == 128 && bn == 64) return launch_tiles_shape<128, 64, WBF>(a, epi, form, parts, s, ln_done);
+  if (bm == 64 && bn == 128) return launch_tiles_shape<64, 128, WBF>(a, epi, form, parts, s, ln_done);
+  if (bm == 64 && bn == 64) return launch_tiles_shape<64, 64, WBF>(a, epi, form, parts, s, ln_done);
+  return hipErrorInvalidValue;
+}
+
+// The planner's choice of tile shape and form.
+void plan_tiles(GemmArgs& a, int num_cus, int* bm, int* bn, int* form, int* parts) {
+  *bm = 64;
+  *bn = 64;
+  *parts = gemm_split_parts(a, num_cus, 64, 64);
+  if (*parts > 1) {
+    *form = 2;
+    return;
+  }
+  // 128x128 tiles once they fill the chip about twice over; otherwise 64x64 tiles, with the
+  // last partial round cut along K where that applies, or 128x128 tiles cut that way
+  const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
+  if (tiles128 >= 2L * num_cus) {
+    *bm = *bn = 128;
+    *form = 1;
+    return;
+  }
+  if (gemm_tail_plan(a, num_cus, 64, 64)) {
+    *form = 3;
+    return;
+  }
+  if (tiles128 > num_cus && gemm_tail_plan(a, num_cus, 128, 128)) {
+    *bm = *bn = 128;
+    *form = 3;
+    return;
+  }
+  *form = 1;
+}
+}  // namespace
 
 namespace {
 hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t s, bool* ln_done);
@@ -1066,24 +1267,13 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done)
                     : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
   if (packed) return hipErrorInvalidValue;  // only the 32-row kernel knows the packed form
-  const int parts = gemm_split_parts(a, num_cus);
-  if (parts > 1)
-    return a.w_bf16 ? launch_gemm_split<true>(a, epi, parts, s, ln_done)
-                    : launch_gemm_split<false>(a, epi, parts, s, ln_done);
-  // 128x128 tiles once they fill the chip about twice over, 64x64 tiles otherwise
-  const long tiles128 = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
-  if (a.w_bf16) {
-    if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, true>(a, epi, s);
-    GemmArgs t = a;
-    if (gemm_tail_plan(t, num_cus)) return launch_gemm_tail<true>(t, epi, s);
-    return launch_gemm_tile<64, 64, true>(a, epi, s);
-  }
-  if (tiles128 >= 2L * num_cus) return launch_gemm_tile<128, 128, false>(a, epi, s);
-  {
-    GemmArgs t = a;
-    if (gemm_tail_plan(t, num_cus)) return launch_gemm_tail<false>(t, epi, s);
-  }
-  return launch_gemm_tile<64, 64, false>(a, epi, s);
+  // Tile forms.  A forced plan (benchmarks, tests) or the planner's choice.
+  int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
+  GemmArgs t = a;
+  if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
+  else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
+  return a.w_bf16 ? launch_tiles<true>(t, epi, bm, bn, form, parts, s, ln_done)
+                  : launch_tiles<false>(t, epi, bm, bn, form, parts, s, ln_done);
 }
 }  // namespace
 
