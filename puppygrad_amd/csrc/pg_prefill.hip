@@ -688,6 +688,14 @@ __global__ __launch_bounds__(256) void k_tail_reduce(GemmArgs a) {
 // Grid: x = head, y = block of queries, longest rows first (blocks are handed out x
 // fastest: every head's long blocks start before any short one).
 // ---------------------------------------------------------------------------
+// The value the lane 32 away holds (v_permlane32_swap: one VALU instruction, no LDS trip).
+__device__ __forceinline__ float other_half(float x) {
+  typedef unsigned u2x __attribute__((ext_vector_type(2)));
+  const u2x r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  // r.x holds lanes 0..31 of x in both halves, r.y lanes 32..63
+  return (threadIdx.x & 32) ? __uint_as_float(r.x) : __uint_as_float(r.y);
+}
+
 __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict__ qkv, int T,
                                                         int C, int P, float* __restrict__ kcache,
                                                         float* __restrict__ vcache,
@@ -766,42 +774,69 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
     __builtin_amdgcn_wave_barrier();
     if (tile + NWV <= last_tile) fetch_v(tile + NWV);
 
-    // S^T = K . Q^T
-    f16v sacc;
+    // S^T = K . Q^T in two independent chains (even and odd j), and between its MFMAs the
+    // LDS reads of the V operands of the second product: a wavefront issues in order, so a
+    // read placed in front of the MFMA that needs it would idle the matrix core for the LDS
+    // latency 32 times a tile.
+    f16v sacc, sacc1;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) sacc[v] = 0.0f;
+    for (int v = 0; v < 16; ++v) { sacc[v] = 0.0f; sacc1[v] = 0.0f; }
+    float vop0[16], vop1[16];  // V^T operands of step v: dims l32 and 32 + l32 of its key
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 8; j += 2) {
       sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].x, qr[j].x, sacc, 0, 0, 0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].y, qr[j].y, sacc, 0, 0, 0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].z, qr[j].z, sacc, 0, 0, 0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].w, qr[j].w, sacc, 0, 0, 0);
-    }
-    if (tile + NWV <= last_tile) fetch_k(tile + NWV);
-    // lane holds keys k0 + 8*(v/4) + 4*half + v%4 of query qi
-    float mx = -INFINITY;
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].x, qr[j + 1].x, sacc1, 0, 0, 0);
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
-      const float sv = (key <= qi && key < T) ? sacc[v] * 0.125f : -INFINITY;
-      sacc[v] = sv;
-      mx = fmaxf(mx, sv);
+      for (int v = 2 * j; v < 2 * j + 4; ++v) {
+        const int key = 8 * (v >> 2) + 4 * half + (v & 3);
+        vop0[v] = vs[key][l32];
+        vop1[v] = vs[key][32 + l32];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].y, qr[j].y, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].y, qr[j + 1].y, sacc1, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].z, qr[j].z, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].z, qr[j + 1].z, sacc1, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].w, qr[j].w, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].w, qr[j + 1].w, sacc1, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    sacc += sacc1;
+    if (tile + NWV <= last_tile) fetch_k(tile + NWV);
+    // lane holds keys k0 + 8*(v/4) + 4*half + v%4 of query qi.  Only the diagonal tile has
+    // keys to mask (later keys of the block, and keys past T in the last block).
+    if (diag) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (!(key <= qi && key < T)) sacc[v] = -INFINITY;
+      }
+    }
+    // The softmax works on the raw dot products: with c = log2(e) / 8,
+    // exp(s / 8 - m / 8) = exp2(s c - m c), one fused multiply-add and one v_exp_f32 per
+    // score (the matrix core waits while this wavefront's other instructions issue, so the
+    // softmax is kept short; v_exp_f32 is exact to 1 ulp).
+    float mx = fmaxf(fmaxf(sacc[0], sacc[1]), sacc[2]);
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, sacc[v]), sacc[v + 1]);
+    mx = fmaxf(mx, sacc[15]);
+    mx = fmaxf(mx, other_half(mx));
     const float m_new = fmaxf(m_run, mx);
     // Every tile a wavefront sees holds a key <= qi for each of its queries (tiles before
     // the diagonal hold only such keys, and the diagonal tile's first key is q0 <= qi), so
-    // m_new is finite from its first tile on; a wavefront that never gets a tile keeps the
-    // neutral (-inf, 0, 0).
-    const float corr = (m_run == -INFINITY) ? 0.0f : expf(m_run - m_new);
+    // m_new is finite from its first tile on (and exp2(-inf - finite) = 0 starts the
+    // running values); a wavefront that never gets a tile keeps the neutral (-inf, 0, 0).
+    constexpr float kC = 0.125f * 1.44269504088896341f;
+    const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * kC);
+    const float mc = m_new * kC;
     float psum = 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const float pv = (m_new == -INFINITY) ? 0.0f : expf(sacc[v] - m_new);
+      const float pv = __builtin_amdgcn_exp2f(fmaf(sacc[v], kC, -mc));
       sacc[v] = pv;
       psum += pv;
     }
-    psum += __shfl_xor(psum, 32, 64);
+    psum += other_half(psum);
     l_run = l_run * corr + psum;
     m_run = m_new;
 #pragma unroll
@@ -810,9 +845,8 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
     // (8*(v/4) + 4 + v%4) of half 1; the B operand is this lane's own P value.
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int key = 8 * (v >> 2) + 4 * half + (v & 3);
-      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key][l32], sacc[v], o0, 0, 0, 0);
-      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[key][32 + l32], sacc[v], o1, 0, 0, 0);
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vop0[v], sacc[v], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vop1[v], sacc[v], o1, 0, 0, 0);
     }
     __builtin_amdgcn_wave_barrier();
   }
@@ -825,12 +859,12 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
   float M = Ms[0][l32];
 #pragma unroll
   for (int w = 1; w < NWV; ++w) M = fmaxf(M, Ms[w][l32]);
-  const float mine = (m_run == -INFINITY) ? 0.0f : expf(m_run - M);
+  const float mine = (m_run == -INFINITY) ? 0.0f : expf((m_run - M) * 0.125f);
   float L = 0.0f;
 #pragma unroll
   for (int w = 0; w < NWV; ++w) {
     const float mw = Ms[w][l32];
-    L += ((mw == -INFINITY) ? 0.0f : expf(mw - M)) * Ls[w][l32];
+    L += ((mw == -INFINITY) ? 0.0f : expf((mw - M) * 0.125f)) * Ls[w][l32];
   }
   // O^T of the wavefronts through LDS (the V tiles' space: [wave][d 0..63][query])
   float (*ob)[KT + 1] = reinterpret_cast<float (*)[KT + 1]>(Vs[wave]);
@@ -1204,6 +1238,15 @@ void plan_tiles(GemmArgs& a, int num_cus, int* bm, int* bn, int* form, int* part
   *bn = 64;
   *parts = gemm_split_parts(a, num_cus, 64, 64);
   if (*parts > 1) {
+    *form = 2;
+    return;
+  }
+  // A projection whose rows are normalised afterwards and whose tiles leave CUs idle: two
+  // parts, so that the LayerNorm rides on the reduce instead of being a launch of its own.
+  if (a.ln_out && a.ws && a.N % 4 == 0 && a.N <= 4096 && a.ldc == a.N &&
+      (long)((a.M + 63) / 64) * ((a.N + 63) / 64) * 2 < 3L * num_cus && a.K >= 512 &&
+      (size_t)2 * a.M * a.N <= a.ws_floats) {
+    *parts = 2;
     *form = 2;
     return;
   }
