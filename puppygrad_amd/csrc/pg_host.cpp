@@ -117,6 +117,12 @@ struct pg_kv_cache {
   uint32_t* d_tok = nullptr;      // [B] token the next step embeds
   uint32_t* d_out_ids = nullptr;  // [P][B] ids produced by greedy decode
   uint32_t* h_ids = nullptr;      // pinned staging, [P][B]
+  // pinned staging of the prompts of full-sequence forwards, used in turn: the copy to the
+  // device is queued without waiting, and a buffer is reused once the copy of two calls ago
+  // has been made
+  uint32_t* h_prompt[2] = {nullptr, nullptr};
+  hipEvent_t ev_prompt[2] = {nullptr, nullptr};
+  unsigned prompt_turn = 0;
   // streamed greedy generation: ids the persistent kernel writes straight into pinned host
   // memory as it selects them ([P + 1], batch 1), and the device's address of that block
   uint32_t* h_stream = nullptr;
@@ -657,8 +663,20 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   if (hd != 64 && (st = SCR.alloc(n * g.H * n))) return st;
   if (all_logits_dst && (st = LOG.alloc(n * g.V))) return st;
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
-  PG_HIP(hipMemcpyAsync(d_ids, ids, n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
-  PG_HIP(hipStreamSynchronize(s));  // ids is the caller's pageable memory
+  {
+    // ids is the caller's pageable memory: through pinned staging, so that the stream need
+    // not drain before the first launch (a prefill queued behind another starts at once)
+    const unsigned turn = c->prompt_turn++ & 1;
+    if (!c->h_prompt[turn]) {
+      PG_HIP(hipHostMalloc(&c->h_prompt[turn], g.P * sizeof(uint32_t), hipHostMallocDefault));
+      PG_HIP(hipEventCreateWithFlags(&c->ev_prompt[turn], hipEventDisableTiming));
+    } else {
+      PG_HIP(hipEventSynchronize(c->ev_prompt[turn]));
+    }
+    memcpy(c->h_prompt[turn], ids, n * sizeof(uint32_t));
+    PG_HIP(hipMemcpyAsync(d_ids, c->h_prompt[turn], n * sizeof(uint32_t), hipMemcpyHostToDevice, s));
+    PG_HIP(hipEventRecord(c->ev_prompt[turn], s));
+  }
 #define PG_MARK(bk) \
   do {              \
     if (marks) PG_HIP(marks->mark(s, ProfileMarks::bk)); \
@@ -1288,6 +1306,10 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->d_force);
     if (c->h_status) (void)hipHostFree(c->h_status);
     if (c->h_stream) (void)hipHostFree(c->h_stream);
+    for (int i = 0; i < 2; ++i) {
+      if (c->h_prompt[i]) (void)hipHostFree(c->h_prompt[i]);
+      if (c->ev_prompt[i]) (void)hipEventDestroy(c->ev_prompt[i]);
+    }
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
