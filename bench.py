@@ -259,7 +259,7 @@ def secondary_workloads(xl_cfg, xl_weights):
                                  launch_ms=round(d["launch_s"] * 1e3, 3),
                                  algorithmic_bytes_per_forward=int(d["algo_bytes"]))}
     ids = synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size)
-    out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 10, 2)
+    out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 60, 6)
     del model, w
     # GPT-2 355M: batch-16 decode steps from 128-token prompts
     cfg = Gpt2Config(**synth.GPT2_MEDIUM)
@@ -428,7 +428,7 @@ def _devinfo():
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by what the same
 # counter reads for a plain copy kernel of known size
 # (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the counters and the factors).
-TRAFFIC_RATIO_XL = 1.031
+TRAFFIC_RATIO_XL = 1.028
 TRAFFIC_SOURCE = "profiles/k_decode_persistent_1600_xl_decode_traffic.txt"
 
 
