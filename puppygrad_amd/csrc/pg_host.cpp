@@ -72,6 +72,9 @@ struct pg_gpt2_model {
   int attn_splits = 1;              // key splits per head in the persistent kernel
   // tunables (pg_hip_options; defaults filled in at creation)
   int item_keys = 128;              // keys per attention item of the persistent kernel
+  bool item_keys_auto = true;       // not set by the caller: 256-key items for launches that stay
+                                    // within 256 positions (one split per head: no merge hop)
+  bool item_keys_256_ok = false;    // the device holds the grid of the 256-key instance
   int attn_blocks_per_cu = 4;       // per-operation / batched decode attention
   int gemm_split_items = 3;         // tile GEMM split-K
   int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
@@ -538,6 +541,13 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   p.epoch0 = c->epoch;
   p.ns = m->attn_splits;
   p.item_keys = m->item_keys;
+  // Past 128 positions a 128-key item needs two splits per head and a merge hop; a launch that
+  // ends within 256 positions runs the 256-key instance instead (355M from 128 tokens: +6 %;
+  // beyond 256 positions the shorter items win by 1-4 %).
+  // (chosen when most of the launch lies past 128: up to there both need one split and the
+  // shorter items are 4 % faster)
+  if (m->item_keys_auto && m->item_keys_256_ok && pos0 + n_fwd / 2 > 128 && pos0 + n_fwd <= 256)
+    p.item_keys = 256;
   p.status = c->status;
 #ifdef PG_DECODE_PROF_BUILD
   // Development builds only: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
@@ -1008,6 +1018,7 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   m->w_bf16 = bf ? 1 : 0;
   m->w_i8 = i8 ? 1 : 0;
   m->item_keys = opts.attn_item_keys ? (int)opts.attn_item_keys : pgk::persistent_default_item_keys();
+  m->item_keys_auto = opts.attn_item_keys == 0;
   m->attn_blocks_per_cu = opts.attn_blocks_per_cu ? (int)opts.attn_blocks_per_cu : 4;
   m->gemm_split_items = opts.gemm_split_items_per_cu ? (int)opts.gemm_split_items_per_cu : 3;
   hipDeviceProp_t prop;
@@ -1150,6 +1161,11 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
       PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &blocks_per_cu, i8 ? 1 : bf ? 2 : 4,
                                                    m->item_keys));
       shape_ok = (long long)blocks_per_cu * m->num_cus >= grid;
+      if (shape_ok && m->item_keys_auto) {
+        int b256 = 0;
+        PG_HIP(pgk::persistent_max_blocks_per_cu((int)g.C, &b256, i8 ? 1 : bf ? 2 : 4, 256));
+        m->item_keys_256_ok = (long long)b256 * m->num_cus >= grid;
+      }
     }
     if (shape_ok) {
       // key splits per head at the longest context (the kernel uses as few as the position
