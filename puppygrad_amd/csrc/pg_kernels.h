@@ -76,7 +76,8 @@ struct BatchStrides {
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
                               float* part_m, float* part_l, hipStream_t s, int batch = 1,
-                              BatchStrides bs = BatchStrides{}, int append_C = 0);
+                              BatchStrides bs = BatchStrides{}, int append_C = 0,
+                              float* direct_out = nullptr, int out_packed = 0);
 // blocks_per_cu: (head, split) blocks per CU to aim for (tunable, 4 by default).
 int choose_nsplit(int n_keys, int H, int num_cus, int blocks_per_cu = 4);
 

@@ -302,7 +302,11 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
                                                           int pos, int P, int nsplit,
                                                           float* part_acc, float* part_m,
                                                           float* part_l, BatchStrides bs,
-                                                          int append_C) {
+                                                          int append_C, float* direct_out,
+                                                          int out_packed) {
+  // direct_out (only with nsplit == 1): the block's result is the head's attention output
+  // and is written there (row blockIdx.z, packed or row-major), with no partials and no
+  // merge launch.
   // append_C > 0: the rows of position pos are not in the cache yet.  They are the k and v
   // parts of this step's interleaved qkv row (q + append_C, q + 2 append_C); the block whose
   // split holds pos uses them from there and writes them to the cache panels
@@ -422,6 +426,11 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
       const float f = wm[w] == -INFINITY ? 0.0f : expf(wm[w] - M);
       t += f * accs[w][tid];
       l += f * wl[w];
+    }
+    if (direct_out) {
+      const size_t b = blockIdx.z, i = (size_t)h * 64 + tid;
+      direct_out[out_packed ? packed32_index(b, i) : b * bs.out + i] = t / l;
+      return;
     }
     part_acc[pidx * 64 + tid] = t;
     if (tid == 0) {
@@ -925,20 +934,22 @@ int choose_nsplit(int n_keys, int H, int num_cus, int blocks_per_cu) {
 hipError_t launch_attn_decode(const float* q, const float* kcache, const float* vcache, int pos,
                               int P, int H, int head_dim, int nsplit, float* part_acc,
                               float* part_m, float* part_l, hipStream_t s, int batch,
-                              BatchStrides bs, int append_C) {
+                              BatchStrides bs, int append_C, float* direct_out, int out_packed) {
+  if (direct_out && (head_dim != kHeadDim || nsplit != 1 || (out_packed && batch > 32)))
+    return hipErrorInvalidValue;
   if (head_dim == kHeadDim) {
     const int per = (pos + 1 + nsplit - 1) / nsplit;
     const dim3 grid(nsplit, H, batch);
     // steps of 16 keys a block needs for its split: the chunk is sized to it
     if (per <= 32)
       hipLaunchKernelGGL(k_attn_decode64<2>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
-                         nsplit, part_acc, part_m, part_l, bs, append_C);
+                         nsplit, part_acc, part_m, part_l, bs, append_C, direct_out, out_packed);
     else if (per <= 64)
       hipLaunchKernelGGL(k_attn_decode64<4>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
-                         nsplit, part_acc, part_m, part_l, bs, append_C);
+                         nsplit, part_acc, part_m, part_l, bs, append_C, direct_out, out_packed);
     else
       hipLaunchKernelGGL(k_attn_decode64<8>, grid, dim3(kBlock), 0, s, q, kcache, vcache, pos, P,
-                         nsplit, part_acc, part_m, part_l, bs, append_C);
+                         nsplit, part_acc, part_m, part_l, bs, append_C, direct_out, out_packed);
   } else {
     hipLaunchKernelGGL(k_attn_decode_any, dim3(1, H, batch), dim3(kBlock),
                        (pos + 1) * sizeof(float), s, q, kcache, vcache, pos, P, head_dim, part_acc,
