@@ -674,10 +674,11 @@ __global__ __launch_bounds__(256) void k_tail_reduce(GemmArgs a) {
 // interleaved qkv[T][3C] buffer.  A block of eight wavefronts owns 32 queries of one head;
 // the wavefronts take the key tiles 0..diagonal (32 keys each) round-robin, each with its
 // own running (max, sum, O), merged through LDS at the end:
-//   S^T (keys x queries) = K . Q^T        32 MFMA steps; both operands come straight from
-//                                         registers: lane (l, half) holds dims
+//   S^T (keys x queries) = K . Q^T        32 MFMA steps; lane (l, half) holds dims
 //                                         32 half .. 32 half + 31 of key l / query l, and step
-//                                         s pairs dim s with dim 32 + s
+//                                         s pairs dim s with dim 32 + s.  Q stays in registers;
+//                                         K rows are loaded row-wise (coalesced) into a
+//                                         per-wavefront LDS tile and read back in that form
 //   online softmax per query (a lane holds 16 keys of one query; one xor-32 swap)
 //   O^T (d x queries)   += V^T . P^T      16 MFMA steps over the 32 keys, twice (d halves),
 //                                         V rows staged in LDS
@@ -704,6 +705,10 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
   constexpr int NWV = 8;   // wavefronts per block
   // per wavefront: V rows [key][d] of the current tile; reused as [d][query] for the merge
   __shared__ __attribute__((aligned(16))) float Vs[NWV][KT * (64 + 4)];
+  // ... and its K rows [key][d]: loaded row-wise like V (sixteen lanes per 256-byte row; a lane
+  // that fetched its own operand dims straight from memory touched 64 cache lines per load
+  // instruction) and read back as the MFMA operand of lane (key, half)
+  __shared__ __attribute__((aligned(16))) float Ks[NWV][KT * (64 + 4)];
   __shared__ float Ms[NWV][32], Ls[NWV][32];
   static_assert(KT * (64 + 4) >= 64 * (KT + 1), "the merge tile fits the V tile's space");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -731,14 +736,17 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
   const int qi = q0 + l32;                // this lane's query
 
   float (*vs)[64 + 4] = reinterpret_cast<float (*)[64 + 4]>(Vs[wave]);
+  float (*ks)[64 + 4] = reinterpret_cast<float (*)[64 + 4]>(Ks[wave]);
   const int last_tile = min(q0 + 31, T - 1) / KT;
-  // K operand: lane (key l32, half) holds K[key][32 half + s]; V rows as this lane loads
-  // them: 8 pieces of (key i / 16, 4 dims)
-  f4 kr[8], vreg[8];
+  // K and V rows as this lane loads them: 8 pieces of (key i / 16, 4 dims) each
+  f4 kreg[8], vreg[8];
   auto fetch_k = [&](int tile) {
-    const int kk = min(tile * KT + l32, T - 1);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) kr[j] = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + 32 * half + 4 * j);
+    for (int j = 0; j < 8; ++j) {
+      const int i = lane + 64 * j;
+      const int kk = min(tile * KT + (i >> 4), T - 1);
+      kreg[j] = *reinterpret_cast<const f4*>(kbase + (size_t)kk * C3 + (i & 15) * 4);
+    }
   };
   auto fetch_v = [&](int tile) {
 #pragma unroll
@@ -761,18 +769,19 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
       const int i = lane + 64 * j;
       const int key = i >> 4, d4 = (i & 15) * 4;
       *reinterpret_cast<f4*>(&vs[key][d4]) = vreg[j];
-      if (diag && k0 + key < T)
+      *reinterpret_cast<f4*>(&ks[key][d4]) = kreg[j];
+      if (diag && k0 + key < T) {
         *reinterpret_cast<f4*>(vcache + ((size_t)h * P + k0 + key) * 64 + d4) = vreg[j];
-    }
-    if (diag && k0 + l32 < T) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        *reinterpret_cast<f4*>(kcache + ((size_t)h * P + k0 + l32) * 64 + 32 * half + 4 * j) = kr[j];
+        *reinterpret_cast<f4*>(kcache + ((size_t)h * P + k0 + key) * 64 + d4) = kreg[j];
+      }
     }
     // each wavefront has its own LDS tile and LDS executes a wavefront's accesses in
     // order, so only the compiler has to be kept from reordering
     __builtin_amdgcn_wave_barrier();
-    if (tile + NWV <= last_tile) fetch_v(tile + NWV);
+    if (tile + NWV <= last_tile) {
+      fetch_v(tile + NWV);
+      fetch_k(tile + NWV);
+    }
 
     // S^T = K . Q^T in two independent chains (even and odd j), and between its MFMAs the
     // LDS reads of the V operands of the second product: a wavefront issues in order, so a
@@ -782,10 +791,18 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
 #pragma unroll
     for (int v = 0; v < 16; ++v) { sacc[v] = 0.0f; sacc1[v] = 0.0f; }
     float vop0[16], vop1[16];  // V^T operands of step v: dims l32 and 32 + l32 of its key
+    // K operand of lane (key l32, half): dims 32 half + 4 j .. + 3, read a pair of j ahead
+    const f4* krow = reinterpret_cast<const f4*>(&ks[l32][32 * half]);
+    f4 ka = krow[0], kb = krow[1];
 #pragma unroll
     for (int j = 0; j < 8; j += 2) {
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].x, qr[j].x, sacc, 0, 0, 0);
-      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].x, qr[j + 1].x, sacc1, 0, 0, 0);
+      const f4 k0v = ka, k1v = kb;
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k0v.x, qr[j].x, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1v.x, qr[j + 1].x, sacc1, 0, 0, 0);
+      if (j + 2 < 8) {
+        ka = krow[j + 2];
+        kb = krow[j + 3];
+      }
 #pragma unroll
       for (int v = 2 * j; v < 2 * j + 4; ++v) {
         const int key = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -793,16 +810,15 @@ __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict_
         vop1[v] = vs[key][32 + l32];
       }
       __builtin_amdgcn_sched_barrier(0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].y, qr[j].y, sacc, 0, 0, 0);
-      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].y, qr[j + 1].y, sacc1, 0, 0, 0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].z, qr[j].z, sacc, 0, 0, 0);
-      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].z, qr[j + 1].z, sacc1, 0, 0, 0);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j].w, qr[j].w, sacc, 0, 0, 0);
-      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j + 1].w, qr[j + 1].w, sacc1, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k0v.y, qr[j].y, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1v.y, qr[j + 1].y, sacc1, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k0v.z, qr[j].z, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1v.z, qr[j + 1].z, sacc1, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(k0v.w, qr[j].w, sacc, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(k1v.w, qr[j + 1].w, sacc1, 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
     sacc += sacc1;
-    if (tile + NWV <= last_tile) fetch_k(tile + NWV);
     // lane holds keys k0 + 8*(v/4) + 4*half + v%4 of query qi.  Only the diagonal tile has
     // keys to mask (later keys of the block, and keys past T in the last block).
     if (diag) {
