@@ -42,12 +42,17 @@ def test_dense_matches_oracle(rows, k, n):
                                       (37, 64, 50), (1000, 1024, 4096), (33, 16, 129), (64, 6400, 1600),
                                       (20, 768, 50257), (512, 768, 2304), (1024, 768, 2304),
                                       (512, 768, 3072), (16, 1024, 3072), (32, 1600, 6400),
-                                      (16, 4096, 1024), (16, 1600, 4800)])
+                                      (16, 4096, 1024), (16, 1600, 4800),
+                                      (100, 48, 100), (333, 112, 260), (200, 32, 64), (64, 16, 52),
+                                      (1024, 3072, 768), (1024, 1600, 4800)])
 def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised.
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
     # parts; (512, 768, 2304), (1024, 768, 2304) and (512, 768, 3072) have 288 / 576 / 384
     # tiles of 64x64 on 256 CUs and cut only the tiles of the last partial round.
+    # K = 48 and 112 are not multiples of 32 and take k-tiles of 16 columns; K = 16 and 32 are a
+    # single k-tile (the pipelined loop's shortest cases); (1024, 3072, 768) has a deep K on 192
+    # tiles and is cut in four; (1024, 1600, 4800) runs 128x128 tiles with the last round cut.
     # 16 rows with K <= 1024 take the row-streaming kernel of the decode batch; other shapes
     # of up to 32 rows the register-fed MFMA kernel (with and without a cut of K over blocks).
     rng = np.random.default_rng(rows * 7 + n)
