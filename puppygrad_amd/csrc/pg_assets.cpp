@@ -16,6 +16,7 @@
 #include <cstring>
 #include <fstream>
 #include <map>
+#include <mutex>
 #include <memory>
 #include <sstream>
 #include <string>
@@ -316,8 +317,10 @@ struct pg_tensor_store {
   const uint8_t* data = nullptr;  // first byte after the header
   size_t data_len = 0;
   std::map<std::string, TensorInfo> tensors;
-  // A tensor whose bytes do not start on a 4-byte boundary is copied here on first use.
+  // A tensor whose bytes do not start on a 4-byte boundary is copied here on first use (under
+  // the lock: lookups of one store may come from several threads).
   mutable std::map<std::string, std::vector<float>> realigned;
+  mutable std::mutex realigned_mu;
 
   ~pg_tensor_store() {
     if (map && map != MAP_FAILED) munmap(map, map_len);
@@ -451,6 +454,7 @@ Lookup lookup_f32(const pg_tensor_store& st, const std::string& name,
   const uint8_t* p = st.data + t.begin;
   const size_t n = (size_t)(t.end - t.begin) / 4;
   if (((uintptr_t)p & 3u) != 0) {
+    std::lock_guard<std::mutex> lock(st.realigned_mu);
     auto& copy = st.realigned[name];
     if (copy.size() != n) {
       copy.resize(n);
