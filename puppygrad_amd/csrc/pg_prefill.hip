@@ -32,13 +32,15 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 // of C, each wavefront a (BM/2) x (BN/2) part made of 32x32 MFMA blocks
 // (v_mfma_f32_32x32x2_f32: A operand lane l -> A[l%32][l/32], B operand lane l ->
 // B[l/32][l%32], D lane l, register v -> D[8*(v/4) + 4*(l/32) + v%4][l%32]).
-// A and W tiles of BK = 16 columns are staged in LDS transposed ([k][row]) so that
-// the operand reads of a wavefront are 32 consecutive floats (no bank conflicts);
-// the next tile's global loads are in flight while the current one is multiplied.
+// A and W tiles of 32 columns (16 where K is not a multiple of 32) are staged in LDS
+// transposed ([k][row]) so that the operand reads of a wavefront are 32 consecutive floats;
+// the k loop is software-pipelined by hand (see the loop): the LDS stores of the next tile,
+// the global loads of the one after it and the LDS reads of the next tile's operands all sit
+// between the MFMAs of the current tile.
 // Rows past M or N are clamped on load and masked on store; K must be a multiple
 // of 16.
 // ---------------------------------------------------------------------------
-constexpr int BK = 16;
+constexpr int BK = 16;  // granularity of K (the short k-tile); planners count in these
 
 // W tile load: 4 consecutive k of one row as f32 (16 bytes) or bf16 (8 bytes, widened
 // to f32 exactly by a 16-bit shift).
