@@ -9,6 +9,9 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libpuppygrad_hip.so"
+# Development build with the persistent decode kernel's in-kernel timestamps compiled in
+# (python -m puppygrad_amd.build --stamps; read by puppygrad_amd.decode_stamps).
+STAMPS_LIB_PATH = PKG_DIR / "libpuppygrad_hip_stamps.so"
 SOURCES = ["pg_kernels.hip", "pg_decode.hip", "pg_prefill.hip", "pg_ops_dev.hip", "pg_sample.hip",
            "pg_host.cpp", "pg_assets.cpp"]
 
@@ -17,17 +20,19 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def build_library(verbose: bool = True) -> Path:
+def build_library(verbose: bool = True, stamps: bool = False) -> Path:
     """Compile every source to an object, then link the shared library."""
     objs = []
     procs = []
+    lib = STAMPS_LIB_PATH if stamps else LIB_PATH
+    extra = ["-DPG_DECODE_PROF_BUILD"] if stamps else []
     for src in SOURCES:
         path = CSRC / src
         if not path.exists():
             continue
-        obj = CSRC / (path.stem + ".o")
+        obj = CSRC / (path.stem + (".stamps.o" if stamps else ".o"))
         cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
-               *DEVICE_FLAGS, "-Wno-unused-command-line-argument", "-c", str(path), "-o", str(obj)]
+               *DEVICE_FLAGS, *extra, "-Wno-unused-command-line-argument", "-c", str(path), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
@@ -39,14 +44,14 @@ def build_library(verbose: bool = True) -> Path:
             raise RuntimeError(f"hipcc failed on {src}:\n{text}")
         if verbose and text.strip():
             print(text, flush=True)
-    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *objs, "-lpthread"]
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib), *objs, "-lpthread"]
     if verbose:
         print(" ".join(link), flush=True)
     subprocess.run(link, check=True)
-    return LIB_PATH
+    return lib
 
 
 if __name__ == "__main__":
-    build_library()
-    print(f"built {LIB_PATH}")
+    built = build_library(stamps="--stamps" in sys.argv[1:])
+    print(f"built {built}")
     sys.exit(0)
