@@ -544,95 +544,159 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 
 // ---------------------------------------------------------------------------
 // A batch of at most 32 rows against W on the matrix cores.  A block owns 32 rows of W;
-// its eight wavefronts cut the block's K range into eight pieces, and each multiplies its
-// piece straight out of registers: lane (l, half) loads 16 bytes of row n0 + l of W and
-// the same columns of input row l, and feeds them to MFMA 32x32x2 as the B and A operands
-// (which columns meet in one MFMA step does not matter for a sum over all of them).  No
-// LDS staging and no barrier in the stream; the eight 32x32 partial tiles are added in
-// wavefront order through LDS at the end.  With gridDim.y > 1 the K range is cut over
-// blocks as well and the raw tile goes to a.ws[part][M][N] for k_splitk_reduce.
-template <int EPI, bool WBF>
+// its eight wavefronts cut the block's K range into eight pieces.  MFMA 32x32x2 wants lane
+// (l, half) to hold columns of row l, but a load in that form touches 64 separate 64-byte
+// pieces of memory and the address path of the CU, not HBM, then sets the pace.  So a
+// wavefront loads 64 bytes of each of the 32 rows per step with four lanes to a row (16
+// pieces per load), turns the tile through a wavefront-private piece of LDS (no block
+// barrier: LDS operations of one wavefront execute in order) and reads it back with lane
+// (l, half) on row l.  The input rows take the same route unless they are in the packed
+// form, which is already laid out for the operand (XP).  Which columns meet in one MFMA
+// step does not matter for a sum over all of them.  Loads run PD steps ahead; every load
+// is issued (past the end it re-reads the last step) so that the count in flight is known
+// at compile time.  The eight 32x32 partial tiles are added in wavefront order through
+// LDS at the end.  With gridDim.y > 1 the K range is cut over blocks as well and the raw
+// tile goes to a.ws[part][M][N] for k_splitk_reduce.
+template <int EPI, bool WBF, bool XP>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
-  constexpr int U = WBF ? 16 : 8;  // columns per unit: 16 bytes of W per lane, two lane halves
-  constexpr int D = 7;             // units requested together
-  __shared__ float red[8][32][33];
+  constexpr int KS = WBF ? 32 : 16;      // columns per step: 64 bytes of a row of W
+  constexpr int XR = KS / 8;             // float4 of input per lane and step
+  constexpr int WSTR = 20;               // row stride of the W tile (floats; 64 bytes + pad)
+  constexpr int XSTR = KS + 4;           // row stride of the input tile
+  constexpr int SLAB = 32 * WSTR + 32 * XSTR;  // per wavefront; the reduce tile [32][33] fits
+  constexpr int PD = 2;                  // steps requested ahead (3, 4, 6 measured slower)
+  static_assert(SLAB >= 32 * 33, "reduce tile");
+  __shared__ __attribute__((aligned(16))) float slab[8][SLAB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
   const int n0 = (int)blockIdx.x * 32;
-  const int units = a.K / U;
+  const int steps = a.K / KS;
   const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
-  const int u0 = (int)(((long)piece * units) / pieces), u1 = (int)(((long)(piece + 1) * units) / pieces);
+  const int s0 = (int)(((long)piece * steps) / pieces), s1 = (int)(((long)(piece + 1) * steps) / pieces);
+  float* wt = slab[wave];
+  float* xt = slab[wave] + 32 * WSTR;
 
-  const size_t wrow = (size_t)min(n0 + l32, a.N - 1) * a.K + (U / 2) * half;
-  // this lane's input columns of unit u: xrow + u * xstep (and xrow + u * xstep + xnext for
-  // the second float4 of a 16-column unit).  Packed: the 32 lanes of a half read 512
-  // contiguous bytes; row-major: 32 rows lda floats apart.
-  const size_t xr = (size_t)min(l32, a.M - 1);
-  const float* xrow = a.a_packed ? a.A + packed32_index(xr, (size_t)(U / 2) * half)
-                                 : a.A + xr * a.lda + (U / 2) * half;
-  const size_t xstep = a.a_packed ? (size_t)U * 32 : (size_t)U;
-  const size_t xnext = a.a_packed ? 128 : 4;
+  // loads: four lanes to a row of W (q, t); rows q and 16 + q
+  const int q = lane >> 2, t = lane & 3;
+  const size_t rowbytes = (size_t)a.K * (WBF ? 2 : 4);
+  const char* wpa = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + q, a.N - 1) * rowbytes + 16 * t;
+  const char* wpb = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + 16 + q, a.N - 1) * rowbytes + 16 * t;
+  // input: packed, straight into operand form (k-block kb of row l32 at (kb * 32 + l32) * 4);
+  // row-major, KS / 4 lanes to a row
+  constexpr int XL = KS / 4;             // lanes to an input row
+  const int xq = lane / XL, xc = lane % XL;
+  const float* xp[XR];
+  int xw[XR];                            // where the lane's float4 goes in xt
+#pragma unroll
+  for (int j = 0; j < XR; ++j) {
+    if (XP) {
+      // f32 W: block 4 s + 2 u + half, u = j; bf16 W: block 8 s + 4 u + 2 half + e, j = 2 u + e
+      const int kb = WBF ? 4 * (j >> 1) + 2 * half + (j & 1) : 2 * j + half;
+      xp[j] = a.A + ((size_t)kb * 32 + min(l32, a.M - 1)) * 4;
+      xw[j] = 0;
+    } else {
+      const int r = xq + (64 / XL) * j;
+      xp[j] = a.A + (size_t)min(r, a.M - 1) * a.lda + 4 * xc;
+      xw[j] = r * XSTR + 4 * xc;
+    }
+  }
+  const size_t xstep = XP ? (size_t)(KS / 4) * 128 : (size_t)KS;
 
   f16v acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 
-  for (int u = u0; u < u1; u += D) {
-    f4 wv[D], xa[D], xb[D];
+  f4 rw[PD][2], rx[PD][XR];
+  auto load_step = [&](int s, f4* w, f4* x) {
+    const size_t sc = (size_t)min(s, s1 - 1);
+    w[0] = *reinterpret_cast<const f4*>(wpa + sc * 64);
+    w[1] = *reinterpret_cast<const f4*>(wpb + sc * 64);
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-      if (u + i >= u1) break;  // (wavefront-uniform)
-      const size_t unit = (size_t)(u + i), k = unit * U;
+    for (int j = 0; j < XR; ++j) x[j] = *reinterpret_cast<const f4*>(xp[j] + sc * xstep);
+  };
+  auto mul_step = [&](const f4* w, const f4* x) {
+    *reinterpret_cast<f4*>(wt + q * WSTR + 4 * t) = w[0];
+    *reinterpret_cast<f4*>(wt + (16 + q) * WSTR + 4 * t) = w[1];
+    if (!XP) {
+#pragma unroll
+      for (int j = 0; j < XR; ++j) *reinterpret_cast<f4*>(xt + xw[j]) = x[j];
+    }
+    __builtin_amdgcn_wave_barrier();
+    f4 wo[2], xo[XR];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) wo[u] = *reinterpret_cast<const f4*>(wt + l32 * WSTR + 4 * (2 * u + half));
+#pragma unroll
+    for (int j = 0; j < XR; ++j) {
+      if (XP) xo[j] = x[j];
+      else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xt + l32 * XSTR + 8 * (2 * (j >> 1) + half) + 4 * (j & 1));
+      else xo[j] = *reinterpret_cast<const f4*>(xt + l32 * XSTR + 4 * (2 * j + half));
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
       if (WBF) {
-        // 8 bf16 columns: widened below; the matching 8 input columns are two float4
-        wv[i] = *reinterpret_cast<const f4*>(reinterpret_cast<const unsigned short*>(a.W) + wrow + k);
-        xa[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep);
-        xb[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep + xnext);
-      } else {
-        wv[i] = *reinterpret_cast<const f4*>(a.W + wrow + k);
-        xa[i] = *reinterpret_cast<const f4*>(xrow + unit * xstep);
-      }
-    }
+        // 8 bf16 columns, widened; the matching 8 input columns are two float4
+        const unsigned* p = reinterpret_cast<const unsigned*>(&wo[u]);
+        float w8[8];
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-      if (u + i < u1) {  // wave-uniform
-        if (WBF) {
-          const unsigned* p = reinterpret_cast<const unsigned*>(&wv[i]);
-          float w8[8];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            w8[2 * q] = __uint_as_float(p[q] << 16);
-            w8[2 * q + 1] = __uint_as_float(p[q] & 0xffff0000u);
-          }
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].x, w8[0], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].y, w8[1], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].z, w8[2], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].w, w8[3], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].x, w8[4], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].y, w8[5], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].z, w8[6], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i].w, w8[7], acc, 0, 0, 0);
-        } else {
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].x, wv[i].x, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].y, wv[i].y, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].z, wv[i].z, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i].w, wv[i].w, acc, 0, 0, 0);
+        for (int c = 0; c < 4; ++c) {
+          w8[2 * c] = __uint_as_float(p[c] << 16);
+          w8[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
         }
+        const f4 xa = xo[2 * u], xb = xo[2 * u + 1];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc, 0, 0, 0);
+      } else {
+        const f4 xa = xo[u];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc, 0, 0, 0);
       }
     }
+  };
+  if (s1 > s0) {
+#pragma unroll
+    for (int i = 0; i < PD; ++i) load_step(s0 + i, rw[i], rx[i]);
+    int s = s0;
+    // rounds whose requests all exist: nothing conditional, the waits are exact
+    for (; s + 2 * PD <= s1; s += PD) {
+#pragma unroll
+      for (int i = 0; i < PD; ++i) {
+        mul_step(rw[i], rx[i]);
+        load_step(s + i + PD, rw[i], rx[i]);
+      }
+    }
+    // the last one or two rounds (all conditions wavefront-uniform)
+#pragma unroll
+    for (int i = 0; i < PD; ++i) {
+      if (s + i < s1) mul_step(rw[i], rx[i]);
+      if (s + i + PD < s1) load_step(s + i + PD, rw[i], rx[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < PD; ++i)
+      if (s + PD + i < s1) mul_step(rw[i], rx[i]);
   }
+  float (*red)[33] = reinterpret_cast<float (*)[33]>(slab[wave]);
+  auto red_at = [&](int w, int b, int nl) -> float& { return slab[w][b * 33 + nl]; };
 
   // acc[v] is row (batch index) 8 (v / 4) + 4 half + v % 4 of column l32
 #pragma unroll
-  for (int v = 0; v < 16; ++v) red[wave][8 * (v >> 2) + 4 * half + (v & 3)][l32] = acc[v];
+  for (int v = 0; v < 16; ++v) red[8 * (v >> 2) + 4 * half + (v & 3)][l32] = acc[v];
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
     const int idx = tid + 512 * q, b = idx >> 5, nl = idx & 31, n = n0 + nl;
     if (b >= a.M || n >= a.N) continue;
-    float sum = red[0][b][nl];
+    float sum = red_at(0, b, nl);
 #pragma unroll
-    for (int w = 1; w < 8; ++w) sum += red[w][b][nl];
+    for (int w = 1; w < 8; ++w) sum += red_at(w, b, nl);
     if (gridDim.y > 1) {
       a.ws[((size_t)blockIdx.y * a.M + b) * a.N + n] = sum;
       continue;
@@ -1108,11 +1172,11 @@ bool gemm_prefers_gemv_rows(const GemmArgs& a) {
   return a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024;
 }
 int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
-  const int U = a.w_bf16 ? 16 : 8;
+  const int U = a.w_bf16 ? 32 : 16;  // columns per step of the kernel
   if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
   const long tiles = (a.N + 31) / 32;
   long parts = std::max<long>(1, num_cus / tiles);
-  parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 16));
+  parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 8));
   parts = std::min<long>(parts, 8);
   if (parts > 1) {
     if (!a.ws || a.N % 4 != 0) parts = 1;
@@ -1120,17 +1184,24 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   }
   return (int)std::max<long>(parts, 1);
 }
+template <bool WBF, bool XP>
+hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP>), grid, dim3(512), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP>), grid, dim3(512), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP>), grid, dim3(512), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  return hipSuccess;
+}
 template <bool WBF>
 hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
   const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)parts);
-  if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF>), grid, dim3(512), 0, s, a);
-  else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF>), grid, dim3(512), 0, s, a);
-  else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF>), grid, dim3(512), 0, s, a);
-  else
-    return hipErrorInvalidValue;
+  const hipError_t e = a.a_packed ? launch_gemm_rows32_x<WBF, true>(a, epi, grid, s)
+                                  : launch_gemm_rows32_x<WBF, false>(a, epi, grid, s);
+  if (e != hipSuccess) return e;
   if (parts > 1) return launch_splitk_reduce(a, epi, parts, s, ln_done);
   return hipGetLastError();
 }
@@ -1319,12 +1390,12 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     if (packed || a.w_bf16) return hipErrorInvalidValue;
     return launch_gemm_tile<64, 64, 2>(a, epi, s);
   }
-  if (gemm_prefers_gemv_rows(a)) {
+  if (!a.plan_form && gemm_prefers_gemv_rows(a)) {
     if (packed) return hipErrorInvalidValue;
     return a.w_bf16 ? launch_gemv_rows<true>(a, epi, num_cus, s) : launch_gemv_rows<false>(a, epi, num_cus, s);
   }
   // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
-  if (const int rp = gemm_rows32_parts(a, num_cus))
+  if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
     return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done)
                     : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
   if (packed) return hipErrorInvalidValue;  // only the 32-row kernel knows the packed form
