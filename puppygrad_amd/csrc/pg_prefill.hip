@@ -557,10 +557,13 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // at compile time.  The eight 32x32 partial tiles are added in wavefront order through
 // LDS at the end.  With gridDim.y > 1 the K range is cut over blocks as well and the raw
 // tile goes to a.ws[part][M][N] for k_splitk_reduce.
-template <int EPI, bool WBF, bool XP>
+// M16: at most 16 input rows, MFMA 16x16x4 (half the matrix-core time and half the input
+// traffic of the 32-row form): lane (i, kq) holds columns 4 kq .. 4 kq + 3 of a step's
+// piece of input row i and of W rows i and 16 + i.
+template <int EPI, bool WBF, bool XP, bool M16>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   constexpr int KS = WBF ? 32 : 16;      // columns per step: 64 bytes of a row of W
-  constexpr int XR = KS / 8;             // float4 of input per lane and step
+  constexpr int XR = M16 ? KS / 16 : KS / 8;  // float4 of input per lane and step
   constexpr int WSTR = 20;               // row stride of the W tile (floats; 64 bytes + pad)
   constexpr int XSTR = KS + 4;           // row stride of the input tile
   constexpr int SLAB = 32 * WSTR + 32 * XSTR;  // per wavefront; the reduce tile [32][33] fits
@@ -568,7 +571,9 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   static_assert(SLAB >= 32 * 33, "reduce tile");
   __shared__ __attribute__((aligned(16))) float slab[8][SLAB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int half = lane >> 5, l32 = lane & 31;
+  // operand position of the lane: row orow, 16-byte piece opc of the row's 64 bytes
+  const int orow = M16 ? (lane & 15) : (lane & 31);
+  const int opc = M16 ? (lane >> 4) : (lane >> 5);
   const int n0 = (int)blockIdx.x * 32;
   const int steps = a.K / KS;
   const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
@@ -581,7 +586,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   const size_t rowbytes = (size_t)a.K * (WBF ? 2 : 4);
   const char* wpa = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + q, a.N - 1) * rowbytes + 16 * t;
   const char* wpb = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + 16 + q, a.N - 1) * rowbytes + 16 * t;
-  // input: packed, straight into operand form (k-block kb of row l32 at (kb * 32 + l32) * 4);
+  // input: packed, straight into operand form (k-block kb of row r at (kb * 32 + r) * 4);
   // row-major, KS / 4 lanes to a row
   constexpr int XL = KS / 4;             // lanes to an input row
   const int xq = lane / XL, xc = lane % XL;
@@ -590,9 +595,11 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
   for (int j = 0; j < XR; ++j) {
     if (XP) {
-      // f32 W: block 4 s + 2 u + half, u = j; bf16 W: block 8 s + 4 u + 2 half + e, j = 2 u + e
-      const int kb = WBF ? 4 * (j >> 1) + 2 * half + (j & 1) : 2 * j + half;
-      xp[j] = a.A + ((size_t)kb * 32 + min(l32, a.M - 1)) * 4;
+      // the k-blocks of the lane's operand piece(s); see the reads in mul_step
+      int kb;
+      if (M16) kb = WBF ? 2 * opc + j : opc;
+      else kb = WBF ? 4 * (j >> 1) + 2 * opc + (j & 1) : 2 * j + opc;
+      xp[j] = a.A + ((size_t)kb * 32 + min(orow, a.M - 1)) * 4;
       xw[j] = 0;
     } else {
       const int r = xq + (64 / XL) * j;
@@ -602,9 +609,11 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   }
   const size_t xstep = XP ? (size_t)(KS / 4) * 128 : (size_t)KS;
 
-  f16v acc;
+  f16v acc;       // 32-row form
+  f4 acc16[2];    // 16-row form: W rows 0..15 and 16..31
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  acc16[0] = acc16[1] = f4{0.f, 0.f, 0.f, 0.f};
 
   f4 rw[PD][2], rx[PD][XR];
   auto load_step = [&](int s, f4* w, f4* x) {
@@ -613,6 +622,15 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     w[1] = *reinterpret_cast<const f4*>(wpb + sc * 64);
 #pragma unroll
     for (int j = 0; j < XR; ++j) x[j] = *reinterpret_cast<const f4*>(xp[j] + sc * xstep);
+  };
+  // 8 bf16 -> 8 floats
+  auto widen8 = [](const f4& v, float* w8) {
+    const unsigned* p = reinterpret_cast<const unsigned*>(&v);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      w8[2 * c] = __uint_as_float(p[c] << 16);
+      w8[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
+    }
   };
   auto mul_step = [&](const f4* w, const f4* x) {
     *reinterpret_cast<f4*>(wt + q * WSTR + 4 * t) = w[0];
@@ -623,41 +641,71 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     }
     __builtin_amdgcn_wave_barrier();
     f4 wo[2], xo[XR];
+    if (M16) {
+      // W rows orow and 16 + orow, piece opc; the same piece of input row orow
 #pragma unroll
-    for (int u = 0; u < 2; ++u) wo[u] = *reinterpret_cast<const f4*>(wt + l32 * WSTR + 4 * (2 * u + half));
+      for (int g = 0; g < 2; ++g) wo[g] = *reinterpret_cast<const f4*>(wt + (16 * g + orow) * WSTR + 4 * opc);
 #pragma unroll
-    for (int j = 0; j < XR; ++j) {
-      if (XP) xo[j] = x[j];
-      else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xt + l32 * XSTR + 8 * (2 * (j >> 1) + half) + 4 * (j & 1));
-      else xo[j] = *reinterpret_cast<const f4*>(xt + l32 * XSTR + 4 * (2 * j + half));
+      for (int j = 0; j < XR; ++j) {
+        if (XP) xo[j] = x[j];
+        else xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + (WBF ? 8 : 4) * opc + 4 * j);
+      }
+    } else {
+      // pieces opc and 2 + opc of W row orow
+#pragma unroll
+      for (int u = 0; u < 2; ++u) wo[u] = *reinterpret_cast<const f4*>(wt + orow * WSTR + 4 * (2 * u + opc));
+#pragma unroll
+      for (int j = 0; j < XR; ++j) {
+        if (XP) xo[j] = x[j];
+        else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + 8 * (2 * (j >> 1) + opc) + 4 * (j & 1));
+        else xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + 4 * (2 * j + opc));
+      }
     }
     __builtin_amdgcn_wave_barrier();
+    if (M16) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      if (WBF) {
-        // 8 bf16 columns, widened; the matching 8 input columns are two float4
-        const unsigned* p = reinterpret_cast<const unsigned*>(&wo[u]);
-        float w8[8];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          w8[2 * c] = __uint_as_float(p[c] << 16);
-          w8[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
+      for (int g = 0; g < 2; ++g) {
+        if (WBF) {
+          float w8[8];
+          widen8(wo[g], w8);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].x, w8[0], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].y, w8[1], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].z, w8[2], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].w, w8[3], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].x, w8[4], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].y, w8[5], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].z, w8[6], acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].w, w8[7], acc16[g], 0, 0, 0);
+        } else {
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].x, wo[g].x, acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].y, wo[g].y, acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].z, wo[g].z, acc16[g], 0, 0, 0);
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].w, wo[g].w, acc16[g], 0, 0, 0);
         }
-        const f4 xa = xo[2 * u], xb = xo[2 * u + 1];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc, 0, 0, 0);
-      } else {
-        const f4 xa = xo[u];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (WBF) {
+          // 8 bf16 columns, widened; the matching 8 input columns are two float4
+          float w8[8];
+          widen8(wo[u], w8);
+          const f4 xa = xo[2 * u], xb = xo[(2 * u + 1) % XR];
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc, 0, 0, 0);
+        } else {
+          const f4 xa = xo[u % XR];
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc, 0, 0, 0);
+        }
       }
     }
   };
@@ -686,9 +734,17 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   float (*red)[33] = reinterpret_cast<float (*)[33]>(slab[wave]);
   auto red_at = [&](int w, int b, int nl) -> float& { return slab[w][b * 33 + nl]; };
 
-  // acc[v] is row (batch index) 8 (v / 4) + 4 half + v % 4 of column l32
+  if (M16) {
+    // acc16[g][r] is row (batch index) 4 (lane / 16) + r of column 16 g + lane % 16
 #pragma unroll
-  for (int v = 0; v < 16; ++v) red[8 * (v >> 2) + 4 * half + (v & 3)][l32] = acc[v];
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[4 * opc + r][16 * g + orow] = acc16[g][r];
+  } else {
+    // acc[v] is row (batch index) 8 (v / 4) + 4 (lane / 32) + v % 4 of column lane % 32
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[8 * (v >> 2) + 4 * opc + (v & 3)][orow] = acc[v];
+  }
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
@@ -1168,8 +1224,12 @@ hipError_t launch_gemv_rows(const GemmArgs& a, int epi, int num_cus, hipStream_t
 // up, or cutting less, were all measured slower: the reduce launch and the shorter pieces
 // cost more than the idle CUs), at least sixteen units per block and part, bounded by the
 // workspace.
+// Whole rows of W per wavefront (k_gemv_rows) only where the matrix-core kernel does not
+// take the shape (its 16-row form is as fast or faster from K = 768 on: 124M c_attn 7.9 against
+// 10.9 us, 355M c_fc 9.4 against 10.2 us with the weights coming from HBM).
 bool gemm_prefers_gemv_rows(const GemmArgs& a) {
-  return a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024;
+  if (!(a.M <= 16 && a.K % 4 == 0 && a.K >= 4 && a.K <= 1024)) return false;
+  return a.K % (a.w_bf16 ? 32 : 16) != 0 || a.lda % 4 != 0;
 }
 int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 32 : 16;  // columns per step of the kernel
@@ -1184,17 +1244,22 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   }
   return (int)std::max<long>(parts, 1);
 }
-template <bool WBF, bool XP>
-hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
+template <bool WBF, bool XP, bool M16>
+hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16>), grid, dim3(512), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipSuccess;
+}
+template <bool WBF, bool XP>
+hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
+  return a.M <= 16 ? launch_gemm_rows32_m<WBF, XP, true>(a, epi, grid, s)
+                   : launch_gemm_rows32_m<WBF, XP, false>(a, epi, grid, s);
 }
 template <bool WBF>
 hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
@@ -1389,6 +1454,11 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   if (a.w_scale) {  // int8 rows: the 64x64 tile form dequantises them as it loads
     if (packed || a.w_bf16) return hipErrorInvalidValue;
     return launch_gemm_tile<64, 64, 2>(a, epi, s);
+  }
+  if (a.plan_form == 4) {  // forced: the 32-row kernel
+    const int rp = gemm_rows32_parts(a, num_cus);
+    if (!rp) return hipErrorInvalidValue;
+    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done) : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
   }
   if (!a.plan_form && gemm_prefers_gemv_rows(a)) {
     if (packed) return hipErrorInvalidValue;
