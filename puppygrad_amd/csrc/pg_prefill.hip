@@ -560,8 +560,11 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // M16: at most 16 input rows, MFMA 16x16x4 (half the matrix-core time and half the input
 // traffic of the 32-row form): lane (i, kq) holds columns 4 kq .. 4 kq + 3 of a step's
 // piece of input row i and of W rows i and 16 + i.
-template <int EPI, bool WBF, bool XP, bool M16>
+// NR: rows of W per block; 16 (16-row form only) where 32-row blocks would leave half of
+// the CUs without one.
+template <int EPI, bool WBF, bool XP, bool M16, int NR>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
+  static_assert(NR == 32 || (NR == 16 && M16), "rows per block");
   constexpr int KS = WBF ? 32 : 16;      // columns per step: 64 bytes of a row of W
   constexpr int XR = M16 ? KS / 16 : KS / 8;  // float4 of input per lane and step
   constexpr int WSTR = 20;               // row stride of the W tile (floats; 64 bytes + pad)
@@ -574,7 +577,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   // operand position of the lane: row orow, 16-byte piece opc of the row's 64 bytes
   const int orow = M16 ? (lane & 15) : (lane & 31);
   const int opc = M16 ? (lane >> 4) : (lane >> 5);
-  const int n0 = (int)blockIdx.x * 32;
+  const int n0 = (int)blockIdx.x * NR;
   const int steps = a.K / KS;
   const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
   const int s0 = (int)(((long)piece * steps) / pieces), s1 = (int)(((long)(piece + 1) * steps) / pieces);
@@ -619,7 +622,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   auto load_step = [&](int s, f4* w, f4* x) {
     const size_t sc = (size_t)min(s, s1 - 1);
     w[0] = *reinterpret_cast<const f4*>(wpa + sc * 64);
-    w[1] = *reinterpret_cast<const f4*>(wpb + sc * 64);
+    if (NR == 32) w[1] = *reinterpret_cast<const f4*>(wpb + sc * 64);
 #pragma unroll
     for (int j = 0; j < XR; ++j) x[j] = *reinterpret_cast<const f4*>(xp[j] + sc * xstep);
   };
@@ -634,7 +637,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   };
   auto mul_step = [&](const f4* w, const f4* x) {
     *reinterpret_cast<f4*>(wt + q * WSTR + 4 * t) = w[0];
-    *reinterpret_cast<f4*>(wt + (16 + q) * WSTR + 4 * t) = w[1];
+    if (NR == 32) *reinterpret_cast<f4*>(wt + (16 + q) * WSTR + 4 * t) = w[1];
     if (!XP) {
 #pragma unroll
       for (int j = 0; j < XR; ++j) *reinterpret_cast<f4*>(xt + xw[j]) = x[j];
@@ -644,7 +647,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     if (M16) {
       // W rows orow and 16 + orow, piece opc; the same piece of input row orow
 #pragma unroll
-      for (int g = 0; g < 2; ++g) wo[g] = *reinterpret_cast<const f4*>(wt + (16 * g + orow) * WSTR + 4 * opc);
+      for (int g = 0; g < NR / 16; ++g) wo[g] = *reinterpret_cast<const f4*>(wt + (16 * g + orow) * WSTR + 4 * opc);
 #pragma unroll
       for (int j = 0; j < XR; ++j) {
         if (XP) xo[j] = x[j];
@@ -664,7 +667,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     __builtin_amdgcn_wave_barrier();
     if (M16) {
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
+      for (int g = 0; g < NR / 16; ++g) {
         if (WBF) {
           float w8[8];
           widen8(wo[g], w8);
@@ -737,7 +740,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   if (M16) {
     // acc16[g][r] is row (batch index) 4 (lane / 16) + r of column 16 g + lane % 16
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
+    for (int g = 0; g < NR / 16; ++g)
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[4 * opc + r][16 * g + orow] = acc16[g][r];
   } else {
@@ -748,8 +751,8 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
-    const int idx = tid + 512 * q, b = idx >> 5, nl = idx & 31, n = n0 + nl;
-    if (b >= a.M || n >= a.N) continue;
+    const int idx = tid + 512 * q, b = idx / NR, nl = idx % NR, n = n0 + nl;
+    if (idx >= 32 * NR || b >= a.M || n >= a.N) continue;
     float sum = red_at(0, b, nl);
 #pragma unroll
     for (int w = 1; w < 8; ++w) sum += red_at(w, b, nl);
@@ -1235,7 +1238,8 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 32 : 16;  // columns per step of the kernel
   if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
   const long tiles = (a.N + 31) / 32;
-  long parts = std::max<long>(1, num_cus / tiles);
+  // (a cut in two plus its reduce launch costs more than it saves: 355M c_attn and c_fc)
+  long parts = tiles * 4 > num_cus ? 1 : std::max<long>(1, num_cus / tiles);
   parts = std::min<long>(parts, std::max<long>(1, (a.K / U) / 8));
   parts = std::min<long>(parts, 8);
   if (parts > 1) {
@@ -1244,28 +1248,32 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   }
   return (int)std::max<long>(parts, 1);
 }
-template <bool WBF, bool XP, bool M16>
-hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
+template <bool WBF, bool XP, bool M16, int NR>
+hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, int parts, hipStream_t s) {
+  const dim3 grid((unsigned)((a.N + NR - 1) / NR), (unsigned)parts);
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipSuccess;
 }
 template <bool WBF, bool XP>
-hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, const dim3& grid, hipStream_t s) {
-  return a.M <= 16 ? launch_gemm_rows32_m<WBF, XP, true>(a, epi, grid, s)
-                   : launch_gemm_rows32_m<WBF, XP, false>(a, epi, grid, s);
+hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s) {
+  if (a.M > 16) return launch_gemm_rows32_m<WBF, XP, false, 32>(a, epi, parts, s);
+  // 16 rows of W per block where K is not cut and 32-row blocks would reach at most half of
+  // the CUs (a CU then pulls half as much of W, and as much of the input)
+  if (parts == 1 && (long)((a.N + 31) / 32) * 2 <= num_cus)
+    return launch_gemm_rows32_m<WBF, XP, true, 16>(a, epi, parts, s);
+  return launch_gemm_rows32_m<WBF, XP, true, 32>(a, epi, parts, s);
 }
 template <bool WBF>
-hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
-  const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)parts);
-  const hipError_t e = a.a_packed ? launch_gemm_rows32_x<WBF, true>(a, epi, grid, s)
-                                  : launch_gemm_rows32_x<WBF, false>(a, epi, grid, s);
+hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s, bool* ln_done) {
+  const hipError_t e = a.a_packed ? launch_gemm_rows32_x<WBF, true>(a, epi, parts, num_cus, s)
+                                  : launch_gemm_rows32_x<WBF, false>(a, epi, parts, num_cus, s);
   if (e != hipSuccess) return e;
   if (parts > 1) return launch_splitk_reduce(a, epi, parts, s, ln_done);
   return hipGetLastError();
@@ -1458,7 +1466,7 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   if (a.plan_form == 4) {  // forced: the 32-row kernel
     const int rp = gemm_rows32_parts(a, num_cus);
     if (!rp) return hipErrorInvalidValue;
-    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done) : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
+    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, num_cus, s, ln_done) : launch_gemm_rows32<false>(a, epi, rp, num_cus, s, ln_done);
   }
   if (!a.plan_form && gemm_prefers_gemv_rows(a)) {
     if (packed) return hipErrorInvalidValue;
@@ -1466,8 +1474,8 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   }
   // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
   if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
-    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, s, ln_done)
-                    : launch_gemm_rows32<false>(a, epi, rp, s, ln_done);
+    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, num_cus, s, ln_done)
+                    : launch_gemm_rows32<false>(a, epi, rp, num_cus, s, ln_done);
   if (packed) return hipErrorInvalidValue;  // only the 32-row kernel knows the packed form
   // Tile forms.  A forced plan (benchmarks, tests) or the planner's choice.
   int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;

@@ -44,7 +44,8 @@ def test_dense_matches_oracle(rows, k, n):
                                       (512, 768, 3072), (16, 1024, 3072), (32, 1600, 6400),
                                       (16, 4096, 1024), (16, 1600, 4800),
                                       (100, 48, 100), (333, 112, 260), (200, 32, 64), (64, 16, 52),
-                                      (1024, 3072, 768), (1024, 1600, 4800)])
+                                      (1024, 3072, 768), (1024, 1600, 4800),
+                                      (16, 100, 52), (24, 768, 768), (16, 768, 1000)])
 def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised.
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
@@ -53,8 +54,11 @@ def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # K = 48 and 112 are not multiples of 32 and take k-tiles of 16 columns; K = 16 and 32 are a
     # single k-tile (the pipelined loop's shortest cases); (1024, 3072, 768) has a deep K on 192
     # tiles and is cut in four; (1024, 1600, 4800) runs 128x128 tiles with the last round cut.
-    # 16 rows with K <= 1024 take the row-streaming kernel of the decode batch; other shapes
-    # of up to 32 rows the register-fed MFMA kernel (with and without a cut of K over blocks).
+    # Up to 32 rows take the MFMA kernel of the decode batch: 16 rows its 16x16x4 form, with 16
+    # rows of W per block where 32 would leave CUs idle ((16, 768, 2304), (16, 1024, 3072),
+    # (16, 768, 1000) with a ragged last block) and 32 otherwise ((16, 1600, 4800); (16, 4096,
+    # 1024) with K cut over blocks); 17..32 rows the 32x32x2 form ((32, 1600, 6400), (20, 768,
+    # 50257), (24, 768, 768)).  (16, 100, 52): K is no multiple of 16, the row-streaming kernel.
     rng = np.random.default_rng(rows * 7 + n)
     x = rng.standard_normal(rows * k).astype(np.float32)
     w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
