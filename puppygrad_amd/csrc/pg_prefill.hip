@@ -1307,7 +1307,9 @@ hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
 //    fewer than 1.5 tiles per CU, about split_items_per_cu work items per CU, a part at least
 //    128 deep.
 //  - Tall operands whose tiles occupy at most half of the CUs: the same, a part at least 192
-//    deep.
+//    deep (128 with tiles for at most a quarter of the CUs).
+//  - Tall operands with more than half a tile and at most one tile per CU and a K of
+//    768..2047: two or three parts, about 1.75 work items per CU.
 //  - Tall operands with up to two tiles per CU and a deep K (the MLP's second projection):
 //    up to four parts of at least 768 columns; more blocks per CU hide each other's waits
 //    and the parts even out the load.
@@ -1318,10 +1320,15 @@ int gemm_split_parts(const GemmArgs& a, int num_cus, int bm, int bn) {
   if (!a.ws || a.N % 4 != 0) return 1;
   int parts = 1;
   if (a.M < 64 ? tiles * 2 < 3L * num_cus : tiles * 2 <= num_cus) {
-    const int depth = a.M < 64 ? 128 : 192;
+    const int depth = a.M < 64 || tiles * 4 <= num_cus ? 128 : 192;
     parts = (int)(((long)std::max(a.split_items_per_cu, 1) * num_cus) / tiles);
     parts = std::min(parts, a.K / depth);
     parts = std::min(parts, 8);
+  } else if (a.M >= 64 && tiles <= num_cus && a.K >= 768 && a.K < 2048) {
+    // a few rows of tiles (prompts of 65..256 tokens): one tile per CU walks its k loop at one
+    // memory latency per k-tile; about 1.75 items per CU overlap each other's waits
+    parts = (int)((7L * num_cus + 2 * tiles) / (4 * tiles));
+    parts = std::max(1, std::min(parts, a.K / 256));
   } else if (a.M >= 64 && tiles <= 2L * num_cus && a.K >= 2048) {
     parts = std::min(4, a.K / 768);
   }
