@@ -562,16 +562,20 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // piece of input row i and of W rows i and 16 + i.
 // NR: rows of W per block; 16 (16-row form only) where 32-row blocks would leave half of
 // the CUs without one.
-template <int EPI, bool WBF, bool XP, bool M16, int NR>
+// MT: tiles of 32 input rows (2: up to 64 rows, row-major input only; the W operands of a step
+// are used twice).
+template <int EPI, bool WBF, bool XP, bool M16, int NR, int MT>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   static_assert(NR == 32 || (NR == 16 && M16), "rows per block");
+  static_assert(MT == 1 || (MT == 2 && !M16 && !XP), "input rows");
   constexpr int KS = WBF ? 32 : 16;      // columns per step: 64 bytes of a row of W
-  constexpr int XR = M16 ? KS / 16 : KS / 8;  // float4 of input per lane and step
+  constexpr int XR = M16 ? KS / 16 : MT * KS / 8;  // float4 of input per lane and step
+  constexpr int XT = KS / 8;             // of those, per tile of 32 rows
   constexpr int WSTR = 20;               // row stride of the W tile (floats; 64 bytes + pad)
   constexpr int XSTR = KS + 4;           // row stride of the input tile
-  constexpr int SLAB = 32 * WSTR + 32 * XSTR;  // per wavefront; the reduce tile [32][33] fits
+  // per wavefront: W tile, input tile; the reduce tile [32 MT][33] lies over them
+  constexpr int SLAB = 32 * WSTR + 32 * MT * XSTR > 32 * MT * 33 ? 32 * WSTR + 32 * MT * XSTR : 32 * MT * 33;
   constexpr int PD = 2;                  // steps requested ahead (3, 4, 6 measured slower)
-  static_assert(SLAB >= 32 * 33, "reduce tile");
   __shared__ __attribute__((aligned(16))) float slab[8][SLAB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // operand position of the lane: row orow, 16-byte piece opc of the row's 64 bytes
@@ -612,10 +616,12 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   }
   const size_t xstep = XP ? (size_t)(KS / 4) * 128 : (size_t)KS;
 
-  f16v acc;       // 32-row form
+  f16v acc[MT];   // 32-row form
   f4 acc16[2];    // 16-row form: W rows 0..15 and 16..31
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[mt][v] = 0.0f;
   acc16[0] = acc16[1] = f4{0.f, 0.f, 0.f, 0.f};
 
   f4 rw[PD][2], rx[PD][XR];
@@ -659,9 +665,12 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       for (int u = 0; u < 2; ++u) wo[u] = *reinterpret_cast<const f4*>(wt + orow * WSTR + 4 * (2 * u + opc));
 #pragma unroll
       for (int j = 0; j < XR; ++j) {
+        // tile mt = j / XT of the input rows, operand jj = j % XT of the step
+        const int mt = j / XT, jj = j % XT;
+        const float* xr = xt + (32 * mt + orow) * XSTR;
         if (XP) xo[j] = x[j];
-        else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + 8 * (2 * (j >> 1) + opc) + 4 * (j & 1));
-        else xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + 4 * (2 * j + opc));
+        else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xr + 8 * (2 * (jj >> 1) + opc) + 4 * (jj & 1));
+        else xo[j] = *reinterpret_cast<const f4*>(xr + 4 * (2 * jj + opc));
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -693,21 +702,27 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
           // 8 bf16 columns, widened; the matching 8 input columns are two float4
           float w8[8];
           widen8(wo[u], w8);
-          const f4 xa = xo[2 * u], xb = xo[(2 * u + 1) % XR];
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc, 0, 0, 0);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const f4 xa = xo[mt * XT + 2 * u], xb = xo[mt * XT + (2 * u + 1) % XT];
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc[mt], 0, 0, 0);
+          }
         } else {
-          const f4 xa = xo[u % XR];
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc, 0, 0, 0);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const f4 xa = xo[mt * XT + u % XT];
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc[mt], 0, 0, 0);
+          }
         }
       }
     }
@@ -744,15 +759,17 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[4 * opc + r][16 * g + orow] = acc16[g][r];
   } else {
-    // acc[v] is row (batch index) 8 (v / 4) + 4 (lane / 32) + v % 4 of column lane % 32
+    // acc[mt][v] is row (batch index) 32 mt + 8 (v / 4) + 4 (lane / 32) + v % 4 of column lane % 32
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red[8 * (v >> 2) + 4 * opc + (v & 3)][orow] = acc[v];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) red[32 * mt + 8 * (v >> 2) + 4 * opc + (v & 3)][orow] = acc[mt][v];
   }
   __syncthreads();
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
+  for (int q = 0; q < 2 * MT; ++q) {
     const int idx = tid + 512 * q, b = idx / NR, nl = idx % NR, n = n0 + nl;
-    if (idx >= 32 * NR || b >= a.M || n >= a.N) continue;
+    if (idx >= 32 * MT * NR || b >= a.M || n >= a.N) continue;
     float sum = red_at(0, b, nl);
 #pragma unroll
     for (int w = 1; w < 8; ++w) sum += red_at(w, b, nl);
@@ -1236,7 +1253,7 @@ bool gemm_prefers_gemv_rows(const GemmArgs& a) {
 }
 int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   const int U = a.w_bf16 ? 32 : 16;  // columns per step of the kernel
-  if (a.M > 32 || a.K % U != 0 || a.lda % 4 != 0) return 0;
+  if (a.M > (a.a_packed || a.c_packed || a.ln_packed ? 32 : 64) || a.K % U != 0 || a.lda % 4 != 0) return 0;
   const long tiles = (a.N + 31) / 32;
   // (a cut in two plus its reduce launch costs more than it saves: 355M c_attn and c_fc)
   long parts = tiles * 4 > num_cus ? 1 : std::max<long>(1, num_cus / tiles);
@@ -1248,21 +1265,25 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   }
   return (int)std::max<long>(parts, 1);
 }
-template <bool WBF, bool XP, bool M16, int NR>
+template <bool WBF, bool XP, bool M16, int NR, int MT = 1>
 hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, int parts, hipStream_t s) {
   const dim3 grid((unsigned)((a.N + NR - 1) / NR), (unsigned)parts);
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16, NR>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipSuccess;
 }
 template <bool WBF, bool XP>
 hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s) {
+  if (a.M > 32) {
+    if constexpr (XP) return hipErrorInvalidValue;  // the packed form holds 32 rows
+    else return launch_gemm_rows32_m<WBF, false, false, 32, 2>(a, epi, parts, s);
+  }
   if (a.M > 16) return launch_gemm_rows32_m<WBF, XP, false, 32>(a, epi, parts, s);
   // 16 rows of W per block where K is not cut and 32-row blocks would reach at most half of
   // the CUs (a CU then pulls half as much of W, and as much of the input)
@@ -1456,7 +1477,7 @@ hipError_t launch_gemm(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
 bool gemm_takes_rows32(int M, int K, int lda, int w_bf16) {
   GemmArgs a{};
   a.M = M; a.K = K; a.lda = lda; a.w_bf16 = w_bf16; a.N = 32;
-  return !gemm_prefers_gemv_rows(a) && gemm_rows32_parts(a, 1) != 0;
+  return M <= 32 && !gemm_prefers_gemv_rows(a) && gemm_rows32_parts(a, 1) != 0;
 }
 
 namespace {

@@ -45,7 +45,8 @@ def test_dense_matches_oracle(rows, k, n):
                                       (16, 4096, 1024), (16, 1600, 4800),
                                       (100, 48, 100), (333, 112, 260), (200, 32, 64), (64, 16, 52),
                                       (1024, 3072, 768), (1024, 1600, 4800),
-                                      (16, 100, 52), (24, 768, 768), (16, 768, 1000)])
+                                      (16, 100, 52), (24, 768, 768), (16, 768, 1000),
+                                      (48, 768, 2304), (33, 1600, 1600), (64, 3072, 768)])
 def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised.
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
@@ -58,7 +59,10 @@ def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows of W per block where 32 would leave CUs idle ((16, 768, 2304), (16, 1024, 3072),
     # (16, 768, 1000) with a ragged last block) and 32 otherwise ((16, 1600, 4800); (16, 4096,
     # 1024) with K cut over blocks); 17..32 rows the 32x32x2 form ((32, 1600, 6400), (20, 768,
-    # 50257), (24, 768, 768)).  (16, 100, 52): K is no multiple of 16, the row-streaming kernel.
+    # 50257), (24, 768, 768)); 33..64 rows that form with two tiles of input rows ((48, 768,
+    # 2304), (33, 1600, 1600) and (64, 3072, 768) with K cut over blocks, (37, 64, 50) ragged,
+    # (64, 16, 52) with a single step for eight wavefronts).  (16, 100, 52): K is no multiple
+    # of 16, the row-streaming kernel.
     rng = np.random.default_rng(rows * 7 + n)
     x = rng.standard_normal(rows * k).astype(np.float32)
     w = (rng.standard_normal(n * k) * 0.02).astype(np.float32)
