@@ -373,6 +373,13 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
                      "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
                      "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
     }
+    # A short prompt reads every weight once for few rows: below about 52 rows the weights'
+    # bytes at the HBM peak take longer than the flops at the MFMA peak, and HBM is the bound.
+    wbytes = weight_bytes(cfg)
+    if wbytes / (HBM_PEAK_GBS * 1e9) > flops / (FP32_MFMA_PEAK_TFLOPS * 1e12):
+        gbs = wbytes / sec / 1e9
+        result["roofline"] = hbm_roofline(gbs, "whole prefill (k_gemm_rows32, k_attn_prefill64, reduce + LayerNorm, lm_head)",
+                                          algorithmic_bytes_per_step=int(wbytes))
     print(json.dumps(result), flush=True)
     return 0
 
