@@ -17,7 +17,7 @@ def batch_case(seed, B, n, cfg):
 
 
 @pytest.mark.parametrize("prefill_path", [0, 1], ids=["gemm_prefill", "token_prefill"])
-@pytest.mark.parametrize("B,n", [(3, 21), (16, 17), (2, 5), (17, 6), (20, 9), (32, 7)])
+@pytest.mark.parametrize("B,n", [(3, 21), (16, 17), (2, 5), (17, 6), (20, 9), (32, 7), (40, 5)])
 def test_batched_steps_match_oracle(B, n, prefill_path):
     cfg = Gpt2Config(vocab_size=257, n_positions=48, n_embd=128, n_layer=2, n_head=2)
     w, ids = batch_case(B * 100 + n, B, n, cfg)
