@@ -543,7 +543,7 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// A batch of at most 32 rows against W on the matrix cores.  A block owns 32 rows of W;
+// A batch of at most 32 rows (64 with MT = 2) against W on the matrix cores.  A block owns 32 rows of W;
 // its eight wavefronts cut the block's K range into eight pieces.  MFMA 32x32x2 wants lane
 // (l, half) to hold columns of row l, but a load in that form touches 64 separate 64-byte
 // pieces of memory and the address path of the CU, not HBM, then sets the pace.  So a
@@ -552,10 +552,11 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // barrier: LDS operations of one wavefront execute in order) and reads it back with lane
 // (l, half) on row l.  The input rows take the same route unless they are in the packed
 // form, which is already laid out for the operand (XP).  Which columns meet in one MFMA
-// step does not matter for a sum over all of them.  Loads run PD steps ahead; every load
-// is issued (past the end it re-reads the last step) so that the count in flight is known
-// at compile time.  The eight 32x32 partial tiles are added in wavefront order through
-// LDS at the end.  With gridDim.y > 1 the K range is cut over blocks as well and the raw
+// step does not matter for a sum over all of them.  Loads run PD steps ahead: whole rounds
+// of PD steps issue every load unconditionally, so that the count in flight is known at
+// compile time, and a peeled tail handles the rest (only a wavefront with fewer than PD
+// steps re-reads its last step in the prologue).  The eight 32x32 partial tiles are added
+// in wavefront order through LDS at the end.  With gridDim.y > 1 the K range is cut over blocks as well and the raw
 // tile goes to a.ws[part][M][N] for k_splitk_reduce.
 // M16: at most 16 input rows, MFMA 16x16x4 (half the matrix-core time and half the input
 // traffic of the 32-row form): lane (i, kq) holds columns 4 kq .. 4 kq + 3 of a step's
