@@ -389,20 +389,29 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts)
     return (red[0] + red[1]) + (red[2] + red[3]);
   };
   f4 c[4];
+  // all partial sums of the row are requested before the first is used (columns past the end
+  // re-read the last float4)
+  f4 v[4][8], lg[4], lb[4];  // (and the LayerNorm's scale and shift for the lane's columns)
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (256 * q >= n4) continue;  // (block-uniform)
+    const size_t n = (size_t)min((int)threadIdx.x + 256 * q, n4 - 1) * 4;
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+      v[q][p] = *reinterpret_cast<const f4*>(a.ws + (size_t)min(p, parts - 1) * stride + m * a.N + n);
+    lg[q] = *reinterpret_cast<const f4*>(a.ln_g + n);
+    lb[q] = *reinterpret_cast<const f4*>(a.ln_b + n);
+  }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int i = (int)threadIdx.x + 256 * q;
     c[q] = f4{0.f, 0.f, 0.f, 0.f};
     if (i < n4) {
       const size_t n = (size_t)i * 4;
-      f4 v[8];
-#pragma unroll
-      for (int p = 0; p < 8; ++p)
-        v[p] = *reinterpret_cast<const f4*>(a.ws + (size_t)min(p, parts - 1) * stride + m * a.N + n);
-      f4 s = v[0];
+      f4 s = v[q][0];
 #pragma unroll
       for (int p = 1; p < 8; ++p)
-        if (p < parts) s += v[p];
+        if (p < parts) s += v[q][p];
       const f4 b = a.bias ? *reinterpret_cast<const f4*>(a.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
       float r[4] = {b.x + s.x, b.y + s.y, b.z + s.z, b.w + s.w};
 #pragma unroll
@@ -432,7 +441,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts)
     const int i = (int)threadIdx.x + 256 * q;
     if (i < n4) {
       const size_t n = (size_t)i * 4;
-      const f4 g = *reinterpret_cast<const f4*>(a.ln_g + n), b = *reinterpret_cast<const f4*>(a.ln_b + n);
+      const f4 g = lg[q], b = lb[q];
       f4 o;
       o.x = (c[q].x - mean) * inv * g.x + b.x;
       o.y = (c[q].y - mean) * inv * g.y + b.y;
