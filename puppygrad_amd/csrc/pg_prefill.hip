@@ -626,6 +626,17 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   }
   const size_t xstep = XP ? (size_t)(KS / 4) * 128 : (size_t)KS;
 
+  // bias and residual of the outputs this thread writes at the end: requested now, so that
+  // the write-out does not wait for them (K not cut over blocks)
+  float ebias[2 * MT], eres[2 * MT];
+#pragma unroll
+  for (int qq = 0; qq < 2 * MT; ++qq) {
+    const int idx = tid + 512 * qq, b = idx / NR, n = n0 + idx % NR;
+    const bool live = gridDim.y == 1 && idx < 32 * MT * NR && b < a.M && n < a.N;
+    ebias[qq] = live && a.bias ? a.bias[n] : 0.0f;
+    eres[qq] = live && EPI == GEMM_RESID ? a.resid[(size_t)b * a.ldc + n] : 0.0f;
+  }
+
   f16v acc[MT];   // 32-row form
   f4 acc16[2];    // 16-row form: W rows 0..15 and 16..31
 #pragma unroll
@@ -787,9 +798,9 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       a.ws[((size_t)blockIdx.y * a.M + b) * a.N + n] = sum;
       continue;
     }
-    float c = (a.bias ? a.bias[n] : 0.0f) + sum;
+    float c = ebias[q] + sum;
     if (EPI == GEMM_GELU) c = gelu_tanh(c);
-    if (EPI == GEMM_RESID) c = a.resid[(size_t)b * a.ldc + n] + c;
+    if (EPI == GEMM_RESID) c = eres[q] + c;
     a.C[a.c_packed ? packed32_index((size_t)b, (size_t)n) : (size_t)b * a.ldc + n] = c;
   }
 }
