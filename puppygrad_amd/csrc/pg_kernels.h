@@ -142,6 +142,7 @@ struct GemmArgs {
   int lda, ldc;
   float* ws = nullptr;    // optional workspace for the split-K form (may be nullptr)
   size_t ws_floats = 0;   // its size
+  int rows_per_block = 0;  // 32-row kernel: rows of W a block owns (filled by its launcher)
   int tail_first = 0;     // filled by gemm_tail_plan: first tile of the tail that is cut along K,
   int tail_parts = 1;     // and the number of parts
   int band_rows = 1;      // tile numbering of the tile forms (set by the launcher)

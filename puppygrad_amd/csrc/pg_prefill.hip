@@ -570,8 +570,8 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // M16: at most 16 input rows, MFMA 16x16x4 (half the matrix-core time and half the input
 // traffic of the 32-row form): lane (i, kq) holds columns 4 kq .. 4 kq + 3 of a step's
 // piece of input row i and of W rows i and 16 + i.
-// NR: rows of W per block; 16 (16-row form only) where 32-row blocks would leave half of
-// the CUs without one.
+// NR: the most rows of W a block can own (16: 16-row form with one group of W rows); how many
+// it does own is a.rows_per_block.
 // MT: tiles of 32 input rows (2: up to 64 rows, row-major input only; the W operands of a step
 // are used twice).
 template <int EPI, bool WBF, bool XP, bool M16, int NR, int MT>
@@ -591,7 +591,9 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   // operand position of the lane: row orow, 16-byte piece opc of the row's 64 bytes
   const int orow = M16 ? (lane & 15) : (lane & 31);
   const int opc = M16 ? (lane >> 4) : (lane >> 5);
-  const int n0 = (int)blockIdx.x * NR;
+  // the block owns rows n0 .. n1 - 1 (a.rows_per_block <= NR of them: the launcher spreads the
+  // rows over as many blocks as there are CUs); lanes past n1 re-read row n1 - 1
+  const int n0 = (int)blockIdx.x * a.rows_per_block, n1 = min(n0 + a.rows_per_block, a.N);
   const int steps = a.K / KS;
   const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
   const int s0 = (int)(((long)piece * steps) / pieces), s1 = (int)(((long)(piece + 1) * steps) / pieces);
@@ -601,8 +603,8 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   // loads: four lanes to a row of W (q, t); rows q and 16 + q
   const int q = lane >> 2, t = lane & 3;
   const size_t rowbytes = (size_t)a.K * (WBF ? 2 : 4);
-  const char* wpa = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + q, a.N - 1) * rowbytes + 16 * t;
-  const char* wpb = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + 16 + q, a.N - 1) * rowbytes + 16 * t;
+  const char* wpa = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + q, n1 - 1) * rowbytes + 16 * t;
+  const char* wpb = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + 16 + q, n1 - 1) * rowbytes + 16 * t;
   // input: packed, straight into operand form (k-block kb of row r at (kb * 32 + r) * 4);
   // row-major, KS / 4 lanes to a row
   constexpr int XL = KS / 4;             // lanes to an input row
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
   for (int qq = 0; qq < 2 * MT; ++qq) {
     const int idx = tid + 512 * qq, b = idx / NR, n = n0 + idx % NR;
-    const bool live = gridDim.y == 1 && idx < 32 * MT * NR && b < a.M && n < a.N;
+    const bool live = gridDim.y == 1 && idx < 32 * MT * NR && b < a.M && n < n1;
     ebias[qq] = live && a.bias ? a.bias[n] : 0.0f;
     eres[qq] = live && EPI == GEMM_RESID ? a.resid[(size_t)b * a.ldc + n] : 0.0f;
   }
@@ -790,7 +792,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
   for (int q = 0; q < 2 * MT; ++q) {
     const int idx = tid + 512 * q, b = idx / NR, nl = idx % NR, n = n0 + nl;
-    if (idx >= 32 * MT * NR || b >= a.M || n >= a.N) continue;
+    if (idx >= 32 * MT * NR || b >= a.M || n >= n1) continue;
     float sum = red_at(0, b, nl);
 #pragma unroll
     for (int w = 1; w < 8; ++w) sum += red_at(w, b, nl);
@@ -1287,8 +1289,10 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   return (int)std::max<long>(parts, 1);
 }
 template <bool WBF, bool XP, bool M16, int NR, int MT = 1>
-hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, int parts, hipStream_t s) {
-  const dim3 grid((unsigned)((a.N + NR - 1) / NR), (unsigned)parts);
+hipError_t launch_gemm_rows32_m(const GemmArgs& a0, int epi, int parts, int rows, hipStream_t s) {
+  GemmArgs a = a0;
+  a.rows_per_block = rows;
+  const dim3 grid((unsigned)((a.N + rows - 1) / rows), (unsigned)parts);
   if (epi == GEMM_BIAS)
     hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_GELU)
@@ -1299,18 +1303,24 @@ hipError_t launch_gemm_rows32_m(const GemmArgs& a, int epi, int parts, hipStream
     return hipErrorInvalidValue;
   return hipSuccess;
 }
+// Rows of W per block.  With K cut over blocks: 32.  Otherwise as many as spread the rows over
+// all CUs (a launch is as fast as its busiest CU's bytes allow, and a block reads the input
+// rows whole whatever its share of W), at least 8 and at most 32.
+int rows32_block_rows(const GemmArgs& a, int parts, int num_cus) {
+  if (parts > 1) return 32;
+  return std::max(8, std::min(32, (a.N + num_cus - 1) / num_cus));
+}
 template <bool WBF, bool XP>
 hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s) {
+  const int rows = rows32_block_rows(a, parts, num_cus);
   if (a.M > 32) {
     if constexpr (XP) return hipErrorInvalidValue;  // the packed form holds 32 rows
-    else return launch_gemm_rows32_m<WBF, false, false, 32, 2>(a, epi, parts, s);
+    else return launch_gemm_rows32_m<WBF, false, false, 32, 2>(a, epi, parts, rows, s);
   }
-  if (a.M > 16) return launch_gemm_rows32_m<WBF, XP, false, 32>(a, epi, parts, s);
-  // 16 rows of W per block where K is not cut and 32-row blocks would reach at most half of
-  // the CUs (a CU then pulls half as much of W, and as much of the input)
-  if (parts == 1 && (long)((a.N + 31) / 32) * 2 <= num_cus)
-    return launch_gemm_rows32_m<WBF, XP, true, 16>(a, epi, parts, s);
-  return launch_gemm_rows32_m<WBF, XP, true, 32>(a, epi, parts, s);
+  if (a.M > 16) return launch_gemm_rows32_m<WBF, XP, false, 32>(a, epi, parts, rows, s);
+  // the 16-row form with one group of 16 rows of W where a block owns no more
+  if (rows <= 16) return launch_gemm_rows32_m<WBF, XP, true, 16>(a, epi, parts, rows, s);
+  return launch_gemm_rows32_m<WBF, XP, true, 32>(a, epi, parts, rows, s);
 }
 template <bool WBF>
 hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s, bool* ln_done) {
