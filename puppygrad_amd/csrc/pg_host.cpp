@@ -758,11 +758,15 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   const int B = (int)c->B, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(),
             P = (int)g.P;
   hipStream_t s = c->stream;
-  // With at least one (sequence, head) pair per CU and up to 256 keys a block takes all keys of
-  // its pair and writes the attention output itself: no partials and no merge launch (355M
-  // B = 16 from 128 tokens: -3.5 % per step; with 528 keys the longer serial chunks cost more
-  // than the merge launch: XL B = 32 +1.3 %).
-  const bool one_split = hd == pgk::kHeadDim && H * B >= m->num_cus && pos + 1 <= 256;
+  // With at least one (sequence, head) pair per CU a block takes all keys of its pair and writes
+  // the attention output itself: no partials and no merge launch (355M B = 16: -3.5 % per step
+  // at 128..192 keys, -6 % at 300, -5 % at 600).  Beyond 256 keys only where the pairs fill whole
+  // rounds of CUs: with 800 pairs on 256 CUs the longer serial chunks of the last, short round
+  // cost more than the merge launch (XL B = 32 at 528 keys: +1.6 %).
+  const int pairs = H * B, rounds = (pairs + m->num_cus - 1) / m->num_cus;
+  const bool whole_rounds = (long)rounds * m->num_cus * 10 <= (long)pairs * 11;
+  const bool one_split =
+      hd == pgk::kHeadDim && pairs >= m->num_cus && (pos + 1 <= 256 || whole_rounds);
   const int nsplit = hd != pgk::kHeadDim ? 1 : one_split
                          ? 1 : pgk::choose_nsplit((int)pos + 1, H * B, m->num_cus, m->attn_blocks_per_cu);
   pgk::BatchStrides bs;
