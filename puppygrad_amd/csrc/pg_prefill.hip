@@ -374,7 +374,10 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a, int parts) {
 // (layer_norm_in_place, cpu.rs:119-143: mean, biased variance in a second pass, eps inside
 // the root) into a.ln_out: the projection back to n_embd and the LayerNorm that reads its
 // result are one launch.  N <= 4096, a multiple of 4; ldc == N.
-template <int EPI>
+// EARLY: everything a thread reads is requested before the first use (a few rows: the launch
+// is a chain of memory round trips and this takes two out of it); otherwise column block by
+// column block, with few registers, for the many rows of a long prompt.
+template <int EPI, bool EARLY>
 __global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts) {
   __shared__ float red[4];
   const size_t m = blockIdx.x;
@@ -389,23 +392,27 @@ __global__ __launch_bounds__(256) void k_splitk_reduce_ln(GemmArgs a, int parts)
     return (red[0] + red[1]) + (red[2] + red[3]);
   };
   f4 c[4];
-  // all partial sums of the row are requested before the first is used (columns past the end
-  // re-read the last float4)
-  f4 v[4][8], lg[4], lb[4];  // (and the LayerNorm's scale and shift for the lane's columns)
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    if (256 * q >= n4) continue;  // (block-uniform)
+  // the partial sums of the row, and the LayerNorm's scale and shift for the lane's columns
+  // (columns past the end re-read the last float4)
+  f4 v[4][8], lg[4], lb[4];
+  auto request = [&](int q) {
     const size_t n = (size_t)min((int)threadIdx.x + 256 * q, n4 - 1) * 4;
 #pragma unroll
     for (int p = 0; p < 8; ++p)
       v[q][p] = *reinterpret_cast<const f4*>(a.ws + (size_t)min(p, parts - 1) * stride + m * a.N + n);
     lg[q] = *reinterpret_cast<const f4*>(a.ln_g + n);
     lb[q] = *reinterpret_cast<const f4*>(a.ln_b + n);
+  };
+  if (EARLY) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (256 * q < n4) request(q);  // (block-uniform)
   }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int i = (int)threadIdx.x + 256 * q;
     c[q] = f4{0.f, 0.f, 0.f, 0.f};
+    if (!EARLY && 256 * q < n4) request(q);
     if (i < n4) {
       const size_t n = (size_t)i * 4;
       f4 s = v[q][0];
@@ -1203,12 +1210,19 @@ namespace {
 // LayerNorm of the result in the same launch (*ln_done tells).
 hipError_t launch_splitk_reduce(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
   if (a.ln_out && a.N % 4 == 0 && a.N <= 4096 && a.ldc == a.N) {
-    if (epi == GEMM_BIAS)
-      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_BIAS>, dim3(a.M), dim3(256), 0, s, a, parts);
+    const bool early = a.M <= 64;
+    if (epi == GEMM_BIAS && early)
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_BIAS, true>), dim3(a.M), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_BIAS)
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_BIAS, false>), dim3(a.M), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_GELU && early)
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_GELU, true>), dim3(a.M), dim3(256), 0, s, a, parts);
     else if (epi == GEMM_GELU)
-      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_GELU>, dim3(a.M), dim3(256), 0, s, a, parts);
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_GELU, false>), dim3(a.M), dim3(256), 0, s, a, parts);
+    else if (epi == GEMM_RESID && early)
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_RESID, true>), dim3(a.M), dim3(256), 0, s, a, parts);
     else if (epi == GEMM_RESID)
-      hipLaunchKernelGGL(k_splitk_reduce_ln<GEMM_RESID>, dim3(a.M), dim3(256), 0, s, a, parts);
+      hipLaunchKernelGGL((k_splitk_reduce_ln<GEMM_RESID, false>), dim3(a.M), dim3(256), 0, s, a, parts);
     else
       return hipErrorInvalidValue;
     *ln_done = true;
