@@ -258,6 +258,7 @@ def secondary_workloads(xl_cfg, xl_weights):
         "roofline": hbm_roofline(d["achieved"], d["kernel"], launches=d["launches"],
                                  launch_ms=round(d["launch_s"] * 1e3, 3),
                                  algorithmic_bytes_per_forward=int(d["algo_bytes"]))}
+    out["gpt2_124m_prefill_32"] = measure_short_prefill(model, cfg, ids, 32, 60, 6)
     ids = synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size)
     out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 60, 6)
     del model, w
@@ -271,6 +272,26 @@ def secondary_workloads(xl_cfg, xl_weights):
     out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 512, 24, True)
     del model
     return out
+
+
+def measure_short_prefill(model, cfg, ids, T, steps, warmup):
+    """First-token latency of a short prompt (BASELINE config 1's 32 tokens): one prefill of T
+    tokens into an empty cache.  With so few rows every weight is read once and the flops are
+    cheap: the bound is the weights' bytes at the HBM peak."""
+    cache = model.new_kv_cache()
+    for _ in range(max(1, warmup)):
+        model.prefill(ids, cache).argmax()
+    t0 = time.time()
+    for _ in range(steps):
+        lg = model.prefill(ids, cache)
+    lg.argmax()
+    sec = (time.time() - t0) / steps
+    wbytes = weight_bytes(cfg)
+    return {"workload": f"GPT-2 124M fp32 B=1 prefill of a {T}-token prompt into an empty KV cache (first-token latency)",
+            "value": round(T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 4),
+            "roofline": hbm_roofline(wbytes / sec / 1e9,
+                                     "whole prefill (k_gemm_rows32, k_attn_prefill64, k_splitk_reduce_ln, lm_head)",
+                                     algorithmic_bytes_per_step=int(wbytes))}
 
 
 def measure_prefill(model, cfg, ids, T, steps, warmup):
