@@ -339,6 +339,18 @@ pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t
 pg_status pg_op_dense_in_out_dev(int32_t device, void* stream, const float* x, uint64_t rows,
                                  uint64_t in_features, uint64_t out_features, const float* weight,
                                  const float* bias, float* out);
+/* QuantizedRows::from_f32 (cpu.rs:38-55) for values[rows][cols]: q[rows][cols] int8 and
+ * scales[rows] (max|row| / 127, 1 for an all-zero row; q = round(v / scale) clamped to
+ * [-127, 127]). */
+pg_status pg_op_quantize_rows_dev(int32_t device, void* stream, const float* values, uint64_t rows,
+                                  uint64_t cols, int8_t* q, float* scales);
+/* quantized_transposed_dense_projection_into (cpu.rs:99-117): out[r][o] = bias[o] +
+ * quantized_dot(x row r, weight row o) with every weight used as (float)q * scale
+ * (cpu.rs:173-184).  bias may be NULL (the reference's Whisper model takes its logits as bare
+ * quantized_dot values, src/models/whisper/model.rs:1528, 1547). */
+pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                                    uint64_t in_features, uint64_t out_features, const int8_t* q,
+                                    const float* scales, const float* bias, float* out);
 /* layer_norm_in_place (cpu.rs:119-143), gelu_in_place (145-150), softmax_in_place per row
  * (152-165), add_in_place (167-171), argmax_logits (generation.rs:269-279; out is a device
  * pointer to one id). */

@@ -145,6 +145,8 @@ SIGNATURES = {
     "pg_device_upload": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
     "pg_device_download": (C.c_int, [C.c_int32, _vp, _vp, C.c_size_t]),
     "pg_op_dense_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64, _vp, _vp, _vp]),
+    "pg_op_quantize_rows_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, _vp, _vp]),
+    "pg_op_quantized_dense_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64, _vp, _vp, _vp, _vp]),
     "pg_op_dense_in_out_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, C.c_uint64, _vp,
                                          _vp, _vp]),
     "pg_op_layer_norm_dev": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, C.c_uint64, _vp, _vp, C.c_float]),

@@ -259,7 +259,7 @@ pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t
   pgk::GemmArgs ga{};
   ga.A = x; ga.W = weight; ga.bias = bias; ga.resid = nullptr; ga.C = out;
   ga.M = (int)rows; ga.N = (int)out_f; ga.K = (int)in_f; ga.lda = (int)in_f; ga.ldc = (int)out_f;
-  if (rows >= 16 && pgk::gemm_supported(ga)) {
+  if (rows >= 2 && pgk::gemm_supported(ga)) {  // (one row, or a K the GEMM kernels do not take: row by row)
     int cus = 0;
     PG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
     PG_HIP(pgk::launch_gemm(ga, pgk::GEMM_BIAS, cus, st));  // no workspace: never cut along K
@@ -289,6 +289,40 @@ pg_status pg_op_dense_in_out_dev(int32_t device, void* stream, const float* x, u
                      static_cast<hipStream_t>(stream), x, (int)rows, (int)in_f, (int)out_f, weight,
                      bias, out);
   PG_HIP(hipGetLastError());
+  return PG_OK;
+}
+
+pg_status pg_op_quantize_rows_dev(int32_t device, void* stream, const float* values, uint64_t rows,
+                                  uint64_t cols, int8_t* q, float* scales) {
+  if (!values || !q || !scales) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (cols == 0 || cols > (1u << 24) || rows > (1u << 30))
+    return pgh::fail(PG_INVALID_INPUT, "quantize_rows: cols must be in [1,16777216]");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  if (rows == 0) return PG_OK;
+  PG_HIP(pgk::launch_quantize_rows(values, q, scales, (size_t)rows, (int)cols,
+                                   static_cast<hipStream_t>(stream)));
+  return PG_OK;
+}
+
+pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
+                                    uint64_t in_f, uint64_t out_f, const int8_t* q,
+                                    const float* scales, const float* bias, float* out) {
+  if (!x || !q || !scales || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
+  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
+    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  pg_status s;
+  if ((s = select_device(device))) return s;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // one matrix-vector launch per input row (the reference's callers have one: the last hidden
+  // state against the token embedding)
+  for (uint64_t r = 0; r < rows; ++r) {
+    pgk::GemvArgs a{};
+    a.W = reinterpret_cast<const float*>(q); a.w_scale = scales; a.bias = bias;
+    a.x = x + r * in_f; a.y = out + r * out_f;
+    a.K = (int)in_f; a.nout = (int)out_f;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_NONE, pgk::EPI_BIAS, st));
+  }
   return PG_OK;
 }
 

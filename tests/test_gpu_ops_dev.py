@@ -53,6 +53,38 @@ def test_dense_with_in_out_weights_matches_oracle(rows, in_f, out_f):
         d.free()
 
 
+@pytest.mark.parametrize("rows,in_f,out_f", [(1, 384, 51865), (2, 100, 37), (1, 16, 8), (3, 1280, 1000),
+                                             (1, 7, 5)])
+def test_quantized_rows_and_quantized_dense_match_oracle(rows, in_f, out_f):
+    """QuantizedRows::from_f32 bit for bit (incl. an all-zero row and a row whose largest value is
+    negative), then the quantised projection against quantized_dot (cpu.rs:99-117, 173-184), with
+    a bias and without one (the Whisper logits, model.rs:1528)."""
+    rng = np.random.default_rng(in_f * 7 + out_f)
+    w = (rng.standard_normal((out_f, in_f)) / np.sqrt(in_f)).astype(np.float32)
+    w[0] = 0.0
+    w[out_f - 1, 0] = -3.0
+    x = rng.standard_normal((rows, in_f)).astype(np.float32)
+    b = rng.standard_normal(out_f).astype(np.float32)
+    lib = _lib.load()
+    dw, dq, ds = DeviceArray(w), DeviceArray(np.zeros((out_f, in_f)), np.int8), DeviceArray(np.zeros(out_f))
+    ok(lib.pg_op_quantize_rows_dev(0, None, dw.ptr, out_f, in_f, dq.ptr, ds.ptr))
+    q_want, s_want = oracle.quantize_rows(w, out_f, in_f)
+    np.testing.assert_array_equal(dq.download(), q_want)
+    np.testing.assert_array_equal(ds.download(), s_want)
+    dx, db, dy = DeviceArray(x), DeviceArray(b), DeviceArray(np.zeros((rows, out_f)))
+    idx = np.unique(np.concatenate([np.arange(min(out_f, 40)), rng.integers(0, out_f, 60), [out_f - 1]]))
+    dots = np.array([[oracle.quantized_dot(x[r], q_want, s_want, int(o)) for o in idx] for r in range(rows)],
+                    np.float32)
+    ok(lib.pg_op_quantized_dense_dev(0, None, dx.ptr, rows, in_f, out_f, dq.ptr, ds.ptr, db.ptr, dy.ptr))
+    np.testing.assert_allclose(dy.download()[:, idx], dots + b[idx], atol=2e-5, rtol=1e-4)
+    ok(lib.pg_op_quantized_dense_dev(0, None, dx.ptr, rows, in_f, out_f, dq.ptr, ds.ptr, None, dy.ptr))
+    np.testing.assert_allclose(dy.download()[:, idx], dots, atol=2e-5, rtol=1e-4)
+    assert lib.pg_op_quantized_dense_dev(0, None, dx.ptr, rows, 0, out_f, dq.ptr, ds.ptr, None, dy.ptr) == _lib.PG_INVALID_INPUT
+    assert lib.pg_op_quantize_rows_dev(0, None, dw.ptr, out_f, in_f, None, ds.ptr) == _lib.PG_INVALID_INPUT
+    for d in (dw, dq, ds, dx, db, dy):
+        d.free()
+
+
 @pytest.mark.parametrize("Tq,Tk,state,heads,causal", [(1, 1, 8, 2, 0), (5, 5, 24, 3, 1), (6, 1500, 384, 6, 0),
                                                       (40, 40, 384, 6, 1), (3, 700, 1280, 20, 0),
                                                       (9, 4, 64, 1, 1), (2, 33, 512, 2, 0)])
