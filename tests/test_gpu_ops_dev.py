@@ -53,6 +53,25 @@ def test_dense_with_in_out_weights_matches_oracle(rows, in_f, out_f):
         d.free()
 
 
+@pytest.mark.parametrize("rows", [2, 5, 8, 16, 17, 31, 33, 47, 64, 65])
+def test_dense_on_device_over_the_small_batch_forms(rows):
+    """2..64 rows take the small-batch projection kernel in its 16-row, 32-row and two-tile forms
+    (65: the tile GEMM), with ragged row blocks (N no multiple of the block height), a single
+    k step for eight wavefronts (K = 16) and N below one block."""
+    lib = _lib.load()
+    for in_f, out_f in [(768, 2304), (1600, 100), (16, 52), (160, 1000), (64, 7)]:
+        rng = np.random.default_rng(rows * 131 + in_f + out_f)
+        x = rng.standard_normal((rows, in_f)).astype(np.float32)
+        w = (rng.standard_normal((out_f, in_f)) / np.sqrt(in_f)).astype(np.float32)
+        b = rng.standard_normal(out_f).astype(np.float32)
+        dx, dw, db, dy = DeviceArray(x), DeviceArray(w), DeviceArray(b), DeviceArray(np.zeros((rows, out_f)))
+        ok(lib.pg_op_dense_dev(0, None, dx.ptr, rows, in_f, out_f, dw.ptr, db.ptr, dy.ptr))
+        want = x.astype(np.float64) @ w.astype(np.float64).T + b
+        np.testing.assert_allclose(dy.download(), want, atol=3e-5, rtol=1e-5, err_msg=f"{rows}x{in_f}x{out_f}")
+        for d in (dx, dw, db, dy):
+            d.free()
+
+
 @pytest.mark.parametrize("rows,in_f,out_f", [(1, 384, 51865), (2, 100, 37), (1, 16, 8), (3, 1280, 1000),
                                              (1, 7, 5)])
 def test_quantized_rows_and_quantized_dense_match_oracle(rows, in_f, out_f):
