@@ -25,7 +25,7 @@ def test_bf16_rounding_is_nearest_even():
     np.testing.assert_array_equal(synth.round_bf16(bits.view(np.float32)).view(np.uint32), want)
 
 
-@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(128, 2, 21), (192, 3, 5), (100, 5, 18)])
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(128, 2, 21), (192, 3, 5), (100, 5, 18), (128, 2, 36)])
 def test_bf16_storage_matches_oracle_on_rounded_weights(n_embd, n_head, n_prompt):
     cfg = Gpt2Config(vocab_size=263, n_positions=40, n_embd=n_embd, n_layer=2, n_head=n_head)
     w = synth.random_weights(cfg, 0x5EED0500 + n_embd, perturb=True)
