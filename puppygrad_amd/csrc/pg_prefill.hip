@@ -581,13 +581,18 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 // it does own is a.rows_per_block.
 // MT: tiles of 32 input rows (2: up to 64 rows, row-major input only; the W operands of a step
 // are used twice).
-template <int EPI, bool WBF, bool XP, bool M16, int NR, int MT>
+// WT: W holds f32 (0), bf16 (1) or int8 rows with a.w_scale (2; a weight is (float)q * scale,
+// formed when its piece is read back; row-major input of up to 32 rows only).
+template <int EPI, int WT, bool XP, bool M16, int NR, int MT>
 __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   static_assert(NR == 32 || (NR == 16 && M16), "rows per block");
-  static_assert(MT == 1 || (MT == 2 && !M16 && !XP), "input rows");
-  constexpr int KS = WBF ? 32 : 16;      // columns per step: 64 bytes of a row of W
-  constexpr int XR = M16 ? KS / 16 : MT * KS / 8;  // float4 of input per lane and step
-  constexpr int XT = KS / 8;             // of those, per tile of 32 rows
+  static_assert(MT == 1 || (MT == 2 && !M16 && !XP && WT != 2), "input rows");
+  static_assert(WT != 2 || !XP, "int8 rows: row-major input");
+  constexpr int CPP = WT == 2 ? 16 : WT == 1 ? 8 : 4;  // columns in a 16-byte piece of a W row
+  constexpr int XF = CPP / 4;            // float4 of input that meet one piece
+  constexpr int KS = 4 * CPP;            // columns per step: 64 bytes of a row of W
+  constexpr int XR = M16 ? XF : MT * 2 * XF;  // float4 of input per lane and step
+  constexpr int XT = 2 * XF;             // of those, per tile of 32 rows
   constexpr int WSTR = 20;               // row stride of the W tile (floats; 64 bytes + pad)
   constexpr int XSTR = KS + 4;           // row stride of the input tile
   // per wavefront: W tile, input tile; the reduce tile [32 MT][33] lies over them
@@ -609,7 +614,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 
   // loads: four lanes to a row of W (q, t); rows q and 16 + q
   const int q = lane >> 2, t = lane & 3;
-  const size_t rowbytes = (size_t)a.K * (WBF ? 2 : 4);
+  const size_t rowbytes = (size_t)a.K * (WT == 2 ? 1 : WT == 1 ? 2 : 4);
   const char* wpa = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + q, n1 - 1) * rowbytes + 16 * t;
   const char* wpb = reinterpret_cast<const char*>(a.W) + (size_t)min(n0 + 16 + q, n1 - 1) * rowbytes + 16 * t;
   // input: packed, straight into operand form (k-block kb of row r at (kb * 32 + r) * 4);
@@ -622,9 +627,8 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   for (int j = 0; j < XR; ++j) {
     if (XP) {
       // the k-blocks of the lane's operand piece(s); see the reads in mul_step
-      int kb;
-      if (M16) kb = WBF ? 2 * opc + j : opc;
-      else kb = WBF ? 4 * (j >> 1) + 2 * opc + (j & 1) : 2 * j + opc;
+      // (float4 e of piece pi is k-block XF pi + e; 32-row form: j = XF u + e, pi = 2 u + opc)
+      const int kb = M16 ? XF * opc + j : XF * (2 * (j / XF) + opc) + j % XF;
       xp[j] = a.A + ((size_t)kb * 32 + min(orow, a.M - 1)) * 4;
       xw[j] = 0;
     } else {
@@ -662,13 +666,29 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < XR; ++j) x[j] = *reinterpret_cast<const f4*>(xp[j] + sc * xstep);
   };
-  // 8 bf16 -> 8 floats
-  auto widen8 = [](const f4& v, float* w8) {
+  // int8 rows: the scale of the W row(s) whose operand this lane holds
+  float wsc[2] = {1.0f, 1.0f};
+  if (WT == 2) {
+    wsc[0] = a.w_scale[min(n0 + orow, n1 - 1)];
+    wsc[1] = a.w_scale[min(n0 + 16 + orow, n1 - 1)];
+  }
+  // a 16-byte piece of a W row -> its CPP columns as floats
+  auto widen = [](const f4& v, float* wv, float scale) {
     const unsigned* p = reinterpret_cast<const unsigned*>(&v);
+    if (WT == 0) {
+      wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
+    } else if (WT == 1) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      w8[2 * c] = __uint_as_float(p[c] << 16);
-      w8[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
+      for (int c = 0; c < 4; ++c) {
+        wv[2 * c] = __uint_as_float(p[c] << 16);
+        wv[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          wv[4 * c + b] = (float)((int)(p[c] << (24 - 8 * b)) >> 24) * scale;
     }
   };
   auto mul_step = [&](const f4* w, const f4* x) {
@@ -681,13 +701,13 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     __builtin_amdgcn_wave_barrier();
     f4 wo[2], xo[XR];
     if (M16) {
-      // W rows orow and 16 + orow, piece opc; the same piece of input row orow
+      // W rows orow and 16 + orow, piece opc; the same piece (CPP columns) of input row orow
 #pragma unroll
       for (int g = 0; g < NR / 16; ++g) wo[g] = *reinterpret_cast<const f4*>(wt + (16 * g + orow) * WSTR + 4 * opc);
 #pragma unroll
       for (int j = 0; j < XR; ++j) {
         if (XP) xo[j] = x[j];
-        else xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + (WBF ? 8 : 4) * opc + 4 * j);
+        else xo[j] = *reinterpret_cast<const f4*>(xt + orow * XSTR + CPP * opc + 4 * j);
       }
     } else {
       // pieces opc and 2 + opc of W row orow
@@ -695,65 +715,31 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       for (int u = 0; u < 2; ++u) wo[u] = *reinterpret_cast<const f4*>(wt + orow * WSTR + 4 * (2 * u + opc));
 #pragma unroll
       for (int j = 0; j < XR; ++j) {
-        // tile mt = j / XT of the input rows, operand jj = j % XT of the step
-        const int mt = j / XT, jj = j % XT;
-        const float* xr = xt + (32 * mt + orow) * XSTR;
+        // tile mt of the input rows, piece 2 u + opc, float4 e of the piece's columns
+        const int mt = j / XT, u = (j % XT) / XF, e = j % XF;
         if (XP) xo[j] = x[j];
-        else if (WBF) xo[j] = *reinterpret_cast<const f4*>(xr + 8 * (2 * (jj >> 1) + opc) + 4 * (jj & 1));
-        else xo[j] = *reinterpret_cast<const f4*>(xr + 4 * (2 * jj + opc));
+        else xo[j] = *reinterpret_cast<const f4*>(xt + (32 * mt + orow) * XSTR + CPP * (2 * u + opc) + 4 * e);
       }
     }
     __builtin_amdgcn_wave_barrier();
+    float wv[CPP];
     if (M16) {
 #pragma unroll
       for (int g = 0; g < NR / 16; ++g) {
-        if (WBF) {
-          float w8[8];
-          widen8(wo[g], w8);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].x, w8[0], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].y, w8[1], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].z, w8[2], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].w, w8[3], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].x, w8[4], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].y, w8[5], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].z, w8[6], acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[XR - 1].w, w8[7], acc16[g], 0, 0, 0);
-        } else {
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].x, wo[g].x, acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].y, wo[g].y, acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].z, wo[g].z, acc16[g], 0, 0, 0);
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[0].w, wo[g].w, acc16[g], 0, 0, 0);
-        }
+        widen(wo[g], wv, wsc[g]);
+#pragma unroll
+        for (int c = 0; c < CPP; ++c)
+          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[c / 4][c % 4], wv[c], acc16[g], 0, 0, 0);
       }
     } else {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        if (WBF) {
-          // 8 bf16 columns, widened; the matching 8 input columns are two float4
-          float w8[8];
-          widen8(wo[u], w8);
+        widen(wo[u], wv, wsc[0]);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const f4 xa = xo[mt * XT + 2 * u], xb = xo[mt * XT + (2 * u + 1) % XT];
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, w8[0], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, w8[1], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, w8[2], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, w8[3], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.x, w8[4], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.y, w8[5], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.z, w8[6], acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xb.w, w8[7], acc[mt], 0, 0, 0);
-          }
-        } else {
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const f4 xa = xo[mt * XT + u % XT];
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.x, wo[u].x, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.y, wo[u].y, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.z, wo[u].z, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa.w, wo[u].w, acc[mt], 0, 0, 0);
-          }
-        }
+          for (int c = 0; c < CPP; ++c)
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xo[mt * XT + u * XF + c / 4][c % 4], wv[c], acc[mt], 0, 0, 0);
       }
     }
   };
@@ -1289,8 +1275,9 @@ bool gemm_prefers_gemv_rows(const GemmArgs& a) {
   return a.K % (a.w_bf16 ? 32 : 16) != 0 || a.lda % 4 != 0;
 }
 int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
-  const int U = a.w_bf16 ? 32 : 16;  // columns per step of the kernel
-  if (a.M > (a.a_packed || a.c_packed || a.ln_packed ? 32 : 64) || a.K % U != 0 || a.lda % 4 != 0) return 0;
+  const int U = a.w_scale ? 64 : a.w_bf16 ? 32 : 16;  // columns per step of the kernel
+  if (a.M > (a.a_packed || a.c_packed || a.ln_packed || a.w_scale ? 32 : 64) || a.K % U != 0 || a.lda % 4 != 0)
+    return 0;
   const long tiles = (a.N + 31) / 32;
   // (a cut in two plus its reduce launch costs more than it saves: 355M c_attn and c_fc)
   long parts = tiles * 4 > num_cus ? 1 : std::max<long>(1, num_cus / tiles);
@@ -1302,17 +1289,17 @@ int gemm_rows32_parts(const GemmArgs& a, int num_cus) {
   }
   return (int)std::max<long>(parts, 1);
 }
-template <bool WBF, bool XP, bool M16, int NR, int MT = 1>
+template <int WT, bool XP, bool M16, int NR, int MT = 1>
 hipError_t launch_gemm_rows32_m(const GemmArgs& a0, int epi, int parts, int rows, hipStream_t s) {
   GemmArgs a = a0;
   a.rows_per_block = rows;
   const dim3 grid((unsigned)((a.N + rows - 1) / rows), (unsigned)parts);
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_BIAS, WT, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_GELU, WT, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WBF, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_rows32<GEMM_RESID, WT, XP, M16, NR, MT>), grid, dim3(512), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipSuccess;
@@ -1324,22 +1311,28 @@ int rows32_block_rows(const GemmArgs& a, int parts, int num_cus) {
   if (parts > 1) return 32;
   return std::max(8, std::min(32, (a.N + num_cus - 1) / num_cus));
 }
-template <bool WBF, bool XP>
+template <int WT, bool XP>
 hipError_t launch_gemm_rows32_x(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s) {
   const int rows = rows32_block_rows(a, parts, num_cus);
   if (a.M > 32) {
-    if constexpr (XP) return hipErrorInvalidValue;  // the packed form holds 32 rows
-    else return launch_gemm_rows32_m<WBF, false, false, 32, 2>(a, epi, parts, rows, s);
+    // (the packed form holds 32 rows; the int8 form's input tile is sized for 32)
+    if constexpr (XP || WT == 2) return hipErrorInvalidValue;
+    else return launch_gemm_rows32_m<WT, false, false, 32, 2>(a, epi, parts, rows, s);
   }
-  if (a.M > 16) return launch_gemm_rows32_m<WBF, XP, false, 32>(a, epi, parts, rows, s);
+  if (a.M > 16) return launch_gemm_rows32_m<WT, XP, false, 32>(a, epi, parts, rows, s);
   // the 16-row form with one group of 16 rows of W where a block owns no more
-  if (rows <= 16) return launch_gemm_rows32_m<WBF, XP, true, 16>(a, epi, parts, rows, s);
-  return launch_gemm_rows32_m<WBF, XP, true, 32>(a, epi, parts, rows, s);
+  if (rows <= 16) return launch_gemm_rows32_m<WT, XP, true, 16>(a, epi, parts, rows, s);
+  return launch_gemm_rows32_m<WT, XP, true, 32>(a, epi, parts, rows, s);
 }
-template <bool WBF>
+template <int WT>
 hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, int num_cus, hipStream_t s, bool* ln_done) {
-  const hipError_t e = a.a_packed ? launch_gemm_rows32_x<WBF, true>(a, epi, parts, num_cus, s)
-                                  : launch_gemm_rows32_x<WBF, false>(a, epi, parts, num_cus, s);
+  hipError_t e;
+  if constexpr (WT == 2) {
+    e = a.a_packed ? hipErrorInvalidValue : launch_gemm_rows32_x<2, false>(a, epi, parts, num_cus, s);
+  } else {
+    e = a.a_packed ? launch_gemm_rows32_x<WT, true>(a, epi, parts, num_cus, s)
+                   : launch_gemm_rows32_x<WT, false>(a, epi, parts, num_cus, s);
+  }
   if (e != hipSuccess) return e;
   if (parts > 1) return launch_splitk_reduce(a, epi, parts, s, ln_done);
   return hipGetLastError();
@@ -1532,14 +1525,16 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   // (Every block stages all input vectors; beyond 16 x 1024 values that costs more than it
   // saves.)
   const bool packed = a.a_packed || a.c_packed || a.ln_packed;
-  if (a.w_scale) {  // int8 rows: the 64x64 tile form dequantises them as it loads
+  if (a.w_scale) {  // int8 rows: up to 32 input rows on the 32-row kernel, else the 64x64 tile form
     if (packed || a.w_bf16) return hipErrorInvalidValue;
+    if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
+      return launch_gemm_rows32<2>(a, epi, rp, num_cus, s, ln_done);
     return launch_gemm_tile<64, 64, 2>(a, epi, s);
   }
   if (a.plan_form == 4) {  // forced: the 32-row kernel
     const int rp = gemm_rows32_parts(a, num_cus);
     if (!rp) return hipErrorInvalidValue;
-    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, num_cus, s, ln_done) : launch_gemm_rows32<false>(a, epi, rp, num_cus, s, ln_done);
+    return a.w_bf16 ? launch_gemm_rows32<1>(a, epi, rp, num_cus, s, ln_done) : launch_gemm_rows32<0>(a, epi, rp, num_cus, s, ln_done);
   }
   if (!a.plan_form && gemm_prefers_gemv_rows(a)) {
     if (packed) return hipErrorInvalidValue;
@@ -1547,8 +1542,8 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   }
   // other decode batches of up to 32 rows: 32 rows of W per block on the matrix cores
   if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
-    return a.w_bf16 ? launch_gemm_rows32<true>(a, epi, rp, num_cus, s, ln_done)
-                    : launch_gemm_rows32<false>(a, epi, rp, num_cus, s, ln_done);
+    return a.w_bf16 ? launch_gemm_rows32<1>(a, epi, rp, num_cus, s, ln_done)
+                    : launch_gemm_rows32<0>(a, epi, rp, num_cus, s, ln_done);
   if (packed) return hipErrorInvalidValue;  // only the 32-row kernel knows the packed form
   // Tile forms.  A forced plan (benchmarks, tests) or the planner's choice.
   int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
