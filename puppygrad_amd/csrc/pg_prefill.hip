@@ -1226,7 +1226,7 @@ hipError_t launch_splitk_reduce(const GemmArgs& a, int epi, int parts, hipStream
   return hipGetLastError();
 }
 
-template <int BM, int BN, bool WBF, int BKT>
+template <int BM, int BN, int WBF, int BKT>
 hipError_t launch_gemm_split(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = (tiles + 7) / 8 * 8;
@@ -1339,7 +1339,7 @@ hipError_t launch_gemm_rows32(const GemmArgs& a, int epi, int parts, int num_cus
 }
 
 // Tiles with the tail cut along K (SPLIT = 2); a carries tail_first / tail_parts.
-template <int BM, int BN, bool WBF, int BKT>
+template <int BM, int BN, int WBF, int BKT>
 hipError_t launch_gemm_tail(const GemmArgs& a, int epi, hipStream_t s) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   const int grid = a.tail_first + (tiles - a.tail_first) * a.tail_parts;
@@ -1415,13 +1415,13 @@ bool gemm_tail_plan(GemmArgs& a, int num_cus, int bm, int bn) {
 namespace {
 // form: 1 whole tiles, 2 every tile cut along K into `parts` (a.ws), 3 only the last partial
 // round of tiles cut (a.tail_first / a.tail_parts are set in a)
-template <int BM, int BN, bool WBF, int BKT>
+template <int BM, int BN, int WBF, int BKT>
 hipError_t launch_tiles_depth(const GemmArgs& a, int epi, int form, int parts, hipStream_t s, bool* ln_done) {
   if (form == 2) return launch_gemm_split<BM, BN, WBF, BKT>(a, epi, parts, s, ln_done);
   if (form == 3) return launch_gemm_tail<BM, BN, WBF, BKT>(a, epi, s);
   return launch_gemm_tile<BM, BN, WBF, BKT>(a, epi, s);
 }
-template <int BM, int BN, bool WBF>
+template <int BM, int BN, int WBF>
 hipError_t launch_tiles_shape(const GemmArgs& a, int epi, int form, int parts, hipStream_t s, bool* ln_done) {
   // k-tiles of 32 columns where K allows
   if (a.K % 32 == 0 && !a.plan_bk16) return launch_tiles_depth<BM, BN, WBF, 32>(a, epi, form, parts, s, ln_done);
@@ -1444,7 +1444,8 @@ int choose_band(int tiles_m, int run, int bm, int bn) {
   return best;
 }
 
-template <bool WBF>
+// WBF: 0 f32, 1 bf16, 2 int8 rows (k_gemm's WT)
+template <int WBF>
 hipError_t launch_tiles(const GemmArgs& a0, int epi, int bm, int bn, int form, int parts, hipStream_t s,
                         bool* ln_done) {
   GemmArgs a = a0;
@@ -1529,7 +1530,11 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     if (packed || a.w_bf16) return hipErrorInvalidValue;
     if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
       return launch_gemm_rows32<2>(a, epi, rp, num_cus, s, ln_done);
-    return launch_gemm_tile<64, 64, 2>(a, epi, s);
+    int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
+    GemmArgs t = a;
+    if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
+    else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
+    return launch_tiles<2>(t, epi, bm, bn, form, parts, s, ln_done);
   }
   if (a.plan_form == 4) {  // forced: the 32-row kernel
     const int rp = gemm_rows32_parts(a, num_cus);
@@ -1550,8 +1555,8 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   GemmArgs t = a;
   if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
   else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
-  return a.w_bf16 ? launch_tiles<true>(t, epi, bm, bn, form, parts, s, ln_done)
-                  : launch_tiles<false>(t, epi, bm, bn, form, parts, s, ln_done);
+  return a.w_bf16 ? launch_tiles<1>(t, epi, bm, bn, form, parts, s, ln_done)
+                  : launch_tiles<0>(t, epi, bm, bn, form, parts, s, ln_done);
 }
 }  // namespace
 
