@@ -624,8 +624,8 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
   return persistent_end(c, &run, done, stopped);
 }
 
-// pg_op_linear: inputs of at least this many rows take the GEMM kernels.
-constexpr size_t kGemmMinRows = 16;
+// pg_op_dense: inputs of at least this many rows take the GEMM kernels.
+constexpr size_t kGemmMinRows = 2;
 // Sequences at least this long take the GEMM path in prefill / forward; shorter ones run as
 // that many single-token forwards (124M: 3 x 0.17 ms against 0.6 ms for the launches of one
 // GEMM pass; XL: 3 x 1.2 ms against 3.3 ms).
