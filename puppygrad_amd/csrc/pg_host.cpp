@@ -637,15 +637,20 @@ bool gemm_path_ok(const pg_gpt2_model* m, size_t n) {
          (g.hd() == 64 || n * g.H * n * sizeof(float) <= (256u << 20));
 }
 
-// Full-sequence forward of sequence b over ids[0..n) (Gpt2Model::forward,
-// src/models/gpt2/rust.rs:831-882, block_forward at 1053-1134) with MFMA GEMMs and
-// tiled causal attention; K and V of every position land in the cache.  The last
-// position's logits go to the cache's logits row b; with all_logits set, the logits
-// of every position are also copied to dst ([n][V], host).
-pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, const uint32_t* ids,
-                            size_t n, float* all_logits_dst, ProfileMarks* marks = nullptr) {
+// Full-sequence forward of the nb sequences b .. b + nb - 1 over ids[nb][n] (each one
+// Gpt2Model::forward, src/models/gpt2/rust.rs:831-882, block_forward at 1053-1134) with MFMA
+// GEMMs over all nb * n rows at once and tiled causal attention per sequence; K and V of every
+// position land in the cache.  The last position's logits go to the cache's logits rows
+// b .. b + nb - 1; with all_logits set (nb = 1), the logits of every position are also copied
+// to dst ([n][V], host).
+pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, size_t nb,
+                            const uint32_t* ids, size_t n_seq, float* all_logits_dst,
+                            ProfileMarks* marks = nullptr) {
   const Cfg& g = m->cfg;
-  const int T = (int)n, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(), P = (int)g.P;
+  if (nb < 1 || (all_logits_dst && nb != 1)) return fail(PG_INVALID_INPUT, "sequence batch");
+  const size_t n = nb * n_seq;  // rows of the activation matrices
+  const int T = (int)n, Ts = (int)n_seq, C = (int)g.C, I = (int)g.I, H = (int)g.H, hd = (int)g.hd(),
+            P = (int)g.P;
   hipStream_t s = c->stream;
   pg_status st;
   // The activations of the sequence live in one block that stays with the cache between
@@ -674,7 +679,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
       at += sizes[i];
     }
   }
-  if (hd != 64 && (st = SCR.alloc(n * g.H * n))) return st;
+  if (hd != 64 && (st = SCR.alloc(n_seq * g.H * n_seq))) return st;
   if (all_logits_dst && (st = LOG.alloc(n * g.V))) return st;
   uint32_t* d_ids = reinterpret_cast<uint32_t*>(IDS.p);
   {
@@ -682,7 +687,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     // not drain before the first launch (a prefill queued behind another starts at once)
     const unsigned turn = c->prompt_turn++ & 1;
     if (!c->h_prompt[turn]) {
-      PG_HIP(hipHostMalloc(&c->h_prompt[turn], g.P * sizeof(uint32_t), hipHostMallocDefault));
+      PG_HIP(hipHostMalloc(&c->h_prompt[turn], c->B * g.P * sizeof(uint32_t), hipHostMallocDefault));
       PG_HIP(hipEventCreateWithFlags(&c->ev_prompt[turn], hipEventDisableTiming));
     } else {
       PG_HIP(hipEventSynchronize(c->ev_prompt[turn]));
@@ -695,7 +700,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
   do {              \
     if (marks) PG_HIP(marks->mark(s, ProfileMarks::bk)); \
   } while (0)
-  PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s, m->w_bf16));
+  PG_HIP(pgk::launch_embed_rows(X.p, m->wte, m->wpe, d_ids, T, C, s, m->w_bf16, Ts));
   PG_MARK(kNone);
   // (ln_g / ln_b: the LayerNorm that reads this projection's result, written to XN by the
   // same call: fused into the projection's reduce where it has one)
@@ -720,8 +725,8 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     const float* next_b = l + 1 < g.L ? m->layers[l + 1].ln_1_b : nullptr;
     PG_HIP(gemm(XN.p, C, w.c_attn_w, w.c_attn_b, QKV.p, 3 * C, 3 * C, C, pgk::GEMM_BIAS));
     PG_MARK(kQkv);
-    PG_HIP(pgk::launch_attn_prefill(QKV.p, T, C, H, hd, P, c->k_panel(l, b), c->v_panel(l, b),
-                                    ATT.p, SCR.p, s));
+    PG_HIP(pgk::launch_attn_prefill(QKV.p, Ts, C, H, hd, P, c->k_panel(l, b), c->v_panel(l, b),
+                                    ATT.p, SCR.p, s, (int)nb, g.H * g.P * g.hd()));
     PG_MARK(kAttention);
     PG_HIP(gemm(ATT.p, C, w.c_proj_w, w.c_proj_b, X.p, C, C, C, pgk::GEMM_RESID, w.ln_2_g, w.ln_2_b));
     PG_MARK(kAttnProj);
@@ -736,11 +741,26 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, co
     PG_HIP(hipMemcpyAsync(all_logits_dst, LOG.p, n * g.V * sizeof(float), hipMemcpyDeviceToHost,
                           s));
   }
-  // last position -> the cache's logits row (LN_f + lm_head, rust.rs:982-1002)
-  pgk::GemvArgs a{};
-  a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
-  a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
-  PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+  // last position of every sequence -> the cache's logits rows (LN_f + lm_head, rust.rs:982-1002)
+  if (nb == 1) {
+    pgk::GemvArgs a{};
+    a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.w_scale = m->lm_s; a.bias = nullptr; a.x = X.p + (n - 1) * g.C; a.y = c->logits_buf + b * g.V;
+    a.K = C; a.nout = (int)g.V; a.ln_g = m->ln_f_g; a.ln_b = m->ln_f_b; a.eps = g.eps;
+    PG_HIP(pgk::launch_gemv(a, pgk::PRO_LN, pgk::EPI_BIAS, s));
+  } else {
+    // the nb last rows, gathered and normalised, against wte in one projection
+    PG_HIP(hipMemcpy2DAsync(ATT.p, g.C * sizeof(float), X.p + (n_seq - 1) * g.C,
+                            n_seq * g.C * sizeof(float), g.C * sizeof(float), nb,
+                            hipMemcpyDeviceToDevice, s));
+    PG_HIP(pgk::launch_layer_norm_rows(ATT.p, XN.p, (int)nb, C, m->ln_f_g, m->ln_f_b, g.eps, s));
+    pgk::GemmArgs a{};
+    a.A = XN.p; a.w_bf16 = m->w_bf16; a.W = m->lm_w; a.bias = nullptr; a.resid = nullptr;
+    a.C = c->logits_buf + b * g.V;
+    a.M = (int)nb; a.N = (int)g.V; a.K = C; a.lda = C; a.ldc = (int)g.V;
+    if (m->w_i8) a.w_scale = m->lm_s;
+    a.split_items_per_cu = m->gemm_split_items;
+    PG_HIP(pgk::launch_gemm(a, pgk::GEMM_BIAS, m->num_cus, s));
+  }
   PG_MARK(kLogits);
 #undef PG_MARK
   PG_HIP(hipStreamSynchronize(s));
@@ -1403,8 +1423,10 @@ pg_status pg_gpt2_prefill_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
   c->seq_len = 0;  // cache.clear() (rust.rs:918)
   c->logits_valid = false;
   if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) {
-    for (size_t b = 0; b < c->B; ++b)
-      if ((s = run_sequence_gemm(m, c, b, ids + b * n, n, nullptr))) return s;
+    // all sequences in one pass over the weights, in groups of at most about 8192 rows
+    const size_t group = std::max<size_t>(1, std::min<size_t>(c->B, 8192 / n));
+    for (size_t b = 0; b < c->B; b += group)
+      if ((s = run_sequence_gemm(m, c, b, std::min(group, c->B - b), ids + b * n, n, nullptr))) return s;
     c->seq_len = n;
     return finish_logits(c, out);
   }
@@ -1446,7 +1468,7 @@ pg_status pg_gpt2_prefill_profiled(const pg_gpt2_model* m, pg_kv_cache* c, const
   c->logits_valid = false;
   ProfileMarks marks;
   if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) {
-    if ((s = run_sequence_gemm(m, c, 0, ids, n, nullptr, &marks))) return s;
+    if ((s = run_sequence_gemm(m, c, 0, 1, ids, n, nullptr, &marks))) return s;
     PG_HIP(marks.collect(profile));
   } else {
     for (size_t i = 0; i < n; ++i) {
@@ -1510,7 +1532,7 @@ pg_status pg_gpt2_forward(const pg_gpt2_model* m, const uint32_t* ids, size_t n,
   pg_kv_cache* c = nullptr;
   if ((s = pg_kv_cache_create(m, 1, &c))) return s;
   std::unique_ptr<pg_kv_cache, void (*)(pg_kv_cache*)> holder(c, pg_kv_cache_destroy);
-  if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) return run_sequence_gemm(m, c, 0, ids, n, dst);
+  if (gemm_path_ok(m, n) && m->opts.prefill_path == 0) return run_sequence_gemm(m, c, 0, 1, ids, n, dst);
   for (size_t i = 0; i < n; ++i) {
     if (use_persistent(m, c)) {
       if ((s = run_persistent(m, c, nullptr, false, false, ids[i], i, 1, false, -1, nullptr,

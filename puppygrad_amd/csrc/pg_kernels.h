@@ -181,11 +181,14 @@ bool gemm_tail_plan(GemmArgs& a, int num_cus, int bm = 64, int bn = 64);
 hipError_t launch_gemm(const GemmArgs& a, int epilogue, int num_cus, hipStream_t s);
 // Causal attention over qkv[T][3C] -> out[T][C]; also appends K, V to the cache panels.
 // scratch ([T*H][T] floats) is only used when head_dim != 64.
+// nseq sequences of T positions each, one after the other in qkv / out; sequence i's panels
+// lie kv_stride floats after sequence i - 1's.
 hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
                                float* kcache, float* vcache, float* out, float* scratch,
-                               hipStream_t s);
+                               hipStream_t s, int nseq = 1, size_t kv_stride = 0);
+// rows rows; row t is position t % period of its sequence
 hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C, hipStream_t s, int w_bf16 = 0);
+                             int rows, int C, hipStream_t s, int w_bf16 = 0, int period = 0);
 // (dst_packed: dst is a packed activation matrix, rows <= 32)
 hipError_t launch_layer_norm_rows(const float* src, float* dst, int rows, int cols, const float* g,
                                   const float* b, float eps, hipStream_t s, int dst_packed = 0);

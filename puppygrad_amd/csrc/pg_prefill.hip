@@ -858,7 +858,12 @@ __device__ __forceinline__ float other_half(float x) {
 __global__ __launch_bounds__(512) void k_attn_prefill64(const float* __restrict__ qkv, int T,
                                                         int C, int P, float* __restrict__ kcache,
                                                         float* __restrict__ vcache,
-                                                        float* __restrict__ out) {
+                                                        float* __restrict__ out, size_t kv_stride) {
+  // blockIdx.z: the sequence (T rows of qkv and out each, panels kv_stride apart)
+  qkv += (size_t)blockIdx.z * T * 3 * C;
+  out += (size_t)blockIdx.z * T * C;
+  kcache += (size_t)blockIdx.z * kv_stride;
+  vcache += (size_t)blockIdx.z * kv_stride;
   constexpr int KT = 32;   // keys per tile
   constexpr int NWV = 8;   // wavefronts per block
   // per wavefront: V rows [key][d] of the current tile; reused as [d][query] for the merge
@@ -1099,15 +1104,16 @@ __global__ void k_attn_prefill_any(const float* qkv, int T, int C, int H, int hd
 
 // x[t] = wte[ids[t]] + wpe[t]   (rust.rs:839-846)
 __global__ void k_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C, int w_bf16) {
+                             int T, int C, int w_bf16, int period) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (t < T && i < C) {
+    const int pos = t % period;
     const size_t idx = (size_t)ids[t] * C + i;
     const float e =
         w_bf16 ? __uint_as_float((unsigned)reinterpret_cast<const unsigned short*>(wte)[idx] << 16)
                : wte[idx];
-    x[(size_t)t * C + i] = e + wpe[(size_t)t * C + i];
+    x[(size_t)t * C + i] = e + wpe[(size_t)pos * C + i];
   }
 }
 
@@ -1562,23 +1568,27 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
 
 hipError_t launch_attn_prefill(const float* qkv, int T, int C, int H, int head_dim, int P,
                                float* kcache, float* vcache, float* out, float* scratch,
-                               hipStream_t s) {
+                               hipStream_t s, int nseq, size_t kv_stride) {
+  if (nseq < 1 || nseq > 65535) return hipErrorInvalidValue;
   if (head_dim == 64) {
     const int qblocks = (T + 31) / 32;
-    hipLaunchKernelGGL(k_attn_prefill64, dim3(H, qblocks), dim3(512), 0, s, qkv, T, C, P, kcache,
-                       vcache, out);
+    hipLaunchKernelGGL(k_attn_prefill64, dim3(H, qblocks, nseq), dim3(512), 0, s, qkv, T, C, P, kcache,
+                       vcache, out, kv_stride);
   } else {
+    // (test-sized models: one launch per sequence, all using the same scratch in turn)
     const int n = T * H;
-    hipLaunchKernelGGL(k_attn_prefill_any, dim3((n + 127) / 128), dim3(128), 0, s, qkv, T, C, H,
-                       head_dim, P, kcache, vcache, out, scratch);
+    for (int i = 0; i < nseq; ++i)
+      hipLaunchKernelGGL(k_attn_prefill_any, dim3((n + 127) / 128), dim3(128), 0, s,
+                         qkv + (size_t)i * T * 3 * C, T, C, H, head_dim, P, kcache + i * kv_stride,
+                         vcache + i * kv_stride, out + (size_t)i * T * C, scratch);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_embed_rows(float* x, const float* wte, const float* wpe, const uint32_t* ids,
-                             int T, int C, hipStream_t s, int w_bf16) {
+                             int T, int C, hipStream_t s, int w_bf16, int period) {
   hipLaunchKernelGGL(k_embed_rows, dim3((C + 255) / 256, T), dim3(256), 0, s, x, wte, wpe, ids, T,
-                     C, w_bf16);
+                     C, w_bf16, period > 0 ? period : T);
   return hipGetLastError();
 }
 
