@@ -7,8 +7,12 @@ from .gpt2 import (GPT2_EOS_TOKEN_ID, DeviceLogits, GenerationStats, Gpt2BlockWe
                    Gpt2Error, Gpt2GenerationConfig, Gpt2HipConfig, Gpt2KvCache, Gpt2Model,
                    Gpt2OperationProfile, Gpt2Output, Gpt2Weights, LogitsSampler, TensorStore, TextGenerationConfig,
                    argmax_logits, generate, load_weights)
+from .runtime import (Gpt2Runtime, Gpt2Tokenizer, IncrementalTextStreamer, escape_raw_token,
+                      is_incremental_decode_safe)
 
 __all__ = ["GPT2_EOS_TOKEN_ID", "DeviceLogits", "GenerationStats", "Gpt2BlockWeights",
            "Gpt2Config", "Gpt2Error", "Gpt2GenerationConfig", "Gpt2HipConfig", "Gpt2KvCache",
-           "Gpt2Model", "Gpt2OperationProfile", "Gpt2Output", "Gpt2Weights", "LogitsSampler", "TensorStore",
+           "Gpt2Model", "Gpt2OperationProfile", "Gpt2Output", "Gpt2Runtime", "Gpt2Tokenizer", "Gpt2Weights",
+           "IncrementalTextStreamer", "LogitsSampler", "TensorStore", "escape_raw_token",
+           "is_incremental_decode_safe",
            "TextGenerationConfig", "argmax_logits", "generate", "load_weights"]

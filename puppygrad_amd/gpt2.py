@@ -289,6 +289,7 @@ class GenerationStats:
     decode_time: float = 0.0
     first_token_time: Optional[float] = None
     gpu_decode_time: float = 0.0
+    tokenize_time: float = 0.0  # host time of the prompt's encode; set by Gpt2Runtime
 
     @property
     def total_generation_time(self) -> float:
