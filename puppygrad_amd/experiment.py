@@ -33,6 +33,7 @@ from typing import Iterable, List, Optional, Sequence
 from . import _lib, synth
 from .gpt2 import (GPT2_EOS_TOKEN_ID, GenerationStats, Gpt2Config, Gpt2HipConfig, Gpt2Model,
                    Gpt2OperationProfile, TextGenerationConfig)
+from .runtime import Gpt2Runtime
 
 
 @dataclass
@@ -150,7 +151,7 @@ def average_row(backend: str, quantized_weights: bool, prompt_index: Optional[in
         mlp_fc_chunk_size=0, mlp_projection_chunk_size=0, logits_chunk_size=0,
         attention_head_parallel_threshold=0, quantized_weights=quantized_weights,
         max_new_tokens=max_new_tokens, runs=runs, prompt_tokens=prompt_tokens,
-        generated_tokens=generated, load_ms=load_time * 1e3, tokenize_ms=0.0,
+        generated_tokens=generated, load_ms=load_time * 1e3, tokenize_ms=_mean([getattr(s, "tokenize_time", 0.0) for s in stats]) * 1e3,
         prefill_ms=prefill * 1e3, time_to_first_token_ms=_mean(first) * 1e3 if first else None,
         decode_ms=decode * 1e3, total_generation_ms=total * 1e3,
         decode_ms_min=dsum.min, decode_ms_median=dsum.median, decode_ms_p95=dsum.p95,
@@ -169,21 +170,51 @@ def average_row(backend: str, quantized_weights: bool, prompt_index: Optional[in
         profile_final_logits_ms=bucket("final_logits"), profile_decoding_ms=bucket("decoding"))
 
 
-def run_experiment(model: Gpt2Model, prompts: Sequence[Sequence[int]],
-                   token_counts: Sequence[int], runs: int, warmup_runs: int = 0,
-                   load_time: float = 0.0, profile_runs: int = 1, quantized_weights: bool = False,
+def load_experiment_prompts(prompt: Optional[str], prompt_file: Optional[str]) -> List[str]:
+    """load_experiment_prompts (src/main.rs:4009-4030): the non-empty trimmed lines of the
+    file, or the one prompt."""
+    if prompt_file is not None:
+        try:
+            with open(prompt_file, encoding="utf-8") as f:
+                text = f.read()
+        except OSError as e:
+            raise ValueError(f"failed to read --prompt-file {prompt_file}: {e}")
+        prompts = [line.strip() for line in text.splitlines() if line.strip()]
+        if not prompts:
+            raise ValueError(f"--prompt-file {prompt_file} contains no prompts")
+        return prompts
+    if prompt is None:
+        raise ValueError("experiment gpt2 requires --prompt or --prompt-file")
+    return [prompt]
+
+
+def run_experiment(model, prompts: Sequence, token_counts: Sequence[int], runs: int,
+                   warmup_runs: int = 0, load_time: float = 0.0, profile_runs: int = 1,
+                   quantized_weights: bool = False,
                    prompt_labels: Optional[Sequence[str]] = None,
                    eos_token_id: Optional[int] = GPT2_EOS_TOKEN_ID) -> List[Gpt2ExperimentRow]:
-    """The loops of run_gpt2_experiment (src/main.rs:3478-3527) over prompts given as token
-    ids: per token budget and prompt, `warmup_runs` untimed generations, `runs` timed ones
-    and `profile_runs` profiled ones; one row per prompt, plus an "<aggregate>" row over
-    all of them when there are several prompts.  Generation is greedy with GPT-2's EOS id
-    (Gpt2GenerationConfig::new, src/models/gpt2/options.rs:156-162) unless another, or
-    None, is given."""
+    """The loops of run_gpt2_experiment (src/main.rs:3478-3527): per token budget and prompt,
+    `warmup_runs` untimed generations, `runs` timed ones and `profile_runs` profiled ones; one
+    row per prompt, plus an "<aggregate>" row over all of them when there are several prompts.
+    `model` is a Gpt2Model with prompts given as token ids, or a Gpt2Runtime with prompts given
+    as text (then the tokenizer's and the text streamer's host time are in the rows, as in the
+    reference, which runs stream_greedy_text_with_stats).  Generation is greedy with GPT-2's EOS
+    id (Gpt2GenerationConfig::new, src/models/gpt2/options.rs:156-162) unless another, or None,
+    is given."""
     if runs == 0:
         raise ValueError("experiment --runs must be > 0")
+    text = hasattr(model, "tokenizer")
+    if text:
+        runtime = model
+
+        class _Text:  # the id-prompt interface over the runtime's text entry point
+            @staticmethod
+            def stream_token_ids_with_stats(prompt, generation, profiled=False):
+                out = runtime.stream_text_with_stats(prompt, generation, lambda _t: None, profiled)
+                return out if profiled else out[:2]
+        model = _Text
     labels = list(prompt_labels) if prompt_labels is not None else [
-        f"<{len(p)} token ids>" for p in prompts]
+        p if text else f"<{len(p)} token ids>" for p in prompts]
     rows = []
     for max_new in token_counts:
         generation = TextGenerationConfig(max_new, eos_token_id=eos_token_id)
@@ -275,6 +306,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     ap.add_argument("--model-dir", help="directory with config.json and model.safetensors")
     ap.add_argument("--prompt-tokens", default="32",
                     help="comma-separated prompt lengths; ids are seeded uniform draws")
+    ap.add_argument("--prompt", help="text prompt (needs --model-dir with a tokenizer.json)")
+    ap.add_argument("--prompt-file", help="one text prompt per line (needs --model-dir)")
     ap.add_argument("--max-new-tokens", default="16")
     ap.add_argument("--runs", type=int, default=3)
     ap.add_argument("--warmup-runs", type=int, default=1)
@@ -286,8 +319,18 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         raise SystemExit("experiment --runs must be > 0")
     hip = Gpt2HipConfig(weight_storage=_lib.PG_STORE_INT8 if args.quantized_weights
                         else _lib.PG_STORE_F32)
+    text_prompts = None
+    if args.prompt is not None or args.prompt_file is not None:
+        if not args.model_dir:
+            raise SystemExit("--prompt / --prompt-file need --model-dir (tokenizer.json)")
+        try:
+            text_prompts = load_experiment_prompts(args.prompt, args.prompt_file)
+        except ValueError as e:
+            raise SystemExit(str(e))
     t0 = time.perf_counter()
-    if args.model_dir:
+    if text_prompts is not None:
+        model = Gpt2Runtime.from_dir(args.model_dir, hip)
+    elif args.model_dir:
         model = Gpt2Model.from_dir(args.model_dir, hip)
     else:
         kw = {"small": synth.GPT2_SMALL, "medium": synth.GPT2_MEDIUM, "large": synth.GPT2_LARGE,
@@ -295,10 +338,12 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         cfg = Gpt2Config(**kw)
         model = Gpt2Model.new(cfg, synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 1), hip)
     load_time = time.perf_counter() - t0
-    print(f"loaded GPT-2 with {model.describe()}", file=sys.stderr)
-    vocab = model.config.vocab_size
-    prompts = [list(synth.token_ids(n, synth.TOKEN_SEED_BASE + 1, vocab))
-               for n in _usize_list("prompt-tokens", args.prompt_tokens)]
+    core = model.model if text_prompts is not None else model
+    print(f"loaded GPT-2 with {core.describe()}", file=sys.stderr)
+    vocab = core.config.vocab_size
+    prompts = text_prompts if text_prompts is not None else [
+        list(synth.token_ids(n, synth.TOKEN_SEED_BASE + 1, vocab))
+        for n in _usize_list("prompt-tokens", args.prompt_tokens)]
     rows = run_experiment(model, prompts, _usize_list("max-new-tokens", args.max_new_tokens),
                           args.runs, args.warmup_runs, load_time, args.profile_runs,
                           args.quantized_weights)

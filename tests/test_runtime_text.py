@@ -177,3 +177,37 @@ def test_runtime_from_dir_needs_the_tokenizer_file(tmp_path):
     (path / "tokenizer.json").unlink()
     with pytest.raises(Gpt2Error, match="failed to load tokenizer"):
         Gpt2Runtime.from_dir(path)
+
+
+def test_experiment_prompts_come_from_a_file_or_one_string(tmp_path):
+    """load_experiment_prompts (src/main.rs:4009-4030)."""
+    from puppygrad_amd import experiment as ex
+    f = tmp_path / "prompts.txt"
+    f.write_text("  first prompt \n\n\tsecond\n   \n")
+    assert ex.load_experiment_prompts("ignored", str(f)) == ["first prompt", "second"]
+    assert ex.load_experiment_prompts("only", None) == ["only"]
+    f.write_text(" \n\n")
+    with pytest.raises(ValueError, match="contains no prompts"):
+        ex.load_experiment_prompts(None, str(f))
+    with pytest.raises(ValueError, match="failed to read --prompt-file"):
+        ex.load_experiment_prompts(None, str(tmp_path / "missing.txt"))
+    with pytest.raises(ValueError, match="requires --prompt or --prompt-file"):
+        ex.load_experiment_prompts(None, None)
+
+
+@pytest.mark.gpu
+def test_experiment_rows_over_text_prompts_carry_the_host_text_time(tmp_path):
+    from puppygrad_amd import experiment as ex
+    path, cfg, w = _model_dir(tmp_path)
+    rt = Gpt2Runtime.from_dir(path)
+    prompts = ["hello there, quick fox", "the lazy dog"]
+    rows = ex.run_experiment(rt, prompts, [6], runs=2, warmup_runs=1, profile_runs=1,
+                             eos_token_id=None)
+    assert [r.prompt for r in rows] == prompts + ["<aggregate>"]
+    assert [r.prompt_index for r in rows] == [0, 1, None]
+    for r, p in zip(rows, prompts):
+        assert r.prompt_tokens == len(rt.tokenizer.encode(p)) and r.generated_tokens == 6.0
+        assert r.tokenize_ms > 0.0 and r.profile_tokenization_ms > 0.0 and r.profile_decoding_ms > 0.0
+        assert r.profile_qkv_projection_ms > 0.0 and r.decode_ms > 0.0
+    assert rows[2].runs == 4
+    assert ex.format_csv(rows).count("\n") == 4
