@@ -68,12 +68,16 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "batch-decode"],
                     help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound); "
                          "batch-decode: a step is one greedy step of --batch sequences")
-    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=None,
+                    help="sequences of a batched step (batch-decode: 16 by default; prefill: 1)")
     ap.add_argument("--bf16", action="store_true", help="store the weights as bf16 (fp32 arithmetic)")
     ap.add_argument("--int8", action="store_true",
                     help="store the weights as int8 rows with f32 scales (the reference's "
                          "quantized_weights; fp32 arithmetic); --workload decode")
     args = ap.parse_args()
+    args.batch_given = args.batch is not None
+    if args.batch is None:
+        args.batch = 16
     if args.gpus != 1:
         log("bench.py: this path runs on ONE GPU (a batch-1 decode step has one all-reduce of "
             "n_embd floats after every projection pair to offer to a second GPU: latency-bound); "
@@ -97,9 +101,6 @@ def main() -> int:
     path = {"auto": _lib.PG_DECODE_AUTO, "kernels": _lib.PG_DECODE_KERNELS,
             "persistent": _lib.PG_DECODE_PERSISTENT}[args.decode_path]
     storage = _lib.PG_STORE_BF16 if args.bf16 else _lib.PG_STORE_INT8 if args.int8 else _lib.PG_STORE_F32
-    if args.bf16 and args.workload == "prefill":
-        log("bench.py: --bf16 is for --workload decode or batch-decode")
-        return 2
     if args.int8 and (args.workload != "decode" or args.bf16):
         log("bench.py: --int8 is for --workload decode, without --bf16")
         return 2
@@ -270,6 +271,7 @@ def secondary_workloads(xl_cfg, xl_weights):
     # GPT-2 XL with bf16-stored weights: batch-32 decode steps from 512-token prompts
     model = Gpt2Model.new(xl_cfg, xl_weights, Gpt2HipConfig(weight_storage=_lib.PG_STORE_BF16))
     out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 512, 24, True)
+    out["gpt2_xl_bf16_prefill_b32_512"] = measure_batch_prefill_bf16(model, xl_cfg, 32, 512, 3)
     del model
     return out
 
@@ -354,18 +356,64 @@ def measure_batch_decode(model, cfg, B, n_prefill, steps, bf16):
                                      algorithmic_bytes_per_step=int(wbytes + kvb))}
 
 
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
+
+
+def prefill_flops(cfg, B, T):
+    """(all, projections only) algorithmic flops of B prompts of T tokens."""
+    C_, I, L, V = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size
+    gemm_flops = 2.0 * B * T * L * (3 * C_ * C_ + C_ * C_ + 2 * C_ * I)
+    attn_flops = 4.0 * B * C_ * (T * (T + 1) / 2) * L
+    return gemm_flops + attn_flops + 2.0 * B * V * C_, gemm_flops
+
+
+def bf16_prefill_roofline(flops, gemm_flops, sec):
+    """bf16 rows: the projections run on the bf16 matrix cores, every f32 input cut into three
+    bf16 parts (exact products, f32 sums): three matrix instructions' worth of work per
+    algorithmic product, so a third of the bf16 peak is this form's ceiling."""
+    achieved = flops / sec / 1e12
+    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4), "traffic": None, "passes": 3,
+            "executed": round((2 * gemm_flops + flops) / sec / 1e12, 2),
+            "kernel": "whole prefill (k_gemm_b3 on the bf16 matrix cores, k_attn_prefill64 and lm_head in f32)",
+            "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)}
+
+
+def measure_batch_prefill_bf16(model, cfg, B, T, steps):
+    """B prompts of T tokens through the layers at once, weights stored as bf16."""
+    from puppygrad_amd import synth
+    ids = np.stack([synth.token_ids(T, synth.TOKEN_SEED_BASE + 100 + b, cfg.vocab_size) for b in range(B)])
+    cache = model.new_kv_cache(B)
+    model.prefill_batch(ids, cache).argmax()
+    t0 = time.time()
+    for _ in range(steps):
+        lg = model.prefill_batch(ids, cache)
+    lg.argmax()
+    sec = (time.time() - t0) / steps
+    flops, gemm_flops = prefill_flops(cfg, B, T)
+    return {"workload": f"GPT-2 n_embd={cfg.n_embd} B={B} prefill of {T} tokens each into empty KV caches, "
+                        f"weights stored as bf16, f32 inputs and sums",
+            "value": round(B * T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 3),
+            "roofline": bf16_prefill_roofline(flops, gemm_flops, sec)}
+
+
 def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
     """Secondary workload (prompt processing, e.g. GPT-2 124M with 1024 tokens): a step is one
-    prefill of n_prefill tokens into an empty cache through the GEMM path.  Algorithmic
+    prefill of n_prefill tokens into an empty cache through the GEMM path; with --batch B > 1
+    (given explicitly) B prompts of that length at once (pg_gpt2_prefill_batch).  Algorithmic
     flops: the four projections of every layer over all tokens, causal attention
     (QK^T and PV over the lower triangle), and the lm_head row of the last token."""
-    C_, I, L, V, T = cfg.n_embd, cfg.n_inner, cfg.n_layer, cfg.vocab_size, n_prefill
-    gemm_flops = 2.0 * T * L * (3 * C_ * C_ + C_ * C_ + 2 * C_ * I)
-    attn_flops = 4.0 * C_ * (T * (T + 1) / 2) * L
-    flops = gemm_flops + attn_flops + 2.0 * V * C_
-    cache = model.new_kv_cache()
+    from puppygrad_amd import synth
+    T = n_prefill
+    B = args.batch if args.batch_given else 1
+    flops, gemm_flops = prefill_flops(cfg, B, T)
+    cache = model.new_kv_cache(B)
+    if B > 1:
+        ids = np.stack([synth.token_ids(T, synth.TOKEN_SEED_BASE + 100 + b, cfg.vocab_size) for b in range(B)])
 
     def one():
+        if B > 1:
+            return model.prefill_batch(ids, cache)
         cache.seq_len = 0
         return model.prefill(ids, cache)
 
@@ -379,13 +427,14 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
     sec = wall / args.steps
     info = _devinfo()
     achieved = flops / sec / 1e12
+    stored = "bf16-stored weights" if args.bf16 else "fp32"
     result = {
-        "metric": f"prefill tokens/sec, GPT-2 {args.model} fp32 bs=1, {T}-token prompt",
-        "value": round(T / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "metric": f"prefill tokens/sec, GPT-2 {args.model} {stored} bs={B}, {T}-token prompt",
+        "value": round(B * T / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": max(1, args.warmup), "ms_per_step": round(sec * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"GPT-2 {args.model} fp32 B=1 prefill of {T} tokens into an empty KV cache",
+        "config": {"workload": f"GPT-2 {args.model} {stored} B={B} prefill of {T} tokens into an empty KV cache",
                    "weights": "seeded N(0,0.02), biases 0, LayerNorm gamma 1 beta 0",
                    "device": info.name.decode() or info.arch.decode(), "compute_units": info.compute_units,
                    "backend": model.describe()},
@@ -394,9 +443,11 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
                      "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
                      "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
     }
+    if args.bf16:
+        result["roofline"] = bf16_prefill_roofline(flops, gemm_flops, sec)
     # A short prompt reads every weight once for few rows: below about 52 rows the weights'
     # bytes at the HBM peak take longer than the flops at the MFMA peak, and HBM is the bound.
-    wbytes = weight_bytes(cfg)
+    wbytes = weight_bytes(cfg, bf16=args.bf16)
     if wbytes / (HBM_PEAK_GBS * 1e9) > flops / (FP32_MFMA_PEAK_TFLOPS * 1e12):
         gbs = wbytes / sec / 1e9
         result["roofline"] = hbm_roofline(gbs, "whole prefill (k_gemm_rows32, k_attn_prefill64, reduce + LayerNorm, lm_head)",

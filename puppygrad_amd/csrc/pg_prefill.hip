@@ -341,6 +341,236 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same product for W stored as bf16, on the bf16 matrix cores, without giving up f32
+// inputs: every input value is cut into three bf16 numbers whose sum is the value exactly
+// (its 24 significant bits in three groups of 8, by truncation), W's values are bf16 as they
+// are, so x . w = hi . w + mid . w + lo . w with every product exact in f32 and the sums
+// accumulated in f32 as before.  Three v_mfma_f32_32x32x16_bf16 do per 16 columns what eight
+// v_mfma_f32_32x32x2_f32 of four times the duration did.  (A NaN or an infinity in the input
+// gives NaN in its row of the result, as inf - inf does in the split.)
+// 256 threads = 4 wavefronts (2 x 2) on a BM x BN tile; k-tiles of 32 columns, staged in LDS
+// row-major ([row][32 bf16] = 64 bytes, the three input planes and W): the operand of a lane
+// is 16 consecutive bytes of its row (8 columns; lanes 32..63 take the second 8 of a 16-column
+// step), and the 16-byte pieces of a row are permuted (lds_piece_turn) so that the lanes of
+// one read hit different banks.  Two LDS buffers; the next tile's global loads are in flight
+// while the current one is multiplied.  K must be a multiple of 32.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+
+// The 16-byte pieces of LDS row `row` are stored permuted by this value (xor): the rows that a
+// group of 8 or of 16 lanes reads in one cycle then lie on different banks, whether the LDS
+// serves 32 or 64 banks a cycle.
+__device__ __forceinline__ int lds_piece_turn(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+
+struct Split3 {
+  u2v hi, mid, lo;  // four bf16 each, lowest column in the low half of .x
+};
+__device__ __forceinline__ Split3 split3_bf16(f4 x) {
+  unsigned h[4], m[4], l[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    h[j] = __float_as_uint(x[j]) & 0xffff0000u;
+    const float r1 = x[j] - __uint_as_float(h[j]);  // exact: the 16 low bits of the significand
+    m[j] = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(m[j]);    // exact: at most 8 significant bits left
+    l[j] = __float_as_uint(r2);
+  }
+  Split3 r;
+  r.hi.x = (h[0] >> 16) | h[1];
+  r.hi.y = (h[2] >> 16) | h[3];
+  r.mid.x = (m[0] >> 16) | m[1];
+  r.mid.y = (m[2] >> 16) | m[3];
+  r.lo.x = (l[0] >> 16) | (l[1] & 0xffff0000u);
+  r.lo.y = (l[2] >> 16) | (l[3] & 0xffff0000u);
+  return r;
+}
+
+template <int BM, int BN, int EPI>
+__global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
+  constexpr int KT = 32;                     // columns per k-tile
+  constexpr int WM = BM / 2, WN = BN / 2;    // per-wavefront tile
+  constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
+  constexpr int ALD = BM / 32;               // float4 loads of A per thread and tile (8 lanes per row)
+  constexpr int BLD = BN / 64;               // 16-byte loads of W per thread and tile (4 lanes per row)
+  // [buffer][plane][row][piece]: a row is four 16-byte pieces
+  __shared__ u4v As[2][3][BM][4];
+  __shared__ u4v Bs[2][BN][4];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (a.N + BN - 1) / BN;
+  const int tiles_all = ((a.M + BM - 1) / BM) * tiles_n;
+  int tile;
+  {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int per_xcd = ((int)gridDim.x + 7) >> 3;
+    tile = xcd * per_xcd + slot;
+  }
+  if (tile >= tiles_all) return;
+  int tm, tn;
+  tile_coords(tile, (a.M + BM - 1) / BM, tiles_n, a.band_rows, &tm, &tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // global loads: A eight lanes to a row (a float4 each), W four lanes to a row (8 bf16 each)
+  const int ar = tid >> 3, ak = (tid & 7) * 4;
+  const int br = tid >> 2, bp = tid & 3;
+  const float* Ag[ALD];
+  const unsigned short* Wg[BLD];
+#pragma unroll
+  for (int i = 0; i < ALD; ++i) Ag[i] = a.A + (size_t)min(m0 + ar + 32 * i, a.M - 1) * a.lda + ak;
+#pragma unroll
+  for (int i = 0; i < BLD; ++i)
+    Wg[i] = reinterpret_cast<const unsigned short*>(a.W) + (size_t)min(n0 + br + 64 * i, a.N - 1) * a.K + bp * 8;
+
+  f16v acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int T = a.K / KT;
+  const int half = lane >> 5, l32 = lane & 31;
+  // two sets of load registers: a tile is requested two tiles' arithmetic before it is stored
+  f4 ra0[ALD], ra1[ALD];
+  u4v rb0[BLD], rb1[BLD];
+  auto load_tile = [&](int t, f4 (&ra)[ALD], u4v (&rb)[BLD]) __attribute__((always_inline)) {
+    const size_t k = (size_t)t * KT;
+#pragma unroll
+    for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + k);
+#pragma unroll
+    for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const u4v*>(Wg[i] + k);
+  };
+  auto store_tile = [&](int buf, f4 (&ra)[ALD], u4v (&rb)[BLD]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < ALD; ++i) {
+      const int row = ar + 32 * i;
+      const int piece = (ak >> 3) ^ lds_piece_turn(row);
+      const Split3 sp = split3_bf16(ra[i]);
+      const int h8 = (ak >> 2) & 1;  // which half of the piece
+      reinterpret_cast<u2v*>(&As[buf][0][row][piece])[h8] = sp.hi;
+      reinterpret_cast<u2v*>(&As[buf][1][row][piece])[h8] = sp.mid;
+      reinterpret_cast<u2v*>(&As[buf][2][row][piece])[h8] = sp.lo;
+    }
+#pragma unroll
+    for (int i = 0; i < BLD; ++i) {
+      const int row = br + 64 * i;
+      Bs[buf][row][bp ^ lds_piece_turn(row)] = rb[i];
+    }
+  };
+  // the operands of one 16-column step of a tile: three planes of MB row blocks, NB column blocks
+  struct Ops {
+    u4v a[3][MB], b[NB];
+  };
+  auto read_ops = [&](int buf, int kc, Ops& o) __attribute__((always_inline)) {
+    const int piece = 2 * kc + half;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int row = wn * WN + 32 * j + l32;
+      o.b[j] = Bs[buf][row][piece ^ lds_piece_turn(row)];
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+      const int row = wm * WM + 32 * i + l32;
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) o.a[pl][i] = As[buf][pl][row][piece ^ lds_piece_turn(row)];
+    }
+  };
+  auto mfma_ops = [&](const Ops& o) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pl = 2; pl >= 0; --pl)  // the small terms first
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, o.a[pl][i]),
+                                                             __builtin_bit_cast(bf16x8, o.b[j]),
+                                                             acc[i][j], 0, 0, 0);
+  };
+  constexpr int NM = 3 * MB * NB;  // MFMAs per 16-column step
+  // A tile in two halves, each a run of NM MFMAs with the other work of the wavefront placed
+  // between them (an MFMA keeps the matrix core busy for 32 clocks, during which the
+  // wavefront can issue a handful of other instructions):
+  //   first 16 columns of tile t   + LDS reads of its second 16 columns
+  //                                + tile t+1 from its load registers, cut in three, to the other LDS buffer
+  //   barrier
+  //   second 16 columns of tile t  + LDS reads of tile t+1's first 16 columns
+  //                                + request of tile t+3 into the load registers just emptied
+  // (r, rb) hold tile t+1.
+  Ops o0, o1;
+  auto tile_step = [&](auto more_c, int t, f4 (&r)[ALD], u4v (&rb)[BLD]) __attribute__((always_inline)) {
+    constexpr bool more = decltype(more_c)::value;  // a tile t+1 exists
+    mfma_ops(o0);
+    read_ops(t & 1, 1, o1);
+    if (more) store_tile((t + 1) & 1, r, rb);
+#pragma unroll
+    for (int g = 0; g < NM; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // a few VALU
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_ops(o1);
+    if (more) {
+      read_ops((t + 1) & 1, 0, o0);
+      load_tile(min(t + 3, T - 1), r, rb);  // past the end: the last tile again, never used
+    }
+#pragma unroll
+    for (int g = 0; g < NM; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (T > 0) {
+    load_tile(0, ra0, rb0);
+    load_tile(min(1, T - 1), ra1, rb1);
+    store_tile(0, ra0, rb0);
+    __syncthreads();
+    read_ops(0, 0, o0);
+    load_tile(min(2, T - 1), ra0, rb0);
+    const std::true_type yes;
+    const std::false_type no;
+    int t = 0;
+    for (; t + 2 < T; t += 2) {
+      tile_step(yes, t, ra1, rb1);
+      tile_step(yes, t + 1, ra0, rb0);
+    }
+    if (T - t == 2) {
+      tile_step(yes, t, ra1, rb1);
+      tile_step(no, t + 1, ra0, rb0);
+    } else {
+      tile_step(no, t, ra1, rb1);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int n = n0 + wn * WN + 32 * j + l32;
+      if (n >= a.N) continue;
+      const float bias = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (m >= a.M) continue;
+        float c = bias + acc[i][j][v];
+        if (EPI == GEMM_GELU) c = gelu_tanh(c);
+        if (EPI == GEMM_RESID) c = a.resid[(size_t)m * a.ldc + n] + c;
+        a.C[(size_t)m * a.ldc + n] = c;
+      }
+    }
+}
+
 // C = epilogue(bias + part[0] + part[1] + ...) for the split-K form of k_gemm; one
 // float4 of a row per thread (N is a multiple of 4 whenever the split is used).
 template <int EPI>
@@ -1175,6 +1405,8 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
   for (int i = threadIdx.x; i < cols; i += 256) out_at(i) = (row[i] - mean) * inv * g[i] + b[i];
 }
 
+int choose_band_fwd(int tiles_m, int run, int bm, int bn);
+
 template <int BM, int BN, int WBF, int BKT = BK>
 hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
@@ -1188,6 +1420,41 @@ hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
+}
+
+// The bf16 matrix-core form (k_gemm_b3): W stored as bf16, whole 128 x 128 tiles.
+bool gemm_b3_ok(const GemmArgs& a) {
+  return a.w_bf16 && !a.w_scale && a.K % 32 == 0 && a.K >= 32 && !a.a_packed && !a.c_packed;
+}
+template <int BM, int BN>
+hipError_t launch_gemm_b3_shape(const GemmArgs& a0, int epi, hipStream_t s) {
+  GemmArgs a = a0;
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int tiles = tiles_m * tiles_n;
+  a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band_fwd(tiles_m, std::max(1, (tiles + 7) / 8), BM, BN);
+  const int grid = (tiles + 7) / 8 * 8;
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_BIAS>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_GELU>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_RESID>), dim3(grid), dim3(256), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+// 128 x 128 tiles (two workgroups to a CU); 128 x 256 for a long K where those still fill the
+// chip twice over (measured: 4096 x 1600 x 6400, 275 against 302 us); a.plan_bn forces one.
+hipError_t launch_gemm_b3(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
+  if (!gemm_b3_ok(a)) return hipErrorInvalidValue;
+  const long tiles_wide = (long)((a.M + 127) / 128) * ((a.N + 255) / 256);
+  const bool wide = a.plan_bn ? a.plan_bn == 256 : a.K >= 4096 && tiles_wide >= 2L * num_cus;
+  return wide ? launch_gemm_b3_shape<128, 256>(a, epi, s) : launch_gemm_b3_shape<128, 128>(a, epi, s);
+}
+// Whether the planner sends a product there: from a quarter of a tile per CU on (below that a
+// tile's own k loop, one workgroup deep, is longer than the f32 forms cut along K).
+bool gemm_b3_pays(const GemmArgs& a, int num_cus) {
+  return gemm_b3_ok(a) && (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * 4 >= num_cus;
 }
 
 }  // namespace
@@ -1450,6 +1717,8 @@ int choose_band(int tiles_m, int run, int bm, int bn) {
   return best;
 }
 
+int choose_band_fwd(int tiles_m, int run, int bm, int bn) { return choose_band(tiles_m, run, bm, bn); }
+
 // WBF: 0 f32, 1 bf16, 2 int8 rows (k_gemm's WT)
 template <int WBF>
 hipError_t launch_tiles(const GemmArgs& a0, int epi, int bm, int bn, int form, int parts, hipStream_t s,
@@ -1542,6 +1811,7 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
     return launch_tiles<2>(t, epi, bm, bn, form, parts, s, ln_done);
   }
+  if (a.plan_form == 5) return launch_gemm_b3(a, epi, num_cus, s);  // forced: the bf16 matrix-core form
   if (a.plan_form == 4) {  // forced: the 32-row kernel
     const int rp = gemm_rows32_parts(a, num_cus);
     if (!rp) return hipErrorInvalidValue;
@@ -1559,6 +1829,8 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   // Tile forms.  A forced plan (benchmarks, tests) or the planner's choice.
   int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
   GemmArgs t = a;
+  // bf16 rows and enough tiles: on the bf16 matrix cores
+  if (!form && gemm_b3_pays(a, num_cus)) return launch_gemm_b3(a, epi, num_cus, s);
   if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
   else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
   return a.w_bf16 ? launch_tiles<1>(t, epi, bm, bn, form, parts, s, ln_done)

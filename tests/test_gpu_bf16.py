@@ -47,6 +47,27 @@ def test_bf16_storage_matches_oracle_on_rounded_weights(n_embd, n_head, n_prompt
     assert np.abs(model.forward(ids).logits - full).max() <= 2e-2 * scale
 
 
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(832, 13, 400), (768, 12, 512)])
+def test_bf16_long_prompts_on_the_bf16_matrix_cores(n_embd, n_head, n_prompt):
+    """Prompts long enough that c_attn and c_fc run as 128 x 128 tiles on the bf16 matrix cores,
+    the f32 inputs cut into three bf16 parts (exact products, f32 sums): a ragged last row tile
+    (400 = 3 x 128 + 16), widths that are no multiple of the tile (2496, 3328) and ones that
+    are, against the oracle on the rounded weights at the f32 tolerance."""
+    cfg = Gpt2Config(vocab_size=300, n_positions=512, n_embd=n_embd, n_layer=1, n_head=n_head)
+    w = synth.random_weights(cfg, 0x5EED0520 + n_head, perturb=True)
+    ids = synth.token_ids(n_prompt, 0x70C00520, cfg.vocab_size)
+    model = Gpt2Model.new(cfg, w, BF16)
+    ref = oracle.Model(cfg, synth.bf16_rounded(w), oracle.rust_config(8))
+    cache, rc = model.new_kv_cache(), ref.new_kv_cache()
+    want = ref.prefill(ids, rc)
+    assert_logits_close(model.prefill(ids, cache).to_host(), want)
+    full = model.forward(ids).logits
+    assert_logits_close(full, ref.forward(ids))
+    if n_prompt < cfg.n_positions:
+        tok = int(np.argmax(want))
+        assert_logits_close(model.forward_one(tok, cache).to_host(), ref.forward_one(tok, rc))
+
+
 def test_bf16_batched_steps():
     cfg = Gpt2Config(vocab_size=257, n_positions=48, n_embd=128, n_layer=2, n_head=2)
     B, n = 6, 20
