@@ -387,7 +387,9 @@ __device__ __forceinline__ Split3 split3_bf16(f4 x) {
   return r;
 }
 
-template <int BM, int BN, int EPI>
+// SPLIT = 1: the k-tiles are cut into gridDim.y parts, the raw partial tiles go to
+// a.ws[part][M][N] and k_splitk_reduce(_ln) finishes them, as for k_gemm.
+template <int BM, int BN, int EPI, int SPLIT = 0>
 __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
   constexpr int KT = 32;                     // columns per k-tile
   constexpr int WM = BM / 2, WN = BN / 2;    // per-wavefront tile
@@ -432,13 +434,16 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  const int T = a.K / KT;
+  const int T_all = a.K / KT;
+  const int kt0 = SPLIT ? (int)(((long)blockIdx.y * T_all) / gridDim.y) : 0;
+  const int kt1 = SPLIT ? (int)(((long)(blockIdx.y + 1) * T_all) / gridDim.y) : T_all;
+  const int T = kt1 - kt0;  // this block's k-tiles [kt0, kt1)
   const int half = lane >> 5, l32 = lane & 31;
   // two sets of load registers: a tile is requested two tiles' arithmetic before it is stored
   f4 ra0[ALD], ra1[ALD];
   u4v rb0[BLD], rb1[BLD];
   auto load_tile = [&](int t, f4 (&ra)[ALD], u4v (&rb)[BLD]) __attribute__((always_inline)) {
-    const size_t k = (size_t)t * KT;
+    const size_t k = (size_t)(kt0 + t) * KT;
 #pragma unroll
     for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + k);
 #pragma unroll
@@ -558,6 +563,15 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
     for (int j = 0; j < NB; ++j) {
       const int n = n0 + wn * WN + 32 * j + l32;
       if (n >= a.N) continue;
+      if (SPLIT) {
+        float* part = a.ws + (size_t)blockIdx.y * a.M * a.N;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+          if (m < a.M) part[(size_t)m * a.N + n] = acc[i][j][v];
+        }
+        continue;
+      }
       const float bias = a.bias ? a.bias[n] : 0.0f;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -1406,6 +1420,7 @@ __global__ __launch_bounds__(256) void k_layer_norm_rows(const float* src, float
 }
 
 int choose_band_fwd(int tiles_m, int run, int bm, int bn);
+hipError_t launch_splitk_reduce_fwd(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done);
 
 template <int BM, int BN, int WBF, int BKT = BK>
 hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
@@ -1451,10 +1466,31 @@ hipError_t launch_gemm_b3(const GemmArgs& a, int epi, int num_cus, hipStream_t s
   const bool wide = a.plan_bn ? a.plan_bn == 256 : a.K >= 4096 && tiles_wide >= 2L * num_cus;
   return wide ? launch_gemm_b3_shape<128, 256>(a, epi, s) : launch_gemm_b3_shape<128, 128>(a, epi, s);
 }
-// Whether the planner sends a product there: from a quarter of a tile per CU on (below that a
-// tile's own k loop, one workgroup deep, is longer than the f32 forms cut along K).
-bool gemm_b3_pays(const GemmArgs& a, int num_cus) {
-  return gemm_b3_ok(a) && (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * 4 >= num_cus;
+// Whether the planner sends a product there whole: from a quarter of a tile per CU on (below
+// that a tile's own k loop, one workgroup deep, is too long).
+bool gemm_b3_pays(const GemmArgs& a, int num_cus, int min_share = 4) {
+  return gemm_b3_ok(a) && (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * min_share >= num_cus;
+}
+// Fewer tiles than that (prompts of 65 to a few hundred tokens): the k-tiles cut into up to 8
+// parts so that about two items per CU exist, each at least four k-tiles long; 0 where that
+// does not apply (no workspace, N no multiple of 4, K too short, hardly any tiles).
+int gemm_b3_split_parts(const GemmArgs& a, int num_cus) {
+  if (!gemm_b3_ok(a) || !a.ws || a.N % 4 != 0 || a.M <= 64) return 0;
+  const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
+  if (!a.plan_parts && tiles < 12) return 0;  // (a dozen short items: the f32 forms' 64 x 64 tiles do better)
+  int parts = a.plan_parts ? a.plan_parts : (int)((2L * num_cus + tiles - 1) / tiles);
+  parts = std::min(parts, a.K / 32 / 4);
+  parts = std::min(parts, 8);  // what the reduce kernels take
+  while (parts > 1 && (size_t)parts * a.M * a.N > a.ws_floats) --parts;
+  return parts >= 2 ? parts : 0;
+}
+hipError_t launch_gemm_b3_split(const GemmArgs& a0, int epi, int parts, hipStream_t s, bool* ln_done) {
+  GemmArgs a = a0;
+  const int tiles_m = (a.M + 127) / 128, tiles_n = (a.N + 127) / 128;
+  const int tiles = tiles_m * tiles_n;
+  a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band_fwd(tiles_m, std::max(1, (tiles + 7) / 8), 128, 128);
+  hipLaunchKernelGGL((k_gemm_b3<128, 128, GEMM_BIAS, 1>), dim3((tiles + 7) / 8 * 8, parts), dim3(256), 0, s, a);
+  return launch_splitk_reduce_fwd(a, epi, parts, s, ln_done);
 }
 
 }  // namespace
@@ -1718,6 +1754,9 @@ int choose_band(int tiles_m, int run, int bm, int bn) {
 }
 
 int choose_band_fwd(int tiles_m, int run, int bm, int bn) { return choose_band(tiles_m, run, bm, bn); }
+hipError_t launch_splitk_reduce_fwd(const GemmArgs& a, int epi, int parts, hipStream_t s, bool* ln_done) {
+  return launch_splitk_reduce(a, epi, parts, s, ln_done);
+}
 
 // WBF: 0 f32, 1 bf16, 2 int8 rows (k_gemm's WT)
 template <int WBF>
@@ -1812,6 +1851,10 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     return launch_tiles<2>(t, epi, bm, bn, form, parts, s, ln_done);
   }
   if (a.plan_form == 5) return launch_gemm_b3(a, epi, num_cus, s);  // forced: the bf16 matrix-core form
+  if (a.plan_form == 6) {                                           // forced: the same, cut along K
+    const int bp = gemm_b3_split_parts(a, num_cus);
+    return bp ? launch_gemm_b3_split(a, epi, bp, s, ln_done) : hipErrorInvalidValue;
+  }
   if (a.plan_form == 4) {  // forced: the 32-row kernel
     const int rp = gemm_rows32_parts(a, num_cus);
     if (!rp) return hipErrorInvalidValue;
@@ -1830,7 +1873,12 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
   GemmArgs t = a;
   // bf16 rows and enough tiles: on the bf16 matrix cores
-  if (!form && gemm_b3_pays(a, num_cus)) return launch_gemm_b3(a, epi, num_cus, s);
+  // bf16 rows: on the bf16 matrix cores; whole tiles from half a tile per CU on, else cut
+  // along K (measured crossover, XL c_attn / c_fc: 128 to 150 tiles), else whole again
+  if (!form && gemm_b3_pays(a, num_cus, 2)) return launch_gemm_b3(a, epi, num_cus, s);
+  if (!form)
+    if (const int bp = gemm_b3_split_parts(a, num_cus)) return launch_gemm_b3_split(a, epi, bp, s, ln_done);
+  if (!form && gemm_b3_pays(a, num_cus, 4)) return launch_gemm_b3(a, epi, num_cus, s);
   if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
   else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;
   return a.w_bf16 ? launch_tiles<1>(t, epi, bm, bn, form, parts, s, ln_done)
