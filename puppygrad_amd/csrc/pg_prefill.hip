@@ -966,24 +966,59 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       }
     }
     __builtin_amdgcn_wave_barrier();
-    float wv[CPP];
-    if (M16) {
+    if constexpr (WT == 1) {
+      // bf16 rows: on the bf16 matrix cores.  A piece of a W row is the operand as it is (8
+      // consecutive columns); the 8 input values that meet it are cut into three bf16 parts
+      // whose sum is the value exactly (split3_bf16), so the three products are exact and the
+      // sums f32 as in the other forms.
+      auto cut8 = [](const f4& lo4, const f4& hi4, u4v (&part)[3]) {
+        const Split3 s0 = split3_bf16(lo4), s1 = split3_bf16(hi4);
+        part[0] = u4v{s0.hi.x, s0.hi.y, s1.hi.x, s1.hi.y};
+        part[1] = u4v{s0.mid.x, s0.mid.y, s1.mid.x, s1.mid.y};
+        part[2] = u4v{s0.lo.x, s0.lo.y, s1.lo.x, s1.lo.y};
+      };
+      if (M16) {
+        u4v xp3[3];
+        cut8(xo[0], xo[1], xp3);
 #pragma unroll
-      for (int g = 0; g < NR / 16; ++g) {
-        widen(wo[g], wv, wsc[g]);
+        for (int g = 0; g < NR / 16; ++g)
 #pragma unroll
-        for (int c = 0; c < CPP; ++c)
-          acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[c / 4][c % 4], wv[c], acc16[g], 0, 0, 0);
+          for (int pl = 2; pl >= 0; --pl)
+            acc16[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
+                                                              __builtin_bit_cast(bf16x8, wo[g]), acc16[g], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            u4v xp3[3];
+            cut8(xo[mt * XT + u * XF], xo[mt * XT + u * XF + 1], xp3);
+#pragma unroll
+            for (int pl = 2; pl >= 0; --pl)
+              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
+                                                                __builtin_bit_cast(bf16x8, wo[u]), acc[mt], 0, 0, 0);
+          }
       }
     } else {
+      float wv[CPP];
+      if (M16) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        widen(wo[u], wv, wsc[0]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int g = 0; g < NR / 16; ++g) {
+          widen(wo[g], wv, wsc[g]);
 #pragma unroll
           for (int c = 0; c < CPP; ++c)
-            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xo[mt * XT + u * XF + c / 4][c % 4], wv[c], acc[mt], 0, 0, 0);
+            acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[c / 4][c % 4], wv[c], acc16[g], 0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          widen(wo[u], wv, wsc[0]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int c = 0; c < CPP; ++c)
+              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(xo[mt * XT + u * XF + c / 4][c % 4], wv[c], acc[mt], 0, 0, 0);
+        }
       }
     }
   };
