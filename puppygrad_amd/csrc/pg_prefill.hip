@@ -585,6 +585,205 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same for W stored as f32: both the input and W are cut into three bf16 parts when their
+// tile is staged and all nine products of the parts are formed, whose sum is x . w exactly —
+// nothing is given up against the f32 matrix instruction, which takes 512 clocks for the 16
+// columns that nine bf16 ones cover in 288.  k-tiles of 16 columns (a row of a plane is 32
+// bytes, two 16-byte pieces, swapped in every second group of four rows against bank
+// conflicts), so that two LDS buffers of six planes are 48 KB and two workgroups share a CU.
+// A tile's 9 MB NB MFMAs run in two halves: the first with the cut + LDS stores of tile t+1
+// between them, then the barrier, the second with the operand reads of tile t+1 and the
+// request of tile t+3.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int lds_piece_turn2(int row) { return ((row >> 2) ^ (row >> 3)) & 1; }
+
+template <int BM, int BN, int EPI, int SPLIT = 0>
+__global__ __launch_bounds__(256) void k_gemm_b9(GemmArgs a) {
+  constexpr int KT = 16;
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MB = WM / 32, NB = WN / 32;
+  constexpr int ALD = BM / 64, BLD = BN / 64;  // float4 loads per thread and tile (4 lanes per row)
+  __shared__ u4v As[2][3][BM][2];
+  __shared__ u4v Bs[2][3][BN][2];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (a.N + BN - 1) / BN;
+  const int tiles_all = ((a.M + BM - 1) / BM) * tiles_n;
+  int tile;
+  {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int per_xcd = ((int)gridDim.x + 7) >> 3;
+    tile = xcd * per_xcd + slot;
+  }
+  if (tile >= tiles_all) return;
+  int tm, tn;
+  tile_coords(tile, (a.M + BM - 1) / BM, tiles_n, a.band_rows, &tm, &tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int lr = tid >> 2, lk = (tid & 3) * 4;  // four lanes to a row, a float4 each
+  const float* Ag[ALD];
+  const float* Wg[BLD];
+#pragma unroll
+  for (int i = 0; i < ALD; ++i) Ag[i] = a.A + (size_t)min(m0 + lr + 64 * i, a.M - 1) * a.lda + lk;
+#pragma unroll
+  for (int i = 0; i < BLD; ++i) Wg[i] = a.W + (size_t)min(n0 + lr + 64 * i, a.N - 1) * a.K + lk;
+
+  f16v acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int T_all = a.K / KT;
+  const int kt0 = SPLIT ? (int)(((long)blockIdx.y * T_all) / gridDim.y) : 0;
+  const int kt1 = SPLIT ? (int)(((long)(blockIdx.y + 1) * T_all) / gridDim.y) : T_all;
+  const int T = kt1 - kt0;
+  const int half = lane >> 5, l32 = lane & 31;
+  struct Regs {
+    f4 a[ALD], b[BLD];
+  };
+  Regs r0, r1;
+  auto load_tile = [&](int t, Regs& r) __attribute__((always_inline)) {
+    const size_t k = (size_t)(kt0 + t) * KT;
+#pragma unroll
+    for (int i = 0; i < ALD; ++i) r.a[i] = *reinterpret_cast<const f4*>(Ag[i] + k);
+#pragma unroll
+    for (int i = 0; i < BLD; ++i) r.b[i] = *reinterpret_cast<const f4*>(Wg[i] + k);
+  };
+  auto store_tile = [&](int buf, const Regs& r) __attribute__((always_inline)) {
+    const int h8 = (lk >> 2) & 1;
+#pragma unroll
+    for (int i = 0; i < ALD + BLD; ++i) {
+      const int row = lr + 64 * (i < ALD ? i : i - ALD);
+      const int piece = (lk >> 3) ^ lds_piece_turn2(row);
+      const Split3 sp = split3_bf16(i < ALD ? r.a[i] : r.b[i - ALD]);
+      if (i < ALD) {
+        reinterpret_cast<u2v*>(&As[buf][0][row][piece])[h8] = sp.hi;
+        reinterpret_cast<u2v*>(&As[buf][1][row][piece])[h8] = sp.mid;
+        reinterpret_cast<u2v*>(&As[buf][2][row][piece])[h8] = sp.lo;
+      } else {
+        reinterpret_cast<u2v*>(&Bs[buf][0][row][piece])[h8] = sp.hi;
+        reinterpret_cast<u2v*>(&Bs[buf][1][row][piece])[h8] = sp.mid;
+        reinterpret_cast<u2v*>(&Bs[buf][2][row][piece])[h8] = sp.lo;
+      }
+    }
+  };
+  struct Ops {
+    u4v a[3][MB], b[3][NB];
+  };
+  auto read_ops = [&](int buf, Ops& o) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pl = 0; pl < 3; ++pl) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int row = wn * WN + 32 * j + l32;
+        o.b[pl][j] = Bs[buf][pl][row][half ^ lds_piece_turn2(row)];
+      }
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int row = wm * WM + 32 * i + l32;
+        o.a[pl][i] = As[buf][pl][row][half ^ lds_piece_turn2(row)];
+      }
+    }
+  };
+  // MFMAs [g0, g1) of a tile's nine plane pairs (the small terms first), MB NB each
+  auto mfma_ops = [&](const Ops& o, int g0, int g1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int g = g0; g < g1; ++g) {
+      const int pa = 2 - g / 3, pw = 2 - g % 3;
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, o.a[pa][i]),
+                                                             __builtin_bit_cast(bf16x8, o.b[pw][j]),
+                                                             acc[i][j], 0, 0, 0);
+    }
+  };
+  constexpr int G1 = 5;  // plane pairs before the barrier
+  // tile t's operands are in `cur`; `r` holds tile t+1; `nxt` receives tile t+1's operands
+  auto tile_step = [&](auto more_c, int t, const Ops& cur, Ops& nxt, Regs& r) __attribute__((always_inline)) {
+    constexpr bool more = decltype(more_c)::value;
+    mfma_ops(cur, 0, G1);
+    if (more) store_tile((t + 1) & 1, r);
+#pragma unroll
+    for (int g = 0; g < G1 * MB * NB; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // a few VALU
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_ops(cur, G1, 9);
+    if (more) {
+      read_ops((t + 1) & 1, nxt);
+      load_tile(min(t + 3, T - 1), r);  // past the end: the last tile again, never used
+    }
+#pragma unroll
+    for (int g = 0; g < (9 - G1) * MB * NB; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (T > 0) {
+    Ops o0, o1;
+    load_tile(0, r0);
+    load_tile(min(1, T - 1), r1);
+    store_tile(0, r0);
+    __syncthreads();
+    read_ops(0, o0);
+    load_tile(min(2, T - 1), r0);
+    const std::true_type yes;
+    const std::false_type no;
+    int t = 0;
+    for (; t + 2 < T; t += 2) {
+      tile_step(yes, t, o0, o1, r1);
+      tile_step(yes, t + 1, o1, o0, r0);
+    }
+    if (T - t == 2) {
+      tile_step(yes, t, o0, o1, r1);
+      tile_step(no, t + 1, o1, o0, r0);
+    } else {
+      tile_step(no, t, o0, o1, r1);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int n = n0 + wn * WN + 32 * j + l32;
+      if (n >= a.N) continue;
+      if (SPLIT) {
+        float* part = a.ws + (size_t)blockIdx.y * a.M * a.N;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+          if (m < a.M) part[(size_t)m * a.N + n] = acc[i][j][v];
+        }
+        continue;
+      }
+      const float bias = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+        if (m >= a.M) continue;
+        float c = bias + acc[i][j][v];
+        if (EPI == GEMM_GELU) c = gelu_tanh(c);
+        if (EPI == GEMM_RESID) c = a.resid[(size_t)m * a.ldc + n] + c;
+        a.C[(size_t)m * a.ldc + n] = c;
+      }
+    }
+}
+
 // C = epilogue(bias + part[0] + part[1] + ...) for the split-K form of k_gemm; one
 // float4 of a row per thread (N is a multiple of 4 whenever the split is used).
 template <int EPI>
@@ -1501,6 +1700,29 @@ hipError_t launch_gemm_b3(const GemmArgs& a, int epi, int num_cus, hipStream_t s
   const bool wide = a.plan_bn ? a.plan_bn == 256 : a.K >= 4096 && tiles_wide >= 2L * num_cus;
   return wide ? launch_gemm_b3_shape<128, 256>(a, epi, s) : launch_gemm_b3_shape<128, 128>(a, epi, s);
 }
+// f32 rows on the bf16 matrix cores (k_gemm_b9), whole tiles or cut along K into `parts`.
+hipError_t launch_gemm_b9(const GemmArgs& a0, int epi, int parts, hipStream_t s, bool* ln_done) {
+  if (a0.w_bf16 || a0.w_scale || a0.a_packed || a0.c_packed || a0.K % 16 != 0) return hipErrorInvalidValue;
+  GemmArgs a = a0;
+  const int tiles_m = (a.M + 127) / 128, tiles_n = (a.N + 127) / 128;
+  const int tiles = tiles_m * tiles_n;
+  a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band_fwd(tiles_m, std::max(1, (tiles + 7) / 8), 128, 128);
+  const int grid = (tiles + 7) / 8 * 8;
+  if (parts > 1) {
+    if (!a.ws || (size_t)parts * a.M * a.N > a.ws_floats || a.N % 4 != 0 || parts > 8) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((k_gemm_b9<128, 128, GEMM_BIAS, 1>), dim3(grid, parts), dim3(256), 0, s, a);
+    return launch_splitk_reduce_fwd(a, epi, parts, s, ln_done);
+  }
+  if (epi == GEMM_BIAS)
+    hipLaunchKernelGGL((k_gemm_b9<128, 128, GEMM_BIAS>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_GELU)
+    hipLaunchKernelGGL((k_gemm_b9<128, 128, GEMM_GELU>), dim3(grid), dim3(256), 0, s, a);
+  else if (epi == GEMM_RESID)
+    hipLaunchKernelGGL((k_gemm_b9<128, 128, GEMM_RESID>), dim3(grid), dim3(256), 0, s, a);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
 // Whether the planner sends a product there whole: from a quarter of a tile per CU on (below
 // that a tile's own k loop, one workgroup deep, is too long).
 bool gemm_b3_pays(const GemmArgs& a, int num_cus, int min_share = 4) {
@@ -1886,6 +2108,7 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     return launch_tiles<2>(t, epi, bm, bn, form, parts, s, ln_done);
   }
   if (a.plan_form == 5) return launch_gemm_b3(a, epi, num_cus, s);  // forced: the bf16 matrix-core form
+  if (a.plan_form == 7) return launch_gemm_b9(a, epi, std::max(1, a.plan_parts), s, ln_done);  // forced: f32 rows there
   if (a.plan_form == 6) {                                           // forced: the same, cut along K
     const int bp = gemm_b3_split_parts(a, num_cus);
     return bp ? launch_gemm_b3_split(a, epi, bp, s, ln_done) : hipErrorInvalidValue;
@@ -1908,6 +2131,18 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
   GemmArgs t = a;
   // bf16 rows and enough tiles: on the bf16 matrix cores
+  // f32 rows of long inputs (1024 rows and more): on the bf16 matrix cores as nine exact
+  // products per value pair (k_gemm_b9) where that was measured faster than the f32-core
+  // forms: whole 128 x 128 tiles from 0.75 of a tile per CU on (XL c_fc at 1024 rows 199 ->
+  // 176 us, at 4096 rows 818 -> 590 us), tiles cut in four along K between a quarter and
+  // 0.56 of a tile per CU (XL second MLP projection at 1024 rows 213 -> 177 us)
+  if (!form && !a.w_bf16 && !a.w_scale && a.M >= 1024 && a.K % 16 == 0) {
+    const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
+    if (tiles * 4 > 3L * num_cus) return launch_gemm_b9(a, epi, 1, s, ln_done);
+    if (tiles * 4 >= num_cus && tiles * 16 < 9L * num_cus && a.K >= 1024 && a.ws && a.N % 4 == 0 &&
+        (size_t)4 * a.M * a.N <= a.ws_floats)
+      return launch_gemm_b9(a, epi, 4, s, ln_done);
+  }
   // bf16 rows: on the bf16 matrix cores; whole tiles from half a tile per CU on, else cut
   // along K (measured crossover, XL c_attn / c_fc: 128 to 150 tiles), else whole again
   if (!form && gemm_b3_pays(a, num_cus, 2)) return launch_gemm_b3(a, epi, num_cus, s);

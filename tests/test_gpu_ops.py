@@ -46,7 +46,8 @@ def test_dense_matches_oracle(rows, k, n):
                                       (100, 48, 100), (333, 112, 260), (200, 32, 64), (64, 16, 52),
                                       (1024, 3072, 768), (1024, 1600, 4800),
                                       (16, 100, 52), (24, 768, 768), (16, 768, 1000),
-                                      (48, 768, 2304), (33, 1600, 1600), (64, 3072, 768)])
+                                      (48, 768, 2304), (33, 1600, 1600), (64, 3072, 768),
+                                      (1024, 1024, 4096), (1024, 4096, 1024), (1100, 1600, 1600)])
 def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # rows >= 16 and K % 16 == 0 take the MFMA GEMM; tails in M and N are exercised.
     # (64, 6400, 1600), (16, 1024, 3072) and (32, 1600, 6400) cut the whole K range into
@@ -54,7 +55,11 @@ def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     # tiles of 64x64 on 256 CUs and cut only the tiles of the last partial round.
     # K = 48 and 112 are not multiples of 32 and take k-tiles of 16 columns; K = 16 and 32 are a
     # single k-tile (the pipelined loop's shortest cases); (1024, 3072, 768) has a deep K on 192
-    # tiles and is cut in four; (1024, 1600, 4800) runs 128x128 tiles with the last round cut.
+    # tiles and is cut in four.  From 1024 rows on, products with enough 128x128 tiles run on the
+    # bf16 matrix cores with input and weights cut into three bf16 parts each and all nine
+    # products formed (exact): whole tiles for (1024, 1600, 4800) and (1024, 1024, 4096), tiles
+    # cut in four along K for (1024, 4096, 1024) and (1100, 1600, 1600), whose last tile row is
+    # ragged.
     # Up to 32 rows take the MFMA kernel of the decode batch: 16 rows its 16x16x4 form, with 16
     # rows of W per block where 32 would leave CUs idle ((16, 768, 2304), (16, 1024, 3072),
     # (16, 768, 1000) with a ragged last block) and 32 otherwise ((16, 1600, 4800); (16, 4096,
