@@ -440,7 +440,8 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
                    "backend": model.describe()},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
+                     "kernel": "whole prefill (k_gemm, or k_gemm_b9 from 1024 rows on where it is faster; "
+                               "k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
                      "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
     }
     if args.bf16:
