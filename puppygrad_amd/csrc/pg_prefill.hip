@@ -1,5 +1,7 @@
 // Full-sequence (prefill) kernels for gfx950: fp32 MFMA GEMM with LDS staging and
-// causal attention with LDS-staged K/V tiles.
+// causal attention with LDS-staged K/V tiles; the GEMM also on the bf16 matrix cores with the
+// f32 operands cut into three bf16 parts whose products are exact (k_gemm_b3 for bf16 rows,
+// k_gemm_b9 for f32 rows, the bf16 rows of k_gemm_rows32).
 //
 // They cover Gpt2Model::forward / block_forward / causal_self_attention
 // (src/models/gpt2/rust.rs:831-882, 1053-1134, 1580-1659): the same arithmetic as
