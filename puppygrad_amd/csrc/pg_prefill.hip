@@ -391,13 +391,19 @@ __device__ __forceinline__ Split3 split3_bf16(f4 x) {
 
 // SPLIT = 1: the k-tiles are cut into gridDim.y parts, the raw partial tiles go to
 // a.ws[part][M][N] and k_splitk_reduce(_ln) finishes them, as for k_gemm.
-template <int BM, int BN, int EPI, int SPLIT = 0>
+// WT = 2: W holds int8 rows with a.w_scale[n] per row (QuantizedRows, cpu.rs:26-56).  The int8
+// values are bf16 numbers as they are, so the same three products per value are exact; the
+// row's scale multiplies the row's sum at the end (the reference scales every weight,
+// cpu.rs:173-184: the two differ by rounding only).
+template <int BM, int BN, int EPI, int SPLIT = 0, int WT = 1>
 __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
   constexpr int KT = 32;                     // columns per k-tile
   constexpr int WM = BM / 2, WN = BN / 2;    // per-wavefront tile
   constexpr int MB = WM / 32, NB = WN / 32;  // 32x32 blocks per wavefront
   constexpr int ALD = BM / 32;               // float4 loads of A per thread and tile (8 lanes per row)
-  constexpr int BLD = BN / 64;               // 16-byte loads of W per thread and tile (4 lanes per row)
+  // 16-byte loads of W per thread and tile: bf16 rows 4 lanes per row, int8 rows 2
+  constexpr int BLD = WT == 2 ? BN / 128 : BN / 64;
+  static_assert(BLD >= 1, "tile width");
   // [buffer][plane][row][piece]: a row is four 16-byte pieces
   __shared__ u4v As[2][3][BM][4];
   __shared__ u4v Bs[2][BN][4];
@@ -419,14 +425,18 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
 
   // global loads: A eight lanes to a row (a float4 each), W four lanes to a row (8 bf16 each)
   const int ar = tid >> 3, ak = (tid & 7) * 4;
-  const int br = tid >> 2, bp = tid & 3;
+  const int br = WT == 2 ? tid >> 1 : tid >> 2;   // W row of the lane's load (of a pass)
+  const int bp = WT == 2 ? 2 * (tid & 1) : tid & 3;  // its first 16-byte piece of the row in LDS
   const float* Ag[ALD];
-  const unsigned short* Wg[BLD];
+  const char* Wg[BLD];
 #pragma unroll
   for (int i = 0; i < ALD; ++i) Ag[i] = a.A + (size_t)min(m0 + ar + 32 * i, a.M - 1) * a.lda + ak;
 #pragma unroll
-  for (int i = 0; i < BLD; ++i)
-    Wg[i] = reinterpret_cast<const unsigned short*>(a.W) + (size_t)min(n0 + br + 64 * i, a.N - 1) * a.K + bp * 8;
+  for (int i = 0; i < BLD; ++i) {
+    constexpr int RP = WT == 2 ? 128 : 64;  // rows per pass
+    const size_t row = (size_t)min(n0 + br + RP * i, a.N - 1);
+    Wg[i] = reinterpret_cast<const char*>(a.W) + (WT == 2 ? row * a.K + (tid & 1) * 16 : (row * a.K + bp * 8) * 2);
+  }
 
   f16v acc[MB][NB];
 #pragma unroll
@@ -449,7 +459,7 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
 #pragma unroll
     for (int i = 0; i < ALD; ++i) ra[i] = *reinterpret_cast<const f4*>(Ag[i] + k);
 #pragma unroll
-    for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const u4v*>(Wg[i] + k);
+    for (int i = 0; i < BLD; ++i) rb[i] = *reinterpret_cast<const u4v*>(Wg[i] + k * (WT == 2 ? 1 : 2));
   };
   auto store_tile = [&](int buf, f4 (&ra)[ALD], u4v (&rb)[BLD]) __attribute__((always_inline)) {
 #pragma unroll
@@ -464,8 +474,27 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < BLD; ++i) {
-      const int row = br + 64 * i;
-      Bs[buf][row][bp ^ lds_piece_turn(row)] = rb[i];
+      if constexpr (WT == 2) {
+        // sixteen int8 -> sixteen bf16 (exact), two pieces
+        const int row = br + 128 * i;
+        unsigned hb[16];
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            hb[4 * d + b] = __float_as_uint((float)((int)(rb[i][d] << (24 - 8 * b)) >> 24));
+        u4v lo8, hi8;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo8[e] = (hb[2 * e] >> 16) | (hb[2 * e + 1] & 0xffff0000u);
+          hi8[e] = (hb[8 + 2 * e] >> 16) | (hb[8 + 2 * e + 1] & 0xffff0000u);
+        }
+        Bs[buf][row][bp ^ lds_piece_turn(row)] = lo8;
+        Bs[buf][row][(bp + 1) ^ lds_piece_turn(row)] = hi8;
+      } else {
+        const int row = br + 64 * i;
+        Bs[buf][row][bp ^ lds_piece_turn(row)] = rb[i];
+      }
     }
   };
   // the operands of one 16-column step of a tile: three planes of MB row blocks, NB column blocks
@@ -565,12 +594,13 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
     for (int j = 0; j < NB; ++j) {
       const int n = n0 + wn * WN + 32 * j + l32;
       if (n >= a.N) continue;
+      const float wscale = WT == 2 ? a.w_scale[n] : 1.0f;
       if (SPLIT) {
         float* part = a.ws + (size_t)blockIdx.y * a.M * a.N;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
-          if (m < a.M) part[(size_t)m * a.N + n] = acc[i][j][v];
+          if (m < a.M) part[(size_t)m * a.N + n] = WT == 2 ? wscale * acc[i][j][v] : acc[i][j][v];
         }
         continue;
       }
@@ -579,7 +609,7 @@ __global__ __launch_bounds__(256) void k_gemm_b3(GemmArgs a) {
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + wm * WM + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
         if (m >= a.M) continue;
-        float c = bias + acc[i][j][v];
+        float c = bias + (WT == 2 ? wscale * acc[i][j][v] : acc[i][j][v]);
         if (EPI == GEMM_GELU) c = gelu_tanh(c);
         if (EPI == GEMM_RESID) c = a.resid[(size_t)m * a.ldc + n] + c;
         a.C[(size_t)m * a.ldc + n] = c;
@@ -1673,11 +1703,11 @@ hipError_t launch_gemm_tile(const GemmArgs& a, int epi, hipStream_t s) {
   return hipGetLastError();
 }
 
-// The bf16 matrix-core form (k_gemm_b3): W stored as bf16, whole 128 x 128 tiles.
+// The bf16 matrix-core form (k_gemm_b3): W stored as bf16 or as int8 rows.
 bool gemm_b3_ok(const GemmArgs& a) {
-  return a.w_bf16 && !a.w_scale && a.K % 32 == 0 && a.K >= 32 && !a.a_packed && !a.c_packed;
+  return (a.w_bf16 != 0) != (a.w_scale != nullptr) && a.K % 32 == 0 && a.K >= 32 && !a.a_packed && !a.c_packed;
 }
-template <int BM, int BN>
+template <int BM, int BN, int WT>
 hipError_t launch_gemm_b3_shape(const GemmArgs& a0, int epi, hipStream_t s) {
   GemmArgs a = a0;
   const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
@@ -1685,22 +1715,24 @@ hipError_t launch_gemm_b3_shape(const GemmArgs& a0, int epi, hipStream_t s) {
   a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band_fwd(tiles_m, std::max(1, (tiles + 7) / 8), BM, BN);
   const int grid = (tiles + 7) / 8 * 8;
   if (epi == GEMM_BIAS)
-    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_BIAS>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_BIAS, 0, WT>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_GELU)
-    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_GELU>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_GELU, 0, WT>), dim3(grid), dim3(256), 0, s, a);
   else if (epi == GEMM_RESID)
-    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_RESID>), dim3(grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_gemm_b3<BM, BN, GEMM_RESID, 0, WT>), dim3(grid), dim3(256), 0, s, a);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
 }
-// 128 x 128 tiles (two workgroups to a CU); 128 x 256 for a long K where those still fill the
-// chip twice over (measured: 4096 x 1600 x 6400, 275 against 302 us); a.plan_bn forces one.
+// 128 x 128 tiles (two workgroups to a CU); for bf16 rows 128 x 256 for a long K where those
+// still fill the chip twice over (measured: 4096 x 1600 x 6400, 275 against 302 us);
+// a.plan_bn forces one.
 hipError_t launch_gemm_b3(const GemmArgs& a, int epi, int num_cus, hipStream_t s) {
   if (!gemm_b3_ok(a)) return hipErrorInvalidValue;
+  if (a.w_scale) return launch_gemm_b3_shape<128, 128, 2>(a, epi, s);
   const long tiles_wide = (long)((a.M + 127) / 128) * ((a.N + 255) / 256);
   const bool wide = a.plan_bn ? a.plan_bn == 256 : a.K >= 4096 && tiles_wide >= 2L * num_cus;
-  return wide ? launch_gemm_b3_shape<128, 256>(a, epi, s) : launch_gemm_b3_shape<128, 128>(a, epi, s);
+  return wide ? launch_gemm_b3_shape<128, 256, 1>(a, epi, s) : launch_gemm_b3_shape<128, 128, 1>(a, epi, s);
 }
 // f32 rows on the bf16 matrix cores (k_gemm_b9), whole tiles or cut along K into `parts`.
 hipError_t launch_gemm_b9(const GemmArgs& a0, int epi, int parts, hipStream_t s, bool* ln_done) {
@@ -1748,7 +1780,10 @@ hipError_t launch_gemm_b3_split(const GemmArgs& a0, int epi, int parts, hipStrea
   const int tiles_m = (a.M + 127) / 128, tiles_n = (a.N + 127) / 128;
   const int tiles = tiles_m * tiles_n;
   a.band_rows = a.plan_band ? std::min(a.plan_band, tiles_m) : choose_band_fwd(tiles_m, std::max(1, (tiles + 7) / 8), 128, 128);
-  hipLaunchKernelGGL((k_gemm_b3<128, 128, GEMM_BIAS, 1>), dim3((tiles + 7) / 8 * 8, parts), dim3(256), 0, s, a);
+  if (a.w_scale)
+    hipLaunchKernelGGL((k_gemm_b3<128, 128, GEMM_BIAS, 1, 2>), dim3((tiles + 7) / 8 * 8, parts), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL((k_gemm_b3<128, 128, GEMM_BIAS, 1, 1>), dim3((tiles + 7) / 8 * 8, parts), dim3(256), 0, s, a);
   return launch_splitk_reduce_fwd(a, epi, parts, s, ln_done);
 }
 
@@ -2104,6 +2139,16 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
       return launch_gemm_rows32<2>(a, epi, rp, num_cus, s, ln_done);
     int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
+    if (form == 5) return launch_gemm_b3(a, epi, num_cus, s);
+    if (form == 6) {
+      const int bp = gemm_b3_split_parts(a, num_cus);
+      return bp ? launch_gemm_b3_split(a, epi, bp, s, ln_done) : hipErrorInvalidValue;
+    }
+    // on the bf16 matrix cores (int8 values are bf16 numbers), in the order of the bf16 rows
+    if (!form && gemm_b3_pays(a, num_cus, 2)) return launch_gemm_b3(a, epi, num_cus, s);
+    if (!form)
+      if (const int bp = gemm_b3_split_parts(a, num_cus)) return launch_gemm_b3_split(a, epi, bp, s, ln_done);
+    if (!form && gemm_b3_pays(a, num_cus, 4)) return launch_gemm_b3(a, epi, num_cus, s);
     GemmArgs t = a;
     if (!form) plan_tiles(t, num_cus, &bm, &bn, &form, &parts);
     else if (form == 3 && !gemm_tail_plan(t, num_cus, bm, bn)) return hipErrorInvalidValue;

@@ -47,6 +47,27 @@ def test_int8_storage_matches_the_quantised_oracle(case):
     assert np.abs(model.forward(ids).logits - oracle.Model(cfg, w).forward(ids)).max() > 1e-4
 
 
+@pytest.mark.parametrize("n_embd,n_head,n_prompt", [(832, 13, 400), (768, 12, 512), (1024, 16, 100),
+                                                    (1024, 16, 512)])
+def test_int8_long_prompts_on_the_bf16_matrix_cores(n_embd, n_head, n_prompt):
+    """Prompts of more than 64 tokens whose projections have a dozen 128 x 128 tiles or more run
+    on the bf16 matrix cores (int8 values are bf16 numbers; the inputs are cut into three bf16
+    parts; the row's scale multiplies the row's sum): tiles cut along K, whole tiles for c_fc of
+    the last case (128 tiles), a ragged last row tile and widths that are no multiple of the
+    tile, against the quantised oracle at the f32 tolerance."""
+    cfg = Gpt2Config(vocab_size=300, n_positions=512, n_embd=n_embd, n_layer=1, n_head=n_head)
+    w = synth.random_weights(cfg, 0x5EED0620 + n_head, perturb=True)
+    ids = synth.token_ids(n_prompt, 0x70C00620, cfg.vocab_size)
+    model, ref = Gpt2Model.new(cfg, w, INT8), qref(cfg, w, threads=8)
+    cache, rc = model.new_kv_cache(), ref.new_kv_cache()
+    want = ref.prefill(ids, rc)
+    assert_logits_close(model.prefill(ids, cache).to_host(), want)
+    assert_logits_close(model.forward(ids).logits, ref.forward(ids))
+    if n_prompt < cfg.n_positions:
+        tok = int(np.argmax(want))
+        assert_logits_close(model.forward_one(tok, cache).to_host(), ref.forward_one(tok, rc))
+
+
 def test_int8_extreme_rows():
     """A zero row (scale 1), a row with one huge entry and rows of tiny values keep the
     quantiser's edge cases on the device equal to the oracle's."""
