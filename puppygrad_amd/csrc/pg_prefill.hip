@@ -1116,13 +1116,15 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 
   // bias and residual of the outputs this thread writes at the end: requested now, so that
   // the write-out does not wait for them (K not cut over blocks)
-  float ebias[2 * MT], eres[2 * MT];
+  float ebias[2 * MT], eres[2 * MT], escale[2 * MT];
 #pragma unroll
   for (int qq = 0; qq < 2 * MT; ++qq) {
     const int idx = tid + 512 * qq, b = idx / NR, n = n0 + idx % NR;
     const bool live = gridDim.y == 1 && idx < 32 * MT * NR && b < a.M && n < n1;
     ebias[qq] = live && a.bias ? a.bias[n] : 0.0f;
     eres[qq] = live && EPI == GEMM_RESID ? a.resid[(size_t)b * a.ldc + n] : 0.0f;
+    // int8 rows: the row's scale multiplies the row's sum (also a partial sum of a cut K)
+    escale[qq] = WT == 2 && idx < 32 * MT * NR && b < a.M && n < n1 ? a.w_scale[n] : 1.0f;
   }
 
   f16v acc[MT];   // 32-row form
@@ -1141,30 +1143,9 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < XR; ++j) x[j] = *reinterpret_cast<const f4*>(xp[j] + sc * xstep);
   };
-  // int8 rows: the scale of the W row(s) whose operand this lane holds
-  float wsc[2] = {1.0f, 1.0f};
-  if (WT == 2) {
-    wsc[0] = a.w_scale[min(n0 + orow, n1 - 1)];
-    wsc[1] = a.w_scale[min(n0 + 16 + orow, n1 - 1)];
-  }
-  // a 16-byte piece of a W row -> its CPP columns as floats
-  auto widen = [](const f4& v, float* wv, float scale) {
-    const unsigned* p = reinterpret_cast<const unsigned*>(&v);
-    if (WT == 0) {
-      wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
-    } else if (WT == 1) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        wv[2 * c] = __uint_as_float(p[c] << 16);
-        wv[2 * c + 1] = __uint_as_float(p[c] & 0xffff0000u);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < 4; ++c)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          wv[4 * c + b] = (float)((int)(p[c] << (24 - 8 * b)) >> 24) * scale;
-    }
+  // (f32 rows only) a 16-byte piece of a W row -> its four columns as floats
+  auto widen = [](const f4& v, float* wv) {
+    wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
   };
   auto mul_step = [&](const f4* w, const f4* x) {
     *reinterpret_cast<f4*>(wt + q * WSTR + 4 * t) = w[0];
@@ -1197,37 +1178,64 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       }
     }
     __builtin_amdgcn_wave_barrier();
-    if constexpr (WT == 1) {
-      // bf16 rows: on the bf16 matrix cores.  A piece of a W row is the operand as it is (8
-      // consecutive columns); the 8 input values that meet it are cut into three bf16 parts
-      // whose sum is the value exactly (split3_bf16), so the three products are exact and the
-      // sums f32 as in the other forms.
+    if constexpr (WT != 0) {
+      // bf16 and int8 rows: on the bf16 matrix cores.  A piece of a bf16 W row is the operand
+      // as it is (8 consecutive columns); a piece of an int8 row is 16 columns, converted to
+      // two operands (an int8 value is a bf16 number).  The 8 input values that meet an
+      // operand are cut into three bf16 parts whose sum is the value exactly (split3_bf16), so
+      // the three products are exact and the sums f32 as in the other forms; an int8 row's
+      // scale multiplies its sum at the end.
       auto cut8 = [](const f4& lo4, const f4& hi4, u4v (&part)[3]) {
         const Split3 s0 = split3_bf16(lo4), s1 = split3_bf16(hi4);
         part[0] = u4v{s0.hi.x, s0.hi.y, s1.hi.x, s1.hi.y};
         part[1] = u4v{s0.mid.x, s0.mid.y, s1.mid.x, s1.mid.y};
         part[2] = u4v{s0.lo.x, s0.lo.y, s1.lo.x, s1.lo.y};
       };
+      // operand h (8 columns) of a piece of W
+      auto w_operand = [](const f4& piece, int h) -> u4v {
+        const u4v raw = __builtin_bit_cast(u4v, piece);
+        if (WT == 1) return raw;
+        u4v r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // columns 8 h + 2 e and + 1: bytes 2 (e % 2), 2 (e % 2) + 1 of word 2 h + e / 2
+          const unsigned w = raw[2 * h + e / 2];
+          const unsigned lo = __float_as_uint((float)((int)(w << (24 - 16 * (e % 2))) >> 24));
+          const unsigned hi = __float_as_uint((float)((int)(w << (16 - 16 * (e % 2))) >> 24));
+          r[e] = (lo >> 16) | (hi & 0xffff0000u);
+        }
+        return r;
+      };
+      constexpr int OPS = CPP / 8;  // operands per piece: 1 (bf16), 2 (int8)
       if (M16) {
-        u4v xp3[3];
-        cut8(xo[0], xo[1], xp3);
 #pragma unroll
-        for (int g = 0; g < NR / 16; ++g)
+        for (int h = 0; h < OPS; ++h) {
+          u4v xp3[3];
+          cut8(xo[2 * h], xo[2 * h + 1], xp3);
 #pragma unroll
-          for (int pl = 2; pl >= 0; --pl)
-            acc16[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
-                                                              __builtin_bit_cast(bf16x8, wo[g]), acc16[g], 0, 0, 0);
+          for (int g = 0; g < NR / 16; ++g) {
+            const u4v wop = w_operand(wo[g], h);
+#pragma unroll
+            for (int pl = 2; pl >= 0; --pl)
+              acc16[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
+                                                                __builtin_bit_cast(bf16x8, wop), acc16[g], 0, 0, 0);
+          }
+        }
       } else {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            u4v xp3[3];
-            cut8(xo[mt * XT + u * XF], xo[mt * XT + u * XF + 1], xp3);
+          for (int h = 0; h < OPS; ++h) {
+            const u4v wop = w_operand(wo[u], h);
 #pragma unroll
-            for (int pl = 2; pl >= 0; --pl)
-              acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
-                                                                __builtin_bit_cast(bf16x8, wo[u]), acc[mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) {
+              u4v xp3[3];
+              cut8(xo[mt * XT + u * XF + 2 * h], xo[mt * XT + u * XF + 2 * h + 1], xp3);
+#pragma unroll
+              for (int pl = 2; pl >= 0; --pl)
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xp3[pl]),
+                                                                  __builtin_bit_cast(bf16x8, wop), acc[mt], 0, 0, 0);
+            }
           }
       }
     } else {
@@ -1235,7 +1243,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       if (M16) {
 #pragma unroll
         for (int g = 0; g < NR / 16; ++g) {
-          widen(wo[g], wv, wsc[g]);
+          widen(wo[g], wv);
 #pragma unroll
           for (int c = 0; c < CPP; ++c)
             acc16[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[c / 4][c % 4], wv[c], acc16[g], 0, 0, 0);
@@ -1243,7 +1251,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
       } else {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          widen(wo[u], wv, wsc[0]);
+          widen(wo[u], wv);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1299,6 +1307,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
     float sum = red_at(0, b, nl);
 #pragma unroll
     for (int w = 1; w < 8; ++w) sum += red_at(w, b, nl);
+    if (WT == 2) sum *= escale[q];
     if (gridDim.y > 1) {
       a.ws[((size_t)blockIdx.y * a.M + b) * a.N + n] = sum;
       continue;
@@ -1766,6 +1775,8 @@ bool gemm_b3_pays(const GemmArgs& a, int num_cus, int min_share = 4) {
 // parts so that about two items per CU exist, each at least four k-tiles long; 0 where that
 // does not apply (no workspace, N no multiple of 4, K too short, hardly any tiles).
 int gemm_b3_split_parts(const GemmArgs& a, int num_cus) {
+  // (int8 rows of 33..64 inputs were measured too: XL, 48 tokens, 4.7 ms on the f32-core tiles,
+  // 6.0 ms here)
   if (!gemm_b3_ok(a) || !a.ws || a.N % 4 != 0 || a.M <= 64) return 0;
   const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
   if (!a.plan_parts && tiles < 12) return 0;  // (a dozen short items: the f32 forms' 64 x 64 tiles do better)
