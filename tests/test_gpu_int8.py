@@ -1,7 +1,8 @@
 """int8 weight storage (the reference's `quantized_weights` option): the library quantises
 the block matrices and the lm_head copy of wte on the device and multiplies with
-(float)q * scale; the oracle's quantised path (pinned in test_oracle_int8.py) is the
-reference.  Both sides use identical dequantised values, so the f32 tolerance applies."""
+(float)q * scale (the matrix-vector kernels per weight, the matrix-core kernels per row sum);
+the oracle's quantised path (pinned in test_oracle_int8.py) is the reference.  Both sides use
+identical quantised values and scales, so the f32 tolerance applies."""
 import numpy as np
 import pytest
 
