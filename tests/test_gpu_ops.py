@@ -77,6 +77,24 @@ def test_dense_many_rows_uses_mfma_gemm(rows, k, n):
     np.testing.assert_allclose(got, want, atol=3e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("rows,k,n", [(1024, 1024, 4096), (1024, 1600, 1600), (96, 768, 768)])
+def test_dense_with_selection_weights_returns_the_inputs_bit_for_bit(rows, k, n):
+    """W[o, :] is a unit vector, so out[r, o] must be exactly x[r, o % k] whatever the
+    summation order: every other product is 0.  For the first two shapes the product runs on
+    the bf16 matrix cores with x and W cut into three bf16 parts each (whole tiles; tiles cut
+    in four along K): the parts of a value must add up to the value in all its 24 bits, at any
+    exponent.  (96 rows: the f32 matrix cores, for comparison.)"""
+    rng = np.random.default_rng(rows + n)
+    x = (rng.standard_normal(rows * k) * 10.0 ** rng.uniform(-6, 6, rows * k)).astype(np.float32)
+    x[::97] = np.float32(1.0) + np.float32(2.0) ** -23  # all-but-one low bits clear
+    x[1::97] = np.nextafter(np.float32(2.0), np.float32(0.0))  # 24 ones
+    w = np.zeros((n, k), np.float32)
+    w[np.arange(n), np.arange(n) % k] = 1.0
+    got = hip_dense(x, rows, k, n, w.reshape(-1), np.zeros(n, np.float32)).reshape(rows, n)
+    want = x.reshape(rows, k)[:, np.arange(n) % k]
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_dense_reference_unit_vector():
     # src/models/cpu.rs:312-327
     x, weight = patterned(6, 0.2), patterned(12, 0.1)
