@@ -2067,6 +2067,7 @@ hipError_t launch_splitk_reduce_fwd(const GemmArgs& a, int epi, int parts, hipSt
 template <int WBF>
 hipError_t launch_tiles(const GemmArgs& a0, int epi, int bm, int bn, int form, int parts, hipStream_t s,
                         bool* ln_done) {
+  if (bm <= 0 || bn <= 0) return hipErrorInvalidValue;  // (a forced plan without a tile shape)
   GemmArgs a = a0;
   {
     const int tiles_m = (a.M + bm - 1) / bm, tiles_n = (a.N + bn - 1) / bn;
@@ -2150,6 +2151,10 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
     if (const int rp = a.plan_form ? 0 : gemm_rows32_parts(a, num_cus))
       return launch_gemm_rows32<2>(a, epi, rp, num_cus, s, ln_done);
     int bm = a.plan_bm, bn = a.plan_bn, form = a.plan_form, parts = a.plan_parts;
+    if (form == 4) {  // forced: the 32-row kernel
+      const int rp = gemm_rows32_parts(a, num_cus);
+      return rp ? launch_gemm_rows32<2>(a, epi, rp, num_cus, s, ln_done) : hipErrorInvalidValue;
+    }
     if (form == 5) return launch_gemm_b3(a, epi, num_cus, s);
     if (form == 6) {
       const int bp = gemm_b3_split_parts(a, num_cus);
