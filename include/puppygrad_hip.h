@@ -346,8 +346,10 @@ pg_status pg_op_quantize_rows_dev(int32_t device, void* stream, const float* val
                                   uint64_t cols, int8_t* q, float* scales);
 /* quantized_transposed_dense_projection_into (cpu.rs:99-117): out[r][o] = bias[o] +
  * quantized_dot(x row r, weight row o) with every weight used as (float)q * scale
- * (cpu.rs:173-184).  bias may be NULL (the reference's Whisper model takes its logits as bare
- * quantized_dot values, src/models/whisper/model.rs:1528, 1547). */
+ * (cpu.rs:173-184; with two rows or more and in_features a multiple of 64 the matrix-core
+ * kernels multiply the row's sum by its scale instead: the same value up to rounding).  bias
+ * may be NULL (the reference's Whisper model takes its logits as bare quantized_dot values,
+ * src/models/whisper/model.rs:1528, 1547). */
 pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
                                     uint64_t in_features, uint64_t out_features, const int8_t* q,
                                     const float* scales, const float* bias, float* out);

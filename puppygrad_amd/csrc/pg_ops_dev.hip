@@ -314,6 +314,17 @@ pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x
   pg_status s;
   if ((s = select_device(device))) return s;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  pgk::GemmArgs ga{};
+  ga.A = x; ga.W = reinterpret_cast<const float*>(q); ga.w_scale = scales; ga.bias = bias;
+  ga.resid = nullptr; ga.C = out;
+  ga.M = (int)rows; ga.N = (int)out_f; ga.K = (int)in_f; ga.lda = (int)in_f; ga.ldc = (int)out_f;
+  if (rows >= 2 && in_f % 64 == 0 && pgk::gemm_supported(ga)) {
+    // several rows: the matrix-core kernels (rows of 64-byte pieces; no workspace: never cut along K)
+    int cus = 0;
+    PG_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    PG_HIP(pgk::launch_gemm(ga, pgk::GEMM_BIAS, cus, st));
+    return PG_OK;
+  }
   // one matrix-vector launch per input row (the reference's callers have one: the last hidden
   // state against the token embedding)
   for (uint64_t r = 0; r < rows; ++r) {

@@ -73,11 +73,15 @@ def test_dense_on_device_over_the_small_batch_forms(rows):
 
 
 @pytest.mark.parametrize("rows,in_f,out_f", [(1, 384, 51865), (2, 100, 37), (1, 16, 8), (3, 1280, 1000),
-                                             (1, 7, 5)])
+                                             (1, 7, 5), (12, 384, 1536), (40, 768, 2304), (150, 1280, 5120),
+                                             (300, 1024, 8200)])
 def test_quantized_rows_and_quantized_dense_match_oracle(rows, in_f, out_f):
     """QuantizedRows::from_f32 bit for bit (incl. an all-zero row and a row whose largest value is
     negative), then the quantised projection against quantized_dot (cpu.rs:99-117, 173-184), with
-    a bias and without one (the Whisper logits, model.rs:1528)."""
+    a bias and without one (the Whisper logits, model.rs:1528).  Several rows with a row length
+    that is a multiple of 64 take the matrix-core kernels: 3 and 12 rows the 32-row kernel's two
+    forms, 40 rows the f32-core tiles, 150 and 300 rows the bf16-core tiles (whole 128 x 128
+    tiles; a ragged last tile row and column)."""
     rng = np.random.default_rng(in_f * 7 + out_f)
     w = (rng.standard_normal((out_f, in_f)) / np.sqrt(in_f)).astype(np.float32)
     w[0] = 0.0
