@@ -4,9 +4,13 @@
 // one or many greedy tokens.
 //
 // 256 workgroups of 8 wavefronts, one workgroup per CU, never a grid barrier.  Every
-// activation that crosses workgroups is a 64-bit word {epoch, f32 bits} written with
-// one agent-scope store; a reader polls until the word carries the epoch of the
-// producing (token, layer, phase).
+// activation that crosses workgroups is one f32 word in uncached memory written with one
+// agent-scope store; a word that has not been written yet holds the bit pattern kArm (a NaN
+// no arithmetic here produces; a producer that would store exactly it stores the next
+// pattern), and a reader polls until none of the words it needs is armed.  Each exchanged
+// vector has two buffers used by alternate layer steps; a buffer is armed again, by all
+// workgroups in equal shares, one step after it was read (see "re-arming" in service_wave).
+// Only the per-workgroup argmax candidates still travel as 64-bit words {epoch, value}.
 //
 // Vector memory instructions of a CU complete in issue order, across all of its
 // wavefronts: a poll of global memory sees its answer only after every weight byte the CU
@@ -26,14 +30,14 @@
 //     an attention item do that where there are enough of them), the embedding and the
 //     argmax merge.
 //
-// Per layer:  A  LN1 + c_attn rows            -> qkv_t   (tagged)
-//             B  split-key attention per head -> part_t  (tagged partial acc, m, l)
-//             B2 per-head merge of the splits -> attn_t  (tagged; B writes it directly
-//                                                         when one split holds all keys)
-//             D  c_proj rows + residual       -> xa_t    (tagged)
-//             E  LN2 + c_fc rows + GELU       -> h_t     (tagged)
-//             F  mlp c_proj rows + residual   -> xm_t    (tagged)
-// then LN_f + lm_head rows -> logits (plain) and per-workgroup argmax -> best_t.
+// Per layer:  A  LN1 + c_attn rows            -> qkv_x
+//             B  split-key attention per head -> part_x  (partial acc, m, l)
+//             B2 per-head merge of the splits -> attn_x  (B writes it directly when one
+//                                                         split holds all keys)
+//             D  c_proj rows + residual       -> xa_x
+//             E  LN2 + c_fc rows + GELU       -> h_x
+//             F  mlp c_proj rows + residual   -> xm_x
+// then LN_f + lm_head rows -> logits (plain) and per-workgroup argmax -> best_t (tagged).
 //
 // The weight rows are f32, or int8 with one f32 scale per row (QuantizedRows,
 // src/models/cpu.rs:26-56; template parameter WB): either way a row is a stream of 16-byte
@@ -48,6 +52,7 @@
 
 #include <math.h>
 
+#include <algorithm>
 #include <type_traits>
 
 namespace pgk {
@@ -85,6 +90,24 @@ constexpr bool early_kv(int C) { return C <= 1024; }
 #define PG_LD32(p) __hip_atomic_load(PG_G32(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define PG_ST32(p, v) __hip_atomic_store(PG_G32(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
+// The "not written yet" pattern of an exchanged f32 word, and the bits a producer stores for v.
+constexpr unsigned kArm = 0xFFFFFFFFu;
+// Where the exchanged vectors lie from DecodeParams::xch on, in words (C = n_embd).  There are
+// two sets (`par` picks one; `set` = DecodeParams::xch_set words apart, a multiple of 16), each
+// qkv 3C | attn C | xa C | h 4C | xm C | part (H * ns * 66): one contiguous run of whole 64-byte
+// lines, so that a set is armed with full-line stores.
+struct XchLayout {
+  static constexpr unsigned qkv(unsigned C) { return 0u; }
+  static constexpr unsigned attn(unsigned C) { return 3u * C; }
+  static constexpr unsigned xa(unsigned C) { return 4u * C; }
+  static constexpr unsigned h(unsigned C) { return 5u * C; }
+  static constexpr unsigned xm(unsigned C) { return 9u * C; }
+  static constexpr unsigned part(unsigned C) { return 10u * C; }
+};
+__device__ __forceinline__ unsigned xbits(float v) {
+  const unsigned u = __float_as_uint(v);
+  return u == kArm ? 0xFFFFFFFEu : u;  // (both are NaNs)
+}
 __device__ __forceinline__ u64 pack(unsigned epoch, float v) {
   return ((u64)epoch << 32) | (u64)__float_as_uint(v);
 }
@@ -473,13 +496,23 @@ __device__ __forceinline__ int splits_at(const DecodeParams& p, int pos) {
   return min((pos + p.item_keys) / p.item_keys, p.ns);
 }
 
-// ---- service side: poll tagged words ---------------------------------------------------
-// One tagged word at a wave-uniform base plus a 32-bit byte offset ("scalar base +
-// vector offset" addressing: no 64-bit per-lane addresses are kept across the retries).
-__device__ __forceinline__ u64 ld_tagged(const u64* base, unsigned byte_off) {
+// ---- service side: poll exchanged words -------------------------------------------------
+// One 64-bit word (a tagged word, or a pair of f32 words) at a wave-uniform base plus a
+// 32-bit byte offset ("scalar base + vector offset" addressing: no 64-bit per-lane addresses
+// are kept across the retries).
+__device__ __forceinline__ u64 ld_tagged(const void* base, unsigned byte_off) {
   typedef char __attribute__((address_space(1)))* gcp;
   return __hip_atomic_load((__attribute__((address_space(1))) u64*)((gcp)base + byte_off),
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// One f32 word of an exchanged vector, as its bits.
+__device__ __forceinline__ unsigned ld_word(const unsigned* base, unsigned byte_off) {
+  typedef char __attribute__((address_space(1)))* gcp;
+  return __hip_atomic_load((__attribute__((address_space(1))) unsigned*)((gcp)base + byte_off),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool pair_armed(u64 v) {
+  return (unsigned)v == kArm || (unsigned)(v >> 32) == kArm;
 }
 // ---- probes through the scalar data path ------------------------------------------------
 // Vector loads of a CU return in the order they were issued, whichever wavefront issued
@@ -494,9 +527,8 @@ __device__ __forceinline__ u64 ld_tagged(const u64* base, unsigned byte_off) {
 typedef unsigned u16x __attribute__((ext_vector_type(16)));
 constexpr unsigned kProbeSpinLimit = 1u << 24;  // a few seconds of scalar probes
 constexpr int kProbeSleep = 4;  // units of 64 clocks between two probes of a wavefront
-// Three lines of eight tagged words each: zero iff all 24 carry `epoch`.
-__device__ __forceinline__ unsigned lines3_diff(const u64* a, const u64* b, const u64* c, unsigned epoch) {
-  u16x va, vb, vc;
+__device__ __forceinline__ void lines3_load(const void* a, const void* b, const void* c, u16x& va,
+                                            u16x& vb, u16x& vc) {
   asm volatile(
       "s_load_dwordx16 %0, %3, 0x0 glc\n\t"
       "s_load_dwordx16 %1, %4, 0x0 glc\n\t"
@@ -505,21 +537,44 @@ __device__ __forceinline__ unsigned lines3_diff(const u64* a, const u64* b, cons
       : "=&s"(va), "=&s"(vb), "=&s"(vc)
       : "s"(a), "s"(b), "s"(c)
       : "memory");
+}
+// Three 64-byte lines of eight tagged words each: zero iff all 24 carry `epoch`.
+__device__ __forceinline__ unsigned lines3_diff(const u64* a, const u64* b, const u64* c, unsigned epoch) {
+  u16x va, vb, vc;
+  lines3_load(a, b, c, va, vb, vc);
   unsigned d = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) d |= (va[2 * i + 1] ^ epoch) | (vb[2 * i + 1] ^ epoch) | (vc[2 * i + 1] ^ epoch);
   return d;
 }
-// Spins until lines la, lb, lc (of eight words each) of src carry `epoch`.  Wave-uniform;
-// false on timeout or abort.
-__device__ __forceinline__ bool probe_lines(const u64* src, int la, int lb, int lc, unsigned epoch,
-                                            unsigned* abort_word) {
-  const u64* a = src + 8 * __builtin_amdgcn_readfirstlane(la);
-  const u64* b = src + 8 * __builtin_amdgcn_readfirstlane(lb);
-  const u64* c = src + 8 * __builtin_amdgcn_readfirstlane(lc);
+// Three 64-byte lines of sixteen f32 words each: zero iff one of the 48 is still armed
+// (~w is zero exactly for the armed pattern).
+__device__ __forceinline__ unsigned lines3_written(const unsigned* a, const unsigned* b, const unsigned* c) {
+  u16x va, vb, vc;
+  lines3_load(a, b, c, va, vb, vc);
+  unsigned m = 0xffffffffu;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) m = min(m, min(~va[i], min(~vb[i], ~vc[i])));
+  return m;
+}
+// Spins until lines la, lb, lc (64 bytes each) of src are written: all their tagged words
+// carry `epoch` (TAGGED), or none of their f32 words is armed.  Wave-uniform; false on
+// timeout or abort.
+template <bool TAGGED>
+__device__ __forceinline__ bool probe_lines(const void* src, int la, int lb, int lc, unsigned epoch,
+                                            unsigned* abort_word, lu64p dbg = nullptr) {
+  const char* base = (const char*)src;
+  const char* a = base + 64 * __builtin_amdgcn_readfirstlane(la);
+  const char* b = base + 64 * __builtin_amdgcn_readfirstlane(lb);
+  const char* c = base + 64 * __builtin_amdgcn_readfirstlane(lc);
   unsigned spins = 0;
   for (;;) {
-    if (lines3_diff(a, b, c, epoch) == 0) return true;
+    if (dbg && (threadIdx.x & 63) == 0) dbg[1] = __builtin_amdgcn_s_memtime();  // development stamp
+    if (TAGGED) {
+      if (lines3_diff((const u64*)a, (const u64*)b, (const u64*)c, epoch) == 0) return true;
+    } else {
+      if (lines3_written((const unsigned*)a, (const unsigned*)b, (const unsigned*)c) != 0) return true;
+    }
     if (++spins > kProbeSpinLimit) {
       PG_ST32(abort_word, 1u);
       return false;
@@ -530,26 +585,27 @@ __device__ __forceinline__ bool probe_lines(const u64* src, int la, int lb, int 
 }
 // The same over a vector of LINES lines: the line `first` and two more a third of the
 // vector apart (different rows of a vector come from different workgroups).
-template <int LINES>
-__device__ __forceinline__ bool probe_spread(const u64* src, int first, unsigned epoch, unsigned* abort_word) {
+template <int LINES, bool TAGGED>
+__device__ __forceinline__ bool probe_spread(const void* src, int first, unsigned epoch, unsigned* abort_word,
+                                             lu64p dbg = nullptr) {
   const int l0 = first % LINES;
-  return probe_lines(src, l0, (l0 + LINES / 3) % LINES, (l0 + 2 * (LINES / 3)) % LINES, epoch, abort_word);
+  return probe_lines<TAGGED>(src, l0, (l0 + LINES / 3) % LINES, (l0 + 2 * (LINES / 3)) % LINES, epoch,
+                             abort_word, dbg);
 }
 
-// Waits until src[i] carries `epoch` for every i in [0, 64 NE) and leaves the payloads
-// in dst (LDS): scalar probes of three lines (they differ per workgroup), then a bulk read
-// of lane + 64 e; while that finds stale words, the probe moves to a stale word's line
+// Waits until the tagged words src[i] carry `epoch` for every i in [0, 64 NE) and leaves the
+// payloads in dst (LDS): scalar probes of three lines (they differ per workgroup), then a bulk
+// read of lane + 64 e; while that finds stale words, the probe moves to a stale word's line
 // and the bulk read repeats.  Nothing but the probe line lives across a repeat: the
 // payloads go to LDS at once.
 template <int NE>
-__device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp dst,
-                                          unsigned* abort_word, int probe, lu64p dbg = nullptr) {
+__device__ __forceinline__ bool wave_poll_tagged(const u64* src, unsigned epoch, lfp dst,
+                                                 unsigned* abort_word, int probe) {
   const int lane = opaque((int)threadIdx.x) & 63;
   unsigned rounds = 0;
   int line = probe * 3;
   for (;;) {
-    if (!probe_spread<8 * NE>(src, line, epoch, abort_word)) return false;
-    if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
+    if (!probe_spread<8 * NE, true>(src, line, epoch, abort_word)) return false;
     bool bad = false;
     int bad_e = 0;
     u64 v[NE];
@@ -567,6 +623,44 @@ __device__ __forceinline__ bool wave_poll(const u64* src, unsigned epoch, lfp ds
     if (m == 0) return true;
     const int first = __builtin_ctzll(m);
     line = 8 * __builtin_amdgcn_readlane(bad_e, first) + (first >> 3);
+    if (++rounds > 4096u) {
+      PG_ST32(abort_word, 1u);
+      return false;
+    }
+  }
+}
+// The same for a vector of C = 64 NW f32 words: waits until none is armed.  The bulk read
+// takes the words in pairs (lane + 64 e is pair number; a 64-byte line is eight pairs).
+template <int NW>
+__device__ __forceinline__ bool wave_poll(const unsigned* src, lfp dst, unsigned* abort_word, int probe,
+                                          lu64p dbg = nullptr) {
+  constexpr int PAIRS = NW * 32, NP = cdiv(PAIRS, 64), LINES = NW * 4;
+  typedef __attribute__((address_space(3))) f2* lf2p;
+  const int lane = opaque((int)threadIdx.x) & 63;
+  unsigned rounds = 0;
+  int line = probe * 3;
+  for (;;) {
+    if (!probe_spread<LINES, false>(src, line, 0u, abort_word, dbg)) return false;
+    if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
+    bool bad = false;
+    int bad_e = 0;
+    u64 v[NP];
+#pragma unroll
+    for (int e = 0; e < NP; ++e) v[e] = ld_tagged(src, (unsigned)min(lane + 64 * e, PAIRS - 1) * 8u);
+#pragma unroll
+    for (int e = 0; e < NP; ++e) {
+      if (pair_armed(v[e])) {
+        bad = true;
+        bad_e = e;
+      }
+      if (64 * (e + 1) <= PAIRS || lane + 64 * e < PAIRS)
+        ((lf2p)dst)[lane + 64 * e] = f2{__uint_as_float((unsigned)v[e]), __uint_as_float((unsigned)(v[e] >> 32))};
+    }
+    const unsigned long long m = __ballot(bad);
+    if (dbg && lane == 0) dbg[2] = __builtin_amdgcn_s_memtime();
+    if (m == 0) return true;
+    const int first = __builtin_ctzll(m);
+    line = min(8 * __builtin_amdgcn_readlane(bad_e, first) + (first >> 3), LINES - 1);
     if (++rounds > 4096u) {
       PG_ST32(abort_word, 1u);
       return false;
@@ -686,24 +780,29 @@ __device__ __forceinline__ void attn_wave_partial(KvRegs<KS>& r, ctlp ctl, int k
   }
 }
 
-// ---- this wavefront's share of the 4C tagged words of h ---------------------------------
-// Runs wave + 8 e (64 words each).  Payloads go to dst (LDS); returns 0, or 1 + a run
-// that held a stale word.
+// ---- this wavefront's share of the 4C words of h ----------------------------------------
+// Runs wave + 8 e (64 pairs of words each).  Payloads go to dst (LDS); returns 0, or 1 + a
+// run that held a word not written yet.
 template <int RUNS>
-__device__ __forceinline__ unsigned h_share(const u64* src, unsigned epoch, lfp dst, int wave, int lane) {
+__device__ __forceinline__ unsigned h_share(const unsigned* src, lfp dst, int wave, int lane) {
   constexpr int RPW = cdiv(RUNS, 8);
+  typedef __attribute__((address_space(3))) f2* lf2p;
   u64 v[RPW];
 #pragma unroll
   for (int e = 0; e < RPW; ++e) {
-    const int run = min(wave + 8 * e, RUNS - 1);
-    v[e] = ld_tagged(src, (unsigned)(run * 64 + lane) * 8u);
+    const int run = wave + 8 * e;  // wave-uniform
+    v[e] = 0;
+    if (8 * (e + 1) <= RUNS || run < RUNS) v[e] = ld_tagged(src, (unsigned)(run * 64 + lane) * 8u);
   }
   unsigned code = 0;
 #pragma unroll
   for (int e = 0; e < RPW; ++e) {
-    const int run = min(wave + 8 * e, RUNS - 1);
-    if (tag_of(v[e]) != epoch) code = 1u + (unsigned)run;
-    dst[run * 64 + lane] = val_of(v[e]);
+    const int run = wave + 8 * e;
+    if (8 * (e + 1) <= RUNS || run < RUNS) {
+      if (pair_armed(v[e])) code = 1u + (unsigned)run;
+      ((lf2p)dst)[run * 64 + lane] =
+          f2{__uint_as_float((unsigned)v[e]), __uint_as_float((unsigned)(v[e] >> 32))};
+    }
   }
   // wave-uniform: any lane's stale run will do
   const unsigned long long m = __ballot(code != 0);
@@ -738,7 +837,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
   // merges the per-workgroup (value, index) pairs published with `ep`
   auto merged_token = [&](unsigned ep, unsigned& out) -> bool {
     // staged in xsF (idle between the last mlp projection and the next one)
-    if (!wave_poll<(2 * G) / 64>(p.best_t, ep, lds.xsF, abort_word, wg)) return false;
+    if (!wave_poll_tagged<(2 * G) / 64>(p.best_t, ep, lds.xsF, abort_word, wg)) return false;
     lds_fence();
     // word 2g is the value, 2g+1 the index of workgroup g
     Best b{-INFINITY, 0xffffffffu};
@@ -779,6 +878,15 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       const LayerW w = layer_of(p.layers, l);
       float* kc = p.kv + (size_t)l * p.kv_layer_stride;
       float* vc = kc + p.kv_v_offset;
+      // this layer step's buffers of the exchanged vectors (`par`), and the other ones
+      // (the addresses are formed where they are used: kept across the layer they would
+      // crowd the scalar registers)
+      const unsigned par = (unsigned)(t * p.L + l) & 1u, opar = par ^ 1u;
+#define X_qkv (p.xch + par * p.xch_set + XchLayout::qkv(C))
+#define X_part (p.xch + par * p.xch_set + XchLayout::part(C))
+#define X_attn (p.xch + par * p.xch_set + XchLayout::attn(C))
+#define X_xa (p.xch + par * p.xch_set + XchLayout::xa(C))
+#define X_h (p.xch + par * p.xch_set + XchLayout::h(C))
 
       // the first attention item of this workgroup, known before the layer starts
       const int items = H * ns, n = pos + 1;
@@ -818,8 +926,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
             lds.xraw1[lane + 64 * j] = e + gld_at(p.wpe + (size_t)pos * C, col);
           }
         } else {
-          if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, l - 1, 5), lds.xraw1, abort_word, wg))
-            PG_SERVICE_FAIL();
+          if (!wave_poll<NW>(p.xch + opar * p.xch_set + XchLayout::xm(C), lds.xraw1, abort_word, wg)) PG_SERVICE_FAIL();
         }
         lds_fence();
         wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsA, lane);
@@ -832,17 +939,17 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // All eight wavefronts work on an item: each loads the K/V rows of its slots as
       // soon as the item is known; this wavefront waits for q, stages it in LDS, counts
       // the item in flag[5], and merges the eight partial results.
-      const unsigned epq = epoch_of(p, t, l, 0), epp = epoch_of(p, t, l, 1);
+      const unsigned epp = epoch_of(p, t, l, 1);
 #pragma unroll 1
       for (int item = wg; item < items; item += G) {
         const int h = item / ns, s = item - h * ns;
         const int k0 = s * per, k1 = min(n, k0 + per);
-        u64* dst = p.part_t + (size_t)item * 66;
+        unsigned* dst = X_part + (size_t)item * 66;
         ++bseq;
         if (k0 >= k1) {  // empty split: neutral element of the merge (the streamers skip it too)
-          PG_ST64(dst + lane, pack(epp, 0.0f));
-          if (lane == 0) PG_ST64(dst + 64, pack(epp, -INFINITY));
-          if (lane == 1) PG_ST64(dst + 65, pack(epp, 0.0f));
+          PG_ST32(dst + lane, xbits(0.0f));
+          if (lane == 0) PG_ST32(dst + 64, xbits(-INFINITY));
+          if (lane == 1) PG_ST32(dst + 65, xbits(0.0f));
           continue;
         }
         const bool owns_new = (k1 == n);
@@ -853,16 +960,16 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         {
           bool ok = true;
           unsigned spins = 0;
-          const unsigned off = (unsigned)(h * 64 + lane) * 8u;
+          const unsigned off = (unsigned)(h * 64 + lane) * 4u;
           for (;;) {
             // without the new row, the K and V words are not waited for (q is re-read)
-            const u64 v0 = ld_tagged(p.qkv_t, off);
-            const u64 v1 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 8u : 0u));
-            const u64 v2 = ld_tagged(p.qkv_t, off + (owns_new ? (unsigned)C * 16u : 0u));
-            const bool bad = tag_of(v0) != epq || tag_of(v1) != epq || tag_of(v2) != epq;
-            qn[0] = val_of(v0);
-            qn[1] = val_of(v1);
-            qn[2] = val_of(v2);
+            const unsigned v0 = ld_word(X_qkv, off);
+            const unsigned v1 = ld_word(X_qkv, off + (owns_new ? (unsigned)C * 4u : 0u));
+            const unsigned v2 = ld_word(X_qkv, off + (owns_new ? (unsigned)C * 8u : 0u));
+            const bool bad = v0 == kArm || v1 == kArm || v2 == kArm;
+            qn[0] = __uint_as_float(v0);
+            qn[1] = __uint_as_float(v1);
+            qn[2] = __uint_as_float(v2);
             if (!__any(bad)) break;
             if (++spins > kSpinLimit) {
               PG_ST32(abort_word, 1u);
@@ -921,11 +1028,11 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           }
           if (ns == 1) {
             // the head's only split: this is the attention output itself, no merge hop
-            PG_ST64(p.attn_t + h * 64 + lane, pack(epoch_of(p, t, l, 2), num / den));
+            PG_ST32(X_attn + h * 64 + lane, xbits(num / den));
           } else {
-            PG_ST64(dst + lane, pack(epp, num));
-            if (lane == 0) PG_ST64(dst + 64, pack(epp, M));
-            if (lane == 1) PG_ST64(dst + 65, pack(epp, den));
+            PG_ST32(dst + lane, xbits(num));
+            if (lane == 0) PG_ST32(dst + 64, xbits(M));
+            if (lane == 1) PG_ST32(dst + 65, xbits(den));
           }
         }
       }
@@ -955,17 +1062,17 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         // the head's ns partials (66 words each) are one run of tagged words: probe the
         // last word of every partial, then read them all into LDS (the staging area of
         // the long vector, idle now) and merge from there
-        const u64* src = p.part_t + (size_t)h * ns * 66;
+        const unsigned* src = X_part + (size_t)h * ns * 66;
         const int nw = ns * 66;
         lfp stage = lds.xsF;
         unsigned spins = 0;
         for (;;) {
           {
-            const unsigned off = (unsigned)(min(lane, ns - 1) * 66 + 65) * 8u;
+            const unsigned off = (unsigned)(min(lane, ns - 1) * 66 + 65) * 4u;
             bool ok = true;
             for (;;) {
-              const u64 v = ld_tagged(src, off);
-              if (__all(tag_of(v) == epp)) break;
+              const unsigned v = ld_word(src, off);
+              if (__all(v != kArm)) break;
               if (++spins > kSpinLimit) {
                 PG_ST32(abort_word, 1u);
                 ok = false;
@@ -983,14 +1090,14 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           constexpr int CH = 12;
 #pragma unroll 1
           for (int e0 = 0; e0 * 64 < nw; e0 += CH) {
-            u64 v[CH];
+            unsigned v[CH];
 #pragma unroll
             for (int e = 0; e < CH; ++e)
-              v[e] = ld_tagged(src, (unsigned)min(lane + 64 * (e0 + e), nw - 1) * 8u);
+              v[e] = ld_word(src, (unsigned)min(lane + 64 * (e0 + e), nw - 1) * 4u);
 #pragma unroll
             for (int e = 0; e < CH; ++e) {
-              bad = bad || (tag_of(v[e]) != epp);
-              stage[min(lane + 64 * (e0 + e), nw - 1)] = val_of(v[e]);
+              bad = bad || (v[e] == kArm);
+              stage[min(lane + 64 * (e0 + e), nw - 1)] = __uint_as_float(v[e]);
             }
           }
           if (!__any(bad)) break;
@@ -1011,17 +1118,38 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           den += wq * stage[q * 66 + 65];
           num += wq * stage[q * 66 + lane];
         }
-        PG_ST64(p.attn_t + h * 64 + lane, pack(epa, num / den));
+        PG_ST32(X_attn + h * 64 + lane, xbits(num / den));
       }
       if (merges && lane == 0) ctl->flag[6] = epp;
 
       // ================= D: attention output -> xsD =================
       {
-        if (!wave_poll<NW>(p.attn_t, epa, lds.xsD, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        if (!wave_poll<NW>(X_attn, lds.xsD, abort_word, wg + 1)) PG_SERVICE_FAIL();
         lds_fence();
         if (lane == 0) ctl->flag[1] = epa;
       }
       PG_STAMP(l, 2);
+
+      // ---- re-arming the other buffers ----
+      // The attention output is complete, so every head's items have run; the items of a head
+      // read its q rows and the newest K and V rows, which together are all of qkv: every
+      // workgroup has published its c_attn rows of this step and was therefore done with the
+      // previous step (its last read there, of h or of the block's output, comes before its
+      // LayerNorm of this step).  Nothing reads the other buffers any more, and nothing
+      // writes them before the next step, whose first product needs this step's output of every
+      // workgroup, this one's included: the stores below are waited for before this
+      // wavefront raises the flag of the c_fc rows.  Each workgroup arms a 256th of each.
+      // Each workgroup arms a 256th of the other set, in whole 64-byte lines (a partial line
+      // would be merged into memory by a read and a write).
+      {
+        const int lines = (int)(p.xch_set >> 4);
+        const int l0 = (int)(((long long)wg * lines) / G), l1 = (int)(((long long)(wg + 1) * lines) / G);
+        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+        typedef u4 __attribute__((address_space(1)))* gu4p;
+        gu4p dst = (gu4p)(p.xch + opar * p.xch_set);
+        // a lane writes 16 bytes: four lanes a line, sixteen lines an instruction
+        for (int i = 4 * l0 + lane; i < 4 * l1; i += 64) dst[i] = u4{kArm, kArm, kArm, kArm};
+      }
 
       // ================= E: xa -> xraw2, LN2 -> xsE =================
       {
@@ -1033,12 +1161,13 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           b[j] = gld_at(w.ln_2_b, (unsigned)ln + 64u * j);
         }
         const unsigned ep = epoch_of(p, t, l, 3);
-        if (!wave_poll<NW>(p.xa_t, ep, lds.xraw2, abort_word, wg + 2,
+        if (!wave_poll<NW>(X_xa, lds.xraw2, abort_word, wg + 2,
                            (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 + 13 : (lu64p) nullptr))
           PG_SERVICE_FAIL();
         lds_fence();
         wave_layer_norm<NW>(lds.xraw2, g, b, p.eps, lds.xsE, lane);
         lds_fence();
+        vm_drain();  // the arming stores above have been performed
         if (lane == 0) ctl->flag[2] = ep;
       }
       PG_STAMP(l, 3);
@@ -1048,17 +1177,17 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // (flag[7] counts the rounds); a stale word sends the probe to its run and the
       // round is repeated.
       {
-        constexpr int RUNS = I / 64;
+        constexpr int RUNS = I / 128;  // runs of 64 pairs of words
         const unsigned ep = epoch_of(p, t, l, 4);
-        int run = -1;  // the run a stale word was seen in
+        int run = -1;  // the run a word not written yet was seen in
         unsigned spins = 0;
         for (;;) {
-          if (run < 0 ? !probe_spread<8 * RUNS>(p.h_t, (wg + 3) * 5, ep, abort_word)
-                      : !probe_lines(p.h_t, 8 * run, 8 * run + 3, 8 * run + 7, ep, abort_word))
+          if (run < 0 ? !probe_spread<8 * RUNS, false>(X_h, (wg + 3) * 5, 0u, abort_word)
+                      : !probe_lines<false>(X_h, 8 * run, 8 * run + 3, 8 * run + 7, 0u, abort_word))
             PG_SERVICE_FAIL();
           ++hseq;
           if (lane == 0) ctl->flag[7] = hseq;
-          unsigned code = h_share<RUNS>(p.h_t, ep, lds.xsF, kSW, lane);
+          unsigned code = h_share<RUNS>(X_h, lds.xsF, kSW, lane);
           lvup st = (lvup)&ctl->hstat[min(lane, kSW - 1)];
           bool ok = true;
           unsigned v = 0;
@@ -1083,6 +1212,11 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         if (lane == 0) ctl->flag[3] = ep;
       }
       PG_STAMP(l, 4);
+#undef X_qkv
+#undef X_part
+#undef X_attn
+#undef X_xa
+#undef X_h
     }  // layers
 
     // ================= LN_f -> xsD, then this workgroup's argmax =================
@@ -1096,7 +1230,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       }
       const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
       // staged in xraw1 (the next user is the next token's embedding)
-      if (!wave_poll<NW>(p.xm_t, epoch_of(p, t, p.L - 1, 5), lds.xraw1, abort_word, wg))
+      if (!wave_poll<NW>(p.xch + ((unsigned)(t * p.L + p.L - 1) & 1u) * p.xch_set + XchLayout::xm(C), lds.xraw1, abort_word, wg))
         PG_SERVICE_FAIL();
       lds_fence();
       wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsD, lane);
@@ -1346,6 +1480,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       const int items = H * ns, n = pos + 1, per = (n + ns - 1) / ns;
       const float* kc = p.kv + (size_t)l * p.kv_layer_stride;
       const float* vc = kc + p.kv_v_offset;
+      // this layer step's buffers of the exchanged vectors
+      const unsigned par = (unsigned)(t * p.L + l) & 1u;
       KvRegs<KS> kv;
       bool kv_early = false;
       if constexpr (early_kv(C_)) {
@@ -1381,12 +1517,17 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
           dot_tiles_packed<WB, TA, J>(WA, lds.xsA, SP::KC, lane, scA, v);
         else
           dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
-        const unsigned ep = epoch_of(p, t, l, 0);
+        unsigned* const qkv_x = p.xch + par * p.xch_set + XchLayout::qkv(C);
+        // lane i finishes row i: one store for all of the wavefront's rows
+        float mine = 0.0f;
+        int r = a1;
 #pragma unroll
-        for (int i = 0; i < TA; ++i) {
-          const int r = a0 + wave + kSW * i;
-          if (lane == 0 && r < a1) PG_ST64(p.qkv_t + r, pack(ep, biasA[i] + v[i]));
-        }
+        for (int i = 0; i < TA; ++i)
+          if (lane == i) {
+            mine = biasA[i] + v[i];
+            r = a0 + wave + kSW * i;
+          }
+        if (lane < TA && r < a1) PG_ST32(qkv_x + r, xbits(mine));
       }
       SSTAMP(5);
       // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
@@ -1430,7 +1571,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         else
           dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
         const int r = d0 + wave;
-        if (lane == 0 && r < d1) PG_ST64(p.xa_t + r, pack(epoch_of(p, t, l, 3), lds.xraw1[r] + (biasD + v[0])));
+        if (lane == 0 && r < d1) PG_ST32(p.xch + par * p.xch_set + XchLayout::xa(C) + r, xbits(lds.xraw1[r] + (biasD + v[0])));
       }
       SSTAMP(11);
       PG_SLICE(3, w, wn);
@@ -1452,7 +1593,6 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
           dot_tiles_packed<WB, TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
         else
           dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
-        const unsigned ep = epoch_of(p, t, l, 4);
         // lane i finishes row i: one GELU and one store for all of the wavefront's rows
         float mine = 0.0f;
         int r = e1;
@@ -1462,7 +1602,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
             mine = biasE[i] + v[i];
             r = e0 + wave + kSW * i;
           }
-        if (lane < TE && r < e1) PG_ST64(p.h_t + r, pack(ep, gelu_tanh(mine)));
+        if (lane < TE && r < e1) PG_ST32(p.xch + par * p.xch_set + XchLayout::h(C) + r, xbits(gelu_tanh(mine)));
       }
       SSTAMP(6);
       PG_SLICE(4, w, wn);
@@ -1477,7 +1617,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         if (r == 0) ok = false;
         if (r != 2) break;
         ++hseq;
-        const unsigned code = h_share<I / 64>(p.h_t, epoch_of(p, t, l, 4), lds.xsF, wave, lane);
+        const unsigned code = h_share<I / 128>(p.xch + par * p.xch_set + XchLayout::h(C), lds.xsF, wave, lane);
         lds_fence();
         if (lane == 0) ctl->hstat[wave] = (hseq << 8) | code;
       }
@@ -1501,7 +1641,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         }
         const float v = wsum(acc);
         const int r = d0 + wave;
-        if (lane == 0 && r < d1) PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), lds.xraw2[r] + (biasF + v)));
+        if (lane == 0 && r < d1) PG_ST32(p.xch + par * p.xch_set + XchLayout::xm(C) + r, xbits(lds.xraw2[r] + (biasF + v)));
       } else {
         // the staged part of the row: complete once only the c_attn rows requested after
         // the row's last registers are still in flight
@@ -1534,7 +1674,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         }
         const float v = wsum((a0_ + a1_) + (a2_ + a3_));
         const int r = d0 + wave;
-        if (lane == 0 && r < d1) PG_ST64(p.xm_t + r, pack(epoch_of(p, t, l, 5), lds.xraw2[r] + (biasF + v)));
+        if (lane == 0 && r < d1) PG_ST32(p.xch + par * p.xch_set + XchLayout::xm(C) + r, xbits(lds.xraw2[r] + (biasF + v)));
       }
       SSTAMP(7);
       PG_SLICE(5, w, wn);
@@ -1717,6 +1857,24 @@ hipError_t max_blocks(int C, int* out) {
   return hipSuccess;
 }
 }  // namespace
+
+namespace {
+__global__ void k_arm_exchange(unsigned* x, size_t n, unsigned* status) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = kArm;
+  if (i < 4) status[i] = 0u;
+}
+}  // namespace
+
+size_t persistent_exchange_set_words(int C, size_t part_words) {
+  return ((size_t)XchLayout::part((unsigned)C) + part_words + 15) / 16 * 16;
+}
+
+hipError_t launch_arm_exchange(unsigned* x, size_t n, unsigned* status, hipStream_t s) {
+  const size_t blocks = (std::max<size_t>(n, 4) + 255) / 256;
+  hipLaunchKernelGGL(k_arm_exchange, dim3((unsigned)blocks), dim3(256), 0, s, x, n, status);
+  return hipGetLastError();
+}
 
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
   if (!p.lm_w || (p.w_bytes == 1 && !p.lm_s)) return hipErrorInvalidValue;

@@ -135,9 +135,12 @@ struct pg_kv_cache {
   pg_logits logits{};
   bool logits_valid = false;
   // persistent decode: tagged activation words {epoch, f32} and the launch status
-  unsigned long long *qkv_t = nullptr, *part_t = nullptr, *attn_t = nullptr, *xa_t = nullptr,
-                     *h_t = nullptr, *xm_t = nullptr, *best_t = nullptr;
-  size_t tagged_words = 0;  // total words in the allocation that starts at qkv_t
+  // One uncached block: the tagged argmax words, then the f32 exchange vectors (two buffers each)
+  unsigned long long* best_t = nullptr;
+  unsigned* xch = nullptr;
+  size_t best_words = 0;  // 64-bit words at best_t
+  size_t x_words = 0;     // 32-bit words at xch
+  unsigned xch_set = 0;   // words from one set of exchange vectors to the other
   size_t tagged_bytes = 0;  // size of that allocation as the exchange pool counts it
   unsigned* status = nullptr;
   unsigned* h_status = nullptr;  // pinned
@@ -468,7 +471,7 @@ constexpr unsigned kEpochWrap = 0xE0000000u;
 std::mutex g_persistent_mu;
 
 bool use_persistent(const pg_gpt2_model* m, const pg_kv_cache* c) {
-  return m->persistent && c->B == 1 && c->qkv_t != nullptr;
+  return m->persistent && c->B == 1 && c->best_t != nullptr;
 }
 
 // Set while this thread has a persistent launch in flight: a callback that re-enters the
@@ -512,7 +515,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   const unsigned span = (unsigned)(n_fwd * (g.L + 1) * 8 + 8);
   if (c->epoch > kEpochWrap - span) {
     // epochs would wrap: clear every tag and start over
-    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->qkv_t), c->tagged_words * 2,
+    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->best_t), c->best_words * 2,
                                  c->stream));
     c->epoch = 1;
   }
@@ -525,8 +528,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   p.kv = c->kv;
   p.kv_layer_stride = 2 * g.H * g.P * g.hd();
   p.kv_v_offset = g.H * g.P * g.hd();
-  p.qkv_t = c->qkv_t; p.part_t = c->part_t; p.attn_t = c->attn_t; p.xa_t = c->xa_t;
-  p.h_t = c->h_t; p.xm_t = c->xm_t; p.best_t = c->best_t;
+  p.xch = c->xch; p.xch_set = c->xch_set; p.best_t = c->best_t;
   p.logits = c->logits_buf;
   p.d_tok = c->d_tok;
   p.tok_val = tok;
@@ -564,7 +566,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   c->epoch += span;
   run->lock = std::unique_lock<std::mutex>(g_persistent_mu);
   auto enqueue = [&]() -> pg_status {
-    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(c->status), 4, c->stream));
+    PG_HIP(pgk::launch_arm_exchange(c->xch, c->x_words, c->status, c->stream));
     if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
     PG_HIP(pgk::launch_decode_persistent(p, c->stream));
     if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
@@ -1300,24 +1302,25 @@ pg_status pg_kv_cache_create(const pg_gpt2_model* m, uint32_t batch, pg_kv_cache
   PG_HIP(hipMalloc(&raw->d_out_ids, g.P * B * sizeof(uint32_t)));
   PG_HIP(hipHostMalloc(&raw->h_ids, g.P * B * sizeof(uint32_t), hipHostMallocDefault));
   if (m->persistent && batch == 1) {
-    const size_t n_part = g.H * pgk::kMaxSplits * 66;
-    const size_t words = 3 * g.C + n_part + g.C + g.C + g.I + g.C + 2 * (size_t)m->persistent_grid;
-    PG_HIP(exchange_acquire(raw->device, words * sizeof(unsigned long long),
-                            reinterpret_cast<void**>(&raw->qkv_t), &raw->tagged_bytes));
-    raw->tagged_words = words;
-    raw->part_t = raw->qkv_t + 3 * g.C;
-    raw->attn_t = raw->part_t + n_part;
-    raw->xa_t = raw->attn_t + g.C;
-    raw->h_t = raw->xa_t + g.C;
-    raw->xm_t = raw->h_t + g.I;
-    raw->best_t = raw->xm_t + g.C;
+    // (every vector starts on a 64-byte line: the scalar probes read whole lines; n_embd is a
+    // multiple of 64 here)
+    const size_t n_best = 2 * (size_t)m->persistent_grid;
+    const size_t set_words =
+        pgk::persistent_exchange_set_words((int)g.C, g.H * (size_t)m->attn_splits * 66);
+    const size_t x_words = 2 * set_words;
+    PG_HIP(exchange_acquire(raw->device, n_best * sizeof(unsigned long long) + x_words * sizeof(unsigned),
+                            reinterpret_cast<void**>(&raw->best_t), &raw->tagged_bytes));
+    raw->best_words = n_best;
+    raw->x_words = x_words;
+    raw->xch_set = (unsigned)set_words;
+    raw->xch = reinterpret_cast<unsigned*>(raw->best_t + n_best);
     PG_HIP(hipMalloc(&raw->status, 4 * sizeof(unsigned)));
     PG_HIP(hipHostMalloc(&raw->h_status, 4 * sizeof(unsigned), hipHostMallocDefault));
     PG_HIP(hipMalloc(&raw->d_force, g.P * sizeof(uint32_t)));
     PG_HIP(hipHostMalloc(&raw->h_stream, (g.P + 1) * sizeof(uint32_t),
                          hipHostMallocMapped | hipHostMallocCoherent));
     PG_HIP(hipHostGetDevicePointer(reinterpret_cast<void**>(&raw->h_stream_dev), raw->h_stream, 0));
-    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(raw->qkv_t), words * 2, raw->stream));
+    PG_HIP(pgk::launch_fill_zero(reinterpret_cast<float*>(raw->best_t), n_best * 2, raw->stream));
   }
   // Gpt2LayerKvCache::new zero-fills (src/models/gpt2/rust.rs:258-266).
   PG_HIP(pgk::launch_fill_zero(raw->kv, kv_floats, raw->stream));
@@ -1351,7 +1354,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->d_tok);
     (void)hipFree(c->d_out_ids);
     if (c->h_ids) (void)hipHostFree(c->h_ids);
-    exchange_release(c->device, c->tagged_bytes, c->qkv_t);
+    exchange_release(c->device, c->tagged_bytes, c->best_t);
     (void)hipFree(c->status);
     (void)hipFree(c->d_force);
     if (c->h_status) (void)hipHostFree(c->h_status);
@@ -1386,10 +1389,10 @@ pg_status pg_kv_cache_set_seq_len(pg_kv_cache* c, uint64_t n) {
   return PG_OK;
 }
 
-uint32_t pg_kv_cache_debug_epoch(const pg_kv_cache* c) { return c && c->qkv_t ? c->epoch : 0; }
+uint32_t pg_kv_cache_debug_epoch(const pg_kv_cache* c) { return c && c->best_t ? c->epoch : 0; }
 pg_status pg_kv_cache_debug_set_epoch(pg_kv_cache* c, uint32_t epoch) {
   if (!c) return fail(PG_INVALID_INPUT, "null argument");
-  if (!c->qkv_t) return fail(PG_INVALID_INPUT, "this cache does not use the persistent decode kernel");
+  if (!c->best_t) return fail(PG_INVALID_INPUT, "this cache does not use the persistent decode kernel");
   // words in memory carry epochs below c->epoch: a lower value could meet one of them again
   if (epoch < c->epoch)
     return fail(PG_INVALID_INPUT, "epoch " + std::to_string(epoch) + " is behind the cache's " +

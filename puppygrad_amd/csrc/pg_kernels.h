@@ -208,7 +208,13 @@ struct DecodeParams {
   float* kv;               // [L][2][H][P][64] of this sequence
   size_t kv_layer_stride;  // floats from layer l to l+1
   size_t kv_v_offset;      // floats from the K panel to the V panel of a layer
-  unsigned long long *qkv_t, *part_t, *attn_t, *xa_t, *h_t, *xm_t, *best_t;
+  // Exchanged activations: f32 words in uncached memory, two sets xch_set words apart (used by
+  // alternate layer steps), all holding the "not written yet" pattern when a launch starts
+  // (launch_arm_exchange).  A set, in words: qkv 3C | attn C | xa C | h 4C | xm C | part
+  // (H * ns * 66), rounded up to whole 64-byte lines (persistent_exchange_set_words).
+  unsigned* xch;
+  unsigned xch_set;
+  unsigned long long* best_t;  // [2 * grid] tagged words {epoch, value}: per-workgroup argmax
   float* logits;
   uint32_t* d_tok;
   uint32_t tok_val;
@@ -236,5 +242,10 @@ int persistent_default_item_keys();
 bool persistent_item_keys_ok(int keys);
 hipError_t persistent_max_blocks_per_cu(int C, int* out, int w_bytes = 4, int item_keys = 128);
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
+// Words of one set of DecodeParams::xch for n_embd = C and part_words words of attention partials.
+size_t persistent_exchange_set_words(int C, size_t part_words);
+// Before every launch: the n exchange words at x take the "not written yet" pattern and the
+// four status words are cleared.
+hipError_t launch_arm_exchange(unsigned* x, size_t n, unsigned* status, hipStream_t s);
 
 }  // namespace pgk
