@@ -151,6 +151,9 @@ struct Ctl {
   unsigned flag[8];    // [0] A, [1] D, [2] E, [3] F, [4] lm_head: epoch whose input is staged;
                        // [5] attention item staged (running count), [6] credit of the
                        // second attention hop (epoch), [7] "read your share of h" (running count)
+  unsigned lnflag[3];  // LayerNorm statistics of the A, E and lm_head inputs: epoch they belong to
+  float lninv[3];      // 1 / sqrt(var + eps) ...
+  float lnminv[3];     // ... and mean / sqrt(var + eps) of that input
   unsigned halt;       // 0 run, 1 a wait gave up, 2 stopped at the EOS token
   unsigned lmdone[8];  // per streamer: epoch of its finished lm_head band
   unsigned bdone[8];   // per wavefront: count of the attention item whose partial it has written
@@ -459,6 +462,33 @@ __device__ __forceinline__ bool wait_flag(ctlp ctl, int which, unsigned epoch, u
   return ok;
 }
 
+// The LayerNorm statistics of input `which` (0 A, 1 E, 2 lm_head) for `epoch`, published by the
+// service wavefront a little after the input itself (ln_publish).
+__device__ __forceinline__ bool wait_ln(ctlp ctl, int which, unsigned epoch, unsigned* abort_word, float& inv,
+                                        float& minv) {
+  lvup f = (lvup)&ctl->lnflag[which];
+  lvup h = (lvup)&ctl->halt;
+  unsigned spins = 0;
+  bool ok = true;
+  for (;;) {
+    if (*f == epoch) break;
+    if (*h != 0) {
+      ok = false;
+      break;
+    }
+    if (++spins > kSpinLimit) {
+      ok = false;
+      PG_ST32(abort_word, 1u);
+      *h = 1u;
+      break;
+    }
+  }
+  asm volatile("" ::: "memory");
+  inv = ctl->lninv[which];
+  minv = ctl->lnminv[which];
+  return ok;
+}
+
 // Waits until flag a carries va (returns 1) or flag b carries vb (returns 2); 0 on halt.
 __device__ __forceinline__ int wait_either(ctlp ctl, int a, unsigned va, int b, unsigned vb,
                                            unsigned* abort_word) {
@@ -630,12 +660,21 @@ __device__ __forceinline__ bool wave_poll_tagged(const u64* src, unsigned epoch,
   }
 }
 // The same for a vector of C = 64 NW f32 words: waits until none is armed.  The bulk read
-// takes the words in pairs (lane + 64 e is pair number; a 64-byte line is eight pairs).
+// takes the words in pairs (lane + 64 e is the pair's number; a 64-byte line is eight pairs)
+// and leaves them in v; lanes past the last pair hold a copy of it (pair_valid tells).
 template <int NW>
-__device__ __forceinline__ bool wave_poll(const unsigned* src, lfp dst, unsigned* abort_word, int probe,
+struct Pairs {
+  static constexpr int PAIRS = NW * 32, NP = cdiv(PAIRS, 64), LINES = NW * 4;
+  u64 v[NP];
+};
+template <int NW>
+__device__ __forceinline__ bool pair_valid(int e, int lane) {
+  return 64 * (e + 1) <= Pairs<NW>::PAIRS || lane + 64 * e < Pairs<NW>::PAIRS;
+}
+template <int NW>
+__device__ __forceinline__ bool wave_poll(const unsigned* src, Pairs<NW>& out, unsigned* abort_word, int probe,
                                           lu64p dbg = nullptr) {
-  constexpr int PAIRS = NW * 32, NP = cdiv(PAIRS, 64), LINES = NW * 4;
-  typedef __attribute__((address_space(3))) f2* lf2p;
+  constexpr int PAIRS = Pairs<NW>::PAIRS, NP = Pairs<NW>::NP, LINES = Pairs<NW>::LINES;
   const int lane = opaque((int)threadIdx.x) & 63;
   unsigned rounds = 0;
   int line = probe * 3;
@@ -644,18 +683,14 @@ __device__ __forceinline__ bool wave_poll(const unsigned* src, lfp dst, unsigned
     if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
     bool bad = false;
     int bad_e = 0;
-    u64 v[NP];
 #pragma unroll
-    for (int e = 0; e < NP; ++e) v[e] = ld_tagged(src, (unsigned)min(lane + 64 * e, PAIRS - 1) * 8u);
+    for (int e = 0; e < NP; ++e) out.v[e] = ld_tagged(src, (unsigned)min(lane + 64 * e, PAIRS - 1) * 8u);
 #pragma unroll
-    for (int e = 0; e < NP; ++e) {
-      if (pair_armed(v[e])) {
+    for (int e = 0; e < NP; ++e)
+      if (pair_armed(out.v[e])) {
         bad = true;
         bad_e = e;
       }
-      if (64 * (e + 1) <= PAIRS || lane + 64 * e < PAIRS)
-        ((lf2p)dst)[lane + 64 * e] = f2{__uint_as_float((unsigned)v[e]), __uint_as_float((unsigned)(v[e] >> 32))};
-    }
     const unsigned long long m = __ballot(bad);
     if (dbg && lane == 0) dbg[2] = __builtin_amdgcn_s_memtime();
     if (m == 0) return true;
@@ -667,31 +702,76 @@ __device__ __forceinline__ bool wave_poll(const unsigned* src, lfp dst, unsigned
     }
   }
 }
-
-// layer_norm_in_place (src/models/cpu.rs:119-143) of the C = 64 NW values in raw (LDS;
-// this lane's are lane + 64 j), two-pass mean / biased variance, eps inside the sqrt;
-// writes the result to xs (LDS).
+__device__ __forceinline__ f2 pair_f2(u64 v) {
+  return f2{__uint_as_float((unsigned)v), __uint_as_float((unsigned)(v >> 32))};
+}
+typedef __attribute__((address_space(3))) f2* lf2p;
+// The pairs as they are -> dst (LDS).
 template <int NW>
-__device__ __forceinline__ void wave_layer_norm(lfp raw, const float (&g)[NW], const float (&b)[NW],
-                                                float eps, lfp xs, int lane) {
-  constexpr int C = NW * 64;
-  float x[NW];
+__device__ __forceinline__ void stage_pairs(const Pairs<NW>& in, lfp dst, int lane) {
 #pragma unroll
-  for (int j = 0; j < NW; ++j) x[j] = raw[lane + 64 * j];
+  for (int e = 0; e < Pairs<NW>::NP; ++e)
+    if (pair_valid<NW>(e, lane)) ((lf2p)dst)[lane + 64 * e] = pair_f2(in.v[e]);
+}
+// The input of a projection that follows a LayerNorm.  layer_norm_in_place
+// (src/models/cpu.rs:119-143) gives xn_i = (x_i - mean) * inv * g_i + b_i with
+// inv = 1 / sqrt(var + eps), so a row of the projection is
+//     W . xn + bias = inv * (W . (g * x)) - (mean * inv) * (W . g) + (W . b + bias).
+// The two row constants (W . g, W . b + bias) are computed once per model (k_ln_fold); the
+// streamers multiply with g * x, which is staged here without waiting for any statistic, and
+// apply mean and inv to their sums, which this wavefront works out while they multiply
+// (ln_stats).  raw receives x itself (the residual reads it).
+template <int NW>
+__device__ __forceinline__ void stage_scaled(const Pairs<NW>& in, const f2 (&g2)[Pairs<NW>::NP], lfp raw,
+                                             lfp xg, int lane) {
+#pragma unroll
+  for (int e = 0; e < Pairs<NW>::NP; ++e)
+    if (pair_valid<NW>(e, lane)) {
+      const f2 x = pair_f2(in.v[e]);
+      ((lf2p)raw)[lane + 64 * e] = x;
+      ((lf2p)xg)[lane + 64 * e] = f2{x.x * g2[e].x, x.y * g2[e].y};
+    }
+}
+// Mean and biased variance of the C = 64 NW values (two passes, eps inside the sqrt, as
+// layer_norm_in_place): inv = 1 / sqrt(var + eps), minv = mean * inv.
+template <int NW>
+__device__ __forceinline__ void ln_stats(const Pairs<NW>& in, float eps, int lane, float& inv, float& minv) {
+  constexpr int C = NW * 64;
   float s = 0.0f;
 #pragma unroll
-  for (int j = 0; j < NW; ++j) s += x[j];
+  for (int e = 0; e < Pairs<NW>::NP; ++e)
+    if (pair_valid<NW>(e, lane)) {
+      const f2 x = pair_f2(in.v[e]);
+      s += x.x + x.y;
+    }
   const float mean = wsum(s) / (float)C;
   float v = 0.0f;
 #pragma unroll
-  for (int j = 0; j < NW; ++j) {
-    const float d = x[j] - mean;
-    v += d * d;
-  }
+  for (int e = 0; e < Pairs<NW>::NP; ++e)
+    if (pair_valid<NW>(e, lane)) {
+      const f2 x = pair_f2(in.v[e]);
+      const float d0 = x.x - mean, d1 = x.y - mean;
+      v += d0 * d0 + d1 * d1;
+    }
   const float var = wsum(v) / (float)C;
-  const float inv = 1.0f / sqrtf(var + eps);
+  inv = 1.0f / sqrtf(var + eps);
+  minv = mean * inv;
+}
+// LayerNorm scale of the pairs this lane holds.
+template <int NW>
+__device__ __forceinline__ void load_g2(f2 (&g2)[Pairs<NW>::NP], const float* g, int lane) {
+  typedef const f2 __attribute__((address_space(1)))* gf2p;
 #pragma unroll
-  for (int j = 0; j < NW; ++j) xs[lane + 64 * j] = (x[j] - mean) * inv * g[j] + b[j];
+  for (int e = 0; e < Pairs<NW>::NP; ++e) g2[e] = ((gf2p)g)[min(lane + 64 * e, Pairs<NW>::PAIRS - 1)];
+}
+// Publishes the statistics of input `which` (0 A, 1 E, 2 lm_head) to the streamers.
+__device__ __forceinline__ void ln_publish(ctlp ctl, int which, float inv, float minv, unsigned epoch, int lane) {
+  if (lane == 0) {
+    ctl->lninv[which] = inv;
+    ctl->lnminv[which] = minv;
+  }
+  lds_fence();
+  if (lane == 0) ctl->lnflag[which] = epoch;
 }
 
 // Development timestamps (only when the launch carries a buffer for them): the shader
@@ -904,34 +984,40 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         }
       }
 
-      // ================= A: block input -> LN1 -> xsA =================
+      // ================= A: block input, scaled by the LN1 weights -> xsA =================
       {
         const int ln = opaque(lane);  // per-lane addresses are built here, not hoisted
-        float g[NW], b[NW];
-#pragma unroll
-        for (int j = 0; j < NW; ++j) {
-          g[j] = gld_at(w.ln_1_g, (unsigned)ln + 64u * j);
-          b[j] = gld_at(w.ln_1_b, (unsigned)ln + 64u * j);
-        }
+        f2 g2[Pairs<NW>::NP];
+        load_g2<NW>(g2, w.ln_1_g, ln);
+        Pairs<NW> x;
         if (l == 0) {
           // embedding (rust.rs:966-974)
 #pragma unroll
-          for (int j = 0; j < NW; ++j) {
-            const unsigned col = (unsigned)ln + 64u * j;
+          for (int e = 0; e < Pairs<NW>::NP; ++e) {
+            const unsigned col = 2u * (unsigned)min(ln + 64 * e, Pairs<NW>::PAIRS - 1);
             // (wte is bf16 when the rows are; wpe is always f32)
             typedef const unsigned short __attribute__((address_space(1)))* ghp;
-            const float e = p.w_bytes == 2
-                                ? __uint_as_float((unsigned)((ghp)p.wte)[(size_t)tok * C + col] << 16)
-                                : gld_at(p.wte + (size_t)tok * C, col);
-            lds.xraw1[lane + 64 * j] = e + gld_at(p.wpe + (size_t)pos * C, col);
+            float e0, e1;
+            if (p.w_bytes == 2) {
+              e0 = __uint_as_float((unsigned)((ghp)p.wte)[(size_t)tok * C + col] << 16);
+              e1 = __uint_as_float((unsigned)((ghp)p.wte)[(size_t)tok * C + col + 1] << 16);
+            } else {
+              e0 = gld_at(p.wte + (size_t)tok * C, col);
+              e1 = gld_at(p.wte + (size_t)tok * C, col + 1);
+            }
+            e0 += gld_at(p.wpe + (size_t)pos * C, col);
+            e1 += gld_at(p.wpe + (size_t)pos * C, col + 1);
+            x.v[e] = ((u64)__float_as_uint(e1) << 32) | (u64)__float_as_uint(e0);
           }
         } else {
-          if (!wave_poll<NW>(p.xch + opar * p.xch_set + XchLayout::xm(C), lds.xraw1, abort_word, wg)) PG_SERVICE_FAIL();
+          if (!wave_poll<NW>(p.xch + opar * p.xch_set + XchLayout::xm(C), x, abort_word, wg)) PG_SERVICE_FAIL();
         }
-        lds_fence();
-        wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsA, lane);
+        stage_scaled<NW>(x, g2, lds.xraw1, lds.xsA, lane);
         lds_fence();
         if (lane == 0) ctl->flag[0] = epoch_of(p, t, l, 0);
+        float inv, minv;
+        ln_stats<NW>(x, p.eps, lane, inv, minv);
+        ln_publish(ctl, 0, inv, minv, epoch_of(p, t, l, 0), lane);
       }
       PG_STAMP(l, 0);
 
@@ -1124,7 +1210,9 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 
       // ================= D: attention output -> xsD =================
       {
-        if (!wave_poll<NW>(X_attn, lds.xsD, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        Pairs<NW> x;
+        if (!wave_poll<NW>(X_attn, x, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        stage_pairs<NW>(x, lds.xsD, lane);
         lds_fence();
         if (lane == 0) ctl->flag[1] = epa;
       }
@@ -1151,24 +1239,23 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         for (int i = 4 * l0 + lane; i < 4 * l1; i += 64) dst[i] = u4{kArm, kArm, kArm, kArm};
       }
 
-      // ================= E: xa -> xraw2, LN2 -> xsE =================
+      // ================= E: xa -> xraw2, scaled by the LN2 weights -> xsE =================
       {
         const int ln = opaque(lane);
-        float g[NW], b[NW];
-#pragma unroll
-        for (int j = 0; j < NW; ++j) {
-          g[j] = gld_at(w.ln_2_g, (unsigned)ln + 64u * j);
-          b[j] = gld_at(w.ln_2_b, (unsigned)ln + 64u * j);
-        }
+        f2 g2[Pairs<NW>::NP];
+        load_g2<NW>(g2, w.ln_2_g, ln);
         const unsigned ep = epoch_of(p, t, l, 3);
-        if (!wave_poll<NW>(X_xa, lds.xraw2, abort_word, wg + 2,
+        Pairs<NW> x;
+        if (!wave_poll<NW>(X_xa, x, abort_word, wg + 2,
                            (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 + 13 : (lu64p) nullptr))
           PG_SERVICE_FAIL();
-        lds_fence();
-        wave_layer_norm<NW>(lds.xraw2, g, b, p.eps, lds.xsE, lane);
+        stage_scaled<NW>(x, g2, lds.xraw2, lds.xsE, lane);
         lds_fence();
         vm_drain();  // the arming stores above have been performed
         if (lane == 0) ctl->flag[2] = ep;
+        float inv, minv;
+        ln_stats<NW>(x, p.eps, lane, inv, minv);
+        ln_publish(ctl, 1, inv, minv, ep, lane);
       }
       PG_STAMP(l, 3);
 
@@ -1219,23 +1306,24 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
 #undef X_h
     }  // layers
 
-    // ================= LN_f -> xsD, then this workgroup's argmax =================
+    // ================= final input, scaled by the LN_f weights -> xsD, then this workgroup's argmax =====
     if (!(p.lm_last_only && t + 1 < p.n_fwd)) {
       const int ln = opaque(lane);
-      float g[NW], b[NW];
-#pragma unroll
-      for (int j = 0; j < NW; ++j) {
-        g[j] = gld_at(p.ln_f_g, (unsigned)ln + 64u * j);
-        b[j] = gld_at(p.ln_f_b, (unsigned)ln + 64u * j);
-      }
+      f2 g2[Pairs<NW>::NP];
+      load_g2<NW>(g2, p.ln_f_g, ln);
       const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
-      // staged in xraw1 (the next user is the next token's embedding)
-      if (!wave_poll<NW>(p.xch + ((unsigned)(t * p.L + p.L - 1) & 1u) * p.xch_set + XchLayout::xm(C), lds.xraw1, abort_word, wg))
+      // (the raw values go to xraw1, whose next user is the next token's embedding)
+      Pairs<NW> x;
+      if (!wave_poll<NW>(p.xch + ((unsigned)(t * p.L + p.L - 1) & 1u) * p.xch_set + XchLayout::xm(C), x, abort_word, wg))
         PG_SERVICE_FAIL();
-      lds_fence();
-      wave_layer_norm<NW>(lds.xraw1, g, b, p.eps, lds.xsD, lane);
+      stage_scaled<NW>(x, g2, lds.xraw1, lds.xsD, lane);
       lds_fence();
       if (lane == 0) ctl->flag[4] = epl;
+      {
+        float inv, minv;
+        ln_stats<NW>(x, p.eps, lane, inv, minv);
+        ln_publish(ctl, 2, inv, minv, epl, lane);
+      }
       PG_STAMP(p.L, 5);
       // wait for the streamers' bands
       {
@@ -1498,9 +1586,13 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       // ================= A: c_attn rows =================
       // (biases are scalar loads: requested before each wait, they neither use vector
       // registers while the rows are in flight nor queue behind them)
-      float biasA[TA];
+      // (c_attn follows LN1: per row the constants W . g and W . b + bias, see stage_scaled)
+      float rgA[TA], biasA[TA];
 #pragma unroll
-      for (int i = 0; i < TA; ++i) biasA[i] = cld(w.c_attn_b + row_of(a0, a1, i));
+      for (int i = 0; i < TA; ++i) {
+        rgA[i] = cld(w.c_attn_f + 2 * row_of(a0, a1, i));
+        biasA[i] = cld(w.c_attn_f + 2 * row_of(a0, a1, i) + 1);
+      }
       float scA[TA];  // int8 rows: their scales
 #pragma unroll
       for (int i = 0; i < TA; ++i) scA[i] = kI8 ? cld(w.c_attn_s + row_of(a0, a1, i)) : 1.0f;
@@ -1518,13 +1610,18 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         else
           dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         unsigned* const qkv_x = p.xch + par * p.xch_set + XchLayout::qkv(C);
+        float inv, minv;
+        if (!wait_ln(ctl, 0, epoch_of(p, t, l, 0), abort_word, inv, minv)) {
+          ok = false;
+          break;
+        }
         // lane i finishes row i: one store for all of the wavefront's rows
         float mine = 0.0f;
         int r = a1;
 #pragma unroll
         for (int i = 0; i < TA; ++i)
           if (lane == i) {
-            mine = biasA[i] + v[i];
+            mine = (inv * v[i] - minv * rgA[i]) + biasA[i];
             r = a0 + wave + kSW * i;
           }
         if (lane < TA && r < a1) PG_ST32(qkv_x + r, xbits(mine));
@@ -1577,9 +1674,12 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       PG_SLICE(3, w, wn);
 
       // ================= E: c_fc rows + GELU =================
-      float biasE[TE];
+      float rgE[TE], biasE[TE];  // (c_fc follows LN2)
 #pragma unroll
-      for (int i = 0; i < TE; ++i) biasE[i] = cld(w.c_fc_b + row_of(e0, e1, i));
+      for (int i = 0; i < TE; ++i) {
+        rgE[i] = cld(w.c_fc_f + 2 * row_of(e0, e1, i));
+        biasE[i] = cld(w.c_fc_f + 2 * row_of(e0, e1, i) + 1);
+      }
       float scE[TE];
 #pragma unroll
       for (int i = 0; i < TE; ++i) scE[i] = kI8 ? cld(w.c_fc_s + row_of(e0, e1, i)) : 1.0f;
@@ -1593,13 +1693,18 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
           dot_tiles_packed<WB, TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
         else
           dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
+        float inv, minv;
+        if (!wait_ln(ctl, 1, epoch_of(p, t, l, 3), abort_word, inv, minv)) {
+          ok = false;
+          break;
+        }
         // lane i finishes row i: one GELU and one store for all of the wavefront's rows
         float mine = 0.0f;
         int r = e1;
 #pragma unroll
         for (int i = 0; i < TE; ++i)
           if (lane == i) {
-            mine = biasE[i] + v[i];
+            mine = (inv * v[i] - minv * rgE[i]) + biasE[i];
             r = e0 + wave + kSW * i;
           }
         if (lane < TE && r < e1) PG_ST32(p.xch + par * p.xch_set + XchLayout::h(C) + r, xbits(gelu_tanh(mine)));
@@ -1689,11 +1794,15 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       float* const logits = p.logits;
       Tile<J> T[kLmTiles];
       float ts[kLmTiles];  // int8: the scale of the row in T[k]
+      // (the lm_head follows LN_f: the row's W . g and W . b, see stage_scaled)
+      float trg[kLmTiles], tbb[kLmTiles];
 #pragma unroll
       for (int k = 0; k < kLmTiles; ++k) {
         const int row = min(v0 + wave + kSW * k, v1 - 1);
         load_tile<J>(T[k], wte4 + (size_t)row * SP::KC, SP::KC, lane);
         ts[k] = kI8 ? cld(p.lm_s + row) : 1.0f;
+        trg[k] = cld(p.lm_f + 2 * row);
+        tbb[k] = cld(p.lm_f + 2 * row + 1);
       }
       const unsigned epl = epoch_of(p, t, p.L, 5);
       if (!wait_flag(ctl, 4, epl, abort_word)) {
@@ -1710,6 +1819,11 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       } else {
         load_x<J>(xr, lds.xsD, K4, lane);
       }
+      float inv, minv;
+      if (!wait_ln(ctl, 2, epl, abort_word, inv, minv)) {
+        ok = false;
+        break;
+      }
       Best best{-INFINITY, 0xffffffffu};
       for (int r = v0 + wave; r < v1; r += kSW * kLmTiles) {
 #pragma unroll
@@ -1724,10 +1838,13 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
           } else {
             v = dot_tile<J>(T[k], xr);
           }
+          v = (inv * v - minv * trg[k]) + tbb[k];
           {
             const int row = min(rk + kSW * kLmTiles, v1 - 1);
             load_tile<J>(T[k], wte4 + (size_t)row * SP::KC, SP::KC, lane);
             if (kI8) ts[k] = cld(p.lm_s + row);
+            trg[k] = cld(p.lm_f + 2 * row);
+            tbb[k] = cld(p.lm_f + 2 * row + 1);
           }
           if (rk < v1) {
             if (lane == 0) gst(logits + rk, v);
@@ -1775,6 +1892,7 @@ __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) 
     ctl->bdone[threadIdx.x] = 0u;
     ctl->hstat[threadIdx.x] = 0u;
   }
+  if (threadIdx.x < 3) ctl->lnflag[threadIdx.x] = 0u;
   if (threadIdx.x == 0) ctl->halt = 0u;
   __syncthreads();
 
@@ -1877,7 +1995,7 @@ hipError_t launch_arm_exchange(unsigned* x, size_t n, unsigned* status, hipStrea
 }
 
 hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s) {
-  if (!p.lm_w || (p.w_bytes == 1 && !p.lm_s)) return hipErrorInvalidValue;
+  if (!p.lm_w || !p.lm_f || (p.w_bytes == 1 && !p.lm_s)) return hipErrorInvalidValue;
   if (p.w_bytes == 1) return launch_keys<1>(p, s);
   if (p.w_bytes == 2) return launch_keys<2>(p, s);
   if (p.w_bytes == 4) return launch_keys<4>(p, s);

@@ -85,6 +85,7 @@ struct pg_gpt2_model {
   int w_i8 = 0;
   float* lm_w = nullptr;
   float* lm_s = nullptr;
+  float* lm_f = nullptr;  // [2 V]: LN_f folded into the lm_head rows (pgk::launch_ln_fold)
 };
 
 struct pg_logits {
@@ -522,7 +523,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   pgk::DecodeParams p{};
   p.layers = m->d_layers;
   p.wte = m->wte; p.wpe = m->wpe; p.ln_f_g = m->ln_f_g; p.ln_f_b = m->ln_f_b;
-  p.lm_w = m->lm_w; p.lm_s = m->lm_s; p.w_bytes = m->w_i8 ? 1 : m->w_bf16 ? 2 : 4;
+  p.lm_w = m->lm_w; p.lm_s = m->lm_s; p.lm_f = m->lm_f; p.w_bytes = m->w_i8 ? 1 : m->w_bf16 ? 2 : 4;
   p.C = (int)g.C; p.I = (int)g.I; p.H = (int)g.H; p.L = (int)g.L; p.V = (int)g.V; p.P = (int)g.P;
   p.eps = g.eps;
   p.kv = c->kv;
@@ -1070,12 +1071,16 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   // the f32 wte kept beside its quantised copy)
   auto wel = [&](size_t n) { return bf ? (n + 1) / 2 : i8 ? (n + 3) / 4 : n; };
   auto sel = [&](size_t rows) { return i8 ? round_up(rows, A) : 0; };
-  size_t total = round_up(wel(g.V * g.C), A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A);
+  // (lm_f, c_attn_f, c_fc_f: two constants per row, the LayerNorm in front of the matrix folded
+  // into its rows for the persistent decode kernel)
+  size_t total = round_up(wel(g.V * g.C), A) + round_up(g.P * g.C, A) + 2 * round_up(g.C, A) +
+                 round_up(2 * g.V, A);
   if (i8) total += round_up(g.V * g.C, A) + sel(g.V);
   const size_t per_layer = 6 * round_up(g.C, A) + round_up(wel(3 * g.C * g.C), A) +
                            round_up(3 * g.C, A) + round_up(wel(g.C * g.C), A) +
                            2 * round_up(wel(g.C * g.I), A) + round_up(g.I, A) +
-                           sel(3 * g.C) + 2 * sel(g.C) + sel(g.I);
+                           sel(3 * g.C) + 2 * sel(g.C) + sel(g.I) + round_up(6 * g.C, A) +
+                           round_up(2 * g.I, A);
   total += g.L * per_layer;
   PG_HIP(hipMalloc(&m->arena, total * sizeof(float)));
   m->arena_floats = total;
@@ -1139,6 +1144,10 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   if ((s = upload(m->wpe, weights->wpe))) return s;
   if ((s = upload(m->ln_f_g, weights->ln_f_g))) return s;
   if ((s = upload(m->ln_f_b, weights->ln_f_b))) return s;
+  const int wb = i8 ? 1 : bf ? 2 : 4;
+  m->lm_f = place(2 * g.V);
+  PG_HIP(pgk::launch_ln_fold(m->lm_w, wb, m->lm_s, nullptr, m->ln_f_g, m->ln_f_b, g.V, (int)g.C,
+                             m->lm_f, nullptr));
   m->layers.resize(g.L);
   for (size_t l = 0; l < g.L; ++l) {
     const pg_gpt2_block_view& b = weights->blocks[l];
@@ -1158,6 +1167,8 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     float* c_proj_mlp_w = place(wel(g.I * g.C));
     float* c_proj_mlp_s = i8 ? place(g.C) : nullptr;
     float* c_proj_mlp_b = place(g.C);
+    float* c_attn_f = place(6 * g.C);
+    float* c_fc_f = place(2 * g.I);
     if ((s = upload(ln_1_g, b.ln_1_g))) return s;
     if ((s = upload(ln_1_b, b.ln_1_b))) return s;
     if ((s = upload_t(c_attn_w, b.c_attn_w, g.C, 3 * g.C, c_attn_s))) return s;
@@ -1170,9 +1181,13 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     if ((s = upload(c_fc_b, b.c_fc_b))) return s;
     if ((s = upload_t(c_proj_mlp_w, b.c_proj_mlp_w, g.I, g.C, c_proj_mlp_s))) return s;
     if ((s = upload(c_proj_mlp_b, b.c_proj_mlp_b))) return s;
+    PG_HIP(pgk::launch_ln_fold(c_attn_w, wb, c_attn_s, c_attn_b, ln_1_g, ln_1_b, 3 * g.C, (int)g.C,
+                               c_attn_f, nullptr));
+    PG_HIP(pgk::launch_ln_fold(c_fc_w, wb, c_fc_s, c_fc_b, ln_2_g, ln_2_b, g.I, (int)g.C, c_fc_f,
+                               nullptr));
     m->layers[l] = pgk::LayerW{ln_1_g, ln_1_b, c_attn_w, c_attn_b, c_proj_w,     c_proj_b,
                                ln_2_g, ln_2_b, c_fc_w,   c_fc_b,   c_proj_mlp_w, c_proj_mlp_b,
-                               c_attn_s, c_proj_s, c_fc_s, c_proj_mlp_s};
+                               c_attn_s, c_proj_s, c_fc_s, c_proj_mlp_s, c_attn_f, c_fc_f};
   }
   PG_HIP(hipMalloc(&m->d_layers, g.L * sizeof(pgk::LayerW)));
   struct Guard2 {

@@ -19,6 +19,9 @@ struct LayerW {
   const float *c_proj_mlp_w, *c_proj_mlp_b;  // [C][I], [C]
   // int8 storage only (nullptr otherwise): one f32 scale per row of the matrix
   const float *c_attn_s, *c_proj_s, *c_fc_s, *c_proj_mlp_s;
+  // The LayerNorm in front of c_attn and c_fc folded into two constants per row o (launch_ln_fold):
+  // [2 o] = sum_i W[o,i] g[i], [2 o + 1] = bias[o] + sum_i W[o,i] b[i] (persistent decode kernel)
+  const float *c_attn_f, *c_fc_f;
 };
 
 enum Prologue : int { PRO_NONE = 0, PRO_LN = 1, PRO_ATTN_COMBINE = 2 };
@@ -119,6 +122,11 @@ hipError_t launch_attn_finish(const float* part_acc, const float* part_m, const 
                               int H, int head_dim, int nsplit, float* out, hipStream_t s,
                               int batch = 1, BatchStrides bs = BatchStrides{}, int out_packed = 0);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t s);
+// out[2 o] = sum_i W[o,i] g[i], out[2 o + 1] = (bias ? bias[o] : 0) + sum_i W[o,i] b[i] for the
+// rows of W[rows][cols] as stored (w_bytes 4: f32, 2: bf16, 1: int8 with scales[o]); sums in f64.
+hipError_t launch_ln_fold(const void* W, int w_bytes, const float* scales, const float* bias,
+                          const float* g, const float* b, size_t rows, int cols, float* out,
+                          hipStream_t s);
 // dst[i] = bf16(src[i]), round to nearest even
 hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t s);
 // QuantizedRows::from_f32 (src/models/cpu.rs:38-55) for src[rows][cols]: scales[r] =
@@ -202,6 +210,7 @@ struct DecodeParams {
   // its quantised copy lm_w and row scales lm_s (wte stays f32 for the embedding; with bf16
   // rows wte is bf16 as well).
   const float *lm_w, *lm_s;
+  const float* lm_f;  // [2 V]: LN_f folded into the lm_head rows, as LayerW::c_attn_f
   int w_bytes;
   int C, I, H, L, V, P;
   float eps;

@@ -838,6 +838,39 @@ __global__ void k_fill_zero(float* p, size_t n) {
   for (; i < n; i += stride) p[i] = 0.0f;
 }
 
+// One wavefront per row o of W[rows][cols] as stored: out[2 o] = sum_i W[o,i] g[i] and
+// out[2 o + 1] = bias[o] + sum_i W[o,i] b[i], summed in f64.  WB = bytes per weight.
+template <int WB>
+__global__ void k_ln_fold(const void* W, const float* scales, const float* bias, const float* g,
+                          const float* b, size_t rows, int cols, float* out) {
+  const size_t row = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  double sg = 0.0, sb = 0.0;
+  for (int i = lane; i < cols; i += 64) {
+    float w;
+    if (WB == 4) {
+      w = ((const float*)W)[row * cols + i];
+    } else if (WB == 2) {
+      w = __uint_as_float((unsigned)((const unsigned short*)W)[row * cols + i] << 16);
+    } else {
+      // a stored weight is (float)q * scale (QuantizedRows, src/models/cpu.rs:26-56, 173-184)
+      w = (float)((const signed char*)W)[row * cols + i] * scales[row];
+    }
+    sg += (double)w * (double)g[i];
+    sb += (double)w * (double)b[i];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    sg += __shfl_xor(sg, off, 64);
+    sb += __shfl_xor(sb, off, 64);
+  }
+  if (lane == 0) {
+    out[2 * row] = (float)sg;
+    out[2 * row + 1] = (float)((bias ? (double)bias[row] : 0.0) + sb);
+  }
+}
+
 // transpose_in_out (cpu.rs:281-289): 32x32 tiles through LDS.
 __global__ void k_transpose(const float* src, float* dst, int in_f, int out_f) {
   __shared__ float tile[32][33];
@@ -1033,6 +1066,22 @@ hipError_t launch_f32_to_bf16(const float* src, void* dst, size_t n, hipStream_t
   if (blocks == 0) blocks = 1;
   hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)blocks), dim3(256), 0, s, src,
                      reinterpret_cast<unsigned short*>(dst), n);
+  return hipGetLastError();
+}
+
+hipError_t launch_ln_fold(const void* W, int w_bytes, const float* scales, const float* bias,
+                          const float* g, const float* b, size_t rows, int cols, float* out,
+                          hipStream_t s) {
+  if (rows == 0 || cols <= 0 || (w_bytes == 1 && !scales)) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  if (w_bytes == 4)
+    hipLaunchKernelGGL(k_ln_fold<4>, grid, block, 0, s, W, scales, bias, g, b, rows, cols, out);
+  else if (w_bytes == 2)
+    hipLaunchKernelGGL(k_ln_fold<2>, grid, block, 0, s, W, scales, bias, g, b, rows, cols, out);
+  else if (w_bytes == 1)
+    hipLaunchKernelGGL(k_ln_fold<1>, grid, block, 0, s, W, scales, bias, g, b, rows, cols, out);
+  else
+    return hipErrorInvalidValue;
   return hipGetLastError();
 }
 
