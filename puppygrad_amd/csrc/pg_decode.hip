@@ -74,12 +74,24 @@ constexpr unsigned kSpinLimit = 1u << 21;
 // the width and the context length, so it is a launch parameter with one kernel instance each
 // (template parameter KS = steps per slot).
 constexpr int kItemKeysDefault = 128;
-constexpr int kPace = 4;           // loads per pacing group of a slice
+#ifndef PGX_PACE
+#define PGX_PACE 3
+#endif
+#ifndef PGX_PSLEEP
+#define PGX_PSLEEP 4
+#endif
+constexpr int kPace = PGX_PACE;           // loads per pacing group of a slice
 constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
 // Widths whose instances leave registers free request the K and V rows of a workgroup's first
 // attention item at the top of the layer, before they wait for the layer's input: the rows do
 // not depend on the current token, and on these widths nothing else hides their latency.
 constexpr bool early_kv(int C) { return C <= 1024; }
+#ifndef PGX_S0LATE
+#define PGX_S0LATE 0
+#endif
+#ifndef PGX_KVTOUCH
+#define PGX_KVTOUCH 1
+#endif
 
 // Tagged words and the abort word live in global memory; saying so in the pointer type
 // gets global_ instead of flat_ instructions (a flat access also counts as an LDS one).
@@ -235,6 +247,15 @@ typedef __attribute__((address_space(3))) float* lfp;
 typedef __attribute__((address_space(3))) f4* lf4p;
 typedef volatile __attribute__((address_space(3))) unsigned* lvup;
 typedef __attribute__((address_space(3))) unsigned long long* lu64p;
+
+// Asks for one word of the 64-byte line at base + byte_off so that the line is on its way into
+// the L2 of this die; the word itself is not wanted.  Hidden from the compiler like the
+// LDS-destination loads below (it never waits for it); `sink` is the register the word lands in
+// and has to stay reserved until a later load of this wavefront has been waited for.
+__device__ __forceinline__ void touch_line(const void* base, unsigned byte_off, unsigned& sink) {
+  asm volatile("global_load_dword %0, %1, %2" : "+v"(sink) : "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void touch_done(unsigned& sink) { asm volatile("" : "+v"(sink)); }
 
 // One tile = one weight row (or a run of 64*J float4 of one), 64 lanes wide, J deep.
 template <int J>
@@ -556,7 +577,7 @@ __device__ __forceinline__ bool pair_armed(u64 v) {
 // vector read it replaced.)
 typedef unsigned u16x __attribute__((ext_vector_type(16)));
 constexpr unsigned kProbeSpinLimit = 1u << 24;  // a few seconds of scalar probes
-constexpr int kProbeSleep = 4;  // units of 64 clocks between two probes of a wavefront
+constexpr int kProbeSleep = PGX_PSLEEP;  // units of 64 clocks between two probes of a wavefront
 __device__ __forceinline__ void lines3_load(const void* a, const void* b, const void* c, u16x& va,
                                             u16x& vb, u16x& vc) {
   asm volatile(
@@ -907,6 +928,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
   int stopped = 0;
   unsigned tok = 0;
   unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
+  unsigned kv_sink = 0;         // landing register of the K/V touches (touch_line)
   // a wait gave up: tell the streamers and leave
 #define PG_SERVICE_FAIL()        \
   do {                           \
@@ -1019,6 +1041,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         ln_stats<NW>(x, p.eps, lane, inv, minv);
         ln_publish(ctl, 0, inv, minv, epoch_of(p, t, l, 0), lane);
       }
+
       PG_STAMP(l, 0);
 
       // ================= B: this workgroup's (head, split) items =================
@@ -1299,6 +1322,21 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         if (lane == 0) ctl->flag[3] = ep;
       }
       PG_STAMP(l, 4);
+      // The K/V rows of this workgroup's attention item of the next layer do not depend on the
+      // token: their lines are asked for now, one word each, so that the eight wavefronts'
+      // loads of the rows find them in the L2 when the next layer's q is on its way.
+      touch_done(kv_sink);
+      if (PGX_KVTOUCH && l + 1 < p.L && wg < items) {
+        const int h0 = wg / ns, s0 = wg - h0 * ns;
+        const int k0 = s0 * per, k1 = min(pos, k0 + per);  // (row pos is not in the cache yet)
+        const float* kn_ = p.kv + (size_t)(l + 1) * p.kv_layer_stride + ((size_t)h0 * P + k0) * 64;
+        const float* vn_ = kn_ + p.kv_v_offset;
+        const int nl = (k1 - k0) * 4;  // 64-byte lines of a panel's rows
+        for (int i = lane; i < nl; i += 64) {
+          touch_line(kn_, (unsigned)i * 64u, kv_sink);
+          touch_line(vn_, (unsigned)i * 64u, kv_sink);
+        }
+      }
 #undef X_qkv
 #undef X_part
 #undef X_attn
@@ -1602,7 +1640,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       }
       // (a slice goes out the moment the flag is seen where the registers allow it:
       // the service wavefront has just completed a poll and its next ones are early)
-      PG_SLICE(0, w, wn);
+      if (!PGX_S0LATE || early_kv(C_)) PG_SLICE(0, w, wn);
       {
         float v[TA];
         if constexpr (kPacked)
@@ -1627,6 +1665,20 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         if (lane < TA && r < a1) PG_ST32(qkv_x + r, xbits(mine));
       }
       SSTAMP(5);
+      // Where the first item's K/V rows were not requested at the top of the layer they go out
+      // here, in front of the first slice: the attention waits for them, nothing waits for the
+      // slice before the c_proj rows are used (rows come back in the order they were asked for).
+      if (PGX_S0LATE && !early_kv(C_)) {
+        if (wg < items) {
+          const int h0 = wg / ns, s0 = wg - h0 * ns;
+          const int k0 = s0 * per, k1 = min(n, k0 + per);
+          if (k0 < k1) {
+            attn_load_kv(kv, kc, vc, h0, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
+            kv_early = true;
+          }
+        }
+        PG_SLICE(0, w, wn);
+      }
       // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
       {
 #pragma unroll 1
