@@ -89,6 +89,15 @@ constexpr bool early_kv(int C) { return C <= 1024; }
 #ifndef PGX_S0LATE
 #define PGX_S0LATE 0
 #endif
+#ifndef PGX_DRAINF
+#define PGX_DRAINF 1
+#endif
+#ifndef PGX_BURST
+#define PGX_BURST 3
+#endif
+#ifndef PGX_WTOUCH
+#define PGX_WTOUCH 0
+#endif
 #ifndef PGX_KVTOUCH
 #define PGX_KVTOUCH 1
 #endif
@@ -256,6 +265,10 @@ __device__ __forceinline__ void touch_line(const void* base, unsigned byte_off, 
   asm volatile("global_load_dword %0, %1, %2" : "+v"(sink) : "v"(byte_off), "s"(base) : "memory");
 }
 __device__ __forceinline__ void touch_done(unsigned& sink) { asm volatile("" : "+v"(sink)); }
+// The lines of `bytes` bytes from base on (both multiples of 64).
+__device__ __forceinline__ void touch_region(const void* base, unsigned bytes, unsigned& sink, int lane) {
+  for (unsigned i = (unsigned)lane * 64u; i < bytes; i += 4096u) touch_line(base, i, sink);
+}
 
 // One tile = one weight row (or a run of 64*J float4 of one), 64 lanes wide, J deep.
 template <int J>
@@ -364,6 +377,53 @@ __device__ __forceinline__ void dot_tiles(const Tile<J> (&W)[T], lfp xs, int K4s
           acc[i].w += W[i].w[j].w * x[b].w;
         }
       }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < T; ++i) out[i] = wsum((acc[i].x + acc[i].y) + (acc[i].z + acc[i].w));
+}
+
+// The same where a row is JW full column blocks plus a tail of TL < 64 float4, and the tails
+// of the T rows came in one load: lanes [TL i, TL (i + 1)) of `tail` hold the tail of row i.
+template <int T, int JW, int TL, int J>
+__device__ __forceinline__ void dot_tiles_tail(const Tile<J> (&W)[T], const f4& tail, lfp xs, int lane,
+                                               float (&out)[T]) {
+  static_assert(JW < J && T * TL <= 64, "the tails of all rows fit one load");
+  lf4p x4 = (lf4p)xs;
+  f4 acc[T];
+#pragma unroll
+  for (int i = 0; i < T; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+  constexpr int B = 2;
+#pragma unroll
+  for (int j0 = 0; j0 < JW; j0 += B) {
+    f4 x[B];
+    asm volatile("" ::: "memory");  // keeps the LDS reads of later column blocks down here
+#pragma unroll
+    for (int b = 0; b < B; ++b)
+      if (j0 + b < JW) x[b] = x4[lane + 64 * (j0 + b)];
+#pragma unroll
+    for (int b = 0; b < B; ++b)
+      if (j0 + b < JW) {
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+          acc[i].x += W[i].w[j0 + b].x * x[b].x;
+          acc[i].y += W[i].w[j0 + b].y * x[b].y;
+          acc[i].z += W[i].w[j0 + b].z * x[b].z;
+          acc[i].w += W[i].w[j0 + b].w * x[b].w;
+        }
+      }
+  }
+  {
+    const int g = lane / TL;
+    const f4 xt = x4[64 * JW + lane % TL];
+    const f4 pr = f4{tail.x * xt.x, tail.y * xt.y, tail.z * xt.z, tail.w * xt.w};
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      const bool mine = g == i;
+      acc[i].x += mine ? pr.x : 0.0f;
+      acc[i].y += mine ? pr.y : 0.0f;
+      acc[i].z += mine ? pr.z : 0.0f;
+      acc[i].w += mine ? pr.w : 0.0f;
     }
   }
 #pragma unroll
@@ -1240,6 +1300,14 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         if (lane == 0) ctl->flag[1] = epa;
       }
       PG_STAMP(l, 2);
+#if PGX_WTOUCH & 1
+      // experiment: the register part of the mlp projection rows, asked for one hop ahead
+      {
+        const int d0_ = (int)(((long long)wg * C) / G), d1_ = (int)(((long long)(wg + 1) * C) / G);
+        for (int r = d0_; r < d1_; ++r)
+          touch_region((const char*)w.c_proj_mlp_w + (size_t)r * (I * 4) + 13 * 1024, 12 * 1024, kv_sink, lane);
+      }
+#endif
 
       // ---- re-arming the other buffers ----
       // The attention output is complete, so every head's items have run; the items of a head
@@ -1274,7 +1342,9 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           PG_SERVICE_FAIL();
         stage_scaled<NW>(x, g2, lds.xraw2, lds.xsE, lane);
         lds_fence();
+#if !PGX_DRAINF
         vm_drain();  // the arming stores above have been performed
+#endif
         if (lane == 0) ctl->flag[2] = ep;
         float inv, minv;
         ln_stats<NW>(x, p.eps, lane, inv, minv);
@@ -1319,6 +1389,9 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           run = __builtin_amdgcn_readlane((int)mine, __builtin_ctzll(m)) - 1;
         }
         lds_fence();
+#if PGX_DRAINF
+        vm_drain();  // the arming stores have been performed
+#endif
         if (lane == 0) ctl->flag[3] = ep;
       }
       PG_STAMP(l, 4);
@@ -1452,8 +1525,16 @@ struct StreamPlan {
   static constexpr int TA = cdiv(RA, kSW), TE = cdiv(RE, kSW);
   static constexpr int J = cdiv(KC, 64);
   static constexpr int JF = cdiv(KF, 64);  // 16-byte chunks per lane of one 4C-wide row
+  // A C-wide f32 row that is not a whole number of 64-chunk column blocks (n_embd 1600: six
+  // blocks and 16 chunks) would spend a load on its last 16 chunks.  The tails of all rows a
+  // wavefront owns in a band come in ONE load instead (lanes [TL i, TL (i + 1)) take row i's):
+  // JW full blocks per row plus one tail load per band.
+  static constexpr int TL = KC % 64;
+  static constexpr bool kTail = WB == 4 && TL != 0 && TL * (TA > TE ? TA : TE) <= 64;
+  static constexpr int JW = kTail ? KC / 64 : J;
   // loads per layer and wavefront, in stream order
-  static constexpr int ND = J, NE = TE * J, NF = JF, NA = TA * J, NL = ND + NE + NF + NA;
+  static constexpr int ND = kTail ? JW + 1 : J, NE = kTail ? TE * JW + 1 : TE * J, NF = JF,
+                       NA = kTail ? TA * JW + 1 : TA * J, NL = ND + NE + NF + NA;
   // Loads into registers, in stream order:
   //     c_proj row | c_fc rows | mlp projection row | next layer's c_attn rows
   // The widest model cannot hold the c_fc rows next to much of the mlp projection row in
@@ -1472,7 +1553,8 @@ struct StreamPlan {
     if (!kTight) return k == 0 ? 0 : c1 + (k - 1) * (NL - c1) / 5;
     // C = 1600 (the only width that stages): found by measurement within what the
     // registers allow at each product
-    constexpr int c[7] = {0, 9, 20, 31, 48, 66, 81};
+    constexpr int c[7] = {0, 9, 20, 31, 48, 63, 76};
+    static_assert(!kTight || NL == 76, "the cuts are those of n_embd 1600 with packed tails");
     return c[k];
   }
   // of the loads [0, n): those held in registers
@@ -1533,6 +1615,15 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
                                                 : (unsigned)min(ln + 64 * j, SP::KC - 1);
     return ld_row(reinterpret_cast<const f4*>(W) + (size_t)row * SP::KC, c * 16u);
   };
+  // The tails of this wavefront's T rows of the band [r0, r1) in one load (kTail): lane group
+  // g = lane / TL takes chunks 64 JW .. KC - 1 of row g (groups past the rows repeat the last).
+  auto ld_tail = [&](const float* W, int r0, int r1, int T, int ln) -> f4 {
+    constexpr int TLs = SP::TL ? SP::TL : 1;
+    const int g = min(ln / TLs, T - 1);
+    const int row = min(r0 + wave_id() + kSW * g, r1 - 1);
+    const unsigned off = (unsigned)(row - r0) * (unsigned)(SP::KC * 16) + (unsigned)(64 * SP::JW + ln % TLs) * 16u;
+    return ld_row(reinterpret_cast<const f4*>(W) + (size_t)r0 * SP::KC, off);
+  };
   // One chunk of the 4C-wide mlp projection row (f32 rows are whole runs of 64 chunks).
   auto ld_f = [&](const float* W, int row, int j, int ln) -> f4 {
     const unsigned c = (64 * (j + 1) <= SP::KF) ? (unsigned)ln + 64u * j
@@ -1553,23 +1644,36 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       // at most kPace of this wavefront's loads are still in flight.  What the streamers
       // have in flight delays the service wavefront's polls (in-order return per CU), so
       // this bounds that delay by the time of about two groups instead of a whole slice.
-      if (kPaced && n > N0 && (n - N0) % kPace == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
+      if (kPaced && n - N0 >= PGX_BURST && (n - N0 - PGX_BURST) % kPace == 0)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
       const int m = n < SP::PS ? n : n - SP::FS;  // index among the loads into registers
       if (n >= SP::PS && n < SP::PS + SP::FS) {
         const int j = n - SP::PS;
         ld_row_lds(reinterpret_cast<const f4*>(w.c_proj_mlp_w) + (size_t)row_of(d0, d1, 0) * SP::KF,
                    ((unsigned)ln + 64u * j) * 16u, lds.stage + (wave_id() * SP::FS + j) * 256);
       } else if (m < SP::ND) {
-        WD[0].w[m] = ld_c(w.c_proj_w, row_of(d0, d1, 0), m, ln);
+        if (SP::kTail && m == SP::JW)
+          WD[0].w[SP::JW] = ld_tail(w.c_proj_w, d0, d1, 1, ln);
+        else
+          WD[0].w[m] = ld_c(w.c_proj_w, row_of(d0, d1, 0), m, ln);
       } else if (m < SP::ND + SP::NE) {
-        const int i = (m - SP::ND) / J, j = (m - SP::ND) % J;
-        WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
+        // (with packed tails: the rows' full blocks, then the one tail load, kept in row 0's
+        // last register)
+        const int i = (m - SP::ND) / SP::JW, j = (m - SP::ND) % SP::JW;
+        if (SP::kTail && m - SP::ND == TE * SP::JW)
+          WE[0].w[SP::JW] = ld_tail(w.c_fc_w, e0, e1, TE, ln);
+        else
+          WE[i].w[j] = ld_c(w.c_fc_w, row_of(e0, e1, i), j, ln);
       } else if (m < SP::ND + SP::NE + SP::NF - SP::FS) {
         const int j = m - SP::ND - SP::NE + SP::FS;  // FS <= j < NF
         WF.w[j] = ld_f(w.c_proj_mlp_w, row_of(d0, d1, 0), j, ln);
       } else {
-        const int i = (n - SP::ND - SP::NE - SP::NF) / J, j = (n - SP::ND - SP::NE - SP::NF) % J;
-        WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
+        const int idx = n - SP::ND - SP::NE - SP::NF;
+        const int i = idx / SP::JW, j = idx % SP::JW;
+        if (SP::kTail && idx == TA * SP::JW)
+          WA[0].w[SP::JW] = ld_tail(wn.c_attn_w, a0, a1, TA, ln);
+        else
+          WA[i].w[j] = ld_c(wn.c_attn_w, row_of(a0, a1, i), j, ln);
       }
     }
   };
@@ -1645,6 +1749,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         float v[TA];
         if constexpr (kPacked)
           dot_tiles_packed<WB, TA, J>(WA, lds.xsA, SP::KC, lane, scA, v);
+        else if constexpr (SP::kTail)
+          dot_tiles_tail<TA, SP::JW, SP::TL, J>(WA, WA[0].w[SP::JW], lds.xsA, lane, v);
         else
           dot_tiles<TA, J>(WA, lds.xsA, K4, lane, v);
         unsigned* const qkv_x = p.xch + par * p.xch_set + XchLayout::qkv(C);
@@ -1717,6 +1823,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         float v[1];
         if constexpr (kPacked)
           dot_tiles_packed<WB, 1, J>(WD, lds.xsD, SP::KC, lane, scD, v);
+        else if constexpr (SP::kTail)
+          dot_tiles_tail<1, SP::JW, SP::TL, J>(WD, WD[0].w[SP::JW], lds.xsD, lane, v);
         else
           dot_tiles<1, J>(WD, lds.xsD, K4, lane, v);
         const int r = d0 + wave;
@@ -1743,6 +1851,8 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         float v[TE];
         if constexpr (kPacked)
           dot_tiles_packed<WB, TE, J>(WE, lds.xsE, SP::KC, lane, scE, v);
+        else if constexpr (SP::kTail)
+          dot_tiles_tail<TE, SP::JW, SP::TL, J>(WE, WE[0].w[SP::JW], lds.xsE, lane, v);
         else
           dot_tiles<TE, J>(WE, lds.xsE, K4, lane, v);
         float inv, minv;
