@@ -74,34 +74,12 @@ constexpr unsigned kSpinLimit = 1u << 21;
 // the width and the context length, so it is a launch parameter with one kernel instance each
 // (template parameter KS = steps per slot).
 constexpr int kItemKeysDefault = 128;
-#ifndef PGX_PACE
-#define PGX_PACE 3
-#endif
-#ifndef PGX_PSLEEP
-#define PGX_PSLEEP 4
-#endif
-constexpr int kPace = PGX_PACE;           // loads per pacing group of a slice
+constexpr int kPace = 3;           // loads per pacing group of a slice
 constexpr int kLmTiles = 2;        // lm_head rows in flight per streamer
 // Widths whose instances leave registers free request the K and V rows of a workgroup's first
 // attention item at the top of the layer, before they wait for the layer's input: the rows do
 // not depend on the current token, and on these widths nothing else hides their latency.
 constexpr bool early_kv(int C) { return C <= 1024; }
-#ifndef PGX_S0LATE
-#define PGX_S0LATE 0
-#endif
-#ifndef PGX_DRAINF
-#define PGX_DRAINF 1
-#endif
-#ifndef PGX_BURST
-#define PGX_BURST 3
-#endif
-#ifndef PGX_WTOUCH
-#define PGX_WTOUCH 0
-#endif
-#ifndef PGX_KVTOUCH
-#define PGX_KVTOUCH 1
-#endif
-
 // Tagged words and the abort word live in global memory; saying so in the pointer type
 // gets global_ instead of flat_ instructions (a flat access also counts as an LDS one).
 #define PG_G64(p) ((__attribute__((address_space(1))) unsigned long long*)(p))
@@ -637,7 +615,7 @@ __device__ __forceinline__ bool pair_armed(u64 v) {
 // vector read it replaced.)
 typedef unsigned u16x __attribute__((ext_vector_type(16)));
 constexpr unsigned kProbeSpinLimit = 1u << 24;  // a few seconds of scalar probes
-constexpr int kProbeSleep = PGX_PSLEEP;  // units of 64 clocks between two probes of a wavefront
+constexpr int kProbeSleep = 4;  // units of 64 clocks between two probes of a wavefront
 __device__ __forceinline__ void lines3_load(const void* a, const void* b, const void* c, u16x& va,
                                             u16x& vb, u16x& vc) {
   asm volatile(
@@ -754,7 +732,7 @@ __device__ __forceinline__ bool pair_valid(int e, int lane) {
 }
 template <int NW>
 __device__ __forceinline__ bool wave_poll(const unsigned* src, Pairs<NW>& out, unsigned* abort_word, int probe,
-                                          lu64p dbg = nullptr) {
+                                          unsigned& reads, lu64p dbg = nullptr) {
   constexpr int PAIRS = Pairs<NW>::PAIRS, NP = Pairs<NW>::NP, LINES = Pairs<NW>::LINES;
   const int lane = opaque((int)threadIdx.x) & 63;
   unsigned rounds = 0;
@@ -764,6 +742,7 @@ __device__ __forceinline__ bool wave_poll(const unsigned* src, Pairs<NW>& out, u
     if (dbg && lane == 0) *dbg = __builtin_amdgcn_s_memtime();
     bool bad = false;
     int bad_e = 0;
+    ++reads;  // bulk reads of this vector so far (a development figure)
 #pragma unroll
     for (int e = 0; e < NP; ++e) out.v[e] = ld_tagged(src, (unsigned)min(lane + 64 * e, PAIRS - 1) * 8u);
 #pragma unroll
@@ -989,6 +968,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
   unsigned tok = 0;
   unsigned bseq = 0, hseq = 0;  // running counts of attention items and of reads of h
   unsigned kv_sink = 0;         // landing register of the K/V touches (touch_line)
+  unsigned n_xm = 0, n_attn = 0, n_xa = 0;  // development counts of bulk reads per vector
   // a wait gave up: tell the streamers and leave
 #define PG_SERVICE_FAIL()        \
   do {                           \
@@ -1092,7 +1072,8 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
             x.v[e] = ((u64)__float_as_uint(e1) << 32) | (u64)__float_as_uint(e0);
           }
         } else {
-          if (!wave_poll<NW>(p.xch + opar * p.xch_set + XchLayout::xm(C), x, abort_word, wg)) PG_SERVICE_FAIL();
+          if (!wave_poll<NW>(p.xch + opar * p.xch_set + XchLayout::xm(C), x, abort_word, wg, n_xm))
+            PG_SERVICE_FAIL();
         }
         stage_scaled<NW>(x, g2, lds.xraw1, lds.xsA, lane);
         lds_fence();
@@ -1294,20 +1275,12 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // ================= D: attention output -> xsD =================
       {
         Pairs<NW> x;
-        if (!wave_poll<NW>(X_attn, x, abort_word, wg + 1)) PG_SERVICE_FAIL();
+        if (!wave_poll<NW>(X_attn, x, abort_word, wg + 1, n_attn)) PG_SERVICE_FAIL();
         stage_pairs<NW>(x, lds.xsD, lane);
         lds_fence();
         if (lane == 0) ctl->flag[1] = epa;
       }
       PG_STAMP(l, 2);
-#if PGX_WTOUCH & 1
-      // experiment: the register part of the mlp projection rows, asked for one hop ahead
-      {
-        const int d0_ = (int)(((long long)wg * C) / G), d1_ = (int)(((long long)(wg + 1) * C) / G);
-        for (int r = d0_; r < d1_; ++r)
-          touch_region((const char*)w.c_proj_mlp_w + (size_t)r * (I * 4) + 13 * 1024, 12 * 1024, kv_sink, lane);
-      }
-#endif
 
       // ---- re-arming the other buffers ----
       // The attention output is complete, so every head's items have run; the items of a head
@@ -1317,7 +1290,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // LayerNorm of this step).  Nothing reads the other buffers any more, and nothing
       // writes them before the next step, whose first product needs this step's output of every
       // workgroup, this one's included: the stores below are waited for before this
-      // wavefront raises the flag of the c_fc rows.  Each workgroup arms a 256th of each.
+      // wavefront raises the flag of the mlp projection rows.
       // Each workgroup arms a 256th of the other set, in whole 64-byte lines (a partial line
       // would be merged into memory by a read and a write).
       {
@@ -1337,14 +1310,11 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
         load_g2<NW>(g2, w.ln_2_g, ln);
         const unsigned ep = epoch_of(p, t, l, 3);
         Pairs<NW> x;
-        if (!wave_poll<NW>(X_xa, x, abort_word, wg + 2,
+        if (!wave_poll<NW>(X_xa, x, abort_word, wg + 2, n_xa,
                            (p.prof && t + 1 == p.n_fwd) ? lds.ts + l * 16 + 13 : (lu64p) nullptr))
           PG_SERVICE_FAIL();
         stage_scaled<NW>(x, g2, lds.xraw2, lds.xsE, lane);
         lds_fence();
-#if !PGX_DRAINF
-        vm_drain();  // the arming stores above have been performed
-#endif
         if (lane == 0) ctl->flag[2] = ep;
         float inv, minv;
         ln_stats<NW>(x, p.eps, lane, inv, minv);
@@ -1389,9 +1359,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           run = __builtin_amdgcn_readlane((int)mine, __builtin_ctzll(m)) - 1;
         }
         lds_fence();
-#if PGX_DRAINF
         vm_drain();  // the arming stores have been performed
-#endif
         if (lane == 0) ctl->flag[3] = ep;
       }
       PG_STAMP(l, 4);
@@ -1399,7 +1367,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       // token: their lines are asked for now, one word each, so that the eight wavefronts'
       // loads of the rows find them in the L2 when the next layer's q is on its way.
       touch_done(kv_sink);
-      if (PGX_KVTOUCH && l + 1 < p.L && wg < items) {
+      if (l + 1 < p.L && wg < items) {
         const int h0 = wg / ns, s0 = wg - h0 * ns;
         const int k0 = s0 * per, k1 = min(pos, k0 + per);  // (row pos is not in the cache yet)
         const float* kn_ = p.kv + (size_t)(l + 1) * p.kv_layer_stride + ((size_t)h0 * P + k0) * 64;
@@ -1425,7 +1393,7 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
       const unsigned epl = epoch_of(p, t, p.L, 5), ep_best = epoch_of(p, t, p.L, 6);
       // (the raw values go to xraw1, whose next user is the next token's embedding)
       Pairs<NW> x;
-      if (!wave_poll<NW>(p.xch + ((unsigned)(t * p.L + p.L - 1) & 1u) * p.xch_set + XchLayout::xm(C), x, abort_word, wg))
+      if (!wave_poll<NW>(p.xch + ((unsigned)(t * p.L + p.L - 1) & 1u) * p.xch_set + XchLayout::xm(C), x, abort_word, wg, n_xm))
         PG_SERVICE_FAIL();
       stage_scaled<NW>(x, g2, lds.xraw1, lds.xsD, lane);
       lds_fence();
@@ -1472,6 +1440,11 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
     if (lane == 0) {
       lds.ts[p.L * 16 + 14] = wall_clock64();
       lds.ts[p.L * 16 + 15] = __builtin_amdgcn_s_memtime();
+      // bulk reads of the launch: h rounds, block input, attention output, c_proj output
+      lds.ts[p.L * 16 + 8] = hseq;
+      lds.ts[p.L * 16 + 9] = n_xm;
+      lds.ts[p.L * 16 + 10] = n_attn;
+      lds.ts[p.L * 16 + 11] = n_xa;
     }
     lds_fence();
     for (int i = lane; i < (p.L + 1) * 16; i += 64)
@@ -1644,8 +1617,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       // at most kPace of this wavefront's loads are still in flight.  What the streamers
       // have in flight delays the service wavefront's polls (in-order return per CU), so
       // this bounds that delay by the time of about two groups instead of a whole slice.
-      if (kPaced && n - N0 >= PGX_BURST && (n - N0 - PGX_BURST) % kPace == 0)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
+      if (kPaced && n > N0 && (n - N0) % kPace == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPace) : "memory");
       const int m = n < SP::PS ? n : n - SP::FS;  // index among the loads into registers
       if (n >= SP::PS && n < SP::PS + SP::FS) {
         const int j = n - SP::PS;
@@ -1744,7 +1716,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
       }
       // (a slice goes out the moment the flag is seen where the registers allow it:
       // the service wavefront has just completed a poll and its next ones are early)
-      if (!PGX_S0LATE || early_kv(C_)) PG_SLICE(0, w, wn);
+      PG_SLICE(0, w, wn);
       {
         float v[TA];
         if constexpr (kPacked)
@@ -1771,20 +1743,6 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
         if (lane < TA && r < a1) PG_ST32(qkv_x + r, xbits(mine));
       }
       SSTAMP(5);
-      // Where the first item's K/V rows were not requested at the top of the layer they go out
-      // here, in front of the first slice: the attention waits for them, nothing waits for the
-      // slice before the c_proj rows are used (rows come back in the order they were asked for).
-      if (PGX_S0LATE && !early_kv(C_)) {
-        if (wg < items) {
-          const int h0 = wg / ns, s0 = wg - h0 * ns;
-          const int k0 = s0 * per, k1 = min(n, k0 + per);
-          if (k0 < k1) {
-            attn_load_kv(kv, kc, vc, h0, P, k0, pos, wave * 4 + (lane >> 4), lane & 15);
-            kv_early = true;
-          }
-        }
-        PG_SLICE(0, w, wn);
-      }
       // ---- attention: this wavefront's slots of the workgroup's (head, split) items ----
       {
 #pragma unroll 1
