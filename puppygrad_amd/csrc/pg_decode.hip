@@ -646,6 +646,34 @@ __device__ __forceinline__ unsigned lines3_written(const unsigned* a, const unsi
   for (int i = 0; i < 16; ++i) m = min(m, min(~va[i], min(~vb[i], ~vc[i])));
   return m;
 }
+// Eight single f32 words, `stride` bytes apart from base on: nonzero iff none is armed.
+__device__ __forceinline__ unsigned words8_written(const unsigned* base, unsigned stride, unsigned last) {
+  const char* b = (const char*)base;
+  // (word k of the eight, or the last one asked for again)
+  const char* a0 = b;
+  const char* a1 = b + stride * min(1u, last);
+  const char* a2 = b + stride * min(2u, last);
+  const char* a3 = b + stride * min(3u, last);
+  const char* a4 = b + stride * min(4u, last);
+  const char* a5 = b + stride * min(5u, last);
+  const char* a6 = b + stride * min(6u, last);
+  const char* a7 = b + stride * min(7u, last);
+  unsigned v0, v1, v2, v3, v4, v5, v6, v7;
+  asm volatile(
+      "s_load_dword %0, %8, 0x0 glc\n\t"
+      "s_load_dword %1, %9, 0x0 glc\n\t"
+      "s_load_dword %2, %10, 0x0 glc\n\t"
+      "s_load_dword %3, %11, 0x0 glc\n\t"
+      "s_load_dword %4, %12, 0x0 glc\n\t"
+      "s_load_dword %5, %13, 0x0 glc\n\t"
+      "s_load_dword %6, %14, 0x0 glc\n\t"
+      "s_load_dword %7, %15, 0x0 glc\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(v0), "=&s"(v1), "=&s"(v2), "=&s"(v3), "=&s"(v4), "=&s"(v5), "=&s"(v6), "=&s"(v7)
+      : "s"(a0), "s"(a1), "s"(a2), "s"(a3), "s"(a4), "s"(a5), "s"(a6), "s"(a7)
+      : "memory");
+  return min(min(min(~v0, ~v1), min(~v2, ~v3)), min(min(~v4, ~v5), min(~v6, ~v7)));
+}
 // Spins until lines la, lb, lc (64 bytes each) of src are written: all their tagged words
 // carry `epoch` (TAGGED), or none of their f32 words is armed.  Wave-uniform; false on
 // timeout or abort.
@@ -1209,30 +1237,28 @@ __device__ __forceinline__ void service_wave(const DecodeParams& p, ctlp ctl, co
           h = slot / ns;
           if (slot - h * ns != 0) continue;
         }
-        // the head's ns partials (66 words each) are one run of tagged words: probe the
-        // last word of every partial, then read them all into LDS (the staging area of
-        // the long vector, idle now) and merge from there
+        // the head's ns partials (66 words each) are one run of words: probe the last word of
+        // (up to eight of) the partials through the scalar path, then read them all into LDS
+        // (the staging area of the long vector, idle now) and merge from there
         const unsigned* src = X_part + (size_t)h * ns * 66;
         const int nw = ns * 66;
         lfp stage = lds.xsF;
         unsigned spins = 0;
         for (;;) {
           {
-            const unsigned off = (unsigned)(min(lane, ns - 1) * 66 + 65) * 4u;
             bool ok = true;
             for (;;) {
-              const unsigned v = ld_word(src, off);
-              if (__all(v != kArm)) break;
-              if (++spins > kSpinLimit) {
+              if (words8_written(src + 65, 66u * 4u, (unsigned)(ns - 1)) != 0) break;
+              if (++spins > kProbeSpinLimit) {
                 PG_ST32(abort_word, 1u);
                 ok = false;
                 break;
               }
-              if ((spins & 15) == 0 && PG_LD32(abort_word) != 0) {
+              if ((spins & 127) == 0 && PG_LD32(abort_word) != 0) {
                 ok = false;
                 break;
               }
-              __builtin_amdgcn_s_sleep(2);
+              __builtin_amdgcn_s_sleep(kProbeSleep);
             }
             if (!ok) PG_SERVICE_FAIL();
           }
