@@ -424,8 +424,10 @@ pg_status pg_gpt2_load_config(const char* path, pg_gpt2_config* out);
 /* load_gpt2_tuning (src/main.rs:2564-2586): reads the `hip` object of a puppygrad-tune.json
  * written by the autotune scan (SavedGpt2Tuning, src/main.rs:2611-2623, with `hip` in the place
  * of `rust`) and copies its tunables into the fields of *options that are still 0.  A file
- * that does not exist is not an error (*found = 0); an unreadable or malformed one is
- * PG_ASSET ("failed to read tuning file ...", "failed to parse tuning file ..."). */
+ * that does not exist, or one without a `hip` object (the file is shared between backends: the
+ * reference's own scan writes one with only `rust`), is not an error (*found = 0, the defaults
+ * stand); an unreadable or malformed one is PG_ASSET ("failed to read tuning file ...",
+ * "failed to parse tuning file ..."). */
 pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t* found);
 
 /* Gpt2Runtime::from_dir_with_backend without the tokenizer

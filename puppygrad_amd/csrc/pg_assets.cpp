@@ -603,11 +603,13 @@ pg_status pg_gpt2_load_config(const char* path, pg_gpt2_config* out) {
 pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t* found) {
   if (!path || !options) return fail(PG_INVALID_INPUT, "null argument");
   if (found) *found = 0;
+  errno = 0;  // (an earlier call's value must not decide what a failed open means)
   std::ifstream in(path, std::ios::binary);
   if (!in) {
-    if (errno == ENOENT) return PG_OK;  // load_gpt2_tuning: a missing default file is no error
+    const int why = errno;
+    if (why == ENOENT) return PG_OK;  // load_gpt2_tuning: a missing default file is no error
     return fail(PG_ASSET, std::string("failed to read tuning file ") + path + ": " +
-                              std::strerror(errno));
+                              std::strerror(why ? why : EIO));
   }
   std::stringstream buf;
   buf << in.rdbuf();
@@ -616,10 +618,17 @@ pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t*
   std::string err;
   if (!JsonParser(text.data(), text.data() + text.size()).parse(root, err))
     return fail(PG_ASSET, std::string("failed to parse tuning file ") + path + ": " + err);
-  const Json* hip = root.kind == Json::Obj ? root.find("hip") : nullptr;
-  if (!hip || hip->kind != Json::Obj)
+  if (root.kind != Json::Obj)
     return fail(PG_ASSET, std::string("failed to parse tuning file ") + path +
-                              ": missing field `hip`");
+                              ": expected an object of per-backend tunings");
+  // The file is shared with the other backends: the reference's own `autotune gpt2` writes one
+  // with only a `rust` object (SavedGpt2Tuning, src/main.rs:2564-2623).  Without a `hip`
+  // object there is no tuning for this backend and the defaults stand.
+  const Json* hip = root.find("hip");
+  if (!hip || hip->kind == Json::Null) return PG_OK;
+  if (hip->kind != Json::Obj)
+    return fail(PG_ASSET, std::string("failed to parse tuning file ") + path +
+                              ": invalid type for field `hip`, expected an object");
   struct Field {
     const char* key;
     uint32_t* dst;

@@ -349,8 +349,12 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 // (its 24 significant bits in three groups of 8, by truncation), W's values are bf16 as they
 // are, so x . w = hi . w + mid . w + lo . w with every product exact in f32 and the sums
 // accumulated in f32 as before.  Three v_mfma_f32_32x32x16_bf16 do per 16 columns what eight
-// v_mfma_f32_32x32x2_f32 of four times the duration did.  (A NaN or an infinity in the input
-// gives NaN in its row of the result, as inf - inf does in the split.)
+// v_mfma_f32_32x32x2_f32 of four times the duration did.  An infinity or a NaN in the input
+// stays whole in the first part, so it meets the weights as it would in f32.  One case differs
+// from the f32 product: an infinite WEIGHT meets the zero second and third parts of a value that
+// fits the first (0 * inf), and the sum is NaN where f32 arithmetic gives an infinity.  (Where W
+// is f32 and cut as well, k_gemm_b9, the same happens to an infinite INPUT against a weight
+// whose second or third part is zero.)
 // 256 threads = 4 wavefronts (2 x 2) on a BM x BN tile; k-tiles of 32 columns, staged in LDS
 // row-major ([row][32 bf16] = 64 bytes, the three input planes and W): the operand of a lane
 // is 16 consecutive bytes of its row (8 columns; lanes 32..63 take the second 8 of a 16-column
@@ -374,7 +378,12 @@ __device__ __forceinline__ Split3 split3_bf16(f4 x) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     h[j] = __float_as_uint(x[j]) & 0xffff0000u;
-    const float r1 = x[j] - __uint_as_float(h[j]);  // exact: the 16 low bits of the significand
+    // exact: the 16 low bits of the significand.  An infinity or a NaN stays whole in the first
+    // part (inf - inf would make the other two NaN): its products and sums then behave as in
+    // f32 arithmetic.  (A NaN whose payload lies only in its 16 low bits, which no arithmetic
+    // produces, would read as an infinity.)
+    const bool finite = (__float_as_uint(x[j]) & 0x7f800000u) != 0x7f800000u;
+    const float r1 = finite ? x[j] - __uint_as_float(h[j]) : 0.0f;
     m[j] = __float_as_uint(r1) & 0xffff0000u;
     const float r2 = r1 - __uint_as_float(m[j]);    // exact: at most 8 significant bits left
     l[j] = __float_as_uint(r2);

@@ -100,7 +100,8 @@ def test_malformed_tuning_files_are_asset_errors(tmp_path):
     found = C.c_int32(5)
     assert lib.pg_hip_load_tuning(str(tmp_path / "absent.json").encode(), C.byref(opts), C.byref(found)) == 0
     assert found.value == 0
-    for text, why in [("{", "failed to parse tuning file"), ('{"rust": {}}', "missing field `hip`"),
+    for text, why in [("{", "failed to parse tuning file"), ("[1]", "expected an object of per-backend tunings"),
+                      ('{"hip": 3}', "invalid type for field `hip`"),
                       ('{"hip": {"attn_item_keys": "x"}}', "invalid type for field `attn_item_keys`"),
                       ('{"hip": {"attn_blocks_per_cu": -1}}', "invalid type for field `attn_blocks_per_cu`"),
                       ('{"hip": {"gemm_split_items_per_cu": 2.5}}', "expected u32")]:
@@ -108,6 +109,15 @@ def test_malformed_tuning_files_are_asset_errors(tmp_path):
         p.write_text(text)
         assert lib.pg_hip_load_tuning(str(p).encode(), C.byref(opts), C.byref(found)) == _lib.PG_ASSET
         assert why in lib.pg_last_error_message().decode()
+    # a file the reference's own `autotune gpt2` wrote (SavedGpt2Tuning, main.rs:2611-2623: a `rust`
+    # object and no `hip`) is no tuning for this backend, and no error
+    for text in ['{"rust": {"parallel_attention_min_tokens": 64}}', '{"hip": null}', "{}"]:
+        p.write_text(text)
+        opts = _lib.pg_hip_options()
+        found = C.c_int32(5)
+        assert lib.pg_hip_load_tuning(str(p).encode(), C.byref(opts), C.byref(found)) == 0
+        assert found.value == 0
+        assert (opts.attn_item_keys, opts.attn_blocks_per_cu, opts.gemm_split_items_per_cu) == (0, 0, 0)
     p.write_text('{"hip": {"attn_item_keys": 256, "unknown": 1, "attn_blocks_per_cu": null}}')
     opts = _lib.pg_hip_options()
     assert lib.pg_hip_load_tuning(str(p).encode(), C.byref(opts), C.byref(found)) == 0 and found.value == 1

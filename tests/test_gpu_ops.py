@@ -95,6 +95,44 @@ def test_dense_with_selection_weights_returns_the_inputs_bit_for_bit(rows, k, n)
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,k,n", [(1024, 1024, 4096), (1024, 4096, 1024), (48, 768, 2304)])
+def test_dense_keeps_infinities_and_nans_of_the_input(rows, k, n):
+    """dot (cpu.rs:231-254) carries an infinite or NaN input into the sums as f32 arithmetic
+    does: +inf times a positive weight is +inf, opposite infinities in one row give NaN, a NaN
+    stays a NaN, and rows without such a value are untouched.  48 rows run on the f32 matrix cores
+    and must show exactly that.  The first two shapes run on the bf16 matrix cores with x AND W
+    cut into three bf16 parts each (whole tiles; tiles cut in four along K): a non-finite input
+    stays whole in its first part, so every affected output is non-finite with the reference's
+    sign where it is an infinity; against a weight whose second or third part is zero (about one
+    f32 weight in 130) the product 0 * inf makes it NaN instead, the one stated difference."""
+    rng = np.random.default_rng(rows + k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    x[3, 5] = np.inf           # one infinity: the sign of w[o, 5] decides
+    x[7, 11] = -np.inf
+    x[9, 2], x[9, k - 1] = np.inf, -np.inf   # both in a row: inf - inf somewhere, or +-inf
+    x[12, 40] = np.nan
+    x[rows - 1, k - 3] = np.inf
+    w[5, 5] = 0.0              # inf * 0 is NaN in f32 as well
+    got = hip_dense(x.reshape(-1), rows, k, n, w.reshape(-1), b).reshape(rows, n)
+    with np.errstate(invalid="ignore"):
+        want = oracle.transposed_dense(x.reshape(-1), rows, k, n, w.reshape(-1), b).reshape(rows, n)
+    assert np.isnan(want[3, 5]) and np.isinf(want[3]).sum() == n - 1 and np.isnan(want[12]).all()
+    fin = np.isfinite(want)
+    np.testing.assert_array_equal(np.isfinite(got), fin)
+    np.testing.assert_allclose(got[fin], want[fin], atol=3e-5, rtol=1e-5)
+    assert np.isnan(got[np.isnan(want)]).all()
+    if rows < 1024:
+        np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
+        np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
+    else:
+        inf = np.isinf(got)
+        np.testing.assert_array_equal(got[inf], want[inf])         # an infinity has the reference's sign
+        extra = np.isnan(got) & np.isinf(want)
+        assert extra.sum() <= 0.03 * np.isinf(want).sum(), (extra.sum(), np.isinf(want).sum())
+
+
 def test_dense_reference_unit_vector():
     # src/models/cpu.rs:312-327
     x, weight = patterned(6, 0.2), patterned(12, 0.1)

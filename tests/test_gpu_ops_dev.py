@@ -108,6 +108,38 @@ def test_quantized_rows_and_quantized_dense_match_oracle(rows, in_f, out_f):
         d.free()
 
 
+@pytest.mark.parametrize("rows,in_f,out_f", [(12, 384, 1536), (150, 1280, 5120)])
+def test_quantized_dense_keeps_infinities_and_nans_of_the_input(rows, in_f, out_f):
+    """quantized_dot (cpu.rs:173-184) in f32 arithmetic: an infinite input gives +-inf by the sign
+    of the weight (NaN against a zero weight), a NaN gives NaN.  12 rows run on the 32-row kernel
+    and 150 on the tile kernel, both on the bf16 matrix cores with the inputs cut into three bf16
+    parts: a non-finite value has to stay whole in the first part."""
+    rng = np.random.default_rng(rows)
+    w = (rng.standard_normal((out_f, in_f)) / np.sqrt(in_f)).astype(np.float32)
+    x = rng.standard_normal((rows, in_f)).astype(np.float32)
+    x[1, 3] = np.inf
+    x[2, 7] = -np.inf
+    x[4, 9] = np.nan
+    x[rows - 1, in_f - 1] = np.inf
+    lib = _lib.load()
+    dw, dq, ds = DeviceArray(w), DeviceArray(np.zeros((out_f, in_f)), np.int8), DeviceArray(np.zeros(out_f))
+    ok(lib.pg_op_quantize_rows_dev(0, None, dw.ptr, out_f, in_f, dq.ptr, ds.ptr))
+    q, sc = dq.download(), ds.download()
+    dx, dy = DeviceArray(x), DeviceArray(np.zeros((rows, out_f)))
+    ok(lib.pg_op_quantized_dense_dev(0, None, dx.ptr, rows, in_f, out_f, dq.ptr, ds.ptr, None, dy.ptr))
+    got = dy.download()
+    with np.errstate(invalid="ignore"):
+        want = x @ (q.astype(np.float32) * sc[:, None]).T
+    assert np.isinf(want[1]).sum() > out_f // 2 and np.isnan(want[4]).all()
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
+    np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
+    fin = np.isfinite(want)
+    np.testing.assert_allclose(got[fin], want[fin], atol=5e-5, rtol=1e-4)
+    for d in (dw, dq, ds, dx, dy):
+        d.free()
+
+
 @pytest.mark.parametrize("Tq,Tk,state,heads,causal", [(1, 1, 8, 2, 0), (5, 5, 24, 3, 1), (6, 1500, 384, 6, 0),
                                                       (40, 40, 384, 6, 1), (3, 700, 1280, 20, 0),
                                                       (9, 4, 64, 1, 1), (2, 33, 512, 2, 0)])

@@ -113,6 +113,12 @@ def test_model_directory_tuning_file_is_read(tmp_path):
     assert "attn_item_keys=128" in text and "attn_blocks_per_cu=8" in text
     tuned = load_gpt2_tuning(None, d)
     assert tuned.attn_item_keys == 256
+    # a directory the reference's own scan has tuned (only a `rust` object in the file) loads with
+    # this backend's defaults
+    (d / "puppygrad-tune.json").write_text(json.dumps(
+        {"model": "gpt2", "backend": "rust", "rust": {"parallel_attention_min_tokens": 64}}))
+    text = Gpt2Model.from_dir(d).describe()
+    assert "attn_item_keys=128" in text and "attn_blocks_per_cu=4" in text and "gemm_split_items_per_cu=3" in text
 
 
 def test_autotune_scan_end_to_end(tmp_path):
