@@ -158,3 +158,36 @@ def test_config5_gpt2_xl_bf16_batch32_subsample():
         nxt = np.argmax(logits, axis=1).astype(np.uint32)
         for b in check:
             nxt[b] = int(np.argmax(want[b]))
+
+
+def test_config5_full_depth_sequence0_to_the_context_limit():
+    """Benchmark configuration 5 at its full depth on the full model (XL, 48 layers, bf16 weights,
+    batch 32, 512-token prompts, 511 steps to position 1022): sequence 0 is teacher-forced with
+    the oracle's greedy tokens through every step, the other 31 sequences follow their own argmax.
+    Its logits are compared with the oracle's (on the rounded weights, f32 tolerance) at the first
+    step, at about 1000 keys and at the last two positions, so that what 48 layers of the
+    three-part bf16 products do to the error at nearly full context is pinned, not only its
+    start."""
+    cfg = Gpt2Config(**synth.GPT2_XL)
+    B, n = 32, 512
+    steps = cfg.n_positions - 1 - n  # forwards at positions 512..1022
+    w = synth.bf16_rounded(synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 5))
+    ids = synth.token_ids(B * n, synth.TOKEN_SEED_BASE + 5, cfg.vocab_size).reshape(B, n)
+    model, ref = Gpt2Model.new(cfg, w, BF16), oracle.Model(cfg, w, oracle.rust_config(16))
+    cache = model.new_kv_cache(B)
+    logits = model.prefill_batch(ids, cache).to_host()
+    rc = ref.new_kv_cache()
+    want = ref.prefill(ids[0], rc)
+    assert_logits_close(logits[0], want, what="prefill seq 0")
+    checked = {0, 255, 487, 488, steps - 2, steps - 1}  # positions 512, 767, 999, 1000, 1021, 1022
+    worst = 0.0
+    for step in range(steps):
+        nxt = np.argmax(logits, axis=1).astype(np.uint32)
+        nxt[0] = int(np.argmax(want))
+        logits = model.forward_one_batch(nxt, cache).to_host()
+        want = ref.forward_one(int(nxt[0]), rc)
+        if step in checked:
+            assert_logits_close(logits[0], want, what=f"step {step} (position {n + step}) seq 0")
+            worst = max(worst, float(np.abs(logits[0] - want).max()))
+    assert cache.seq_len == cfg.n_positions - 1 and rc.seq_len == cfg.n_positions - 1
+    print(f"config 5 full depth: max |logit error| of sequence 0 at the checked steps {worst:.2e}")
