@@ -245,7 +245,13 @@ pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* model, pg_kv_cache* c
  * on_token / forward_one until max_new_tokens, n_positions or EOS.  on_token may
  * be NULL; a non-zero return from it stops generation and is reported as
  * PG_INVALID_INPUT.  out_ids must hold n + max_new entries and receives prompt
- * plus generated ids. */
+ * plus generated ids.
+ * A greedy stream without a repeat penalty runs as launches of up to 64 forwards of the fused
+ * decode kernel, and on_token is called while such a launch is running and the process-wide
+ * lock of that kernel is held.  The callback therefore must not call the model (that is
+ * refused with PG_INVALID_INPUT) and must not wait for another thread that does: that thread
+ * cannot start its own launch before this one has ended.  After a callback has asked to stop,
+ * the launch still finishes its forwards (at most 63) before the call returns. */
 typedef int (*pg_on_token)(uint32_t token_id, void* user);
 pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* model, const uint32_t* ids,
                                               size_t n, uint32_t max_new, int64_t eos,
@@ -331,6 +337,11 @@ pg_status pg_device_download(int32_t device, void* dst_host, const void* src_dev
  * (a hipStream_t, NULL for the default stream) and nothing is waited for, so a model that
  * shares these kernels (src/models/whisper/runtime.rs:43-47 is where a backend would plug
  * in) keeps its activations in HBM from one op to the next. */
+/* Limits of these entry points (PG_INVALID_INPUT beyond them): in_features and LayerNorm cols
+ * up to 16320 (a row is staged in 64 KiB of LDS), at most 2^20 rows per dense call.
+ * pg_op_dense_dev and pg_op_dense_in_out_dev need a bias (the reference's signatures take one:
+ * pass zeros for none); pg_op_quantized_dense_dev accepts bias == NULL for the bare
+ * quantized_dot per row. */
 /* transposed_dense_projection_into (cpu.rs:58-75): weight is [out,in]. */
 pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t rows,
                           uint64_t in_features, uint64_t out_features, const float* weight,

@@ -174,10 +174,10 @@ pg_status validate_config(const pg_gpt2_config& c) {
     return fail(PG_INVALID_CONFIG, "layer_norm_epsilon must be > 0");
   // Limits of this backend (no reference counterpart): vectors are staged in
   // 64 KiB of LDS and indices are 32-bit.
-  const uint64_t lds_floats = 16384;
+  const uint64_t lds_floats = pgh::kMaxStagedFloats;
   if (c.n_embd > lds_floats || c.n_inner > lds_floats || c.n_positions > lds_floats)
     return fail(PG_INVALID_CONFIG,
-                "hip backend supports n_embd, n_inner and n_positions up to 16384");
+                "hip backend supports n_embd, n_inner and n_positions up to 16320");
   if (c.vocab_size > (1ull << 31) || c.n_layer > 4096)
     return fail(PG_INVALID_CONFIG, "hip backend supports vocab_size < 2^31 and n_layer <= 4096");
   return PG_OK;
@@ -1962,6 +1962,9 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
         if (take()) continue;
         if (!running) break;  // the kernel has ended without writing this id: it gave up
         if (hipStreamQuery(c->stream) != hipErrorNotReady) running = false;  // one more look
+        // (a token takes the kernel 0.2 - 1.3 ms: a short pause between two looks leaves the
+        // core's memory pipeline to whatever else runs on it)
+        for (int k = 0; k < 32; ++k) __builtin_ia32_pause();
       }
       size_t done = 0;
       bool stopped = false;
@@ -2038,8 +2041,8 @@ pg_status pg_gpt2_stream_token_ids_profiled(const pg_gpt2_model* m, const uint32
 pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in_f,
                       uint64_t out_f, const float* weight, const float* bias, float* out) {
   if (!x || !weight || !bias || !out) return fail(PG_INVALID_INPUT, "null argument");
-  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30))
-    return fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  if (in_f == 0 || in_f > pgh::kMaxStagedFloats || out_f == 0 || out_f > (1u << 30))
+    return fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16320], out_features >= 1");
   pg_status s;
   if ((s = select_device(device))) return s;
   DevBuf dx, dw, db, dy;
@@ -2079,8 +2082,8 @@ pg_status pg_op_dense(int32_t device, const float* x, uint64_t rows, uint64_t in
 pg_status pg_op_layer_norm(int32_t device, float* x, uint64_t rows, uint64_t cols,
                            const float* gamma, const float* beta, float eps) {
   if (!x || !gamma || !beta) return fail(PG_INVALID_INPUT, "null argument");
-  if (cols == 0 || cols > 16384 || rows > (1u << 30))
-    return fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16384]");
+  if (cols == 0 || cols > pgh::kMaxStagedFloats || rows > (1u << 30))
+    return fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16320]");
   pg_status s;
   if ((s = select_device(device))) return s;
   if (rows == 0) return PG_OK;
@@ -2144,8 +2147,8 @@ pg_status pg_op_attention_decode(int32_t device, const float* qkv, uint64_t pos,
                                  float* values, uint64_t max_seq_len, uint64_t n_head,
                                  uint64_t head_dim, float* out) {
   if (!qkv || !keys || !values || !out) return fail(PG_INVALID_INPUT, "null argument");
-  if (n_head == 0 || head_dim == 0 || max_seq_len == 0 || max_seq_len > 16384 ||
-      n_head * head_dim > 16384)
+  if (n_head == 0 || head_dim == 0 || max_seq_len == 0 || max_seq_len > pgh::kMaxStagedFloats ||
+      n_head * head_dim > pgh::kMaxStagedFloats)
     return fail(PG_INVALID_INPUT, "attention: dimensions out of range");
   if (pos >= max_seq_len)
     return fail(PG_INVALID_INPUT, "cache is full at seq_len " + std::to_string(pos));

@@ -8,6 +8,11 @@
 
 namespace pgh {
 
+// Vectors a kernel stages in LDS (a LayerNorm row, the input of a matrix-vector product, the
+// scores of the generic attention kernel) take this many floats at most: 64 KiB of dynamic LDS
+// less the kernels' small static blocks.
+constexpr unsigned long long kMaxStagedFloats = 16320;
+
 // Records `msg` as the calling thread's last error message and returns `s`.
 __attribute__((visibility("hidden"))) pg_status fail(pg_status s, const std::string& msg);
 

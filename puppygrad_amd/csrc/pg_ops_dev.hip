@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <mutex>
 #include <string>
 
@@ -214,8 +215,8 @@ pg_status pg_op_attention_decode_noalloc(int32_t device, void* stream, const flo
                                          uint64_t max_seq_len, uint64_t n_head, uint64_t head_dim,
                                          float* out) {
   if (!qkv || !keys || !values || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
-  if (n_head == 0 || head_dim == 0 || max_seq_len == 0 || max_seq_len > 16384)
-    return pgh::fail(PG_INVALID_INPUT, "attention: dimensions out of range");
+  if (n_head == 0 || head_dim == 0 || max_seq_len == 0 || max_seq_len > pgh::kMaxStagedFloats)
+    return pgh::fail(PG_INVALID_INPUT, "attention: n_head, head_dim >= 1 and max_seq_len in [1,16320]");
   if (n_head > kNoAllocMaxHeads || n_head * head_dim > kNoAllocMaxWidth)
     return pgh::fail(PG_INVALID_INPUT,
                      "attention without allocation: n_head " + std::to_string(n_head) +
@@ -250,8 +251,9 @@ pg_status pg_op_dense_dev(int32_t device, void* stream, const float* x, uint64_t
                           uint64_t in_f, uint64_t out_f, const float* weight, const float* bias,
                           float* out) {
   if (!x || !weight || !bias || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
-  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
-    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  if (in_f == 0 || in_f > pgh::kMaxStagedFloats || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
+    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16320], out_features >= 1, "
+                                       "at most 1048576 rows");
   pg_status s;
   if ((s = select_device(device))) return s;
   if (rows == 0) return PG_OK;
@@ -284,11 +286,16 @@ pg_status pg_op_dense_in_out_dev(int32_t device, void* stream, const float* x, u
   pg_status s;
   if ((s = select_device(device))) return s;
   if (rows == 0) return PG_OK;
-  const dim3 grid((unsigned)((out_f + kBlk - 1) / kBlk), (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock));
-  hipLaunchKernelGGL(k_dense_in_out, grid, dim3(kBlk), kRowsPerBlock * in_f * sizeof(float),
-                     static_cast<hipStream_t>(stream), x, (int)rows, (int)in_f, (int)out_f, weight,
-                     bias, out);
-  PG_HIP(hipGetLastError());
+  // (a launch's second grid dimension holds 65535 blocks: more rows go out in several launches)
+  const uint64_t rows_per_launch = 65535ull * kRowsPerBlock;
+  for (uint64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
+    const uint64_t nr = std::min(rows - r0, rows_per_launch);
+    const dim3 grid((unsigned)((out_f + kBlk - 1) / kBlk), (unsigned)((nr + kRowsPerBlock - 1) / kRowsPerBlock));
+    hipLaunchKernelGGL(k_dense_in_out, grid, dim3(kBlk), kRowsPerBlock * in_f * sizeof(float),
+                       static_cast<hipStream_t>(stream), x + r0 * in_f, (int)nr, (int)in_f, (int)out_f,
+                       weight, bias, out + r0 * out_f);
+    PG_HIP(hipGetLastError());
+  }
   return PG_OK;
 }
 
@@ -309,8 +316,9 @@ pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x
                                     uint64_t in_f, uint64_t out_f, const int8_t* q,
                                     const float* scales, const float* bias, float* out) {
   if (!x || !q || !scales || !out) return pgh::fail(PG_INVALID_INPUT, "null argument");
-  if (in_f == 0 || in_f > 16384 || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
-    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16384], out_features >= 1");
+  if (in_f == 0 || in_f > pgh::kMaxStagedFloats || out_f == 0 || out_f > (1u << 30) || rows > (1u << 20))
+    return pgh::fail(PG_INVALID_INPUT, "dense: in_features must be in [1,16320], out_features >= 1, "
+                                       "at most 1048576 rows");
   pg_status s;
   if ((s = select_device(device))) return s;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -340,8 +348,8 @@ pg_status pg_op_quantized_dense_dev(int32_t device, void* stream, const float* x
 pg_status pg_op_layer_norm_dev(int32_t device, void* stream, float* x, uint64_t rows, uint64_t cols,
                                const float* gamma, const float* beta, float eps) {
   if (!x || !gamma || !beta) return pgh::fail(PG_INVALID_INPUT, "null argument");
-  if (cols == 0 || cols > 16384 || rows > (1u << 30))
-    return pgh::fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16384]");
+  if (cols == 0 || cols > pgh::kMaxStagedFloats || rows > (1u << 30))
+    return pgh::fail(PG_INVALID_INPUT, "layer_norm: cols must be in [1,16320]");
   pg_status s;
   if ((s = select_device(device))) return s;
   if (rows == 0) return PG_OK;

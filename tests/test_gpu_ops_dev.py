@@ -213,4 +213,29 @@ def test_device_ops_refuse_bad_shapes():
     assert b"state must be heads * head_dim" in lib.pg_last_error_message()
     assert lib.pg_op_attention_dev(0, None, one.ptr, one.ptr, one.ptr, 1, 0, 8, 2, 0, one.ptr) == _lib.PG_INVALID_INPUT
     assert lib.pg_op_layer_norm_dev(0, None, None, 1, 8, one.ptr, one.ptr, 1e-5) == _lib.PG_INVALID_INPUT
+    # the limits a row staged in LDS sets, refused before any launch
+    assert lib.pg_op_layer_norm_dev(0, None, one.ptr, 1, 16321, one.ptr, one.ptr, 1e-5) == _lib.PG_INVALID_INPUT
+    assert b"cols must be in [1,16320]" in lib.pg_last_error_message()
+    assert lib.pg_op_dense_dev(0, None, one.ptr, 1, 16321, 4, one.ptr, one.ptr, one.ptr) == _lib.PG_INVALID_INPUT
+    assert b"in_features must be in [1,16320]" in lib.pg_last_error_message()
+    assert lib.pg_op_dense_dev(0, None, one.ptr, (1 << 20) + 1, 8, 4, one.ptr, one.ptr, one.ptr) == _lib.PG_INVALID_INPUT
+    assert lib.pg_op_attention_decode_noalloc(0, None, one.ptr, 0, one.ptr, one.ptr, 16321, 2, 4, one.ptr) == _lib.PG_INVALID_INPUT
+    assert b"max_seq_len in [1,16320]" in lib.pg_last_error_message()
+    # dense without a bias: only the quantised projection takes NULL
+    assert lib.pg_op_dense_dev(0, None, one.ptr, 1, 8, 1, one.ptr, None, one.ptr) == _lib.PG_INVALID_INPUT
     one.free()
+
+
+def test_dense_in_out_more_rows_than_one_launch_holds():
+    """[in,out] dense with 262,200 rows of 2 values: the rows go out in two launches (a launch's
+    second grid dimension ends at 65535 blocks of four rows)."""
+    rows, in_f, out_f = 262200, 2, 3
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((rows, in_f)).astype(np.float32)
+    w = rng.standard_normal((in_f, out_f)).astype(np.float32)
+    b = rng.standard_normal(out_f).astype(np.float32)
+    dx, dw, db, dy = DeviceArray(x), DeviceArray(w), DeviceArray(b), DeviceArray(np.zeros((rows, out_f)))
+    ok(_lib.load().pg_op_dense_in_out_dev(0, None, dx.ptr, rows, in_f, out_f, dw.ptr, db.ptr, dy.ptr))
+    np.testing.assert_allclose(dy.download(), x @ w + b, atol=1e-5, rtol=1e-5)
+    for d in (dx, dw, db, dy):
+        d.free()
