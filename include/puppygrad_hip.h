@@ -261,11 +261,16 @@ pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* model, const 
 
 /* Gpt2OperationProfile (src/models/gpt2/rust.rs:336-347) in seconds, accumulated over the
  * prefill and the decode steps of one generation as forward_one_profiled and
- * prefill_profiled do (rust.rs:906-1006, 1136-1250).  The spans are measured with HIP
- * events between the launches of the per-operation decode path.  On this backend a
- * LayerNorm runs inside the launch of the projection that consumes it, so its time is
- * part of that projection's bucket and layer_norm_s stays 0; tokenization_s and
- * decoding_s are tokenizer work (rust.rs:473-478, 651), 0 for streams of token ids. */
+ * prefill_profiled do (rust.rs:906-1006, 1136-1250), taken from the path generations are
+ * timed on: HIP events between the launches of the GEMM prefill, and for every decode
+ * forward the fused decode kernel's own time stamps (the moment an operation's input is
+ * staged and the moment its rows are published; a hand-over between workgroups counts for the
+ * operation that waits for it), so that the buckets of a generation add up to its prefill
+ * and decode time on the device.  Models the fused kernel does not cover are timed with
+ * events between the launches of the per-operation path instead.  A LayerNorm has no span of
+ * its own on either path (it runs inside, or is folded into, the projection that consumes
+ * it): layer_norm_s only holds the LayerNorm launches of the GEMM prefill.  tokenization_s
+ * and decoding_s are tokenizer work (rust.rs:473-478, 651), 0 for streams of token ids. */
 typedef struct pg_gpt2_operation_profile {
   double tokenization_s;
   double layer_norm_s;
@@ -278,11 +283,11 @@ typedef struct pg_gpt2_operation_profile {
   double decoding_s;
 } pg_gpt2_operation_profile;
 
-/* pg_gpt2_stream_token_ids_with_stats with every forward (the prompt's included, token by
- * token as prefill_profiled does) run as separate launches per operation and timed into
- * `profile` (must not be NULL).  Tokens are the same as the unprofiled stream's; the
- * wall-clock fields of `stats` include the per-step synchronisation the timing needs, so
- * throughput is quoted from the unprofiled call. */
+/* pg_gpt2_stream_token_ids_with_stats with its time on the device split into `profile`
+ * (must not be NULL): the prompt through pg_gpt2_prefill_profiled, every decode forward as a
+ * launch of its own.  Tokens are the same as the unprofiled stream's; the wall-clock fields
+ * of `stats` include the per-step synchronisation the timing needs, so throughput is quoted
+ * from the unprofiled call. */
 pg_status pg_gpt2_stream_token_ids_profiled(const pg_gpt2_model* model, const uint32_t* ids,
                                             size_t n, uint32_t max_new, int64_t eos,
                                             const pg_sampling* sampling, uint64_t seed,

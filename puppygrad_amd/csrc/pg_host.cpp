@@ -142,6 +142,9 @@ struct pg_kv_cache {
   size_t best_words = 0;  // 64-bit words at best_t
   size_t x_words = 0;     // 32-bit words at xch
   unsigned xch_set = 0;   // words from one set of exchange vectors to the other
+  // [grid][L + 1][16] time stamps of a profiled forward of the persistent kernel (allocated on
+  // first use; pg_gpt2_stream_token_ids_profiled)
+  unsigned long long* stamps = nullptr;
   size_t tagged_bytes = 0;  // size of that allocation as the exchange pool counts it
   unsigned* status = nullptr;
   unsigned* h_status = nullptr;  // pinned
@@ -508,7 +511,7 @@ struct PersistentRun {
 pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
                            bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
                            size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
-                           bool timed, PersistentRun* run) {
+                           bool timed, PersistentRun* run, unsigned long long* stamps = nullptr) {
   const Cfg& g = m->cfg;
   if (t_persistent_in_flight)
     return fail(PG_INVALID_INPUT,
@@ -552,6 +555,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   if (m->item_keys_auto && m->item_keys_256_ok && pos0 + n_fwd / 2 > 128 && pos0 + n_fwd <= 256)
     p.item_keys = 256;
   p.status = c->status;
+  p.prof = stamps;  // the kernel's own time stamps of the launch's last forward, if wanted
 #ifdef PG_DECODE_PROF_BUILD
   // Development builds only: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
   // of the last token of each persistent launch (raw u64, [grid][L+1][16]).
@@ -619,10 +623,11 @@ pg_status persistent_end(pg_kv_cache* c, PersistentRun* run, size_t* done, bool*
 pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
                          bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
                          size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
-                         size_t* done, bool* stopped, bool timed) {
+                         size_t* done, bool* stopped, bool timed,
+                         unsigned long long* stamps = nullptr) {
   PersistentRun run;
   pg_status s = persistent_begin(m, c, force_ids, lm_last_only, tok_from_ptr, tok, pos0, n_fwd,
-                                 select_last, eos, out_ids_dev, timed, &run);
+                                 select_last, eos, out_ids_dev, timed, &run, stamps);
   if (s) return s;
   return persistent_end(c, &run, done, stopped);
 }
@@ -1355,6 +1360,7 @@ void pg_kv_cache_destroy(pg_kv_cache* c) {
     (void)hipFree(c->hbuf);
     if (c->gemm_ws) (void)hipFree(c->gemm_ws);
     if (c->seq_scratch) (void)hipFree(c->seq_scratch);
+    if (c->stamps) (void)hipFree(c->stamps);
     (void)hipFree(c->part_acc);
     (void)hipFree(c->part_m);
     (void)hipFree(c->part_l);
@@ -1869,6 +1875,56 @@ static pg_status forward_one_profiled(const pg_gpt2_model* m, pg_kv_cache* c, ui
   return want_logits ? finish_logits(c, out) : PG_OK;
 }
 
+// One forward of the persistent kernel (the path generations are timed on) with its time added
+// to the buckets of `profile`.  The kernel stamps its own phases with the shader clock
+// (workgroup 0: the service wavefront when a phase's input is staged, streamer 0 when its rows
+// are published) and two readings of the 100 MHz clock give the rate.  A span belongs to the
+// operation that is waiting or multiplying in it:
+//   end of the previous layer (or token start) -> c_attn rows published   qkv_projection
+//   -> attention output staged (q hand-over, items, merge, gather)         attention
+//   -> c_proj rows published                                               attention_projection
+//   -> c_fc rows published (hand-over, LayerNorm statistics, product)      mlp_fc_projection
+//   -> mlp projection rows published                                       mlp_projection
+//   last layer -> end of the launch (LN_f, lm_head, argmax)                final_logits
+// so the buckets of a forward add up to the launch's duration.  LayerNorm has no span of its
+// own here (it is folded into the rows that follow it): layer_norm_s stays 0.
+static pg_status forward_one_stamped(const pg_gpt2_model* m, pg_kv_cache* c, uint32_t id,
+                                     pg_gpt2_operation_profile* profile, pg_logits** out) {
+  pg_status s;
+  if ((s = check_compatible(m, c))) return s;
+  if (id >= m->cfg.V)  // rust.rs:951-956
+    return fail(PG_INVALID_INPUT, "token id " + std::to_string(id) + " exceeds vocab_size " +
+                                      std::to_string(m->cfg.V));
+  if ((s = check_step(m, c))) return s;
+  if ((s = select_device(m->device))) return s;
+  const size_t L = m->cfg.L, row = (L + 1) * 16;
+  if (!c->stamps) PG_HIP(hipMalloc(&c->stamps, (size_t)m->persistent_grid * row * 8));
+  if ((s = run_persistent(m, c, nullptr, false, false, id, c->seq_len, 1, false, -1, nullptr, nullptr,
+                          nullptr, false, c->stamps)))
+    return s;
+  std::vector<unsigned long long> t(row);  // workgroup 0's stamps
+  PG_HIP(hipMemcpy(t.data(), c->stamps, row * 8, hipMemcpyDeviceToHost));
+  auto at = [&](size_t layer, int slot) { return (double)t[layer * 16 + slot]; };
+  const double s0 = at(L, 7), w0 = at(L, 13), w1 = at(L, 14), s1 = at(L, 15);
+  if (!(s1 > s0) || !(w1 > w0))
+    return fail(PG_BACKEND, "persistent decode kernel left no time stamps");
+  const double sec_per_tick = (w1 - w0) * 1e-8 / (s1 - s0);  // 100 MHz wall clock over shader ticks
+  double prev = s0;
+  for (size_t l = 0; l < L; ++l) {
+    const double a_store = at(l, 5), d_flag = at(l, 2), d_store = at(l, 11), e_store = at(l, 6),
+                 f_store = at(l, 7);
+    profile->qkv_projection_s += (a_store - prev) * sec_per_tick;
+    profile->attention_s += (d_flag - a_store) * sec_per_tick;
+    profile->attention_projection_s += (d_store - d_flag) * sec_per_tick;
+    profile->mlp_fc_projection_s += (e_store - d_store) * sec_per_tick;
+    profile->mlp_projection_s += (f_store - e_store) * sec_per_tick;
+    prev = f_store;
+  }
+  profile->final_logits_s += (s1 - prev) * sec_per_tick;
+  c->seq_len += 1;  // rust.rs:1004
+  return finish_logits(c, out);
+}
+
 static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t n,
                              uint32_t max_new, int64_t eos, const pg_sampling* sampling,
                              uint64_t seed, pg_on_token on_token, void* user, uint32_t* out_ids,
@@ -1888,9 +1944,17 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
   auto first_start = Clock::now();
   auto prefill_start = Clock::now();
   pg_logits* logits = nullptr;
-  if (profile) {
-    // prefill_profiled (rust.rs:906-927): the checks of prefill, then the prompt token by
-    // token, logits from the last one
+  // The profile describes the path that is timed: the prompt through the GEMM prefill with an
+  // event after each launch, every decode forward through the persistent kernel with its own
+  // time stamps.  (Models the persistent kernel does not cover, or more than 63 layers: the
+  // per-operation launches with events between them, the prompt token by token as
+  // prefill_profiled does, rust.rs:906-927.)
+  const bool stamped = profile && use_persistent(m, c) && m->cfg.L + 1 <= 64;
+  if (profile && stamped) {
+    pg_gpt2_operation_profile pre{};
+    if ((s = pg_gpt2_prefill_profiled(m, c, ids, n, &logits, &pre))) return s;
+    *profile = pre;
+  } else if (profile) {
     if ((s = validate_input(m->cfg, ids, n))) return s;
     if ((s = pg_kv_cache_clear(c))) return s;
     for (size_t i = 0; i < n; ++i)
@@ -1994,7 +2058,9 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
     if (first_token_s < 0) first_token_s = since(first_start);
     bool needs_next = generated < max_new && output.size() < m->cfg.P;
     if (needs_next) {
-      if (profile)
+      if (stamped)
+        s = forward_one_stamped(m, c, tok, profile, &logits);
+      else if (profile)
         s = forward_one_profiled(m, c, tok, true, &marks, profile, &logits);
       else
         s = pg_gpt2_forward_one(m, c, tok, &logits);

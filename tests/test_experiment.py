@@ -140,6 +140,38 @@ def test_profiled_stream_matches_the_plain_stream_and_fills_the_buckets():
 
 
 @pytest.mark.gpu
+def test_profiled_stream_of_the_persistent_path_is_taken_from_its_own_time_stamps():
+    """A GPT-2 width: decode forwards run on the persistent kernel, and the profiled stream takes
+    its buckets from that kernel's own time stamps (one launch per forward) and from events
+    between the launches of the GEMM prefill: same tokens as the plain stream and the oracle,
+    greedy and sampled, every operation bucket filled, and the spans inside the run."""
+    cfg = synth.Gpt2Config(vocab_size=523, n_positions=96, n_embd=768, n_layer=3, n_head=12)
+    w = synth.random_weights(cfg, 0x5EED0233, std=0.08, perturb=True)
+    model, ref = Gpt2Model.new(cfg, w), oracle.Model(cfg, w, oracle.rust_config(8))
+    assert "decode=persistent" in model.describe()
+    ids = list(synth.token_ids(20, 0x70C00233, cfg.vocab_size))
+    gen = TextGenerationConfig(max_new_tokens=16)
+    plain, _ = model.stream_token_ids_with_stats(ids, gen)
+    got, pst, prof = model.stream_token_ids_with_stats(ids, gen, profiled=True)
+    want, _, logits, gaps = ref.stream_token_ids_with_stats(ids, 16, None, want_logits=True)
+    assert got == plain
+    if (gaps > 2 * (1e-4 + 1e-3 * np.abs(logits).max())).all():
+        assert got == want
+    op = [prof.qkv_projection, prof.attention, prof.attention_projection, prof.mlp_fc_projection,
+          prof.mlp_projection, prof.final_logits]
+    assert all(v > 0.0 for v in op), op
+    assert prof.layer_norm >= 0.0 and prof.tokenization == prof.decoding == 0.0
+    assert sum(op) + prof.layer_norm <= pst.prefill_time + pst.decode_time
+    # 15 decode forwards of a few tens of microseconds each, plus the prefill's launches
+    assert 15 * 10e-6 < sum(op) < 15 * 2e-3 + 5e-3, op
+    samp = TextGenerationConfig(max_new_tokens=10, temperature=0.9, top_k=20, seed=7)
+    assert model.stream_token_ids_with_stats(ids, samp)[0] == \
+        model.stream_token_ids_with_stats(ids, samp, profiled=True)[0]
+    toks, lst, _ = model.stream_token_ids_with_stats(ids, TextGenerationConfig(max_new_tokens=200), profiled=True)
+    assert len(toks) == cfg.n_positions and lst.generated_tokens == cfg.n_positions - 20
+
+
+@pytest.mark.gpu
 def test_experiment_rows_on_the_device():
     cfg, w = _c128()
     model = Gpt2Model.new(cfg, w)
