@@ -235,9 +235,12 @@ def measure_decode(model, cfg, ids, n_prefill, steps, warmup, int8=False, bf16=F
             "bytes_per_launch": bytes_per_launch, "algo_bytes": algo_bytes, "persistent": persistent, "kernel": kernel}
 
 
-def hbm_roofline(achieved_gbs, kernel, **extra):
-    return {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel, **extra}
+def hbm_roofline(achieved_gbs, kernel, traffic=None, traffic_source=None, **extra):
+    r = {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": kernel, **extra}
+    if traffic_source:
+        r["traffic_source"] = traffic_source
+    return r
 
 
 def secondary_workloads(xl_cfg, xl_weights):
@@ -256,21 +259,26 @@ def secondary_workloads(xl_cfg, xl_weights):
         "value": round(d["tok_s"], 1), "unit": "tokens/s", "steps": 96, "ms_per_step": round(d["ms_per_step"], 4),
         "gpu_ms_per_step": round(d["gpu_ms_per_step"], 4),
         "reference_metric_tokens_per_s": round(d["tokens"] / d["wall"], 1),
-        "roofline": hbm_roofline(d["achieved"], d["kernel"], launches=d["launches"],
+        "roofline": hbm_roofline(d["achieved"], d["kernel"],
+                                 traffic=round(TRAFFIC_RATIO_124M * d["algo_bytes"] * 96),
+                                 traffic_source=TRAFFIC_SOURCE_124M, launches=d["launches"],
                                  launch_ms=round(d["launch_s"] * 1e3, 3),
                                  algorithmic_bytes_per_forward=int(d["algo_bytes"]))}
     out["gpt2_124m_prefill_32"] = measure_short_prefill(model, cfg, ids, 32, 60, 6)
     ids = synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size)
     out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 60, 6)
     del model, w
-    # GPT-2 355M: batch-16 decode steps from 128-token prompts
+    # GPT-2 355M: batch-16 decode steps around the mean cache length of configuration 3
+    # (128-token prompts + 256 tokens: 129..383 keys, mean 256)
     cfg = Gpt2Config(**synth.GPT2_MEDIUM)
     model = Gpt2Model.new(cfg, synth.random_weights(cfg, synth.WEIGHT_SEED_BASE + 3))
-    out["gpt2_355m_decode_b16"] = measure_batch_decode(model, cfg, 16, 128, 64, False)
+    out["gpt2_355m_decode_b16"] = measure_batch_decode(model, cfg, 16, 220, 64, False,
+                                                       traffic_ratio=TRAFFIC_RATIO_355M_B16)
     del model
-    # GPT-2 XL with bf16-stored weights: batch-32 decode steps from 512-token prompts
+    # GPT-2 XL with bf16-stored weights: batch-32 decode steps around the mean cache length of
+    # configuration 5 (512-token prompts + 512 tokens: 513..1023 keys, mean 768)
     model = Gpt2Model.new(xl_cfg, xl_weights, Gpt2HipConfig(weight_storage=_lib.PG_STORE_BF16))
-    out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 512, 24, True)
+    out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 752, 24, True)
     out["gpt2_xl_bf16_prefill_b32_512"] = measure_batch_prefill_bf16(model, xl_cfg, 32, 512, 3)
     del model
     return out
@@ -331,7 +339,7 @@ def measure_prefill(model, cfg, ids, T, steps, warmup):
                                "frac": round(attn / FP32_MFMA_PEAK_TFLOPS, 4), "flops": int(attn_flops)}}
 
 
-def measure_batch_decode(model, cfg, B, n_prefill, steps, bf16):
+def measure_batch_decode(model, cfg, B, n_prefill, steps, bf16, traffic_ratio=None):
     """B sequences prefilled to n_prefill tokens each, then `steps` greedy steps for all of them.
     A step reads every weight once plus the K/V rows of every sequence: HBM-bound."""
     from puppygrad_amd import synth
@@ -353,6 +361,8 @@ def measure_batch_decode(model, cfg, B, n_prefill, steps, bf16):
                         f"tokens, weights stored as {'bf16' if bf16 else 'f32'}, fp32 arithmetic",
             "value": round(B / sec, 1), "unit": "tokens/s", "steps": n, "ms_per_step": round(sec * 1e3, 4),
             "roofline": hbm_roofline(achieved, "all launches of one batched step",
+                                     traffic=round(traffic_ratio * (wbytes + kvb)) if traffic_ratio else None,
+                                     traffic_source=TRAFFIC_SOURCE_355M_B16 if traffic_ratio else None,
                                      algorithmic_bytes_per_step=int(wbytes + kvb))}
 
 
@@ -508,8 +518,15 @@ def _devinfo():
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by what the same
 # counter reads for a plain copy kernel of known size
 # (profiles/k_decode_persistent_1600_xl_decode_traffic.txt has the counters and the factors).
-TRAFFIC_RATIO_XL = 1.028
+TRAFFIC_RATIO_XL = 1.0256
 TRAFFIC_SOURCE = "profiles/k_decode_persistent_1600_xl_decode_traffic.txt"
+# The same for k_decode_persistent<768> on the 124M decode (127 forwards from 32 tokens) and for
+# the launches of one 355M batch-16 step (16 steps at 224..239 keys), from runs of this file
+# with --model small and with --workload batch-decode.
+TRAFFIC_RATIO_124M = 0.983
+TRAFFIC_SOURCE_124M = "profiles/k_decode_persistent_768_124m_decode.txt"
+TRAFFIC_RATIO_355M_B16 = 1.093
+TRAFFIC_SOURCE_355M_B16 = "profiles/batched_decode_355m_b16_xl_bf16_b32.txt"
 
 
 def measured_traffic(args, n_prefill, persistent, bytes_per_launch):

@@ -3,6 +3,7 @@ a development build of the library takes inside the kernel.
 
     python -m puppygrad_amd.build --stamps
     python -m puppygrad_amd.decode_stamps small|medium|xl [n_prefill] [n_tokens]
+    python -m puppygrad_amd.decode_stamps --read <file of raw stamps> <n_layer>
 
 The build compiles the library with PG_DECODE_PROF_BUILD (libpuppygrad_hip_stamps.so); a launch
 then keeps, for its last token, the shader clock (s_memtime) of every phase of every layer in LDS
@@ -18,34 +19,32 @@ import numpy as np
 from . import build as _build
 
 
-def main(argv):
-    os.environ.setdefault("PUPPYGRAD_HIP_LIB", str(_build.STAMPS_LIB_PATH))
-    # (a caller may name the file of raw stamps itself, to keep it)
-    out = os.environ.setdefault("PG_DECODE_PROF", os.path.join(tempfile.gettempdir(), "pg_decode_stamps.bin"))
-    from . import Gpt2Config, Gpt2Model, synth  # after the environment is set: the library loads on import
-    name = argv[1] if len(argv) > 1 else 'small'
-    kw = {'xl': synth.GPT2_XL, 'small': synth.GPT2_SMALL, 'medium': synth.GPT2_MEDIUM}[name]
-    cfg = Gpt2Config(**kw)
-    npre = int(argv[2]) if len(argv) > 2 else {'xl': 896, 'small': 32, 'medium': 128}[name]
-    ntok = int(argv[3]) if len(argv) > 3 else 33
-    w = synth.random_weights(cfg, 1)
-    ids = synth.token_ids(npre, 2, cfg.vocab_size)
-    m = Gpt2Model.new(cfg, w)
-    c = m.new_kv_cache()
-    m.prefill(ids, c)
-    toks, st = m.decode_greedy(c, ntok)
-    print(name, 'decode', st.gpu_decode_time / (ntok - 1) * 1e3, 'ms/token (with stamps)')
-    L = cfg.n_layer
-    raw = np.fromfile(out, dtype=np.uint64).reshape(-1, L + 1, 16).astype(np.float64)
-    G = raw.shape[0]
-    # per-WG conversion of shader-clock stamps to the global 100 MHz wall clock
+def analyse(path, L, show=print):
+    """Prints the per-hop table from a file of raw stamps ([workgroup][L + 1][16] u64)."""
+    raw = np.fromfile(path, dtype=np.uint64).reshape(-1, L + 1, 16).astype(np.float64)
+    # per-workgroup conversion of shader-clock stamps to the 100 MHz wall clock
     S0, W0, W1, S1 = raw[:, L, 7], raw[:, L, 13], raw[:, L, 14], raw[:, L, 15]
     rate = (S1 - S0) / (W1 - W0)   # shader ticks per wall tick
-    print('shader clock: %.1f MHz (min %.1f max %.1f)' % (rate.mean() * 100, rate.min() * 100, rate.max() * 100))
+    show('shader clock: %.1f MHz (min %.1f max %.1f)' % (rate.mean() * 100, rate.min() * 100, rate.max() * 100))
     a = np.where(raw > 0, (W0[:, None, None] + (raw - S0[:, None, None]) / rate[:, None, None]) * 0.01, 0.0)
-    a[:, L, 13] = W0 * 0.01; a[:, L, 14] = W1 * 0.01
-    t_origin = a[:, L, 7][a[:, L, 7] > 0].min()
-    a = np.where(a > 0, a - t_origin + 1.0, 0.0)
+    # The wall clocks of the eight XCDs are offset against each other by up to a few microseconds
+    # (the same amounts at every event of a run, other amounts in the next run).  Workgroup g runs
+    # on XCD g % 8: each XCD's mean deviation from the all-workgroup mean over the events of
+    # layers 1.. is taken as its offset and removed, so that "first" and "last workgroup" compare
+    # times and not clocks.
+    events = [0, 5, 2, 11, 3, 6, 4, 7]
+    dev = np.zeros(a.shape[0])
+    for k in events:
+        v = a[:, 1:L, k]
+        dev += (v - v.mean(axis=0, keepdims=True)).mean(axis=1)
+    dev /= len(events)
+    off = np.array([dev[x::8].mean() for x in range(8)])
+    show('clock offsets of the XCDs removed (us): ' + ' '.join('%+.2f' % o for o in off))
+    b = a.copy()
+    for x in range(8):
+        b[x::8] -= off[x]
+    a = np.where(a > 0, b, 0.0)
+
     def col(l, k):
         v = a[:, l, k]
         return v[v > 0]
@@ -53,7 +52,7 @@ def main(argv):
     rows = []
     for l in range(1, L):
         F_prev = col(l - 1, 7).max()          # last F store of the previous layer (streamer 0 of each WG)
-        A_flag = col(l, 0)                    # service: xsA staged, flag raised
+        A_flag = col(l, 0)                    # service: xsA staged, flag raised, statistics published
         A_store = col(l, 5)                   # streamer 0: A rows published
         B_done = col(l, 1)                    # service: attention items done (partials / attn published)
         D_flag = col(l, 2)
@@ -74,8 +73,39 @@ def main(argv):
              'F flag->F store (product)', 'LAYER', 'spread A flag', 'spread D flag', 'spread E flag', 'spread F flag',
              'last F store->FIRST A flag', 'last D store->FIRST E flag', 'last E store->FIRST F flag', 'last B done->FIRST D flag']
     for n_, v in zip(names, r.T):
-        print(f'{n_:32s} mean {v.mean():6.2f}  min {v.min():6.2f}  max {v.max():6.2f}')
-    print('token span', a[:, L, 6].max() - a[:, L, 7][a[:, L, 7] > 0].min())
+        show(f'{n_:32s} mean {v.mean():6.2f}  min {v.min():6.2f}  max {v.max():6.2f}')
+    # one workgroup's own clock: the pieces of the c_fc hand-over
+    d = lambda k1, k0: raw[:, 1:L, k1] - raw[:, 1:L, k0]
+    us = lambda v: (v / rate[:, None] * 0.01)
+    if (raw[:, 1:L, 14] > 0).all() and (raw[:, 1:L, 15] > 0).all():
+        show('c_fc input, per workgroup: probe round trip %.2f, probe ok -> vector read back %.2f, -> statistics published %.2f'
+             % (us(d(13, 14)).mean(), us(d(15, 13)).mean(), us(d(3, 15)).mean()))
+    show('tail: last F store -> final input staged %.2f, -> argmax published %.2f (lm_head); token start -> first input staged %.2f'
+         % (us(raw[:, L, 5] - raw[:, L - 1, 7]).mean(), us(raw[:, L, 6] - raw[:, L, 5]).mean(),
+            us(raw[:, 0, 0] - raw[:, L, 7]).mean()))
+
+
+def main(argv):
+    if len(argv) > 3 and argv[1] == '--read':  # a file of raw stamps kept from an earlier run
+        analyse(argv[2], int(argv[3]))
+        return
+    os.environ.setdefault("PUPPYGRAD_HIP_LIB", str(_build.STAMPS_LIB_PATH))
+    # (a caller may name the file of raw stamps itself, to keep it)
+    out = os.environ.setdefault("PG_DECODE_PROF", os.path.join(tempfile.gettempdir(), "pg_decode_stamps.bin"))
+    from . import Gpt2Config, Gpt2Model, synth  # after the environment is set: the library loads on import
+    name = argv[1] if len(argv) > 1 else 'small'
+    kw = {'xl': synth.GPT2_XL, 'small': synth.GPT2_SMALL, 'medium': synth.GPT2_MEDIUM}[name]
+    cfg = Gpt2Config(**kw)
+    npre = int(argv[2]) if len(argv) > 2 else {'xl': 896, 'small': 32, 'medium': 128}[name]
+    ntok = int(argv[3]) if len(argv) > 3 else 33
+    w = synth.random_weights(cfg, 1)
+    ids = synth.token_ids(npre, 2, cfg.vocab_size)
+    m = Gpt2Model.new(cfg, w)
+    c = m.new_kv_cache()
+    m.prefill(ids, c)
+    toks, st = m.decode_greedy(c, ntok)
+    print(name, 'decode', st.gpu_decode_time / (ntok - 1) * 1e3, 'ms/token (with stamps)')
+    analyse(out, cfg.n_layer)
 
 
 if __name__ == "__main__":
