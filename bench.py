@@ -265,6 +265,7 @@ def secondary_workloads(xl_cfg, xl_weights):
                                  launch_ms=round(d["launch_s"] * 1e3, 3),
                                  algorithmic_bytes_per_forward=int(d["algo_bytes"]))}
     out["gpt2_124m_prefill_32"] = measure_short_prefill(model, cfg, ids, 32, 60, 6)
+    out["gpt2_124m_sampled_stream_b1"] = measure_sampled_stream(model, ids, 128)
     ids = synth.token_ids(1024, synth.TOKEN_SEED_BASE + 2, cfg.vocab_size)
     out["gpt2_124m_prefill_1024"] = measure_prefill(model, cfg, ids, 1024, 60, 6)
     del model, w
@@ -282,6 +283,34 @@ def secondary_workloads(xl_cfg, xl_weights):
     out["gpt2_xl_bf16_prefill_b32_512"] = measure_batch_prefill_bf16(model, xl_cfg, 32, 512, 3)
     del model
     return out
+
+
+def measure_sampled_stream(model, ids, n_new):
+    """stream_token_ids_with_stats (rust.rs:548-634) with sampled selection: prompt, then n_new
+    tokens whose selection (sample_logits, generation.rs:300-362) runs on the device between the
+    forwards, no host round trip per token.  Rates are generated tokens over the decode loop's
+    wall time, best of three streams; the greedy stream of the same length stands beside them."""
+    from puppygrad_amd import TextGenerationConfig
+
+    def rate(**kw):
+        best = 0.0
+        for _ in range(3):
+            _, st = model.stream_token_ids_with_stats(ids, TextGenerationConfig(n_new, seed=7, **kw))
+            if st.decode_time > 0:
+                best = max(best, st.generated_tokens / st.decode_time)
+        return best
+
+    greedy = rate()
+    topk = rate(temperature=0.8, top_k=40)
+    topp = rate(temperature=0.8, top_p=0.9)
+    pen = rate(temperature=0.8, top_k=40, repeat_penalty=1.2)
+    return {"workload": f"GPT-2 124M fp32 B=1 streamed generation of {n_new} tokens from a {len(ids)}-token prompt, "
+                        "temperature 0.8 + top_k 40, selection on the device",
+            "value": round(topk, 1), "unit": "tokens/s", "steps": n_new,
+            "greedy_tokens_per_s": round(greedy, 1),
+            "fraction_of_greedy": round(topk / greedy, 3) if greedy > 0 else None,
+            "temperature_0.8_top_p_0.9_tokens_per_s": round(topp, 1),
+            "temperature_0.8_top_k_40_repeat_penalty_1.2_tokens_per_s": round(pen, 1)}
 
 
 def measure_short_prefill(model, cfg, ids, T, steps, warmup):

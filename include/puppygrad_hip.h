@@ -478,6 +478,12 @@ pg_status pg_kv_cache_debug_set_epoch(pg_kv_cache* cache, uint32_t epoch);
  * started, and selections for which it copied the row of logits to the host. */
 void pg_debug_sample_counts(uint64_t* device_draws, uint64_t* host_rows);
 
+/* Test hook: with enabled == 0 the streamed generations select sampled (and penalised) tokens
+ * one call of pg_logits_sample at a time, as a caller of the single-step entry points would,
+ * instead of in trains of launches that keep the selection state on the device.  Both give
+ * the same ids; the switch is there so that tests can show it.  Returns the previous setting. */
+int pg_debug_sample_train(int enabled);
+
 /* Device facts for the benchmark harness. */
 typedef struct pg_device_info {
   char name[128];

@@ -159,6 +159,7 @@ SIGNATURES = {
     "pg_op_attention_decode_noalloc": (C.c_int, [C.c_int32, _vp, _vp, C.c_uint64, _vp, _vp,
                                                  C.c_uint64, C.c_uint64, C.c_uint64, _vp]),
     "pg_debug_sample_counts": (None, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "pg_debug_sample_train": (C.c_int, [C.c_int]),
     "pg_kv_cache_debug_epoch": (C.c_uint32, [_vp]),
     "pg_kv_cache_debug_set_epoch": (C.c_int, [_vp, C.c_uint32]),
     "pg_tensor_store_open": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),

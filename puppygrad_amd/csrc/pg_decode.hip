@@ -90,7 +90,7 @@ constexpr bool early_kv(int C) { return C <= 1024; }
 #define PG_ST32(p, v) __hip_atomic_store(PG_G32(p), (unsigned)(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
 // The "not written yet" pattern of an exchanged f32 word, and the bits a producer stores for v.
-constexpr unsigned kArm = 0xFFFFFFFFu;
+constexpr unsigned kArm = kExchangeArmed;
 // Where the exchanged vectors lie from DecodeParams::xch on, in words (C = n_embd).  There are
 // two sets (`par` picks one; `set` = DecodeParams::xch_set words apart, a multiple of 16), each
 // qkv 3C | attn C | xa C | h 4C | xm C | part (H * ns * 66): one contiguous run of whole 64-byte
@@ -2015,6 +2015,7 @@ __device__ __forceinline__ void streamer_wave(const DecodeParams& p, ctlp ctl, c
 template <int C_, int WB, int KS>
 __global__ __launch_bounds__(kThreads) void k_decode_persistent(DecodeParams p) {
   constexpr int C = C_, I = 4 * C_;
+  if (p.skip && p.skip[0] != 0u) return;  // (the same answer in every workgroup: see DecodeParams)
   // 16-byte LDS accesses run at full speed only on 16-byte boundaries: the dynamic block
   // starts on one whatever the size of the static control block before it
   extern __shared__ __attribute__((aligned(256))) float dyn[];
@@ -2126,7 +2127,7 @@ namespace {
 __global__ void k_arm_exchange(unsigned* x, size_t n, unsigned* status) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) x[i] = kArm;
-  if (i < 4) status[i] = 0u;
+  if (status && i < 4) status[i] = 0u;
 }
 }  // namespace
 

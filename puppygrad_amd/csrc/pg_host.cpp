@@ -29,6 +29,7 @@ thread_local std::string g_err;
 
 // Test hook counters: selections drawn entirely on the device, and selections for which the row
 // of logits was copied to the host.
+std::atomic<bool> g_no_sample_train{false};
 std::atomic<uint64_t> g_device_draws{0}, g_host_draws{0};
 
 pg_status fail(pg_status s, const std::string& msg) {
@@ -505,17 +506,15 @@ struct PersistentRun {
 #endif
 };
 
-// n_fwd cached decoder steps of sequence 0.  Token t is force_ids[t] when force_ids is set
-// (prefill), otherwise the first token comes from d_tok / tok and later ones from the argmax
-// of the previous step.
-pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
-                           bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
-                           size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
-                           bool timed, PersistentRun* run, unsigned long long* stamps = nullptr) {
+// The kernel arguments of one launch: n_fwd cached decoder steps of sequence 0.  Token t is
+// force_ids[t] when force_ids is set (prefill), otherwise the first token comes from d_tok / tok
+// and later ones from the argmax of the previous step.  The epochs the launch will use are taken
+// off the cache's counter.
+pg_status persistent_params(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
+                            bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
+                            size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
+                            unsigned long long* stamps, pgk::DecodeParams* out) {
   const Cfg& g = m->cfg;
-  if (t_persistent_in_flight)
-    return fail(PG_INVALID_INPUT,
-                "a token callback must not call the model while its generation is running");
   const unsigned span = (unsigned)(n_fwd * (g.L + 1) * 8 + 8);
   if (c->epoch > kEpochWrap - span) {
     // epochs would wrap: clear every tag and start over
@@ -556,6 +555,23 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
     p.item_keys = 256;
   p.status = c->status;
   p.prof = stamps;  // the kernel's own time stamps of the launch's last forward, if wanted
+  c->epoch += span;
+  *out = p;
+  return PG_OK;
+}
+
+pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t* force_ids,
+                           bool lm_last_only, bool tok_from_ptr, uint32_t tok, size_t pos0,
+                           size_t n_fwd, bool select_last, int64_t eos, uint32_t* out_ids_dev,
+                           bool timed, PersistentRun* run, unsigned long long* stamps = nullptr) {
+  const Cfg& g = m->cfg;
+  if (t_persistent_in_flight)
+    return fail(PG_INVALID_INPUT,
+                "a token callback must not call the model while its generation is running");
+  pgk::DecodeParams p{};
+  pg_status ps = persistent_params(m, c, force_ids, lm_last_only, tok_from_ptr, tok, pos0, n_fwd,
+                                   select_last, eos, out_ids_dev, stamps, &p);
+  if (ps) return ps;
 #ifdef PG_DECODE_PROF_BUILD
   // Development builds only: PG_DECODE_PROF=<file> dumps the per-workgroup phase timestamps
   // of the last token of each persistent launch (raw u64, [grid][L+1][16]).
@@ -568,7 +584,6 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
     p.prof = reinterpret_cast<unsigned long long*>(run->prof);
   }
 #endif
-  c->epoch += span;
   run->lock = std::unique_lock<std::mutex>(g_persistent_mu);
   auto enqueue = [&]() -> pg_status {
     PG_HIP(pgk::launch_arm_exchange(c->xch, c->x_words, c->status, c->stream));
@@ -1627,6 +1642,23 @@ double pg_rng_next_unit_f64(pg_rng_state* rng) {
   return (double)(pg_rng_next_u64(rng) >> 11) * (1.0 / (double)(1ULL << 53));
 }
 
+// Device and pinned buffers of the sampler, made on first use: the candidates of a top-k
+// selection (count, then (id, logit) pairs) followed by four words of state for generations
+// that run as a train of launches (kCandHalt: the halt word, kCandRng: the generator's state),
+// and the recent ids of the repeat penalty (the train keeps the whole history there).
+constexpr uint64_t kMaxCand = 4096, kMaxRecent = 8192;
+constexpr size_t kCandHalt = 2 * kMaxCand + 4, kCandRng = 2 * kMaxCand + 6;
+constexpr size_t kCandWords = 2 * kMaxCand + 8;
+static pg_status ensure_sample_buffers(pg_kv_cache* c) {
+  if (!c->d_cand) PG_HIP(hipMalloc(&c->d_cand, kCandWords * sizeof(uint32_t)));
+  if (!c->h_cand)
+    PG_HIP(hipHostMalloc(&c->h_cand, kCandWords * sizeof(uint32_t), hipHostMallocDefault));
+  if (!c->d_recent) PG_HIP(hipMalloc(&c->d_recent, kMaxRecent * sizeof(uint32_t)));
+  if (!c->h_recent)
+    PG_HIP(hipHostMalloc(&c->h_recent, kMaxRecent * sizeof(uint32_t), hipHostMallocDefault));
+  return PG_OK;
+}
+
 pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, size_t n_hist,
                            const pg_sampling* sampling, pg_rng_state* rng, uint32_t* out) {
   if (!l || !sampling || !rng || !out) return fail(PG_INVALID_INPUT, "null argument");
@@ -1650,16 +1682,10 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
   // Sampling with top_k: the candidates are chosen on the device (penalty, finite filter, the
   // k first of the stable order) and only they cross to the host, which does the f64
   // arithmetic of the draw exactly as the reference does.
-  constexpr uint64_t kMaxCand = 4096, kMaxRecent = 8192;
   const uint64_t recent = penalised ? std::min<uint64_t>(sampling->repeat_last_n, n_hist) : 0;
   if (sampling->temperature > 0.0f && sampling->has_top_k && sampling->top_k <= kMaxCand &&
       l->vocab <= (uint64_t)pgk::kTopkMaxVocab && recent <= kMaxRecent && (recent == 0 || history)) {
-    if (!c->d_cand) {
-      PG_HIP(hipMalloc(&c->d_cand, (2 * kMaxCand + 4) * sizeof(uint32_t)));
-      PG_HIP(hipHostMalloc(&c->h_cand, (2 * kMaxCand + 4) * sizeof(uint32_t), hipHostMallocDefault));
-      PG_HIP(hipMalloc(&c->d_recent, kMaxRecent * sizeof(uint32_t)));
-      PG_HIP(hipHostMalloc(&c->h_recent, kMaxRecent * sizeof(uint32_t), hipHostMallocDefault));
-    }
+    if ((s = ensure_sample_buffers(c))) return s;
     const int k = (int)sampling->top_k;
     if (recent) {
       std::memcpy(c->h_recent, history + (n_hist - recent), recent * sizeof(uint32_t));
@@ -1689,12 +1715,7 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
   // reference's exact arithmetic.
   if (sampling->temperature > 0.0f && !sampling->has_top_k &&
       l->vocab <= (uint64_t)pgk::kTopkMaxVocab && recent <= kMaxRecent && (recent == 0 || history)) {
-    if (!c->d_cand) {
-      PG_HIP(hipMalloc(&c->d_cand, (2 * kMaxCand + 4) * sizeof(uint32_t)));
-      PG_HIP(hipHostMalloc(&c->h_cand, (2 * kMaxCand + 4) * sizeof(uint32_t), hipHostMallocDefault));
-      PG_HIP(hipMalloc(&c->d_recent, kMaxRecent * sizeof(uint32_t)));
-      PG_HIP(hipHostMalloc(&c->h_recent, kMaxRecent * sizeof(uint32_t), hipHostMallocDefault));
-    }
+    if ((s = ensure_sample_buffers(c))) return s;
     if (recent) {
       std::memcpy(c->h_recent, history + (n_hist - recent), recent * sizeof(uint32_t));
       PG_HIP(hipMemcpyAsync(c->d_recent, c->h_recent, recent * sizeof(uint32_t),
@@ -1732,6 +1753,10 @@ pg_status pg_logits_sample(pg_logits* l, uint32_t row, const uint32_t* history, 
     return PG_OK;
   }
   return sample_logits(adjusted, *sampling, rng, out);
+}
+
+int pg_debug_sample_train(int enabled) {
+  return g_no_sample_train.exchange(enabled == 0) ? 0 : 1;
 }
 
 void pg_debug_sample_counts(uint64_t* device_draws, uint64_t* host_rows) {
@@ -2042,6 +2067,168 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
       // the forwards the reference would have run: one per token pushed, except the last
       c->seq_len += stopped ? done : nf;
       base += nf;
+    }
+    c->logits_valid = false;
+  } else if (!profile && use_persistent(m, c) && m->cfg.V <= (uint64_t)pgk::kTopkMaxVocab &&
+             m->cfg.P <= kMaxRecent && !g_no_sample_train &&
+             (sampling->temperature <= 0.0f || !sampling->has_top_k || sampling->top_k <= kMaxCand)) {
+    // Sampled (or penalised) selection on the persistent path: the reference's loop
+    // (rust.rs:495-531) as a train of launches per chunk of tokens, [select, forward] [select,
+    // forward] ..., enqueued without waiting.  The selection kernels keep the generator's state,
+    // the history of ids and the id of the next forward in device memory and write every id into
+    // pinned host memory, which this thread reads while the train runs.  A selection the device
+    // does not decide (pg_logits_sample explains when), or an EOS id, raises a halt word that
+    // makes the rest of the train fall through; the host then selects that token itself from the
+    // logits that are still in place and starts the next train.
+    constexpr size_t kTrainChunk = 32;
+    constexpr uint32_t kUnset = 0xffffffffu;
+    const size_t N = std::min<size_t>(max_new, m->cfg.P - output.size());  // tokens to select
+    // (top_k up to 128 of a row that fits a block's registers: selection and draw in one
+    // launch; larger ones: launch_topk_select, then the draw among the list it leaves)
+    const int mode = sampling->temperature <= 0.0f ? pgk::kStepGreedy
+                     : !sampling->has_top_k        ? pgk::kStepRow
+                     : pgk::topk_step_supports((int)m->cfg.V, sampling->top_k) ? pgk::kStepTopk
+                                                                               : pgk::kStepList;
+    if ((s = ensure_sample_buffers(c))) return s;
+    volatile uint32_t* slot = c->h_stream;
+    size_t selected = 0;  // tokens selected so far (EOS included)
+    bool ended = N == 0, eos_hit = false;
+    // what the reference's loop does with a selected id
+    auto deliver = [&](uint32_t tok) -> pg_status {
+      ++selected;
+      if (eos >= 0 && (uint32_t)eos == tok) {
+        ended = eos_hit = true;
+        return PG_OK;
+      }
+      output.push_back(tok);
+      if (on_token && on_token(tok, user) != 0)
+        return fail(PG_INVALID_INPUT, "on_token callback stopped generation");
+      generated += 1;
+      if (first_token_s < 0) first_token_s = since(first_start);
+      if (selected == N) ended = true;
+      return PG_OK;
+    };
+    while (!ended) {
+      const size_t nt = std::min(N - selected, kTrainChunk);  // selections of this train
+      const size_t n_hist0 = output.size();
+      // state of the train: history, halt word, generator
+      if (penalised) {
+        std::memcpy(c->h_recent, output.data(), n_hist0 * sizeof(uint32_t));
+        PG_HIP(hipMemcpyAsync(c->d_recent, c->h_recent, n_hist0 * sizeof(uint32_t),
+                              hipMemcpyHostToDevice, c->stream));
+      }
+      c->h_cand[kCandHalt] = 0u;
+      c->h_cand[kCandHalt + 1] = 0u;
+      std::memcpy(&c->h_cand[kCandRng], &rng.state, sizeof(uint64_t));
+      PG_HIP(hipMemcpyAsync(c->d_cand + kCandHalt, c->h_cand + kCandHalt, 4 * sizeof(uint32_t),
+                            hipMemcpyHostToDevice, c->stream));
+      for (size_t j = 0; j < nt; ++j) slot[j] = kUnset;
+      if (t_persistent_in_flight)
+        return fail(PG_INVALID_INPUT,
+                    "a token callback must not call the model while its generation is running");
+      PersistentRun run;
+      run.lock = std::unique_lock<std::mutex>(g_persistent_mu);
+      size_t forwards = 0;  // forwards enqueued
+      auto enqueue = [&]() -> pg_status {
+        PG_HIP(pgk::launch_arm_exchange(c->xch, 0, c->status, c->stream));  // clears the status
+        PG_HIP(hipEventRecord(c->ev0, c->stream));
+        for (size_t j = 0; j < nt; ++j) {
+          const size_t n_hist = n_hist0 + j;
+          const uint64_t recent =
+              penalised ? std::min<uint64_t>(sampling->repeat_last_n, n_hist) : 0;
+          if (mode == pgk::kStepList)
+            PG_HIP(pgk::launch_topk_select(c->logits_buf, (int)m->cfg.V, c->d_recent + (n_hist - recent),
+                                           (int)recent, sampling->repeat_penalty,
+                                           (int)sampling->top_k, c->d_cand, c->stream));
+          pgk::SampleStep a{};
+          a.logits = c->logits_buf;
+          a.V = (int)m->cfg.V;
+          a.mode = mode;
+          a.list = c->d_cand;
+          a.top_k = (int)sampling->top_k;
+          a.hist = c->d_recent;
+          a.n_hist = (int)n_hist;
+          a.recent = (int)recent;
+          a.penalty = sampling->repeat_penalty;
+          a.temperature = (double)sampling->temperature;
+          a.has_top_p = sampling->has_top_p ? 1 : 0;
+          a.top_p = (double)sampling->top_p;
+          a.rng = reinterpret_cast<unsigned long long*>(c->d_cand + kCandRng);
+          a.halt = c->d_cand + kCandHalt;
+          a.abort_word = c->status;
+          a.d_tok = c->d_tok;
+          a.slot = c->h_stream_dev + j;
+          a.eos = (int)eos;
+          const bool forward = selected + j + 1 < N;  // rust.rs:518-528: none after the last token
+          if (forward) {  // (the step arms the exchange words of the forward that follows it)
+            a.arm = c->xch;
+            a.arm_words = c->x_words;
+          }
+          PG_HIP(pgk::launch_sample_step(a, c->stream));
+          if (forward) {
+            pgk::DecodeParams p{};
+            pg_status ps = persistent_params(m, c, nullptr, false, true, 0, c->seq_len + j, 1,
+                                             false, -1, nullptr, nullptr, &p);
+            if (ps) return ps;
+            p.skip = c->d_cand + kCandHalt;
+            PG_HIP(pgk::launch_decode_persistent(p, c->stream));
+            ++forwards;
+          }
+        }
+        PG_HIP(hipEventRecord(c->ev1, c->stream));
+        PG_HIP(hipMemcpyAsync(c->h_status, c->status, 4 * sizeof(unsigned), hipMemcpyDeviceToHost,
+                              c->stream));
+        return PG_OK;
+      };
+      s = enqueue();
+      run.begun = true;  // (whatever was enqueued is waited for before the lock is released)
+      run.stream = c->stream;
+      t_persistent_in_flight = true;
+      if (s) return s;
+      // follow the train
+      size_t j = 0;            // next slot to read
+      uint32_t special = 0;    // a slot value that is not an id
+      pg_status cb = PG_OK;
+      bool running = true;
+      while (!ended && j < nt) {
+        const uint32_t tok = slot[j];
+        if (tok == kUnset) {
+          if (!running) break;  // the train has ended without writing this slot
+          if (hipStreamQuery(c->stream) != hipErrorNotReady) running = false;  // one more look
+          for (int k = 0; k < 32; ++k) __builtin_ia32_pause();
+          continue;
+        }
+        if (tok >= pgk::kSlotAborted) {
+          special = tok;
+          break;
+        }
+        ++j;
+        if (mode != pgk::kStepGreedy) (void)pg_rng_next_u64(&rng);  // the draw the device used
+        g_device_draws.fetch_add(1, std::memory_order_relaxed);
+        if ((cb = deliver(tok))) break;
+      }
+      if ((s = persistent_end(c, &run, nullptr, nullptr))) return s;
+      float ms = 0.0f;
+      PG_HIP(hipEventElapsedTime(&ms, c->ev0, c->ev1));
+      gpu_decode_s += ms * 1e-3;
+      if (cb) return cb;
+      if (special == pgk::kSlotNoCandidate)
+        return fail(PG_INVALID_INPUT,
+                    "token sampling failed: cannot sample from empty or non-finite logits");
+      if (special == pgk::kSlotAborted || (special == 0 && !ended && j < nt))
+        return fail(PG_BACKEND, "persistent decode kernel ended without the expected token");
+      // forwards that ran: one per id the device selected, except an EOS id (its step raised
+      // the halt word) and the last token of all (none was enqueued)
+      c->seq_len += eos_hit ? j - 1 : std::min(j, forwards);
+      if (special == pgk::kSlotUndecided) {
+        // the logits of this selection are still in place: the host's own selection
+        if ((s = finish_logits(c, &logits))) return s;
+        uint32_t tok = 0;
+        if ((s = pg_logits_sample(logits, 0, output.data(), output.size(), sampling, &rng, &tok)))
+          return s;
+        if ((s = deliver(tok))) return s;
+        if (!ended && (s = pg_gpt2_forward_one(m, c, tok, &logits))) return s;
+      }
     }
     c->logits_valid = false;
   } else {

@@ -102,6 +102,49 @@ hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_id
 hipError_t launch_sample_select(const float* logits, int V, const uint32_t* pen_ids, int n_pen,
                                 float penalty, double temperature, int has_top_p, double top_p,
                                 double u, uint32_t* out, hipStream_t s);
+// One selection of a sampled generation that runs as a train of launches (k_sample_step): the
+// same selection as launch_sample_select (kStepRow), the draw among the candidates
+// launch_topk_select left in `list` (kStepList), or the argmax of the penalised row (kStepGreedy,
+// temperature 0), with everything the next launch needs kept on the device.  A step first looks
+// at halt[0] and does nothing when it is set.  Otherwise it draws with the generator state at
+// rng[0] (splitmix64, advanced only when the draw is used), writes the id to d_tok[0], to
+// hist[n_hist] and to *slot (pinned host memory), and raises halt[0] = kStepEos when the id is
+// `eos`.  A selection it cannot decide raises halt[0] = kStepUndecided / kStepNoCandidate and
+// writes kSlotUndecided / kSlotNoCandidate to *slot; abort_word[0] != 0 (the forward before it
+// gave up) raises kStepAborted / kSlotAborted.  The recent ids of the penalty are
+// hist[n_hist - recent .. n_hist).
+// kStepTopk does the top_k selection and the draw in one launch (no launch_topk_select before
+// it), for the shapes topk_step_supports() names.  With `arm` set a step that runs also gives
+// the arm_words exchange words at arm the "not written yet" pattern (launch_arm_exchange's work
+// for the forward that follows it).
+enum : int { kStepRow = 0, kStepList = 1, kStepGreedy = 2, kStepTopk = 3 };
+constexpr unsigned kExchangeArmed = 0xFFFFFFFFu;
+bool topk_step_supports(int V, uint64_t top_k);
+enum : unsigned { kStepEos = 1, kStepUndecided = 2, kStepNoCandidate = 3, kStepAborted = 4 };
+constexpr uint32_t kSlotUndecided = 0xfffffffeu, kSlotNoCandidate = 0xfffffffdu,
+                   kSlotAborted = 0xfffffffcu;
+struct SampleStep {
+  const float* logits;
+  int V;
+  int mode;
+  const uint32_t* list;  // kStepList: launch_topk_select's output for this row
+  int top_k;
+  uint32_t* hist;
+  int n_hist, recent;
+  float penalty;
+  double temperature;
+  int has_top_p;
+  double top_p;
+  unsigned long long* rng;
+  unsigned* halt;
+  const unsigned* abort_word;  // may be null
+  uint32_t* d_tok;
+  uint32_t* slot;
+  int eos;
+  unsigned* arm;
+  size_t arm_words;
+};
+hipError_t launch_sample_step(const SampleStep& a, hipStream_t s);
 // x[b] = wte[ids[b]] + wpe[pos]
 hipError_t launch_embed_batch(float* x, const float* wte, const float* wpe, const uint32_t* ids,
                               int batch, int pos, int C, hipStream_t s, int w_bf16 = 0);
@@ -236,6 +279,9 @@ struct DecodeParams {
   int ns;         // key splits per head at the longest context
   int item_keys;  // keys per (head, split) attention item: 128 or 256
   unsigned* status;  // [0] abort, [1] forwards done, [2] stopped at eos
+  // Optional: the launch does nothing when skip[0] != 0 at its start (a word an earlier launch
+  // on the same stream may have set: see SampleStep::halt).
+  const unsigned* skip;
   // Optional [grid][L+1][8] timestamps (100 MHz wall clock) of the last token's phase
   // completions per workgroup; slot [L][7] holds the token's start.
   unsigned long long* prof;
@@ -254,7 +300,7 @@ hipError_t launch_decode_persistent(const DecodeParams& p, hipStream_t s);
 // Words of one set of DecodeParams::xch for n_embd = C and part_words words of attention partials.
 size_t persistent_exchange_set_words(int C, size_t part_words);
 // Before every launch: the n exchange words at x take the "not written yet" pattern and the
-// four status words are cleared.
+// four status words are cleared (status may be null: then they are left as they are).
 hipError_t launch_arm_exchange(unsigned* x, size_t n, unsigned* status, hipStream_t s);
 
 }  // namespace pgk

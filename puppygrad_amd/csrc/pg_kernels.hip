@@ -568,9 +568,187 @@ __device__ __forceinline__ unsigned order_key(float f) {  // total_cmp order, as
   return (unsigned)b ^ 0x80000000u;
 }
 constexpr int kTopkRows = (kTopkMaxVocab + 1023) / 1024;  // ids are visited in rows of 1024
+
+// The quick way, for rows of at most kTopkRegs * kTopkBlock logits: the row is read once and
+// kept in registers (512 threads, so that a thread's hundred values and its working set fit the
+// registers of two wavefronts per SIMD).  2048 bins laid linearly over the candidates' value
+// range (descending: a higher value never lands in a later bin, equal values share one) are
+// counted, a scan finds the bin in which the k-th candidate of the stable order lies, every
+// candidate of the bins before it is kept, and that one bin is sorted by (value descending, id
+// ascending) to keep its first ones.  When that bin holds more than the sort takes (thousands
+// of equal or nearly equal logits, or an outlier that squeezes the rest of the row into one
+// bin) nothing is decided: out[0] = kTopkUndecided, and the radix select below, which handles
+// every row, runs after it.
+constexpr int kTopkBlock = 512;
+constexpr int kTopkRegs = 100;
+constexpr int kTopkBins = 2048;
+constexpr uint32_t kTopkUndecided = 0xffffffffu;
+__global__ __launch_bounds__(kTopkBlock) void k_topk_bins(const float* logits, int V,
+                                                          const uint32_t* pen_ids, int n_pen,
+                                                          float penalty, int k, uint32_t* out) {
+  constexpr int TB = kTopkBlock, NW = TB / 64, PER = kTopkBins / TB;
+  extern __shared__ unsigned pen_bits[];  // one bit per id: among the recent ids
+  __shared__ unsigned red[64];
+  __shared__ unsigned long long items[2048];
+  __shared__ unsigned count[kTopkBins];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int words = (V + 31) / 32;
+  for (int i = tid; i < words; i += TB) pen_bits[i] = 0u;
+  __syncthreads();
+  for (int i = tid; i < n_pen; i += TB) {
+    const uint32_t id = pen_ids[i];
+    if (id < (uint32_t)V) atomicOr(&pen_bits[id >> 5], 1u << (id & 31));
+  }
+  __syncthreads();
+  auto adjust = [&](int i, float l) {
+    if (n_pen && ((pen_bits[i >> 5] >> (i & 31)) & 1u)) return l < 0.0f ? l * penalty : l / penalty;
+    return l;
+  };
+  auto put = [&](unsigned at, unsigned id, unsigned value_bits) {
+    out[1 + 2 * at] = id;
+    out[2 + 2 * at] = value_bits;
+  };
+  float v[kTopkRegs];
+#pragma unroll
+  for (int r = 0; r < kTopkRegs; ++r) {
+    const int i = r * TB + tid;
+    v[r] = i < V ? logits[i] : NAN;
+  }
+  float vmax = -INFINITY, vmin = INFINITY;
+  unsigned n = 0;
+#pragma unroll
+  for (int r = 0; r < kTopkRegs; ++r) {
+    const int i = r * TB + tid;
+    if (i < V) {
+      const float a = adjust(i, v[r]);
+      v[r] = fabsf(a) <= 3.402823466e+38f ? a : NAN;  // NaN: not a candidate
+    }
+    if (v[r] == v[r]) {
+      vmax = fmaxf(vmax, v[r]);
+      vmin = fminf(vmin, v[r]);
+      ++n;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    vmax = fmaxf(vmax, __shfl_xor(vmax, off, 64));
+    vmin = fminf(vmin, __shfl_xor(vmin, off, 64));
+    n += __shfl_xor(n, off, 64);
+  }
+  if (lane == 0) {
+    red[wave] = __float_as_uint(vmax);
+    red[16 + wave] = __float_as_uint(vmin);
+    red[32 + wave] = n;
+  }
+  for (int i = tid; i < kTopkBins; i += TB) count[i] = 0u;
+  if (tid == 0) {
+    red[48] = 0u;  // candidates written from the bins before the crossing one
+    red[49] = 0u;  // candidates collected from the crossing bin
+  }
+  __syncthreads();
+  unsigned total = 0;
+  for (int w = 0; w < NW; ++w) {
+    vmax = fmaxf(vmax, __uint_as_float(red[w]));
+    vmin = fminf(vmin, __uint_as_float(red[16 + w]));
+    total += red[32 + w];
+  }
+  const unsigned kk = total < (unsigned)k ? total : (unsigned)k;
+  if (kk == 0) {
+    if (tid == 0) out[0] = 0u;
+    return;
+  }
+  const float span = vmax - vmin;
+  const float bin_scale = span > 0.0f ? (float)(kTopkBins - 1) / span : 0.0f;
+  auto bin_of = [&](float x) {
+    const int b = (int)((vmax - x) * bin_scale);
+    return min(max(b, 0), kTopkBins - 1);
+  };
+#pragma unroll
+  for (int r = 0; r < kTopkRegs; ++r)
+    if (v[r] == v[r]) atomicAdd(&count[bin_of(v[r])], 1u);
+  __syncthreads();
+  // inclusive scan of the 2048 counts, PER per thread; the bin whose prefix first reaches kk
+  unsigned c[PER], s = 0;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    c[e] = count[PER * tid + e];
+    s += c[e];
+  }
+  const unsigned own = s;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned o = __shfl_up(s, off, 64);
+    if (lane >= off) s += o;
+  }
+  if (lane == 63) red[wave] = s;
+  __syncthreads();
+  unsigned before = s - own;
+  for (int w = 0; w < wave; ++w) before += red[w];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    if (before < kk && kk <= before + c[e]) {  // true for exactly one bin of the block
+      red[50] = (unsigned)(PER * tid + e);
+      red[51] = before;
+      red[52] = c[e];
+    }
+    before += c[e];
+  }
+  __syncthreads();
+  const int b = (int)red[50];
+  const unsigned above = red[51], nb = red[52];
+  if (nb > 2048u) {
+    if (tid == 0) out[0] = kTopkUndecided;
+    return;
+  }
+  if (tid == 0) out[0] = kk;
+  const unsigned need = kk - above;  // 1 <= need <= nb
+#pragma unroll
+  for (int r = 0; r < kTopkRegs; ++r) {
+    if (v[r] == v[r]) {
+      const int bn = bin_of(v[r]);
+      const unsigned id = (unsigned)(r * TB + tid);
+      if (bn < b) {
+        put(atomicAdd(&red[48], 1u), id, __float_as_uint(v[r]));
+      } else if (bn == b) {
+        items[atomicAdd(&red[49], 1u)] = ((unsigned long long)(~order_key(v[r])) << 32) | id;
+      }
+    }
+  }
+  __syncthreads();
+  if (need < nb) {  // bitonic sort of the next power of two (padding sorts last)
+    unsigned n2 = 1;
+    while (n2 < nb) n2 <<= 1;
+    for (unsigned i = nb + tid; i < n2; i += TB) items[i] = ~0ull;
+    __syncthreads();
+    for (unsigned kq = 2; kq <= n2; kq <<= 1) {
+      for (unsigned j = kq >> 1; j > 0; j >>= 1) {
+        for (unsigned i = tid; i < n2; i += TB) {
+          const unsigned l = i ^ j;
+          if (l > i) {
+            const unsigned long long a = items[i], d = items[l];
+            const bool up = (i & kq) == 0;
+            if ((a > d) == up) {
+              items[i] = d;
+              items[l] = a;
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+  for (unsigned i = tid; i < need; i += TB) {
+    const unsigned key = ~(unsigned)(items[i] >> 32);
+    unsigned bits = key ^ 0x80000000u;  // undo order_key
+    bits ^= (unsigned)(((int)bits >> 31)) >> 1;
+    put(above + i, (unsigned)(items[i] & 0xffffffffu), bits);
+  }
+}
+
 __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V,
                                                       const uint32_t* pen_ids, int n_pen,
-                                                      float penalty, int k, uint32_t* out) {
+                                                      float penalty, int k, uint32_t* out,
+                                                      int only_if_undecided) {
   // out[0] = number of candidates, then (id, logit bits) pairs: one block to copy back
   uint32_t* const out_count = out;
   auto put = [&](unsigned at, int i, float v) {
@@ -580,6 +758,9 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
   extern __shared__ unsigned pen_bits[];  // one bit per id: among the recent ids
   __shared__ unsigned hist[256];
   __shared__ unsigned sh_prefix, sh_remaining, sh_total;
+  // 24 KB used by either way of selecting: the bins' sort items and counts, or the radix
+  // select's compaction cells
+  __shared__ unsigned long long pool[3 * 1024];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int words = (V + 31) / 32;
   for (int i = tid; i < words; i += 1024) pen_bits[i] = 0u;
@@ -595,6 +776,7 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
     return l;
   };
   auto finite = [](float v) { return fabsf(v) <= 3.402823466e+38f; };  // false for NaN and inf
+  if (only_if_undecided && out[0] != kTopkUndecided) return;
   // One pass over the row: thread t visits ids t, t + 1024, ...; eight loads are in flight
   // before the first is used.  f(i, key) sees the finite candidates only.
   constexpr int U = 8;
@@ -660,8 +842,11 @@ __global__ __launch_bounds__(1024) void k_topk_select(const float* logits, int V
   // Ordered compaction.  Id order is (row, wavefront, lane) order; the rank of a candidate
   // among those above T (or among those equal to T) is the sum of the counts of the
   // (row, wavefront) cells before its own plus its rank inside its wavefront.
-  __shared__ unsigned short cell_gt[kTopkRows * 16], cell_eq[kTopkRows * 16];
-  __shared__ unsigned base_gt[kTopkRows * 16], base_eq[kTopkRows * 16];
+  static_assert(kTopkRows * 16 * 12 <= (int)sizeof(pool), "the cells fit the pool");
+  unsigned* const base_gt = reinterpret_cast<unsigned*>(pool);
+  unsigned* const base_eq = base_gt + kTopkRows * 16;
+  unsigned short* const cell_gt = reinterpret_cast<unsigned short*>(base_eq + kTopkRows * 16);
+  unsigned short* const cell_eq = cell_gt + kTopkRows * 16;
   const int rows = (V + 1023) / 1024;
   for (int r = 0; r < rows; ++r) {
     const int i = r * 1024 + tid;
@@ -1019,8 +1204,13 @@ hipError_t launch_topk_select(const float* logits, int V, const uint32_t* pen_id
                               float penalty, int k, uint32_t* out, hipStream_t s) {
   const size_t lds = (size_t)((V + 31) / 32) * sizeof(unsigned);
   if (V < 1 || V > kTopkMaxVocab || k < 1 || n_pen < 0) return hipErrorInvalidValue;
+  // rows that fit the registers: the bins first; the radix select only if they gave up
+  const bool quick = V <= kTopkRegs * kTopkBlock;
+  if (quick)
+    hipLaunchKernelGGL(k_topk_bins, dim3(1), dim3(kTopkBlock), lds, s, logits, V, pen_ids, n_pen,
+                       penalty, k, out);
   hipLaunchKernelGGL(k_topk_select, dim3(1), dim3(1024), lds, s, logits, V, pen_ids, n_pen,
-                     penalty, k, out);
+                     penalty, k, out, quick ? 1 : 0);
   return hipGetLastError();
 }
 

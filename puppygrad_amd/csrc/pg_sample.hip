@@ -31,6 +31,7 @@ namespace pgk {
 namespace {
 
 constexpr int kThreads = 1024;
+constexpr int kWavesPerBlock = kThreads / 64;
 constexpr int kBins = 2048;
 constexpr int kBinCap = 2048;  // candidates of one bin that can be sorted in LDS
 constexpr double kMargin = 1e-9;
@@ -50,8 +51,6 @@ struct Smem {
   float wave_f[2][16];
   unsigned wave_u[16];
   unsigned n_items;
-  int chosen;
-  int status;
 };
 
 __device__ __forceinline__ double shfl_d(double v, int src_lane_xor) {
@@ -67,11 +66,19 @@ __device__ __forceinline__ double shfl_up_d(double v, int delta) {
   return __hiloint2double(hi, lo);
 }
 
-// Inclusive prefix sum over vals[0 .. 2048) in place (two values per thread, 1024 threads).
+// Inclusive prefix sum over vals[0 .. 2048) in place (2048 / TB values per thread of a block of
+// TB threads).
+template <int TB = kThreads>
 __device__ __forceinline__ void block_scan_2048(double* vals, double* wave_tot) {
+  constexpr int PER = 2048 / TB;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const double a = vals[2 * tid], b = vals[2 * tid + 1];
-  double s = a + b;
+  double x[PER], s = 0.0;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    x[e] = vals[PER * tid + e];
+    s += x[e];
+  }
+  const double own = s;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
     const double o = shfl_up_d(s, off);
@@ -79,64 +86,26 @@ __device__ __forceinline__ void block_scan_2048(double* vals, double* wave_tot) 
   }
   if (lane == 63) wave_tot[wave] = s;
   __syncthreads();
-  double base = 0.0;
-  for (int w = 0; w < wave; ++w) base += wave_tot[w];
-  const double incl_b = base + s;
-  vals[2 * tid] = incl_b - b;
-  vals[2 * tid + 1] = incl_b;
+  double run = s - own;
+  for (int w = 0; w < wave; ++w) run += wave_tot[w];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    run += x[e];
+    vals[PER * tid + e] = run;
+  }
   __syncthreads();
 }
 
-}  // namespace
-
-// out[0] = status (0: token drawn with the uniform value, 1: token is the first candidate and
-// the uniform value was not used, 2: undecided, 3: no finite candidate), out[1] = token id.
-__global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits, int V,
-                                                            const uint32_t* pen_ids, int n_pen,
-                                                            float penalty, double temperature,
-                                                            int has_top_p, double top_p, double u,
-                                                            uint32_t* out) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
-  unsigned* pen_bits = reinterpret_cast<unsigned*>(smem_raw + sizeof(Smem));
+// The draw of sample_logits (generation.rs:311-362) among the candidates that for_each
+// enumerates: for_each(f) calls f(id, value) once for every finite candidate, the same ones in
+// every call, each thread of the block taking its share.  Returns 0 with the drawn id in
+// *token_out (every thread holds both), 2 when the draw is not decided here, 3 when there is no
+// candidate.
+template <class Each>
+__device__ __forceinline__ int draw_among(Smem& sm, const Each& for_each, double temperature,
+                                          int has_top_p, double top_p, double u,
+                                          unsigned* token_out) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int words = (V + 31) / 32;
-  for (int i = tid; i < words; i += kThreads) pen_bits[i] = 0u;
-  if (tid == 0) {
-    sm.status = -1;
-    sm.chosen = 0;
-  }
-  __syncthreads();
-  for (int i = tid; i < n_pen; i += kThreads) {
-    const uint32_t id = pen_ids[i];
-    if (id < (uint32_t)V) atomicOr(&pen_bits[id >> 5], 1u << (id & 31));
-  }
-  __syncthreads();
-  // apply_repeat_penalty (generation.rs:281-298): once per distinct recent id
-  auto adjust = [&](int i, float l) {
-    if (n_pen && ((pen_bits[i >> 5] >> (i & 31)) & 1u)) return l < 0.0f ? l * penalty : l / penalty;
-    return l;
-  };
-  auto finite = [](float v) { return fabsf(v) <= 3.402823466e+38f; };  // false for NaN and inf
-  constexpr int U = 8;  // loads in flight per thread
-  auto for_each = [&](auto f) {
-    for (int i0 = tid; i0 < V; i0 += kThreads * U) {
-      float x[U];
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        const int i = i0 + kThreads * k;
-        x[k] = i < V ? logits[i] : INFINITY;
-      }
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        const int i = i0 + kThreads * k;
-        if (i >= V) break;
-        const float v = adjust(i, x[k]);
-        if (finite(v)) f(i, v);
-      }
-    }
-  };
-
   // ---- 1. candidates, largest and smallest value ----
   float vmax = -INFINITY, vmin = INFINITY;
   unsigned n_cand = 0;
@@ -160,17 +129,13 @@ __global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits,
   vmax = sm.wave_f[0][0];
   vmin = sm.wave_f[1][0];
   n_cand = sm.wave_u[0];
-  for (int w = 1; w < 16; ++w) {
+  for (int w = 1; w < kWavesPerBlock; ++w) {
     vmax = fmaxf(vmax, sm.wave_f[0][w]);
     vmin = fminf(vmin, sm.wave_f[1][w]);
     n_cand += sm.wave_u[w];
   }
   if (n_cand == 0) {
-    if (tid == 0) {
-      out[0] = 3u;
-      out[1] = 0u;
-    }
-    return;
+    return 3;
   }
   const double max_logit = (double)vmax / temperature;  // generation.rs:318
   auto weight_of = [&](float v) { return exp((double)v / temperature - max_logit); };
@@ -199,11 +164,7 @@ __global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits,
   const double full = sm.hist[kBins - 1];
   if (!(full > 0.0) || !isfinite(full)) {  // generation.rs:344-346: the first candidate
     // (cannot happen with a finite positive temperature: the largest candidate weighs 1)
-    if (tid == 0) {
-      out[0] = 2u;
-      out[1] = 0u;
-    }
-    return;
+    return 2;
   }
   const double slack = kMargin * full;
 
@@ -275,7 +236,7 @@ __global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits,
     if (lane == 0) sm.wave_u[wave] = (unsigned)first;
     __syncthreads();
     first = (int)sm.wave_u[0];
-    for (int w = 1; w < 16; ++w) first = min(first, (int)sm.wave_u[w]);
+    for (int w = 1; w < kWavesPerBlock; ++w) first = min(first, (int)sm.wave_u[w]);
     __syncthreads();
     if (first == 0x7fffffff) return false;  // the bin's own sum fell short of the bins' prefix
     const double incl = before + sm.weight[first];
@@ -299,11 +260,7 @@ __global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits,
   if (has_top_p && top_p < 1.0) {
     // generation.rs:325-340: the shortest prefix with cumulative / full >= top_p (at least one)
     if (!locate(top_p * full, &token, &reached)) {
-      if (tid == 0) {
-        out[0] = 2u;
-        out[1] = 0u;
-      }
-      return;
+      return 2;
     }
     kept = reached;
   }
@@ -313,23 +270,393 @@ __global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits,
     // u == 0: the walk stops at the first candidate whatever its weight; that is the largest
     // value with the lowest id, which locate() finds for any target inside the first weight
     if (!locate(fmin(kept, 0.5), &token, &reached)) {
-      if (tid == 0) {
-        out[0] = 2u;
-        out[1] = 0u;
-      }
-      return;
+      return 2;
     }
   } else if (!locate(target, &token, &reached)) {
-    if (tid == 0) {
-      out[0] = 2u;
-      out[1] = 0u;
+    return 2;
+  }
+  *token_out = token;
+  return 0;
+}
+
+// The recent ids as a bitmap over the vocabulary (apply_repeat_penalty, generation.rs:281-298:
+// once per distinct recent id).
+template <int TB = kThreads>
+__device__ __forceinline__ void mark_recent(unsigned* pen_bits, int V, const uint32_t* pen_ids,
+                                            int n_pen) {
+  const int tid = threadIdx.x;
+  const int words = (V + 31) / 32;
+  for (int i = tid; i < words; i += TB) pen_bits[i] = 0u;
+  __syncthreads();
+  for (int i = tid; i < n_pen; i += TB) {
+    const uint32_t id = pen_ids[i];
+    if (id < (uint32_t)V) atomicOr(&pen_bits[id >> 5], 1u << (id & 31));
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ bool is_finite(float v) {  // false for NaN and inf
+  return fabsf(v) <= 3.402823466e+38f;
+}
+
+// for_each over a row of logits after the repeat penalty: the finite ones are the candidates.
+struct RowCandidates {
+  const float* logits;
+  int V;
+  const unsigned* pen_bits;
+  int n_pen;
+  float penalty;
+  __device__ __forceinline__ float adjust(int i, float l) const {
+    if (n_pen && ((pen_bits[i >> 5] >> (i & 31)) & 1u)) return l < 0.0f ? l * penalty : l / penalty;
+    return l;
+  }
+  template <class F>
+  __device__ __forceinline__ void operator()(F f) const {
+    constexpr int U = 8;  // loads in flight per thread
+    const int tid = threadIdx.x;
+    for (int i0 = tid; i0 < V; i0 += kThreads * U) {
+      float x[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = i0 + kThreads * k;
+        x[k] = i < V ? logits[i] : INFINITY;
+      }
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = i0 + kThreads * k;
+        if (i >= V) break;
+        const float v = adjust(i, x[k]);
+        if (is_finite(v)) f(i, v);
+      }
     }
+  }
+};
+
+// for_each over the (id, logit) pairs k_topk_select leaves: out[0] pairs, at most k, all finite,
+// the penalty applied.
+struct ListCandidates {
+  const uint32_t* list;
+  int n;
+  template <class F>
+  __device__ __forceinline__ void operator()(F f) const {
+    for (int i = threadIdx.x; i < n; i += kThreads)
+      f((int)list[1 + 2 * i], __uint_as_float(list[2 + 2 * i]));
+  }
+};
+
+}  // namespace
+
+// out[0] = status (0: token drawn with the uniform value, 2: undecided, 3: no finite
+// candidate), out[1] = token id.
+__global__ __launch_bounds__(kThreads) void k_sample_select(const float* logits, int V,
+                                                            const uint32_t* pen_ids, int n_pen,
+                                                            float penalty, double temperature,
+                                                            int has_top_p, double top_p, double u,
+                                                            uint32_t* out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
+  unsigned* pen_bits = reinterpret_cast<unsigned*>(smem_raw + sizeof(Smem));
+  mark_recent(pen_bits, V, pen_ids, n_pen);
+  unsigned token = 0;
+  const int st = draw_among(sm, RowCandidates{logits, V, pen_bits, n_pen, penalty}, temperature,
+                            has_top_p, top_p, u, &token);
+  if (threadIdx.x == 0) {
+    out[0] = (unsigned)st;
+    out[1] = st == 0 ? token : 0u;
+  }
+}
+
+// ---- selections of a generation that runs as a train of launches -------------------------
+// (the sample step, then the forward of the id it chose, then the next sample step, ...).  The
+// generator's state, the history of ids and the id for the next forward live in device memory;
+// the host follows through `slot`, a word of pinned host memory.  A step that cannot decide
+// (or that draws the EOS id) raises `halt`; every later launch of the train looks at that word
+// first and falls through, so the logits the undecided step saw are still there for the host.
+namespace {
+
+// What every step starts with.  False: the step has nothing to do (every thread gets the same
+// answer).  Otherwise the exchange words of the forward that follows are armed here, which
+// saves that forward a launch of its own.
+template <int TB>
+__device__ __forceinline__ bool step_begin(const SampleStep& a) {
+  const int tid = threadIdx.x;
+  if (a.halt[0] != 0u) return false;  // (written only by the last thread of an earlier launch)
+  if (a.abort_word && a.abort_word[0] != 0u) {  // the forward before this step gave up
+    __syncthreads();  // every thread has read halt
+    if (tid == 0) {
+      a.halt[0] = kStepAborted;
+      __hip_atomic_store(a.slot, kSlotAborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    return false;
+  }
+  if (a.arm) {
+    uint4* x = reinterpret_cast<uint4*>(a.arm);
+    const uint4 armed{kExchangeArmed, kExchangeArmed, kExchangeArmed, kExchangeArmed};
+    for (size_t i = tid; i < a.arm_words / 4; i += TB) x[i] = armed;
+  }
+  return true;
+}
+
+// SmallRng's next state and draw (generation.rs:364-386): splitmix64, the top 53 bits as [0, 1)
+__device__ __forceinline__ double next_unit(unsigned long long state_in,
+                                            unsigned long long* state_out) {
+  const unsigned long long state = state_in + 0x9e3779b97f4a7c15ULL;
+  unsigned long long z = state;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+  z ^= z >> 31;
+  *state_out = state;
+  return (double)(z >> 11) * (1.0 / 9007199254740992.0);
+}
+
+// What every step ends with (one thread, after a barrier that every thread of the block has
+// passed): st 0 = `token` is selected, 2 = not decided here, 3 = no candidate.
+__device__ __forceinline__ void step_finish(const SampleStep& a, int st, unsigned token,
+                                            bool drew, unsigned long long state) {
+  auto to_host = [&](unsigned v) {
+    __hip_atomic_store(a.slot, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  };
+  if (st != 0) {
+    a.halt[0] = st == 3 ? kStepNoCandidate : kStepUndecided;
+    to_host(st == 3 ? kSlotNoCandidate : kSlotUndecided);
     return;
   }
-  if (tid == 0) {
-    out[0] = 0u;
-    out[1] = token;
+  if (drew) a.rng[0] = state;  // the draw was used
+  a.d_tok[0] = token;
+  a.hist[a.n_hist] = token;
+  if (a.eos >= 0 && token == (unsigned)a.eos) a.halt[0] = kStepEos;
+  to_host(token);
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(kThreads) void k_sample_step(SampleStep a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
+  unsigned* pen_bits = reinterpret_cast<unsigned*>(smem_raw + sizeof(Smem));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (!step_begin<kThreads>(a)) return;
+  const uint32_t* pen_ids = a.hist + (a.n_hist - a.recent);
+  unsigned token = 0;
+  int st = 0;
+  unsigned long long state = 0;
+  if (a.mode == kStepGreedy) {
+    // temperature 0 with a repeat penalty: the first maximum of the adjusted row in id order
+    // (a NaN never wins; nothing above -inf: id 0)
+    mark_recent(pen_bits, a.V, pen_ids, a.recent);
+    const RowCandidates row{a.logits, a.V, pen_bits, a.recent, a.penalty};
+    float bv = -INFINITY;
+    unsigned bi = 0xffffffffu;
+    constexpr int U = 8;
+    for (int i0 = tid; i0 < a.V; i0 += kThreads * U) {
+      float x[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = i0 + kThreads * k;
+        x[k] = i < a.V ? a.logits[i] : -INFINITY;
+      }
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = i0 + kThreads * k;
+        if (i >= a.V) break;
+        const float v = row.adjust(i, x[k]);
+        if (v > bv) {
+          bv = v;
+          bi = (unsigned)i;
+        }
+      }
+    }
+    auto take = [&](float ov, unsigned oi) {
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    };
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+      take(__shfl_xor(bv, off, 64), (unsigned)__shfl_xor((int)bi, off, 64));
+    if (lane == 0) {
+      sm.wave_f[0][wave] = bv;
+      sm.wave_u[wave] = bi;
+    }
+    __syncthreads();
+    bv = sm.wave_f[0][0];
+    bi = sm.wave_u[0];
+    for (int w = 1; w < kWavesPerBlock; ++w) take(sm.wave_f[0][w], sm.wave_u[w]);
+    token = bi == 0xffffffffu ? 0u : bi;
+  } else {
+    const double u = next_unit(a.rng[0], &state);
+    if (a.mode == kStepList) {
+      const int n = (int)min(a.list[0], (uint32_t)a.top_k);
+      st = draw_among(sm, ListCandidates{a.list, n}, a.temperature, a.has_top_p, a.top_p, u, &token);
+    } else {
+      mark_recent(pen_bits, a.V, pen_ids, a.recent);
+      st = draw_among(sm, RowCandidates{a.logits, a.V, pen_bits, a.recent, a.penalty},
+                      a.temperature, a.has_top_p, a.top_p, u, &token);
+    }
   }
+  __syncthreads();  // every thread has read halt and the generator's state
+  if (tid == 0) step_finish(a, st, token, a.mode != kStepGreedy, state);
+}
+
+// The top_k selection and its draw in one step, for rows of at most kTopkStepRegs *
+// kTopkStepThreads logits and top_k <= kTopkStepMaxK.  The row is read once into registers
+// (512 threads: a thread's 99 values and its working set fit the registers of two
+// wavefronts per SIMD).  A lower bound of the k-th largest candidate comes from the threads'
+// own maxima: each of the eight wavefronts gives the m = ceil(k / 8) largest of its 64 lane
+// maxima, 8 m >= k distinct candidates, so the smallest of them, L, is no larger than the
+// k-th largest of the row.  The candidates >= L (a few more than k for a row of distinct
+// values) are collected in LDS and sorted by (value descending, id ascending); the first k are
+// sample_logits' truncated list (generation.rs:311-315), over which the f64 weights, the top-p
+// prefix and the inverse-CDF walk (generation.rs:316-361) are placed with the margin
+// draw_among uses.  More than 2048 candidates >= L (rows of equal logits): not decided here.
+constexpr int kTopkStepThreads = 512, kTopkStepRegs = 99, kTopkStepMaxK = 128;
+__global__ __launch_bounds__(kTopkStepThreads) void k_topk_step(SampleStep a) {
+  constexpr int TB = kTopkStepThreads, NW = TB / 64, NR = kTopkStepRegs;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
+  unsigned* pen_bits = reinterpret_cast<unsigned*>(smem_raw + sizeof(Smem));
+  unsigned long long* const sorted = reinterpret_cast<unsigned long long*>(sm.hist);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (!step_begin<TB>(a)) return;
+  unsigned long long state = 0;
+  const double u = next_unit(a.rng[0], &state);
+  float v[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) v[r] = a.logits[min(r * TB + tid, a.V - 1)];  // (ids >= V: dropped below)
+  if (a.recent > 0) {
+    mark_recent<TB>(pen_bits, a.V, a.hist + (a.n_hist - a.recent), a.recent);
+    const RowCandidates row{a.logits, a.V, pen_bits, a.recent, a.penalty};
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      const int i = r * TB + tid;
+      if (i < a.V) v[r] = row.adjust(i, v[r]);
+    }
+  }
+  float lm = -INFINITY;  // this thread's largest candidate
+  unsigned n = 0;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    if (!is_finite(v[r]) || r * TB + tid >= a.V) v[r] = NAN;  // NaN: not a candidate
+    if (v[r] == v[r]) {
+      lm = fmaxf(lm, v[r]);
+      ++n;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off, 64);
+  // the m-th largest of the wavefront's lane maxima (-inf when fewer lanes hold a candidate)
+  const int m = (a.top_k + NW - 1) / NW;
+  float bound = -INFINITY;
+  for (int j = 0; j < m; ++j) {
+    float wmax = lm;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, off, 64));
+    bound = wmax;
+    if (!(wmax > -INFINITY)) break;
+    const unsigned long long holders = __ballot(lm == wmax);
+    if (lane == __builtin_ctzll(holders)) lm = -INFINITY;
+  }
+  if (lane == 0) {
+    sm.wave_f[0][wave] = bound;
+    sm.wave_u[wave] = n;
+  }
+  if (tid == 0) sm.n_items = 0u;
+  __syncthreads();
+  float L = sm.wave_f[0][0];
+  unsigned total = sm.wave_u[0];
+  for (int w = 1; w < NW; ++w) {
+    L = fminf(L, sm.wave_f[0][w]);
+    total += sm.wave_u[w];
+  }
+  const unsigned kk = min(total, (unsigned)a.top_k);
+  int st = 0;
+  unsigned token = 0;
+  if (kk == 0) {
+    st = 3;
+  } else {
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (v[r] >= L) {
+        const unsigned at = atomicAdd(&sm.n_items, 1u);
+        if (at < (unsigned)kBinCap)
+          sm.item[at] = ((unsigned long long)(~order_key(v[r])) << 32) | (unsigned)(r * TB + tid);
+      }
+    }
+    __syncthreads();
+    const unsigned ni = sm.n_items;  // >= kk
+    if (ni > (unsigned)kBinCap) {
+      st = 2;
+    } else {
+      // sorted[rank] = item: the items are distinct, an item's rank is the number of items
+      // before it
+      for (unsigned i = tid; i < ni; i += TB) {
+        const unsigned long long mine = sm.item[i];
+        unsigned rank = 0;
+        for (unsigned j = 0; j < ni; ++j) rank += sm.item[j] < mine ? 1u : 0u;
+        sorted[rank] = mine;
+      }
+      __syncthreads();
+      auto value_at = [&](unsigned i) {
+        const unsigned key = ~(unsigned)(sorted[i] >> 32);
+        unsigned bits = key ^ 0x80000000u;  // undo order_key
+        bits ^= (unsigned)(((int)bits >> 31)) >> 1;
+        return __uint_as_float(bits);
+      };
+      const double max_logit = (double)value_at(0) / a.temperature;  // generation.rs:318
+      for (unsigned i = tid; i < (unsigned)kBinCap; i += TB)
+        sm.weight[i] = i < kk ? exp((double)value_at(i) / a.temperature - max_logit) : 0.0;
+      __syncthreads();
+      block_scan_2048<TB>(sm.weight, sm.wave_d);
+      const double full = sm.weight[kBinCap - 1];
+      if (!(full > 0.0) || !isfinite(full)) {
+        st = 2;  // (generation.rs:344-346 takes the first candidate: left to the host)
+      } else {
+        const double slack = kMargin * full;
+        // the first of the `limit` first candidates whose inclusive running weight reaches
+        // `target`; -1 when the target comes within the margin of a boundary between two
+        auto place = [&](double target, unsigned limit) -> int {
+          int first = 0x7fffffff;
+          for (unsigned i = tid; i < limit; i += TB)
+            if (sm.weight[i] >= target) first = min(first, (int)i);
+#pragma unroll
+          for (int off = 32; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, 64));
+          __syncthreads();
+          if (lane == 0) sm.wave_u[wave] = (unsigned)first;
+          __syncthreads();
+          first = (int)sm.wave_u[0];
+          for (int w = 1; w < NW; ++w) first = min(first, (int)sm.wave_u[w]);
+          if (first == 0x7fffffff) return -1;
+          const double incl = sm.weight[first], excl = first ? sm.weight[first - 1] : 0.0;
+          if (first != 0 && !(target - excl > slack)) return -1;
+          if ((unsigned)first + 1 != limit && !(incl - target > slack)) return -1;
+          return first;
+        };
+        unsigned keep = kk;
+        double kept = full;
+        if (a.has_top_p && a.top_p < 1.0) {
+          // generation.rs:325-340: the shortest prefix with cumulative / full >= top_p
+          const int cut = place(a.top_p * full, kk);
+          if (cut < 0) {
+            st = 2;
+          } else {
+            keep = (unsigned)cut + 1;
+            kept = sm.weight[cut];
+          }
+        }
+        if (st == 0) {
+          // generation.rs:348-361: target = u * total, walk until it is used up
+          const int at = place(u * kept, keep);
+          if (at < 0)
+            st = 2;
+          else
+            token = (unsigned)(sorted[at] & 0xffffffffu);
+        }
+      }
+    }
+  }
+  __syncthreads();  // every thread has read halt and the generator's state
+  if (tid == 0) step_finish(a, st, token, true, state);
 }
 
 size_t sample_select_lds_bytes(int V) { return sizeof(Smem) + (size_t)((V + 31) / 32) * sizeof(unsigned); }
@@ -352,6 +679,42 @@ hipError_t launch_sample_select(const float* logits, int V, const uint32_t* pen_
   }
   hipLaunchKernelGGL(k_sample_select, dim3(1), dim3(kThreads), lds, s, logits, V, pen_ids, n_pen,
                      penalty, temperature, has_top_p, top_p, u, out);
+  return hipGetLastError();
+}
+
+bool topk_step_supports(int V, uint64_t top_k) {
+  return V >= 1 && V <= kTopkStepRegs * kTopkStepThreads && top_k >= 1 && top_k <= kTopkStepMaxK;
+}
+
+hipError_t launch_sample_step(const SampleStep& a, hipStream_t s) {
+  if (a.V < 1 || a.V > kTopkMaxVocab || a.recent < 0 || a.recent > a.n_hist || !a.halt ||
+      !a.d_tok || !a.hist || !a.slot || !a.logits)
+    return hipErrorInvalidValue;
+  if (a.mode != kStepGreedy && (!(a.temperature > 0.0) || !a.rng)) return hipErrorInvalidValue;
+  if (a.mode == kStepList && (!a.list || a.top_k < 1)) return hipErrorInvalidValue;
+  if (a.mode == kStepTopk && !topk_step_supports(a.V, (uint64_t)a.top_k)) return hipErrorInvalidValue;
+  if (a.arm && (a.arm_words % 4 != 0 || (reinterpret_cast<uintptr_t>(a.arm) & 15u) != 0))
+    return hipErrorInvalidValue;
+  const size_t lds = a.mode == kStepList ? sizeof(Smem) : sample_select_lds_bytes(a.V);
+  static thread_local int armed_device = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (armed_device != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_sample_step),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)sample_select_lds_bytes(kTopkMaxVocab));
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_topk_step),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)sample_select_lds_bytes(kTopkStepRegs * kTopkStepThreads));
+    if (e != hipSuccess) return e;
+    armed_device = dev;
+  }
+  if (a.mode == kStepTopk)
+    hipLaunchKernelGGL(k_topk_step, dim3(1), dim3(kTopkStepThreads), lds, s, a);
+  else
+    hipLaunchKernelGGL(k_sample_step, dim3(1), dim3(kThreads), lds, s, a);
   return hipGetLastError();
 }
 
