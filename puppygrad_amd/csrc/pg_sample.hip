@@ -137,8 +137,11 @@ __device__ __forceinline__ int draw_among(Smem& sm, const Each& for_each, double
   if (n_cand == 0) {
     return 3;
   }
-  const double max_logit = (double)vmax / temperature;  // generation.rs:318
-  auto weight_of = [&](float v) { return exp((double)v / temperature - max_logit); };
+  // (exp((l - max) / T) for the reference's exp(l / T - max / T): l - max is exact in f64 and
+  // the product with 1 / T is within an ulp or two of the quotient, far inside the margin; the
+  // f64 division would be a third of the arithmetic of the pass over the row)
+  const double vmax_d = (double)vmax, inv_t = 1.0 / temperature;
+  auto weight_of = [&](float v) { return exp(((double)v - vmax_d) * inv_t); };
   // bin of a value: linear over [vmin, vmax], the largest value in bin 0; never decreasing as
   // the value falls (the same monotone expression for every candidate)
   const float span = vmax - vmin;
