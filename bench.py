@@ -65,9 +65,11 @@ def main() -> int:
     ap.add_argument("--no-secondary", action="store_true",
                     help="skip the other configurations (they run only beside the default workload)")
     ap.add_argument("--decode-path", default="auto", choices=["auto", "kernels", "persistent"])
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "batch-decode"],
+    ap.add_argument("--workload", default="decode",
+                    choices=["decode", "prefill", "batch-decode", "sampled-stream"],
                     help="prefill: a step is one prefill of --prefill tokens (GEMM path, MFMA-bound); "
-                         "batch-decode: a step is one greedy step of --batch sequences")
+                         "batch-decode: a step is one greedy step of --batch sequences; "
+                         "sampled-stream: streamed generations of --steps tokens with sampled selection")
     ap.add_argument("--batch", type=int, default=None,
                     help="sequences of a batched step (batch-decode: 16 by default; prefill: 1)")
     ap.add_argument("--bf16", action="store_true", help="store the weights as bf16 (fp32 arithmetic)")
@@ -111,6 +113,12 @@ def main() -> int:
         return bench_prefill(args, cfg, model, ids, n_prefill)
     if args.workload == "batch-decode":
         return bench_batch_decode(args, cfg, model, n_prefill)
+    if args.workload == "sampled-stream":
+        r = measure_sampled_stream(model, ids, min(args.steps + 1, room), name=f"GPT-2 {args.model}")
+        r.update({"metric": f"streamed generation tokens/sec with sampled selection, GPT-2 {args.model} fp32 bs=1",
+                  "n_gpus": 1, "higher_is_better": True, "data": "synthetic", "dtype": "f32"})
+        print(json.dumps(r), flush=True)
+        return 0
 
     d = measure_decode(model, cfg, ids, n_prefill, args.steps, args.warmup, args.int8, args.bf16)
     K, room, launches = args.steps, d["room"], d["launches"]
@@ -285,7 +293,7 @@ def secondary_workloads(xl_cfg, xl_weights):
     return out
 
 
-def measure_sampled_stream(model, ids, n_new):
+def measure_sampled_stream(model, ids, n_new, name="GPT-2 124M"):
     """stream_token_ids_with_stats (rust.rs:548-634) with sampled selection: prompt, then n_new
     tokens whose selection (sample_logits, generation.rs:300-362) runs on the device between the
     forwards, no host round trip per token.  Rates are generated tokens over the decode loop's
@@ -304,7 +312,7 @@ def measure_sampled_stream(model, ids, n_new):
     topk = rate(temperature=0.8, top_k=40)
     topp = rate(temperature=0.8, top_p=0.9)
     pen = rate(temperature=0.8, top_k=40, repeat_penalty=1.2)
-    return {"workload": f"GPT-2 124M fp32 B=1 streamed generation of {n_new} tokens from a {len(ids)}-token prompt, "
+    return {"workload": f"{name} fp32 B=1 streamed generation of {n_new} tokens from a {len(ids)}-token prompt, "
                         "temperature 0.8 + top_k 40, selection on the device",
             "value": round(topk, 1), "unit": "tokens/s", "steps": n_new,
             "greedy_tokens_per_s": round(greedy, 1),

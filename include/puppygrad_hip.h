@@ -246,12 +246,20 @@ pg_status pg_gpt2_decode_greedy_batch(const pg_gpt2_model* model, pg_kv_cache* c
  * be NULL; a non-zero return from it stops generation and is reported as
  * PG_INVALID_INPUT.  out_ids must hold n + max_new entries and receives prompt
  * plus generated ids.
- * A greedy stream without a repeat penalty runs as launches of up to 64 forwards of the fused
- * decode kernel, and on_token is called while such a launch is running and the process-wide
- * lock of that kernel is held.  The callback therefore must not call the model (that is
- * refused with PG_INVALID_INPUT) and must not wait for another thread that does: that thread
- * cannot start its own launch before this one has ended.  After a callback has asked to stop,
- * the launch still finishes its forwards (at most 63) before the call returns. */
+ * On models the fused decode kernel covers, the device runs ahead of the host.  A greedy stream
+ * without a repeat penalty runs as launches of up to 64 forwards of that kernel.  A sampled or
+ * penalised stream (temperature > 0, or a repeat penalty; top_k up to 4096) runs as trains of
+ * up to 32 [selection, forward] launch pairs: the selections (sample_logits,
+ * src/models/generation.rs:281-362) keep the generator's state, the id history and the next id
+ * in device memory and write each id to pinned host memory; a draw the device cannot decide
+ * (see pg_logits_sample) or an EOS id makes the rest of the train fall through, and the host
+ * then selects that token as pg_logits_sample does.  Either way the ids are those of the
+ * reference's loop, one selection and one forward at a time.
+ * on_token is called while such launches are running and the process-wide lock of the fused
+ * kernel is held.  The callback therefore must not call the model (that is refused with
+ * PG_INVALID_INPUT) and must not wait for another thread that does: that thread cannot start
+ * its own launch before this one has ended.  After a callback has asked to stop, the launches
+ * already enqueued still run (at most 63 forwards) before the call returns. */
 typedef int (*pg_on_token)(uint32_t token_id, void* user);
 pg_status pg_gpt2_stream_token_ids_with_stats(const pg_gpt2_model* model, const uint32_t* ids,
                                               size_t n, uint32_t max_new, int64_t eos,
