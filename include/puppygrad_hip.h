@@ -91,7 +91,8 @@ typedef struct pg_hip_options {
   int32_t device;          /* HIP device ordinal */
   uint32_t weight_storage; /* pg_weight_storage: how the dense matrices and wte are kept in HBM */
   uint32_t decode_path;    /* pg_decode_path */
-  uint32_t prefill_path;   /* 0: GEMM prefill for prompts of 16+ tokens; 1: always token by token */
+  uint32_t prefill_path;   /* 0: GEMM prefill for prompts of seq_gemm_min_tokens and more; 1: always
+                              token by token */
   /* Tunables, the counterpart of the thresholds and chunk sizes of Gpt2RustConfig
    * (src/models/gpt2/options.rs:54-96) that the reference's `autotune gpt2` scans
    * (src/main.rs:2732-2870).  0 selects the built-in default. */
@@ -101,6 +102,13 @@ typedef struct pg_hip_options {
                                        blocks per CU the split count aims for (default 4) */
   uint32_t gemm_split_items_per_cu; /* tile GEMM: a product that leaves CUs idle is cut along K
                                        into about this many work items per CU (default 3) */
+  uint32_t gemm_b9_min_rows;        /* f32 weights: products over at least this many input rows
+                                       run on the bf16 matrix cores as nine exact bf16 products
+                                       per value pair where the planner finds enough tiles
+                                       (default 1024; 0xffffffff: never) */
+  uint32_t seq_gemm_min_tokens;     /* prompts of at least this many tokens take the GEMM
+                                       prefill, shorter ones run token by token through the
+                                       decode path (default 4; at most 65536) */
   uint32_t reserved;                /* must be 0 */
 } pg_hip_options;
 

@@ -44,7 +44,8 @@ class pg_hip_options(C.Structure):
     _fields_ = [("device", C.c_int32), ("weight_storage", C.c_uint32),
                 ("decode_path", C.c_uint32), ("prefill_path", C.c_uint32),
                 ("attn_item_keys", C.c_uint32), ("attn_blocks_per_cu", C.c_uint32),
-                ("gemm_split_items_per_cu", C.c_uint32), ("reserved", C.c_uint32)]
+                ("gemm_split_items_per_cu", C.c_uint32), ("gemm_b9_min_rows", C.c_uint32),
+                ("seq_gemm_min_tokens", C.c_uint32), ("reserved", C.c_uint32)]
 
 
 class pg_sampling(C.Structure):

@@ -8,9 +8,14 @@ validates the best one with more runs and saves it to `{model_dir}/puppygrad-tun
 src/main.rs:2564-2586).  This module does the same over the tunables of `Gpt2HipConfig`
 (the counterpart of the thresholds and chunk sizes of `Gpt2RustConfig`): keys per attention
 item of the fused decode kernel, attention blocks per CU of the per-operation / batched
-decode attention, and work items per CU of the split-K tile GEMM.  The saved file has the
-reference's fields with a `hip` object in the place of `rust`; `Gpt2Model.from_dir`
-(pg_gpt2_create_from_dir) reads it.
+decode attention, and three knobs of the GEMM prefill's planner: work items per CU of the
+split-K tile GEMM, the row count from which f32 products move to the bf16 matrix cores, and the
+prompt length from which the GEMM prefill is used at all.  The decode knobs move the reference's
+score (median decode tokens per second); the planner's knobs only move the prompt's share of a
+generation, so `--score total` (median of prompt + generated tokens over the whole generation
+time, a figure the reference's measurement already holds) or `--score prefill` ranks by that
+instead.  The saved file has the reference's fields with a `hip` object in the place of `rust`;
+`Gpt2Model.from_dir` (pg_gpt2_create_from_dir) reads it.
 
     python -m puppygrad_amd.autotune --model medium --prompt-tokens 128 --max-new-tokens 64 \
         --save-tuning puppygrad-tune.json
@@ -103,6 +108,7 @@ class Gpt2AutoTuneMeasurement:
     decode_tokens_per_second_stddev: float = 0.0
     total_tokens_per_second: float = 0.0
     total_tokens_per_second_median: float = 0.0
+    prefill_tokens_per_second_median: float = 0.0  # (not in the reference's struct: for --score prefill)
     prefill_ms: float = 0.0
     decode_ms: float = 0.0
     total_generation_ms: float = 0.0
@@ -119,6 +125,7 @@ def summarize_runs(load_time: float, prompt_count: int, runs_per_prompt: int,
     decode_tps = value_distribution(_rate(float(s.generated_tokens), s.decode_time) for s in stats)
     total_tps = value_distribution(
         _rate(float(s.prompt_tokens + s.generated_tokens), s.total_generation_time) for s in stats)
+    prefill_tps = value_distribution(_rate(float(s.prompt_tokens), s.prefill_time) for s in stats)
     n = max(len(stats), 1)
     return Gpt2AutoTuneMeasurement(
         load_ms=load_time * 1e3, prompt_count=prompt_count, runs_per_prompt=runs_per_prompt,
@@ -126,22 +133,30 @@ def summarize_runs(load_time: float, prompt_count: int, runs_per_prompt: int,
         decode_tokens_per_second_p25=decode_tps.p25, decode_tokens_per_second_median=decode_tps.median,
         decode_tokens_per_second_p95=decode_tps.p95, decode_tokens_per_second_stddev=decode_tps.stddev,
         total_tokens_per_second=_rate(float(prompt_tokens + generated), total),
-        total_tokens_per_second_median=total_tps.median, prefill_ms=prefill * 1e3 / n,
+        total_tokens_per_second_median=total_tps.median,
+        prefill_tokens_per_second_median=prefill_tps.median, prefill_ms=prefill * 1e3 / n,
         decode_ms=decode * 1e3 / n, total_generation_ms=total * 1e3 / n)
 
 
-TUNABLES = ("attn_item_keys", "attn_blocks_per_cu", "gemm_split_items_per_cu")
+TUNABLES = ("attn_item_keys", "attn_blocks_per_cu", "gemm_split_items_per_cu", "gemm_b9_min_rows",
+            "seq_gemm_min_tokens")
+SCORES = {"decode": ("median_decode_tokens_per_second", "decode_tokens_per_second_median"),
+          "total": ("median_total_tokens_per_second", "total_tokens_per_second_median"),
+          "prefill": ("median_prefill_tokens_per_second", "prefill_tokens_per_second_median")}
 
 
 def candidate_grid(base: Gpt2HipConfig, attn_item_keys: Sequence[int], attn_blocks_per_cu: Sequence[int],
-                   gemm_split_items_per_cu: Sequence[int]) -> List[Gpt2HipConfig]:
+                   gemm_split_items_per_cu: Sequence[int], gemm_b9_min_rows: Sequence[int] = (0,),
+                   seq_gemm_min_tokens: Sequence[int] = (0,)) -> List[Gpt2HipConfig]:
     """gpt2_autotune_candidates (src/main.rs:2809-2873): the cross product of the value
     lists, the first list varying slowest."""
     out = []
-    for keys, blocks, items in itertools.product(attn_item_keys, attn_blocks_per_cu,
-                                                 gemm_split_items_per_cu):
+    for keys, blocks, items, b9, seq in itertools.product(attn_item_keys, attn_blocks_per_cu,
+                                                          gemm_split_items_per_cu, gemm_b9_min_rows,
+                                                          seq_gemm_min_tokens):
         out.append(dataclasses.replace(base, attn_item_keys=keys, attn_blocks_per_cu=blocks,
-                                       gemm_split_items_per_cu=items))
+                                       gemm_split_items_per_cu=items, gemm_b9_min_rows=b9,
+                                       seq_gemm_min_tokens=seq))
     if not out:
         raise ValueError("autotune gpt2 generated no candidates")
     return out
@@ -157,6 +172,7 @@ class Gpt2AutoTuneTarget:
     candidates: List[Gpt2HipConfig]
     log: Callable[[str], None] = lambda line: print(line, file=sys.stderr)
     eos_token_id: Optional[int] = GPT2_EOS_TOKEN_ID  # Gpt2GenerationConfig::new; None for small vocabularies
+    score_by: str = "decode"  # key of SCORES; the reference scores by decode
 
     def candidate_configs(self) -> List[Gpt2HipConfig]:
         return list(self.candidates)
@@ -177,15 +193,15 @@ class Gpt2AutoTuneTarget:
         return summarize_runs(load_time, len(self.prompts), options.measured_runs, stats)
 
     def score(self, measurement: Gpt2AutoTuneMeasurement) -> float:
-        return measurement.decode_tokens_per_second_median
+        return getattr(measurement, SCORES[self.score_by][1])
 
 
 def save_gpt2_tuning(path, best_config: Gpt2HipConfig, search_score: float, validation_score: float,
                      validation_measurement: Gpt2AutoTuneMeasurement, max_new_tokens: int,
-                     options: AutoTuneOptions, model: str = "gpt2") -> None:
+                     options: AutoTuneOptions, model: str = "gpt2", score_by: str = "decode") -> None:
     """save_gpt2_tuning (src/main.rs:2927-2958): SavedGpt2Tuning as pretty JSON."""
     saved = {
-        "model": model, "backend": "hip", "score_name": "median_decode_tokens_per_second",
+        "model": model, "backend": "hip", "score_name": SCORES[score_by][0],
         "score": validation_score, "search_score": search_score, "max_new_tokens": max_new_tokens,
         "warmup_runs": options.warmup_runs, "measured_runs": options.measured_runs,
         "prompt_count": validation_measurement.prompt_count,
@@ -218,7 +234,8 @@ def load_gpt2_tuning(tuning_file, model_dir=None, base: Optional[Gpt2HipConfig] 
 
 def run_gpt2_autotune(make_model, prompts, max_new_tokens: int, candidates: List[Gpt2HipConfig],
                       options: AutoTuneOptions, validation_runs: int, save_path=None, model_name="gpt2",
-                      log=lambda line: print(line, file=sys.stderr), eos_token_id=GPT2_EOS_TOKEN_ID):
+                      log=lambda line: print(line, file=sys.stderr), eos_token_id=GPT2_EOS_TOKEN_ID,
+                      score_by: str = "decode"):
     """run_gpt2_autotune (src/main.rs:2732-2807): scan, validate the winner, save it."""
     if options.measured_runs == 0:
         raise ValueError("autotune gpt2 --runs must be > 0")
@@ -226,7 +243,9 @@ def run_gpt2_autotune(make_model, prompts, max_new_tokens: int, candidates: List
         raise ValueError("autotune gpt2 --max-trials must be > 0")
     log(f"autotune: {len(candidates)} candidates, evaluating up to "
         f"{options.max_trials if options.max_trials is not None else len(candidates)}")
-    target = Gpt2AutoTuneTarget(make_model, prompts, max_new_tokens, candidates, log, eos_token_id)
+    if score_by not in SCORES:
+        raise ValueError(f"autotune gpt2 --score must be one of {', '.join(SCORES)}")
+    target = Gpt2AutoTuneTarget(make_model, prompts, max_new_tokens, candidates, log, eos_token_id, score_by)
     result = autotune(target, options)
     validation_options = AutoTuneOptions(options.warmup_runs, validation_runs, None)
     log(f"validating best config with {validation_runs} measured runs")
@@ -234,7 +253,7 @@ def run_gpt2_autotune(make_model, prompts, max_new_tokens: int, candidates: List
     validation_score = target.score(validation)
     if save_path is not None:
         save_gpt2_tuning(save_path, result.best_config, result.best_score, validation_score, validation,
-                         max_new_tokens, validation_options, model_name)
+                         max_new_tokens, validation_options, model_name, score_by)
         log(f"saved tuning config to {save_path}")
     return result, validation, validation_score
 
@@ -253,6 +272,10 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     ap.add_argument("--attn-item-keys", default="128,256")
     ap.add_argument("--attn-blocks-per-cu", default="4")
     ap.add_argument("--gemm-split-items-per-cu", default="3")
+    ap.add_argument("--gemm-b9-min-rows", default="0", help="0: the built-in 1024")
+    ap.add_argument("--seq-gemm-min-tokens", default="0", help="0: the built-in 4")
+    ap.add_argument("--score", choices=sorted(SCORES), default="decode",
+                    help="what ranks the candidates (the reference: decode)")
     ap.add_argument("--quantized-weights", action="store_true")
     ap.add_argument("--save-tuning", help="default: {model-dir}/puppygrad-tune.json, or none without --model-dir")
     args = ap.parse_args(argv)
@@ -273,15 +296,18 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
                for n in _usize_list("prompt-tokens", args.prompt_tokens)]
     candidates = candidate_grid(base, _usize_list("attn-item-keys", args.attn_item_keys),
                                 _usize_list("attn-blocks-per-cu", args.attn_blocks_per_cu),
-                                _usize_list("gemm-split-items-per-cu", args.gemm_split_items_per_cu))
+                                _usize_list("gemm-split-items-per-cu", args.gemm_split_items_per_cu),
+                                _usize_list("gemm-b9-min-rows", args.gemm_b9_min_rows),
+                                _usize_list("seq-gemm-min-tokens", args.seq_gemm_min_tokens))
     options = AutoTuneOptions(args.warmup_runs, args.runs, args.max_trials)
     result, validation, score = run_gpt2_autotune(make_model, prompts, args.max_new_tokens, candidates,
                                                   options, args.validation_runs, save_path,
-                                                  args.model if not args.model_dir else "gpt2")
+                                                  args.model if not args.model_dir else "gpt2",
+                                                  score_by=args.score)
     print("best config:")
     for k in TUNABLES:
         print(f"  --{k.replace('_', '-')} {getattr(result.best_config, k)}")
-    print(f"search score: {result.best_score:.2f} tok/s median")
+    print(f"search score ({SCORES[args.score][0]}): {result.best_score:.2f} tok/s median")
     for trial in result.trials:
         print("  trial " + " ".join(f"{k}={getattr(trial.config, k)}" for k in TUNABLES)
               + f": {trial.score:.2f} tok/s median")

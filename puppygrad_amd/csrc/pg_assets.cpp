@@ -634,7 +634,9 @@ pg_status pg_hip_load_tuning(const char* path, pg_hip_options* options, int32_t*
     uint32_t* dst;
   } fields[] = {{"attn_item_keys", &options->attn_item_keys},
                 {"attn_blocks_per_cu", &options->attn_blocks_per_cu},
-                {"gemm_split_items_per_cu", &options->gemm_split_items_per_cu}};
+                {"gemm_split_items_per_cu", &options->gemm_split_items_per_cu},
+                {"gemm_b9_min_rows", &options->gemm_b9_min_rows},
+                {"seq_gemm_min_tokens", &options->seq_gemm_min_tokens}};
   for (const Field& f : fields) {
     const Json* v = hip->find(f.key);
     if (!v || v->kind == Json::Null) continue;

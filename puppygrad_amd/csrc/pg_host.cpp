@@ -78,6 +78,8 @@ struct pg_gpt2_model {
   bool item_keys_256_ok = false;    // the device holds the grid of the 256-key instance
   int attn_blocks_per_cu = 4;       // per-operation / batched decode attention
   int gemm_split_items = 3;         // tile GEMM split-K
+  int gemm_b9_min_rows = 1024;      // f32 rows on the bf16 matrix cores from this many input rows
+  size_t seq_gemm_min_tokens = 4;   // prompts at least this long take the GEMM prefill
   int w_bf16 = 0;                   // wte and the block matrices are stored as bf16
   // int8 storage (QuantizedRows, src/models/cpu.rs:26-56): the block matrices hold int8 rows
   // with the scales in LayerW; wte stays f32 for the embedding (rust.rs:966-974 reads the f32
@@ -649,14 +651,12 @@ pg_status run_persistent(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_t*
 
 // pg_op_dense: inputs of at least this many rows take the GEMM kernels.
 constexpr size_t kGemmMinRows = 2;
-// Sequences at least this long take the GEMM path in prefill / forward; shorter ones run as
-// that many single-token forwards (124M: 3 x 0.17 ms against 0.6 ms for the launches of one
-// GEMM pass; XL: 3 x 1.2 ms against 3.3 ms).
-constexpr size_t kSeqGemmMinRows = 4;
-
+// Sequences of at least seq_gemm_min_tokens (a tunable, 4 by default) take the GEMM path in
+// prefill / forward; shorter ones run as that many single-token forwards (124M: 3 x 0.17 ms
+// against 0.6 ms for the launches of one GEMM pass; XL: 3 x 1.2 ms against 3.3 ms).
 bool gemm_path_ok(const pg_gpt2_model* m, size_t n) {
   const Cfg& g = m->cfg;
-  return n >= kSeqGemmMinRows && g.C % 16 == 0 && g.I % 16 == 0 &&
+  return n >= m->seq_gemm_min_tokens && n >= 2 && g.C % 16 == 0 && g.I % 16 == 0 &&
          (g.hd() == 64 || n * g.H * n * sizeof(float) <= (256u << 20));
 }
 
@@ -737,6 +737,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, si
     a.ws = WS.p; a.ws_floats = ws_floats;
     if (ln_g) { a.ln_out = XN.p; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; }
     a.split_items_per_cu = m->gemm_split_items;
+    a.b9_min_rows = m->gemm_b9_min_rows;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_layer_norm_rows(X.p, XN.p, T, C, m->layers[0].ln_1_g, m->layers[0].ln_1_b, g.eps, s));
@@ -782,6 +783,7 @@ pg_status run_sequence_gemm(const pg_gpt2_model* m, pg_kv_cache* c, size_t b, si
     a.M = (int)nb; a.N = (int)g.V; a.K = C; a.lda = C; a.ldc = (int)g.V;
     if (m->w_i8) a.w_scale = m->lm_s;
     a.split_items_per_cu = m->gemm_split_items;
+    a.b9_min_rows = m->gemm_b9_min_rows;
     PG_HIP(pgk::launch_gemm(a, pgk::GEMM_BIAS, m->num_cus, s));
   }
   PG_MARK(kLogits);
@@ -833,6 +835,7 @@ pg_status enqueue_forward_batch(const pg_gpt2_model* m, pg_kv_cache* c, const ui
     a.a_packed = pk; a.c_packed = c_packed;
     if (ln_g) { a.ln_out = c->xn_b; a.ln_g = ln_g; a.ln_b = ln_b; a.ln_eps = g.eps; a.ln_packed = pk; }
     a.split_items_per_cu = m->gemm_split_items;
+    a.b9_min_rows = m->gemm_b9_min_rows;
     return pgk::launch_gemm(a, epi, m->num_cus, s);
   };
   PG_HIP(pgk::launch_embed_batch(c->x, m->wte, m->wpe, d_ids, B, (int)pos, C, s, m->w_bf16));
@@ -1065,6 +1068,8 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
     return fail(PG_INVALID_CONFIG, "hip backend attn_blocks_per_cu must be at most 64");
   if (opts.gemm_split_items_per_cu > 16)
     return fail(PG_INVALID_CONFIG, "hip backend gemm_split_items_per_cu must be at most 16");
+  if (opts.seq_gemm_min_tokens > 65536)
+    return fail(PG_INVALID_CONFIG, "hip backend seq_gemm_min_tokens must be at most 65536");
   if (opts.reserved != 0) return fail(PG_INVALID_CONFIG, "hip backend options: reserved must be 0");
   if ((s = select_device(opts.device))) return s;
 
@@ -1078,6 +1083,10 @@ pg_status pg_gpt2_create(const pg_gpt2_config* config, const pg_gpt2_weights_vie
   m->item_keys_auto = opts.attn_item_keys == 0;
   m->attn_blocks_per_cu = opts.attn_blocks_per_cu ? (int)opts.attn_blocks_per_cu : 4;
   m->gemm_split_items = opts.gemm_split_items_per_cu ? (int)opts.gemm_split_items_per_cu : 3;
+  m->gemm_b9_min_rows = opts.gemm_b9_min_rows == 0 ? 1024
+                        : opts.gemm_b9_min_rows > 0x7fffffffu ? 0x7fffffff
+                                                              : (int)opts.gemm_b9_min_rows;
+  m->seq_gemm_min_tokens = opts.seq_gemm_min_tokens ? opts.seq_gemm_min_tokens : 4;
   hipDeviceProp_t prop;
   PG_HIP(hipGetDeviceProperties(&prop, opts.device));
   m->num_cus = prop.multiProcessorCount;
@@ -1278,10 +1287,11 @@ pg_status pg_gpt2_describe(const pg_gpt2_model* m, char* dst, size_t cap) {
   if (!m || !dst || cap == 0) return fail(PG_INVALID_INPUT, "null argument");
   std::snprintf(dst, cap,
                 "hip (device=%d, compute_units=%d, weights=%s, decode=%s, attn_item_keys=%d, "
-                "attn_blocks_per_cu=%d, gemm_split_items_per_cu=%d)",
+                "attn_blocks_per_cu=%d, gemm_split_items_per_cu=%d, gemm_b9_min_rows=%d, "
+                "seq_gemm_min_tokens=%zu)",
                 m->device, m->num_cus, m->w_bf16 ? "bf16" : m->w_i8 ? "int8" : "f32",
                 m->persistent ? "persistent" : "kernels", m->item_keys, m->attn_blocks_per_cu,
-                m->gemm_split_items);
+                m->gemm_split_items, m->gemm_b9_min_rows, m->seq_gemm_min_tokens);
   return PG_OK;
 }
 

@@ -210,6 +210,8 @@ struct GemmArgs {
   // Tunable: a GEMM whose M x N leaves CUs idle is cut along K into about this many work items
   // per CU (gemm_split_parts).
   int split_items_per_cu = 3;
+  // Tunable: f32 rows go to the bf16 matrix cores (k_gemm_b9) from this many input rows on.
+  int b9_min_rows = 1024;
   // A forced plan for the tile forms (benchmarks and tests; 0 = the planner chooses): tile
   // shape, form (1 whole tiles, 2 every tile cut along K into plan_parts, 3 only the last
   // partial round of tiles cut).

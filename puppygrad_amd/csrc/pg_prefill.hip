@@ -349,12 +349,13 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 // (its 24 significant bits in three groups of 8, by truncation), W's values are bf16 as they
 // are, so x . w = hi . w + mid . w + lo . w with every product exact in f32 and the sums
 // accumulated in f32 as before.  Three v_mfma_f32_32x32x16_bf16 do per 16 columns what eight
-// v_mfma_f32_32x32x2_f32 of four times the duration did.  An infinity or a NaN in the input
-// stays whole in the first part, so it meets the weights as it would in f32.  One case differs
-// from the f32 product: an infinite WEIGHT meets the zero second and third parts of a value that
-// fits the first (0 * inf), and the sum is NaN where f32 arithmetic gives an infinity.  (Where W
-// is f32 and cut as well, k_gemm_b9, the same happens to an infinite INPUT against a weight
-// whose second or third part is zero.)
+// v_mfma_f32_32x32x2_f32 of four times the duration did.  An infinity in the input stays whole
+// in the first part and a NaN is NaN in all three, so both meet the weights as they would in
+// f32.  One case differs from the f32 product: an infinite bf16 WEIGHT meets the zero second and
+// third parts of a value that fits the first (0 * inf), and the sum is NaN where f32 arithmetic
+// gives an infinity.  (Where W is f32 and cut as well, k_gemm_b9, any infinity would meet zero
+// parts of the other operand: a block that has cut one computes its tile again in plain f32
+// arithmetic, redo_tile, so the result is the f32 product's for infinite inputs and weights.)
 // 256 threads = 4 wavefronts (2 x 2) on a BM x BN tile; k-tiles of 32 columns, staged in LDS
 // row-major ([row][32 bf16] = 64 bytes, the three input planes and W): the operand of a lane
 // is 16 consecutive bytes of its row (8 columns; lanes 32..63 take the second 8 of a 16-column
@@ -373,17 +374,22 @@ __device__ __forceinline__ int lds_piece_turn(int row) { return ((row >> 1) ^ (r
 struct Split3 {
   u2v hi, mid, lo;  // four bf16 each, lowest column in the low half of .x
 };
+// GUARD: an infinity stays whole in the first part (inf - inf would make the other two NaN), so
+// its products and sums behave as in f32 arithmetic; a NaN is NaN in all three parts and in
+// every sum it meets, as in f32 arithmetic, with or without the guard.  k_gemm_b9, which cuts
+// both operands, does so without the guard (two instructions a value in its busiest loop: 13 %
+// of an XL prefill) and instead repeats a tile in plain f32 arithmetic when one of its values
+// was infinite (tile_has_infinity, redo_tile).
+template <bool GUARD = true>
 __device__ __forceinline__ Split3 split3_bf16(f4 x) {
   unsigned h[4], m[4], l[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     h[j] = __float_as_uint(x[j]) & 0xffff0000u;
-    // exact: the 16 low bits of the significand.  An infinity or a NaN stays whole in the first
-    // part (inf - inf would make the other two NaN): its products and sums then behave as in
-    // f32 arithmetic.  (A NaN whose payload lies only in its 16 low bits, which no arithmetic
-    // produces, would read as an infinity.)
-    const bool finite = (__float_as_uint(x[j]) & 0x7f800000u) != 0x7f800000u;
-    const float r1 = finite ? x[j] - __uint_as_float(h[j]) : 0.0f;
+    // exact: the 16 low bits of the significand
+    // (v_cmp_class: bits 2 and 9 of the mask are -inf and +inf)
+    const bool whole = GUARD && __builtin_amdgcn_class(x[j], 0x204);
+    const float r1 = whole ? 0.0f : x[j] - __uint_as_float(h[j]);
     m[j] = __float_as_uint(r1) & 0xffff0000u;
     const float r2 = r1 - __uint_as_float(m[j]);    // exact: at most 8 significant bits left
     l[j] = __float_as_uint(r2);
@@ -396,6 +402,71 @@ __device__ __forceinline__ Split3 split3_bf16(f4 x) {
   r.lo.x = (l[0] >> 16) | (l[1] & 0xffff0000u);
   r.lo.y = (l[2] >> 16) | (l[3] & 0xffff0000u);
   return r;
+}
+
+// Largest magnitude seen so far (a NaN does not count: it becomes NaN in all three parts and
+// in every sum it meets, as in f32 arithmetic).
+__device__ __forceinline__ float abs_max4(float mx, const f4& v) {
+  return fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+}
+// True for every thread of the block when any thread saw an infinity (mx from abs_max4).
+__device__ __forceinline__ bool tile_has_infinity(float mx, int* flag) {
+  if (mx == INFINITY) *flag = 1;  // (*flag was cleared before the block's first barrier)
+  __syncthreads();
+  return *flag != 0;
+}
+// The block's tile once more in plain f32 arithmetic, sums over columns [k0, k1), finished and
+// written out as the kernel's own epilogue would (SPLIT: the raw partial tile of part `part`):
+// where an operand is infinite the cut values give NaN (a zero part times the infinity) and f32
+// arithmetic gives the reference's result.  The thread's outputs are those of the accumulator
+// layout of the 2 x 2 wavefronts of k_gemm_b3 / k_gemm_b9 (wavefront tile at mbase, nbase).
+// WT: W holds f32 (0), bf16 (1) or int8 (2) rows.  It keeps no more than a dozen sums at a time,
+// so that its registers stay below what the kernel's own loop needs; slow, and next to never run.
+template <int MB, int NB, int WT, int EPI, int SPLIT>
+__device__ __forceinline__ void redo_tile(const GemmArgs& a, int mbase, int nbase, int k0, int k1, int part) {
+  const int lane = threadIdx.x & 63, half = lane >> 5, l32 = lane & 31;
+  auto w_at = [&](int n, int k) -> float {
+    const size_t at = (size_t)n * a.K + k;
+    if (WT == 1) return __uint_as_float((unsigned)reinterpret_cast<const unsigned short*>(a.W)[at] << 16);
+    if (WT == 2) return (float)reinterpret_cast<const signed char*>(a.W)[at];
+    return a.W[at];
+  };
+  for (int i = 0; i < MB; ++i)
+    for (int g = 0; g < 4; ++g) {  // four consecutive rows at a time
+      const int mrow = mbase + 32 * i + 8 * g + 4 * half;
+      float sum[4][NB];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) sum[r][j] = 0.0f;
+      for (int k = k0; k < k1; ++k) {
+        float wv[NB], av[4];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) wv[j] = w_at(min(nbase + 32 * j + l32, a.N - 1), k);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) av[r] = a.A[(size_t)min(mrow + r, a.M - 1) * a.lda + k];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int j = 0; j < NB; ++j) sum[r][j] = fmaf(av[r], wv[j], sum[r][j]);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          const int m = mrow + r, n = nbase + 32 * j + l32;
+          if (m >= a.M || n >= a.N) continue;
+          float c = WT == 2 ? a.w_scale[n] * sum[r][j] : sum[r][j];
+          if (SPLIT) {
+            a.ws[((size_t)part * a.M + m) * a.N + n] = c;
+            continue;
+          }
+          c = (a.bias ? a.bias[n] : 0.0f) + c;
+          if (EPI == GEMM_GELU) c = gelu_tanh(c);
+          if (EPI == GEMM_RESID) c = a.resid[(size_t)m * a.ldc + n] + c;
+          a.C[(size_t)m * a.ldc + n] = c;
+        }
+    }
 }
 
 // SPLIT = 1: the k-tiles are cut into gridDim.y parts, the raw partial tiles go to
@@ -647,8 +718,11 @@ __global__ __launch_bounds__(256) void k_gemm_b9(GemmArgs a) {
   constexpr int ALD = BM / 64, BLD = BN / 64;  // float4 loads per thread and tile (4 lanes per row)
   __shared__ u4v As[2][3][BM][2];
   __shared__ u4v Bs[2][3][BN][2];
+  __shared__ int s_infinity;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) s_infinity = 0;
+  float in_max = 0.0f;  // largest |input| and |weight| this thread has cut
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (a.N + BN - 1) / BN;
   const int tiles_all = ((a.M + BM - 1) / BM) * tiles_n;
@@ -701,7 +775,8 @@ __global__ __launch_bounds__(256) void k_gemm_b9(GemmArgs a) {
     for (int i = 0; i < ALD + BLD; ++i) {
       const int row = lr + 64 * (i < ALD ? i : i - ALD);
       const int piece = (lk >> 3) ^ lds_piece_turn2(row);
-      const Split3 sp = split3_bf16(i < ALD ? r.a[i] : r.b[i - ALD]);
+      in_max = abs_max4(in_max, i < ALD ? r.a[i] : r.b[i - ALD]);
+      const Split3 sp = split3_bf16<false>(i < ALD ? r.a[i] : r.b[i - ALD]);
       if (i < ALD) {
         reinterpret_cast<u2v*>(&As[buf][0][row][piece])[h8] = sp.hi;
         reinterpret_cast<u2v*>(&As[buf][1][row][piece])[h8] = sp.mid;
@@ -795,6 +870,11 @@ __global__ __launch_bounds__(256) void k_gemm_b9(GemmArgs a) {
     } else {
       tile_step(no, t, o0, o1, r1);
     }
+  }
+  __syncthreads();  // (also orders the clearing of s_infinity when the block had no k-tile)
+  if (tile_has_infinity(in_max, &s_infinity)) {
+    redo_tile<MB, NB, 0, EPI, SPLIT>(a, m0 + wm * WM, n0 + wn * WN, kt0 * KT, kt1 * KT, (int)blockIdx.y);
+    return;
   }
 
 #pragma unroll
@@ -2208,7 +2288,7 @@ hipError_t launch_gemm_form(const GemmArgs& a, int epi, int num_cus, hipStream_t
   // forms: whole 128 x 128 tiles from 0.75 of a tile per CU on (XL c_fc at 1024 rows 199 ->
   // 176 us, at 4096 rows 818 -> 590 us), tiles cut in four along K between a quarter and
   // 0.56 of a tile per CU (XL second MLP projection at 1024 rows 213 -> 177 us)
-  if (!form && !a.w_bf16 && !a.w_scale && a.M >= 1024 && a.K % 16 == 0) {
+  if (!form && !a.w_bf16 && !a.w_scale && a.M >= a.b9_min_rows && a.M >= 128 && a.K % 16 == 0) {
     const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128);
     if (tiles * 4 > 3L * num_cus) return launch_gemm_b9(a, epi, 1, s, ln_done);
     if (tiles * 4 >= num_cus && tiles * 16 < 9L * num_cus && a.K >= 1024 && a.ws && a.N % 4 == 0 &&

@@ -224,16 +224,19 @@ class Gpt2HipConfig:
     device: int = 0
     weight_storage: int = _lib.PG_STORE_F32
     decode_path: int = _lib.PG_DECODE_AUTO
-    prefill_path: int = 0  # 0: GEMM prefill for prompts of 16+ tokens, 1: token by token
+    prefill_path: int = 0  # 0: GEMM prefill for prompts of seq_gemm_min_tokens and more, 1: token by token
     # tunables (0 = built-in default): what the autotune scan varies and puppygrad-tune.json holds
     attn_item_keys: int = 0
     attn_blocks_per_cu: int = 0
     gemm_split_items_per_cu: int = 0
+    gemm_b9_min_rows: int = 0
+    seq_gemm_min_tokens: int = 0
 
     def to_c(self) -> _lib.pg_hip_options:
         return _lib.pg_hip_options(self.device, self.weight_storage, self.decode_path,
                                    self.prefill_path, self.attn_item_keys, self.attn_blocks_per_cu,
-                                   self.gemm_split_items_per_cu, 0)
+                                   self.gemm_split_items_per_cu, self.gemm_b9_min_rows,
+                                   self.seq_gemm_min_tokens, 0)
 
 
 @dataclass

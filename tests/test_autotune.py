@@ -68,6 +68,8 @@ def test_candidate_grid_is_the_cross_product_in_order():
     assert [(g.attn_item_keys, g.attn_blocks_per_cu, g.gemm_split_items_per_cu) for g in grid] == \
         [(128, 2, 3), (128, 4, 3), (256, 2, 3), (256, 4, 3)]
     assert all(g.weight_storage == 2 for g in grid)
+    grid = candidate_grid(Gpt2HipConfig(), [128], [4], [3], [512, 2048], [2, 16])
+    assert [(g.gemm_b9_min_rows, g.seq_gemm_min_tokens) for g in grid] == [(512, 2), (512, 16), (2048, 2), (2048, 16)]
     with pytest.raises(ValueError, match="no candidates"):
         candidate_grid(Gpt2HipConfig(), [], [4], [3])
 
@@ -82,13 +84,21 @@ def test_saved_tuning_round_trip(tmp_path):
                            "warmup_runs", "measured_runs", "prompt_count", "hip", "measurement"]
     assert saved["backend"] == "hip" and saved["score_name"] == "median_decode_tokens_per_second"
     assert saved["score"] == 2200.5 and saved["search_score"] == 2190.0 and saved["prompt_count"] == 2
-    assert saved["hip"] == {"attn_item_keys": 256, "attn_blocks_per_cu": 8, "gemm_split_items_per_cu": 2}
+    assert saved["hip"] == {"attn_item_keys": 256, "attn_blocks_per_cu": 8, "gemm_split_items_per_cu": 2,
+                            "gemm_b9_min_rows": 0, "seq_gemm_min_tokens": 0}
     assert saved["measurement"]["decode_tokens_per_second_median"] == 2200.5
     # the library's reader: the default file of a model directory, and an explicit file
     got = load_gpt2_tuning(None, tmp_path / "m")
     assert (got.attn_item_keys, got.attn_blocks_per_cu, got.gemm_split_items_per_cu) == (256, 8, 2)
     got = load_gpt2_tuning(path, None, Gpt2HipConfig(attn_blocks_per_cu=6, weight_storage=1))
     assert (got.attn_item_keys, got.attn_blocks_per_cu, got.weight_storage) == (256, 6, 1)  # explicit wins
+    # the planner's knobs and the score they were ranked by
+    best = Gpt2HipConfig(gemm_b9_min_rows=512, seq_gemm_min_tokens=8)
+    save_gpt2_tuning(tmp_path / "p.json", best, 1.0, 2.0, meas, 8, AutoTuneOptions(1, 5, None), "small", "total")
+    saved = json.loads((tmp_path / "p.json").read_text())
+    assert saved["score_name"] == "median_total_tokens_per_second"
+    got = load_gpt2_tuning(tmp_path / "p.json", None)
+    assert (got.gemm_b9_min_rows, got.seq_gemm_min_tokens, got.attn_item_keys) == (512, 8, 0)
     assert load_gpt2_tuning(None, tmp_path) is None  # no default file: nothing to load
     with pytest.raises(FileNotFoundError, match="does not exist"):
         load_gpt2_tuning(tmp_path / "nope.json", None)
@@ -129,7 +139,8 @@ def test_tunables_are_validated_before_any_device_work():
     w = synth.tiny_weights(cfg)
     for kw, msg in [(dict(attn_item_keys=100), "attn_item_keys must be 0 \\(default\\), 128 or 256"),
                     (dict(attn_blocks_per_cu=65), "attn_blocks_per_cu must be at most 64"),
-                    (dict(gemm_split_items_per_cu=17), "gemm_split_items_per_cu must be at most 16")]:
+                    (dict(gemm_split_items_per_cu=17), "gemm_split_items_per_cu must be at most 16"),
+                    (dict(seq_gemm_min_tokens=65537), "seq_gemm_min_tokens must be at most 65536")]:
         with pytest.raises(Gpt2Error, match=msg) as e:
             Gpt2Model.new(cfg, w, Gpt2HipConfig(**kw))
         assert e.value.kind == "InvalidConfig"

@@ -97,14 +97,13 @@ def test_dense_with_selection_weights_returns_the_inputs_bit_for_bit(rows, k, n)
 
 @pytest.mark.parametrize("rows,k,n", [(1024, 1024, 4096), (1024, 4096, 1024), (48, 768, 2304)])
 def test_dense_keeps_infinities_and_nans_of_the_input(rows, k, n):
-    """dot (cpu.rs:231-254) carries an infinite or NaN input into the sums as f32 arithmetic
-    does: +inf times a positive weight is +inf, opposite infinities in one row give NaN, a NaN
-    stays a NaN, and rows without such a value are untouched.  48 rows run on the f32 matrix cores
-    and must show exactly that.  The first two shapes run on the bf16 matrix cores with x AND W
-    cut into three bf16 parts each (whole tiles; tiles cut in four along K): a non-finite input
-    stays whole in its first part, so every affected output is non-finite with the reference's
-    sign where it is an infinity; against a weight whose second or third part is zero (about one
-    f32 weight in 130) the product 0 * inf makes it NaN instead, the one stated difference."""
+    """dot (cpu.rs:231-254) carries an infinite or NaN input or weight into the sums as f32
+    arithmetic does: +inf times a positive weight is +inf, opposite infinities in one row give
+    NaN, inf times a zero weight gives NaN, a NaN stays a NaN, and rows without such a value are
+    untouched.  48 rows run on the f32 matrix cores.  The first two shapes run on the bf16 matrix
+    cores with x AND W cut into three bf16 parts each (whole tiles; tiles cut in four along K),
+    where a zero part times an infinity would be NaN: a tile that has met an infinity is computed
+    again in f32 arithmetic, so the result is the reference's there as well."""
     rng = np.random.default_rng(rows + k)
     x = rng.standard_normal((rows, k)).astype(np.float32)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
@@ -115,22 +114,18 @@ def test_dense_keeps_infinities_and_nans_of_the_input(rows, k, n):
     x[12, 40] = np.nan
     x[rows - 1, k - 3] = np.inf
     w[5, 5] = 0.0              # inf * 0 is NaN in f32 as well
+    w[n - 2, 17] = -np.inf     # an infinite weight: every row's output n - 2, by the sign of x[:, 17]
     got = hip_dense(x.reshape(-1), rows, k, n, w.reshape(-1), b).reshape(rows, n)
     with np.errstate(invalid="ignore"):
         want = oracle.transposed_dense(x.reshape(-1), rows, k, n, w.reshape(-1), b).reshape(rows, n)
-    assert np.isnan(want[3, 5]) and np.isinf(want[3]).sum() == n - 1 and np.isnan(want[12]).all()
+    assert np.isnan(want[3, 5]) and np.isinf(want[3]).sum() >= n - 2 and np.isnan(want[12]).all()
+    assert np.isinf(want[:, n - 2]).sum() >= rows - 6
     fin = np.isfinite(want)
     np.testing.assert_array_equal(np.isfinite(got), fin)
     np.testing.assert_allclose(got[fin], want[fin], atol=3e-5, rtol=1e-5)
-    assert np.isnan(got[np.isnan(want)]).all()
-    if rows < 1024:
-        np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
-        np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
-    else:
-        inf = np.isinf(got)
-        np.testing.assert_array_equal(got[inf], want[inf])         # an infinity has the reference's sign
-        extra = np.isnan(got) & np.isinf(want)
-        assert extra.sum() <= 0.03 * np.isinf(want).sum(), (extra.sum(), np.isinf(want).sum())
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
+    np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
 
 
 def test_dense_reference_unit_vector():

@@ -99,6 +99,27 @@ def test_per_operation_and_batched_paths_with_other_split_plans(blocks, items):
     assert_logits_close(got, want)
 
 
+def test_planner_tunables_move_the_prompt_to_other_kernels_with_the_same_logits():
+    """seq_gemm_min_tokens decides from which prompt length the GEMM prefill runs,
+    gemm_b9_min_rows from which row count f32 products take the bf16 matrix cores: every
+    setting gives the oracle's logits (the nine-product form is exact in its products)."""
+    cfg = Gpt2Config(vocab_size=97, n_positions=512, n_embd=768, n_layer=1, n_head=12)
+    w = synth.random_weights(cfg, 0x5EED0650, perturb=True)
+    ref = oracle.Model(cfg, w, oracle.rust_config(8))
+    ids = [int(t) for t in synth.token_ids(512, 0x70C00650, 97)]
+    want = {n: ref.prefill(ids[:n], ref.new_kv_cache()) for n in (6, 40, 512)}
+    for kw in (dict(), dict(seq_gemm_min_tokens=2), dict(seq_gemm_min_tokens=48),
+               dict(gemm_b9_min_rows=128), dict(gemm_b9_min_rows=0xffffffff)):
+        model = Gpt2Model.new(cfg, w, Gpt2HipConfig(**kw))
+        text = model.describe()
+        assert f"seq_gemm_min_tokens={kw.get('seq_gemm_min_tokens', 4)}" in text
+        assert f"gemm_b9_min_rows={min(kw.get('gemm_b9_min_rows', 1024), 0x7fffffff)}" in text
+        for n, logits in want.items():
+            cache = model.new_kv_cache()
+            assert_logits_close(model.prefill(ids[:n], cache).to_host(), logits)
+            assert cache.seq_len == n
+
+
 def test_model_directory_tuning_file_is_read(tmp_path):
     cfg = Gpt2Config(vocab_size=300, n_positions=64, n_embd=768, n_layer=1, n_head=12)
     w = synth.random_weights(cfg, 0x5EED0630, perturb=True)
@@ -138,3 +159,14 @@ def test_autotune_scan_end_to_end(tmp_path):
     saved = json.loads((tmp_path / "puppygrad-tune.json").read_text())
     assert saved["hip"]["attn_item_keys"] == result.best_config.attn_item_keys
     assert load_gpt2_tuning(tmp_path / "puppygrad-tune.json").attn_item_keys == result.best_config.attn_item_keys
+    # the planner's knobs ranked by the whole generation's rate
+    candidates = candidate_grid(Gpt2HipConfig(), [128], [4], [3], [0, 128], [4, 512])
+    result, validation, score = run_gpt2_autotune(
+        lambda hip: Gpt2Model.new(cfg, w, hip), prompts, 8, candidates,
+        AutoTuneOptions(warmup_runs=1, measured_runs=2, max_trials=8), validation_runs=2,
+        save_path=tmp_path / "planner.json", log=lines.append, eos_token_id=None, score_by="total")
+    assert len(result.trials) == 4 and result.best_score == max(t.score for t in result.trials)
+    assert all(t.score == t.measurement.total_tokens_per_second_median for t in result.trials)
+    saved = json.loads((tmp_path / "planner.json").read_text())
+    assert saved["score_name"] == "median_total_tokens_per_second"
+    assert saved["hip"]["seq_gemm_min_tokens"] == result.best_config.seq_gemm_min_tokens
