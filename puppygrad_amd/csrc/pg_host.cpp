@@ -2170,7 +2170,12 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
           a.slot = c->h_stream_dev + j;
           a.eos = (int)eos;
           const bool forward = selected + j + 1 < N;  // rust.rs:518-528: none after the last token
-          if (forward) {  // (the step arms the exchange words of the forward that follows it)
+          // The first step of a train arms the exchange words of the forward that follows it.
+          // Later forwards find them as the forward before them left them: with an even number
+          // of layers that is what a launch starts from (the set its first layer uses was armed
+          // again during the last layer before it, and the other set is armed by the first
+          // layer before the second uses it, as between two forwards of one launch).
+          if (forward && (j == 0 || (m->cfg.L & 1) != 0)) {
             a.arm = c->xch;
             a.arm_words = c->x_words;
           }
