@@ -144,6 +144,12 @@ struct pg_kv_cache {
   unsigned* xch = nullptr;
   size_t best_words = 0;  // 64-bit words at best_t
   size_t x_words = 0;     // 32-bit words at xch
+  // The exchange words are as a launch expects them: the last persistent launch on this cache
+  // ran to its end and the model has an even number of layers (the set a launch's first layer
+  // uses was then armed again during the last layer before it, and the other set is armed by
+  // the first layer before the second uses it, as between two forwards of one launch), so the
+  // next launch needs no k_arm_exchange in front of it.
+  bool xch_ready = false;
   unsigned xch_set = 0;   // words from one set of exchange vectors to the other
   // [grid][L + 1][16] time stamps of a profiled forward of the persistent kernel (allocated on
   // first use; pg_gpt2_stream_token_ids_profiled)
@@ -493,6 +499,7 @@ thread_local bool t_persistent_in_flight = false;
 struct PersistentRun {
   std::unique_lock<std::mutex> lock;
   bool begun = false;
+  bool rearms = false;  // a launch that runs to its end leaves the exchange words ready
   hipStream_t stream = nullptr;
   // (a caller that leaves early still waits for the kernel before the lock is released)
   ~PersistentRun() {
@@ -587,8 +594,10 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
   }
 #endif
   run->lock = std::unique_lock<std::mutex>(g_persistent_mu);
+  const bool armed = c->xch_ready;
+  c->xch_ready = false;  // until this launch has ended well (persistent_end)
   auto enqueue = [&]() -> pg_status {
-    PG_HIP(pgk::launch_arm_exchange(c->xch, c->x_words, c->status, c->stream));
+    if (!armed) PG_HIP(pgk::launch_arm_exchange(c->xch, c->x_words, c->status, c->stream));
     if (timed) PG_HIP(hipEventRecord(c->ev0, c->stream));
     PG_HIP(pgk::launch_decode_persistent(p, c->stream));
     if (timed) PG_HIP(hipEventRecord(c->ev1, c->stream));
@@ -603,6 +612,7 @@ pg_status persistent_begin(const pg_gpt2_model* m, pg_kv_cache* c, const uint32_
     return s;
   }
   run->begun = true;
+  run->rearms = (g.L & 1) == 0 && n_fwd > 0;
   run->stream = c->stream;
   t_persistent_in_flight = true;
   return PG_OK;
@@ -632,6 +642,7 @@ pg_status persistent_end(pg_kv_cache* c, PersistentRun* run, size_t* done, bool*
                             "(another kernel may be occupying the device)");
   if (done) *done = c->h_status[1];
   if (stopped) *stopped = c->h_status[2] != 0;
+  c->xch_ready = run->rearms && c->h_status[2] == 0;
   return PG_OK;
 }
 
@@ -2138,6 +2149,7 @@ static pg_status stream_core(const pg_gpt2_model* m, const uint32_t* ids, size_t
                     "a token callback must not call the model while its generation is running");
       PersistentRun run;
       run.lock = std::unique_lock<std::mutex>(g_persistent_mu);
+      c->xch_ready = false;  // (the train arms for itself; what it leaves is not relied on)
       size_t forwards = 0;  // forwards enqueued
       auto enqueue = [&]() -> pg_status {
         PG_HIP(pgk::launch_arm_exchange(c->xch, 0, c->status, c->stream));  // clears the status
