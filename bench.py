@@ -287,7 +287,8 @@ def secondary_workloads(xl_cfg, xl_weights):
     # GPT-2 XL with bf16-stored weights: batch-32 decode steps around the mean cache length of
     # configuration 5 (512-token prompts + 512 tokens: 513..1023 keys, mean 768)
     model = Gpt2Model.new(xl_cfg, xl_weights, Gpt2HipConfig(weight_storage=_lib.PG_STORE_BF16))
-    out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 752, 24, True)
+    out["gpt2_xl_bf16_decode_b32"] = measure_batch_decode(model, xl_cfg, 32, 752, 24, True,
+                                                          traffic_ratio=TRAFFIC_RATIO_XL_BF16_B32)
     out["gpt2_xl_bf16_prefill_b32_512"] = measure_batch_prefill_bf16(model, xl_cfg, 32, 512, 3)
     del model
     return out
@@ -563,6 +564,7 @@ TRAFFIC_SOURCE = "profiles/k_decode_persistent_1600_xl_decode_traffic.txt"
 TRAFFIC_RATIO_124M = 0.983
 TRAFFIC_SOURCE_124M = "profiles/k_decode_persistent_768_124m_decode.txt"
 TRAFFIC_RATIO_355M_B16 = 1.093
+TRAFFIC_RATIO_XL_BF16_B32 = 1.073  # same file, section (c)
 TRAFFIC_SOURCE_355M_B16 = "profiles/batched_decode_355m_b16_xl_bf16_b32.txt"
 
 
