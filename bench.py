@@ -339,6 +339,8 @@ def measure_short_prefill(model, cfg, ids, T, steps, warmup):
             "value": round(T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 4),
             "roofline": hbm_roofline(wbytes / sec / 1e9,
                                      "whole prefill (k_gemm_rows32, k_attn_prefill64, k_splitk_reduce_ln, lm_head)",
+                                     traffic=TRAFFIC_124M_PREFILL_32 if T == 32 else None,
+                                     traffic_source=TRAFFIC_SOURCE_124M_PREFILL if T == 32 else None,
                                      algorithmic_bytes_per_step=int(wbytes))}
 
 
@@ -366,7 +368,9 @@ def measure_prefill(model, cfg, ids, T, steps, warmup):
     return {"workload": f"GPT-2 124M fp32 B=1 prefill of {T} tokens into an empty KV cache, final-position logits",
             "value": round(T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 4),
             "roofline": {"bound": "mfma", "achieved": round(whole, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(whole / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                         "unit": "TFLOP/s", "frac": round(whole / FP32_MFMA_PEAK_TFLOPS, 4),
+                         "traffic": TRAFFIC_124M_PREFILL_1024 if T == 1024 else None,
+                         "traffic_source": TRAFFIC_SOURCE_124M_PREFILL if T == 1024 else None,
                          "kernel": "whole prefill (k_gemm, k_attn_prefill64, LayerNorm, split-K reduces, lm_head)",
                          "algorithmic_flops_per_step": int(flops)},
             "gemm_part": {"ms": round(gemm_s * 1e3, 4), "achieved": round(gemm, 2), "unit": "TFLOP/s",
@@ -563,6 +567,10 @@ TRAFFIC_SOURCE = "profiles/k_decode_persistent_1600_xl_decode_traffic.txt"
 # with --model small and with --workload batch-decode.
 TRAFFIC_RATIO_124M = 0.983
 TRAFFIC_SOURCE_124M = "profiles/k_decode_persistent_768_124m_decode.txt"
+# HBM bytes of one 124M prefill (FETCH_SIZE + WRITE_SIZE of all its launches, scaled)
+TRAFFIC_124M_PREFILL_1024 = 3208200000
+TRAFFIC_124M_PREFILL_32 = 631400000
+TRAFFIC_SOURCE_124M_PREFILL = "profiles/prefill_124m_traffic.txt"
 TRAFFIC_RATIO_355M_B16 = 1.093
 TRAFFIC_RATIO_XL_BF16_B32 = 1.073  # same file, section (c)
 TRAFFIC_SOURCE_355M_B16 = "profiles/batched_decode_355m_b16_xl_bf16_b32.txt"
