@@ -287,6 +287,13 @@ __global__ void k_embed(float* x, const float* wte, const float* wpe, const uint
   if (i < C) x[i] = wte_at(wte, w_bf16, (size_t)t * C + i) + wpe[(size_t)pos * C + i];
 }
 
+// A K or V row is read once per step: a load that leaves no line behind in the caches.
+__device__ __forceinline__ float4 nt_load4(const float4* p) {
+  typedef float f4v __attribute__((ext_vector_type(4)));
+  const f4v v = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+
 // cached_self_attention_into (rust.rs:1721-1740) for head_dim 64, keys split
 // over blockIdx.x.  Sixteen lanes score one key (a float4 each); a wavefront takes
 // 4 keys per step and IT steps per chunk, and requests the K and the V rows of a whole
@@ -363,9 +370,9 @@ __global__ __launch_bounds__(kBlock) void k_attn_decode64(const float* __restric
     const int kfirst = c0 + wave * 4 + sub;
     // a key past the split re-reads the split's last row and is masked below
 #pragma unroll
-    for (int i = 0; i < IT; ++i) kr[i] = K4[(size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4];
+    for (int i = 0; i < IT; ++i) kr[i] = nt_load4(K4 + (size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4);
 #pragma unroll
-    for (int i = 0; i < IT; ++i) vr[i] = V4[(size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4];
+    for (int i = 0; i < IT; ++i) vr[i] = nt_load4(V4 + (size_t)min(kfirst + kGroups * i, k1 - 1) * 16 + d4);
     float sc[IT];
     float cm = -INFINITY;
 #pragma unroll
