@@ -419,16 +419,19 @@ def prefill_flops(cfg, B, T):
     return gemm_flops + attn_flops + 2.0 * B * V * C_, gemm_flops
 
 
-def bf16_prefill_roofline(flops, gemm_flops, sec):
+def bf16_prefill_roofline(flops, gemm_flops, sec, traffic=None, traffic_source=None):
     """bf16 rows: the projections run on the bf16 matrix cores, every f32 input cut into three
     bf16 parts (exact products, f32 sums): three matrix instructions' worth of work per
     algorithmic product, so a third of the bf16 peak is this form's ceiling."""
     achieved = flops / sec / 1e12
-    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4), "traffic": None, "passes": 3,
-            "executed": round((2 * gemm_flops + flops) / sec / 1e12, 2),
-            "kernel": "whole prefill (k_gemm_b3 on the bf16 matrix cores, k_attn_prefill64 and lm_head in f32)",
-            "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)}
+    r = {"bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+         "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4), "traffic": traffic, "passes": 3,
+         "executed": round((2 * gemm_flops + flops) / sec / 1e12, 2),
+         "kernel": "whole prefill (k_gemm_b3 on the bf16 matrix cores, k_attn_prefill64 and lm_head in f32)",
+         "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)}
+    if traffic_source:
+        r["traffic_source"] = traffic_source
+    return r
 
 
 def measure_batch_prefill_bf16(model, cfg, B, T, steps):
@@ -446,7 +449,10 @@ def measure_batch_prefill_bf16(model, cfg, B, T, steps):
     return {"workload": f"GPT-2 n_embd={cfg.n_embd} B={B} prefill of {T} tokens each into empty KV caches, "
                         f"weights stored as bf16, f32 inputs and sums",
             "value": round(B * T / sec, 1), "unit": "tokens/s", "steps": steps, "ms_per_step": round(sec * 1e3, 3),
-            "roofline": bf16_prefill_roofline(flops, gemm_flops, sec)}
+            "roofline": bf16_prefill_roofline(
+                flops, gemm_flops, sec,
+                traffic=TRAFFIC_XL_BF16_PREFILL_B32_512 if (cfg.n_embd, B, T) == (1600, 32, 512) else None,
+                traffic_source=TRAFFIC_SOURCE_XL_BF16_PREFILL if (cfg.n_embd, B, T) == (1600, 32, 512) else None)}
 
 
 def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
@@ -497,7 +503,10 @@ def bench_prefill(args, cfg, model, ids, n_prefill) -> int:
                      "algorithmic_flops_per_step": int(flops), "gemm_flops_per_step": int(gemm_flops)},
     }
     if args.bf16:
-        result["roofline"] = bf16_prefill_roofline(flops, gemm_flops, sec)
+        counted = (cfg.n_embd, B, T) == (1600, 32, 512)
+        result["roofline"] = bf16_prefill_roofline(
+            flops, gemm_flops, sec, traffic=TRAFFIC_XL_BF16_PREFILL_B32_512 if counted else None,
+            traffic_source=TRAFFIC_SOURCE_XL_BF16_PREFILL if counted else None)
     # A short prompt reads every weight once for few rows: below about 52 rows the weights'
     # bytes at the HBM peak take longer than the flops at the MFMA peak, and HBM is the bound.
     wbytes = weight_bytes(cfg, bf16=args.bf16)
@@ -574,6 +583,11 @@ TRAFFIC_SOURCE_124M_PREFILL = "profiles/prefill_124m_traffic.txt"
 TRAFFIC_RATIO_355M_B16 = 1.093
 TRAFFIC_RATIO_XL_BF16_B32 = 1.073  # same file, section (c)
 TRAFFIC_SOURCE_355M_B16 = "profiles/batched_decode_355m_b16_xl_bf16_b32.txt"
+# Bytes through the L2s to and from the fabric per XL bf16 prefill of 32 x 512 tokens (FETCH_SIZE
+# scaled by 1.9994 + WRITE_SIZE over all launches of a step; most of the reads are operand
+# re-reads that the Infinity Cache serves).
+TRAFFIC_XL_BF16_PREFILL_B32_512 = 573030000000
+TRAFFIC_SOURCE_XL_BF16_PREFILL = "profiles/k_gemm_b3_xl_bf16_prefill_b32_512.txt"
 
 
 def measured_traffic(args, n_prefill, persistent, bytes_per_launch):
