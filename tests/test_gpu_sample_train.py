@@ -54,8 +54,8 @@ def replay(model, ids, g):
     return out, generated
 
 
-def small_persistent(width=768, vocab=2003, positions=256, seed=0x5EED0900, std=0.1):
-    cfg = Gpt2Config(vocab_size=vocab, n_positions=positions, n_embd=width, n_layer=2,
+def small_persistent(width=768, vocab=2003, positions=256, seed=0x5EED0900, std=0.1, layers=2):
+    cfg = Gpt2Config(vocab_size=vocab, n_positions=positions, n_embd=width, n_layer=layers,
                      n_head=width // 64)
     w = synth.random_weights(cfg, seed + width, std=std, perturb=True)
     return cfg, w
@@ -98,6 +98,23 @@ def test_sampled_streams_in_trains_pick_the_oracles_ids(width):
         with step_by_step():
             again, _ = model.stream_token_ids_with_stats(ids, g)
         assert again == want, kw
+
+
+def test_trains_of_a_model_with_an_odd_number_of_layers():
+    """With an odd number of layers a forward leaves the other set of exchange words armed than
+    the next one starts from, so every step of a train arms for its forward; with an even number
+    only the first does.  Both must give the oracle's ids, also right after a greedy launch."""
+    cfg, w = small_persistent(768, layers=3, seed=0x5EED0930)
+    model = Gpt2Model.new(cfg, w)
+    assert "decode=persistent" in model.describe()
+    ids = [int(t) for t in synth.token_ids(11, 0x70C00930, cfg.vocab_size)]
+    for i, kw in enumerate((SAMPLINGS[2], SAMPLINGS[1], SAMPLINGS[5])):
+        g = TextGenerationConfig(40, seed=300 + i, **kw)
+        want, want_generated = replay(model, ids, g)
+        # a greedy stream in between: its launch ends with the exchange words in the other state
+        model.stream_token_ids_with_stats(ids, TextGenerationConfig(5, seed=1, temperature=0.0))
+        got, stats = model.stream_token_ids_with_stats(ids, g)
+        assert got == want and stats.generated_tokens == want_generated == 40, kw
 
 
 def test_train_stops_at_eos_at_the_context_limit_and_for_the_callback():
