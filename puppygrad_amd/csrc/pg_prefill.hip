@@ -1124,7 +1124,7 @@ __global__ __launch_bounds__(256) void k_gemv_rows(GemmArgs a) {
 
 // ---------------------------------------------------------------------------
 // A batch of at most 32 rows (64 with MT = 2) against W on the matrix cores.  A block owns 32 rows of W;
-// its eight wavefronts cut the block's K range into eight pieces.  MFMA 32x32x2 wants lane
+// its eight wavefronts take the steps of the block's K range in turn.  MFMA 32x32x2 wants lane
 // (l, half) to hold columns of row l, but a load in that form touches 64 separate 64-byte
 // pieces of memory and the address path of the CU, not HBM, then sets the pace.  So a
 // wavefront loads 64 bytes of each of the 32 rows per step with four lanes to a row (16
@@ -1172,7 +1172,10 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
   const int n0 = (int)blockIdx.x * a.rows_per_block, n1 = min(n0 + a.rows_per_block, a.N);
   const int steps = a.K / KS;
   const int piece = (int)blockIdx.y * 8 + wave, pieces = (int)gridDim.y * 8;
-  const int s0 = (int)(((long)piece * steps) / pieces), s1 = (int)(((long)(piece + 1) * steps) / pieces);
+  // the wavefront's steps are piece, piece + pieces, ...: at any time the wavefronts of a block
+  // (and of the blocks that share its rows of W) read neighbouring 64-byte pieces of a row, whole
+  // cache lines and DRAM pages between them (contiguous K ranges per wavefront: 1.6 % slower steps)
+  const int s0 = 0, s1 = piece < steps ? (steps - piece + pieces - 1) / pieces : 0;
   float* wt = slab[wave];
   float* xt = slab[wave] + 32 * WSTR;
 
@@ -1226,7 +1229,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows32(GemmArgs a) {
 
   f4 rw[PD][2], rx[PD][XR];
   auto load_step = [&](int s, f4* w, f4* x) {
-    const size_t sc = (size_t)min(s, s1 - 1);
+    const size_t sc = (size_t)piece + (size_t)pieces * min(s, s1 - 1);  // local step -> step of the row
     w[0] = *reinterpret_cast<const f4*>(wpa + sc * 64);
     if (NR == 32) w[1] = *reinterpret_cast<const f4*>(wpb + sc * 64);
 #pragma unroll
