@@ -540,25 +540,33 @@ __global__ __launch_bounds__(kTopkStepThreads) void k_topk_step(SampleStep a) {
   unsigned n = 0;
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
-    if (!is_finite(v[r]) || r * TB + tid >= a.V) v[r] = NAN;  // NaN: not a candidate
-    if (v[r] == v[r]) {
-      lm = fmaxf(lm, v[r]);
-      ++n;
-    }
+    bool cand = is_finite(v[r]);
+    if (r * TB + TB > a.V) cand = cand && r * TB + tid < a.V;  // (block-uniform: the last ids)
+    v[r] = cand ? v[r] : NAN;  // NaN: not a candidate
+    lm = fmaxf(lm, v[r]);      // (the maximum of a number and a NaN is the number)
+    n += cand ? 1u : 0u;
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off, 64);
-  // the m-th largest of the wavefront's lane maxima (-inf when fewer lanes hold a candidate)
+  // the m-th largest of the wavefront's lane maxima, equal ones counted each (-inf when fewer
+  // than m lanes hold a candidate): bit by bit from the top of the order key, a bit stays set
+  // when at least m maxima reach the key built so far with that bit set (32 ballots on the
+  // scalar side, where m rounds of a wavefront-wide maximum took m x 6 lane exchanges)
   const int m = (a.top_k + NW - 1) / NW;
   float bound = -INFINITY;
-  for (int j = 0; j < m; ++j) {
-    float wmax = lm;
+  {
+    const unsigned key = order_key(lm);
+    if (__popcll(__ballot(key > order_key(-INFINITY))) >= m) {
+      unsigned prefix = 0;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, off, 64));
-    bound = wmax;
-    if (!(wmax > -INFINITY)) break;
-    const unsigned long long holders = __ballot(lm == wmax);
-    if (lane == __builtin_ctzll(holders)) lm = -INFINITY;
+      for (int bit = 31; bit >= 0; --bit) {
+        const unsigned trial = prefix | (1u << bit);
+        if (__popcll(__ballot(key >= trial)) >= m) prefix = trial;
+      }
+      unsigned bits = prefix ^ 0x80000000u;  // undo order_key
+      bits ^= (unsigned)(((int)bits >> 31)) >> 1;
+      bound = __uint_as_float(bits);
+    }
   }
   if (lane == 0) {
     sm.wave_f[0][wave] = bound;
